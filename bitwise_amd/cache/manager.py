@@ -1,0 +1,153 @@
+"""The cache manager: for every request a block table per cache group and a state slot.
+
+A *group* is a set of caches (one per layer call that writes one) with the same needs: all
+keys, or a window of them.  Every group has a page pool of its own.  A request's pages are
+given back when it ends, is preempted or cancelled, and, in a windowed group, as soon as the
+window has passed them; cached full pages of a finished request stay until the space is
+needed (reference: src/engine.cpp:146-220, src/block_manager.cpp).
+
+Prefix reuse (src/engine.cpp:176-205) is only sound when the reused pages hold everything
+the request has computed: it is on for models with one group that keeps all keys and no
+per-request state outside the pages, and switched off otherwise.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+from .pages import PagePool, StateSlots, block_hash
+
+
+@dataclass(frozen=True)
+class GroupSpec:
+    window: Optional[int] = None       # None: all keys stay
+
+
+@dataclass
+class RequestCache:
+    slot: int
+    tables: List[List[int]]            # per group: page of positions [i*page, (i+1)*page); -1 once given back
+    hashes: List[int] = field(default_factory=list)   # hash chain of this request's registered full pages
+    computed: int = 0                  # tokens whose keys and values are in the cache
+
+
+class CacheManager:
+    def __init__(self, groups: Sequence[GroupSpec], num_pages: int, page_size: int, num_slots: int,
+                 prefix_caching: bool = True, has_state: bool = False):
+        self.groups = list(groups)
+        self.page_size = page_size
+        self.num_pages = num_pages
+        self.prefix_caching = (bool(prefix_caching) and not has_state and len(self.groups) == 1
+                               and self.groups[0].window is None)
+        self.pools = [PagePool(num_pages, page_size, self.prefix_caching) for _ in self.groups]
+        self.slots = StateSlots(num_slots)
+
+    # ------------------------------------------------------------------ requests
+    def open(self) -> Optional[RequestCache]:
+        slot = self.slots.allocate()
+        if slot is None:
+            return None
+        return RequestCache(slot=slot, tables=[[] for _ in self.groups])
+
+    def close(self, rc: RequestCache) -> None:
+        """Give back every page and the slot."""
+        self.release_pages(rc)
+        self.slots.release(rc.slot)
+        rc.slot = -1
+
+    def release_pages(self, rc: RequestCache) -> None:
+        for pool, table in zip(self.pools, rc.tables):
+            for page in table:
+                if page >= 0:
+                    pool.release(page)
+            table.clear()
+        rc.hashes.clear()
+        rc.computed = 0
+
+    # ------------------------------------------------------------------ prefix reuse
+    def admit_prefix(self, rc: RequestCache, tokens: Sequence[int]) -> int:
+        """Take cached pages holding a prefix of ``tokens``.  The page holding the last token
+        is never reused, so that its logits are computed (src/engine.cpp:178-179)."""
+        if not self.prefix_caching or rc.tables[0]:
+            return rc.computed
+        ps = self.page_size
+        full = (len(tokens) - 1) // ps
+        parent = 0
+        pool = self.pools[0]
+        for i in range(full):
+            toks = tokens[i * ps:(i + 1) * ps]
+            h = block_hash(parent, toks)
+            page = pool.lookup(h, toks)
+            if page is None:
+                break
+            rc.tables[0].append(page)
+            rc.hashes.append(h)
+            parent = h
+        rc.computed = len(rc.tables[0]) * ps
+        return rc.computed
+
+    # ------------------------------------------------------------------ growth
+    def first_needed_page(self, group: int, next_position: int) -> int:
+        """Index of the first page a query at ``next_position`` still reads in this group."""
+        w = self.groups[group].window
+        if w is None:
+            return 0
+        return max(0, next_position - w + 1) // self.page_size
+
+    def ensure(self, rc: RequestCache, tokens: int) -> bool:
+        """Make the request's tables cover positions [computed, tokens).  False if a pool ran
+        out; pages taken so far stay with the request (the caller preempts or releases)."""
+        need = (tokens + self.page_size - 1) // self.page_size
+        for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
+            lo = self.first_needed_page(g, rc.computed)
+            while len(table) < need:
+                if len(table) < lo:
+                    table.append(-1)             # wholly before the window: never allocated
+                    continue
+                page = pool.allocate()
+                if page is None:
+                    return False
+                table.append(page)
+        return True
+
+    def pages_missing(self, rc: RequestCache, tokens: int) -> int:
+        """Most pages any pool would have to hand out for ``ensure(rc, tokens)``."""
+        need = (tokens + self.page_size - 1) // self.page_size
+        return max((max(0, need - len(t)) for t in rc.tables), default=0)
+
+    def advance(self, rc: RequestCache, tokens: Sequence[int], computed: int) -> None:
+        """After a step: ``computed`` tokens are in the cache.  Register newly full pages
+        (src/engine.cpp:196-205) and give back pages a window has passed."""
+        rc.computed = computed
+        ps = self.page_size
+        if self.prefix_caching:
+            pool, table = self.pools[0], rc.tables[0]
+            for i in range(len(rc.hashes), computed // ps):
+                toks = tokens[i * ps:(i + 1) * ps]
+                h = block_hash(rc.hashes[i - 1] if i else 0, toks)
+                pool.register_full(table[i], h, toks)
+                rc.hashes.append(h)
+        for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
+            if self.groups[g].window is None:
+                continue
+            lo = min(self.first_needed_page(g, computed), len(table))
+            for i in range(lo):
+                if table[i] >= 0:
+                    pool.release(table[i])
+                    table[i] = -1
+
+    # ------------------------------------------------------------------ accounting
+    def free_pages(self, group: int = 0) -> int:
+        return self.pools[group].available()
+
+    def all_free(self) -> bool:
+        return all(p.available() == p.num_pages for p in self.pools) and self.slots.available() == self.slots.num_slots
+
+    @property
+    def evictions(self) -> int:
+        return sum(p.evictions for p in self.pools)
+
+    def check(self) -> None:
+        for p in self.pools:
+            p.check()

@@ -1,0 +1,40 @@
+"""Engine-side option structs, with the reference's field names and meanings.
+
+SamplingParams: src/engine.h:26-31.  EngineConfig: src/engine.h:38-50, less the fields of
+speculative decoding, static batching and kernel-mode comparison, plus the choices the
+reference fixes at compile time (block_size, src/block_manager.h:20) or does not have
+(dtype, max_model_len).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass
+class SamplingParams:
+    temperature: float = 0.0   # <= 0 means greedy (src/engine.cpp:469)
+    seed: int = 0              # key of the counter-based generator
+    max_new_tokens: int = 32
+    ignore_eos: bool = False
+
+
+@dataclass
+class EngineConfig:
+    num_blocks: int = 512            # pages in every cache group's pool
+    max_batched_tokens: int = 256    # token budget of one step
+    max_num_seqs: int = 32           # running requests at a time
+    prefix_caching: bool = True
+    fingerprint_logits: bool = True
+    block_size: int = 16             # tokens in a page
+    dtype: str = "bfloat16"          # "bfloat16" (serving precision) or "float32" (true 32-bit)
+    max_model_len: int = 0           # 0: the model's max_position_embeddings
+    use_graphs: bool = True          # replay pure-decode steps from captured HIP graphs
+
+    def validate(self) -> None:
+        if self.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
+        if self.block_size not in (8, 16, 32, 64):
+            raise ValueError(f"block_size must be 8, 16, 32 or 64, got {self.block_size}")
+        if self.num_blocks < 1 or self.max_batched_tokens < 1 or self.max_num_seqs < 1:
+            raise ValueError("num_blocks, max_batched_tokens and max_num_seqs must be positive")

@@ -1,0 +1,37 @@
+// C entry points of the kernel library.  Every function launches on the given stream and
+// returns 0, a HIP error code (> 0), or a negative code for arguments it refuses:
+//   -2 sizes or strides out of range, -3 misaligned pointer or stride,
+//   -4 head size not compiled in, -5 page size not supported.
+// All pointers are device pointers.  Nothing here allocates.
+#pragma once
+#include <stdint.h>
+
+extern "C" {
+int bw_embed(const int32_t* tokens, const void* table, int table_is_bf16, float* out, int rows, int width,
+             int vocab, void* stream);
+int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16, int rows,
+               int dim, int ldy, float eps, void* stream);
+int bw_add(float* x, const float* y, long long n, void* stream);
+int bw_swiglu_f32(const float* gate_up, float* h, int rows, int inter, void* stream);
+int bw_gather_rows_f32(const float* x, const int32_t* idx, float* out, int count, int width, int ldx, void* stream);
+int bw_rope_kvwrite(float* qkv, void* q_out, const int32_t* positions, const int32_t* row_seq,
+                    const int32_t* block_table, int table_stride, const float* cos_table, const float* sin_table,
+                    void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads, int head_dim,
+                    int page_size, int write_cache, void* stream);
+int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, int N, int K, int ldx, int ldy,
+                int accumulate, void* stream);
+int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, int epilogue,
+                 void* stream);
+int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
+                     const int32_t* block_table, int table_stride, const float* k_cache, const float* v_cache,
+                     float* out, int out_stride, int rows, int heads, int kv_heads, int head_dim, int page_size,
+                     int window, float scale, void* stream);
+int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
+                      int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
+                      const void* v_cache, void* out, int out_stride, int heads, int kv_heads, int head_dim,
+                      int page_size, int window, float scale, int split, int max_parts, float* part_o,
+                      float* part_ml, void* stream);
+int bw_sample(const float* logits, int vocab, int ld, int rows, const float* temperature, const double* uniform,
+              int32_t* out, void* stream);
+int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out, void* stream);
+}

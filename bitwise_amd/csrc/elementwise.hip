@@ -1,0 +1,277 @@
+// Row-wise kernels around the matrix products: embedding gather, RMSNorm, rotary
+// position encoding fused with the cache write, SwiGLU, residual add, row gather.
+//
+// 32-bit variants follow the reference's operation order exactly
+// (src/kernels.cpp:57-103, :264-298; src/model.cpp:285-297); the bfloat16 variants keep
+// sums of squares, rotation and the residual in 32-bit and round once when they store.
+#include "common.h"
+#include "api.h"
+
+// ------------------------------------------------------------------------- embedding
+
+template <typename TableT>
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const TableT* __restrict__ table,
+                             float* __restrict__ out, int width, int vocab) {
+  const int row = blockIdx.x;
+  const int tok = tokens[row];
+  float* o = out + (size_t)row * width;
+  if (tok < 0 || tok >= vocab) {  // padding rows of a fixed-size batch carry token -1
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = 0.0f;
+    return;
+  }
+  const TableT* e = table + (size_t)tok * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    if constexpr (sizeof(TableT) == 2) o[i] = bf16_to_f32(e[i]);
+    else o[i] = e[i];
+  }
+}
+
+extern "C" int bw_embed(const int32_t* tokens, const void* table, int table_is_bf16, float* out, int rows,
+                        int width, int vocab, void* stream) {
+  if (rows <= 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (table_is_bf16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, tokens, (const bf16_t*)table, out, width, vocab);
+  else
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(rows), dim3(256), 0, s, tokens, (const float*)table, out, width, vocab);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------- RMSNorm, 32-bit
+
+// 16 lanes per row: lane j runs the fused multiply-add chain over i = j, j+16, ... and the
+// lanes are joined by the tree (v[i]+v[i+8]), (+4), (s4[0]+s4[2])+(s4[1]+s4[3])
+// (src/kernels.cpp:57-64, :86-101).  Then inv = 1/sqrt(ss/dim + eps), y = (x*inv)*w
+// (src/kernels.cpp:264-271).
+template <typename WT>
+__global__ void rmsnorm_f32_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                   float* __restrict__ y, int rows, int dim, float eps) {
+  const int sub = threadIdx.x & 15;
+  const int row = blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  const bool live = row < rows;
+  const float* xr = x + (size_t)(live ? row : 0) * dim;
+  float acc = 0.0f;
+  if (live)
+    for (int i = sub; i < dim; i += 16) acc = fmaf(xr[i], xr[i], acc);
+  acc += __shfl_xor(acc, 8, 16);
+  acc += __shfl_xor(acc, 4, 16);
+  acc += __shfl_xor(acc, 2, 16);
+  acc += __shfl_xor(acc, 1, 16);
+  if (!live) return;
+  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+  float* yr = y + (size_t)row * dim;
+  for (int i = sub; i < dim; i += 16) {
+    float wi;
+    if constexpr (sizeof(WT) == 2) wi = bf16_to_f32(w[i]);
+    else wi = w[i];
+    yr[i] = (xr[i] * inv) * wi;
+  }
+}
+
+// ------------------------------------------------------------------------- RMSNorm, bfloat16 out
+
+// One wave per row; lane l sums x[i]^2 over i = l, l+64, ... by fused multiply-adds, the
+// lanes are joined by xor butterflies (32, 16, ..., 1).  All in 32-bit; one rounding at the
+// store.  A row's result depends on that row alone.
+template <typename WT>
+__global__ void rmsnorm_bf16_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                    bf16_t* __restrict__ y, int rows, int dim, int ldy, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* xr = x + (size_t)row * dim;
+  float acc = 0.0f;
+  for (int i = lane; i < dim; i += 64) acc = fmaf(xr[i], xr[i], acc);
+  acc = wave_sum(acc);
+  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+  bf16_t* yr = y + (size_t)row * ldy;
+  for (int i = lane; i < dim; i += 64) {
+    float wi;
+    if constexpr (sizeof(WT) == 2) wi = bf16_to_f32(w[i]);
+    else wi = w[i];
+    yr[i] = f32_to_bf16((xr[i] * inv) * wi);
+  }
+}
+
+extern "C" int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16,
+                          int rows, int dim, int ldy, float eps, void* stream) {
+  if (rows <= 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_is_bf16) {
+    dim3 grid((rows + 3) / 4), block(256);
+    if (weight_is_bf16)
+      hipLaunchKernelGGL(rmsnorm_bf16_kernel<bf16_t>, grid, block, 0, s, x, (const bf16_t*)weight, (bf16_t*)y, rows, dim, ldy, eps);
+    else
+      hipLaunchKernelGGL(rmsnorm_bf16_kernel<float>, grid, block, 0, s, x, (const float*)weight, (bf16_t*)y, rows, dim, ldy, eps);
+  } else {
+    if (ldy != dim) return -2;
+    dim3 grid((rows + 15) / 16), block(256);
+    if (weight_is_bf16)
+      hipLaunchKernelGGL(rmsnorm_f32_kernel<bf16_t>, grid, block, 0, s, x, (const bf16_t*)weight, (float*)y, rows, dim, eps);
+    else
+      hipLaunchKernelGGL(rmsnorm_f32_kernel<float>, grid, block, 0, s, x, (const float*)weight, (float*)y, rows, dim, eps);
+  }
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------- small row ops
+
+__global__ void add_kernel(float* __restrict__ x, const float* __restrict__ y, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] += y[i];
+}
+
+extern "C" int bw_add(float* x, const float* y, long long n, void* stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, y, (size_t)n);
+  return BW_LAUNCH_CHECK();
+}
+
+// h = g * (1/(1+exp(-g))) * u over rows laid out [gate | up] (src/kernels.cpp:291-298).
+__global__ void swiglu_f32_kernel(const float* __restrict__ gate_up, float* __restrict__ h, int rows, int inter) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)rows * inter) return;
+  const int r = (int)(i / inter), c = (int)(i % inter);
+  const float g = gate_up[(size_t)r * 2 * inter + c];
+  const float u = gate_up[(size_t)r * 2 * inter + inter + c];
+  h[i] = g * (1.0f / (1.0f + expf(-g))) * u;
+}
+
+extern "C" int bw_swiglu_f32(const float* gate_up, float* h, int rows, int inter, void* stream) {
+  if (rows <= 0) return 0;
+  size_t n = (size_t)rows * inter;
+  hipLaunchKernelGGL(swiglu_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, gate_up, h, rows, inter);
+  return BW_LAUNCH_CHECK();
+}
+
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ x, const int32_t* __restrict__ idx, T* __restrict__ out,
+                                   int width, int ldx) {
+  const T* src = x + (size_t)idx[blockIdx.x] * ldx;
+  T* dst = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int bw_gather_rows_f32(const float* x, const int32_t* idx, float* out, int count, int width, int ldx,
+                                  void* stream) {
+  if (count <= 0) return 0;
+  hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(count), dim3(256), 0, (hipStream_t)stream, x, idx, out, width, ldx);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------- rotary + cache write
+
+// The tables hold cos and sin of float(pos) * inv_freq[i] (src/kernels.cpp:277-279), built once
+// on the host.  Pairs are (i, i + hd/2): out[i] = x1*c - x2*s, out[i+hd/2] = x2*c + x1*s, as
+// separate products and one subtraction or addition (src/kernels.cpp:283-287).
+// A row whose position is negative is padding and is skipped.
+
+struct RopeArgs {
+  const float* qkv;         // [rows, q_dim + 2*kv_dim] 32-bit, row = [q | k | v]
+  const int32_t* positions;  // [rows]
+  const int32_t* row_seq;    // [rows] -> row of the block table
+  const int32_t* block_table;
+  const float* cos_table;    // [max_pos, hd/2]
+  const float* sin_table;
+  int rows, heads, kv_heads, head_dim, page_size, table_stride, write_cache;
+};
+
+// 32-bit: q and k are rotated in place; k and v go to cache[page][kv_head][slot][hd]
+// (src/model.cpp:291-296, src/kernels.h:97-99).
+__global__ void rope_kvwrite_f32_kernel(RopeArgs a, float* qkv_rw, float* __restrict__ k_cache,
+                                        float* __restrict__ v_cache) {
+  const int row = blockIdx.x;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  const int hd = a.head_dim, half = hd / 2;
+  const int q_dim = a.heads * hd, kv_dim = a.kv_heads * hd;
+  float* r = qkv_rw + (size_t)row * (q_dim + 2 * kv_dim);
+  const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
+  const int slot = pos % a.page_size;
+  const float* ct = a.cos_table + (size_t)pos * half;
+  const float* st = a.sin_table + (size_t)pos * half;
+  const int pairs = (a.heads + a.kv_heads) * half;
+  for (int e = threadIdx.x; e < pairs; e += blockDim.x) {
+    const int hh = e / half, i = e % half;
+    float* v = r + hh * hd;
+    const float x1 = v[i], x2 = v[i + half];
+    const float c = ct[i], s = st[i];
+    const float o1 = x1 * c - x2 * s;
+    const float o2 = x2 * c + x1 * s;
+    v[i] = o1;
+    v[i + half] = o2;
+    if (hh >= a.heads && a.write_cache) {
+      const int h = hh - a.heads;
+      float* dst = k_cache + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * hd;
+      dst[i] = o1;
+      dst[i + half] = o2;
+    }
+  }
+  if (a.write_cache) {
+    const float* vsrc = r + q_dim + kv_dim;
+    for (int e = threadIdx.x; e < kv_dim; e += blockDim.x) {
+      const int h = e / hd, d = e % hd;
+      v_cache[(((size_t)page * a.kv_heads + h) * a.page_size + slot) * hd + d] = vsrc[e];
+    }
+  }
+}
+
+// bfloat16: rotation in 32-bit from the 32-bit projections; q goes to q_out [rows, q_dim],
+// k to cache[page][kv_head][slot][hd], v transposed to cache[page][kv_head][hd][slot], each
+// rounded once.
+__global__ void rope_kvwrite_bf16_kernel(RopeArgs a, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
+                                         bf16_t* __restrict__ v_cache) {
+  const int row = blockIdx.x;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  const int hd = a.head_dim, half = hd / 2;
+  const int q_dim = a.heads * hd, kv_dim = a.kv_heads * hd;
+  const float* r = a.qkv + (size_t)row * (q_dim + 2 * kv_dim);
+  const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
+  const int slot = pos % a.page_size;
+  const float* ct = a.cos_table + (size_t)pos * half;
+  const float* st = a.sin_table + (size_t)pos * half;
+  const int pairs = (a.heads + a.kv_heads) * half;
+  for (int e = threadIdx.x; e < pairs; e += blockDim.x) {
+    const int hh = e / half, i = e % half;
+    const float* v = r + hh * hd;
+    const float x1 = v[i], x2 = v[i + half];
+    const float c = ct[i], s = st[i];
+    const float o1 = x1 * c - x2 * s;
+    const float o2 = x2 * c + x1 * s;
+    if (hh < a.heads) {
+      bf16_t* dst = q_out + (size_t)row * q_dim + hh * hd;
+      dst[i] = f32_to_bf16(o1);
+      dst[i + half] = f32_to_bf16(o2);
+    } else if (a.write_cache) {
+      const int h = hh - a.heads;
+      bf16_t* dst = k_cache + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * hd;
+      dst[i] = f32_to_bf16(o1);
+      dst[i + half] = f32_to_bf16(o2);
+    }
+  }
+  if (a.write_cache) {
+    const float* vsrc = r + q_dim + kv_dim;
+    for (int e = threadIdx.x; e < kv_dim; e += blockDim.x) {
+      const int h = e / hd, d = e % hd;
+      v_cache[(((size_t)page * a.kv_heads + h) * hd + d) * a.page_size + slot] = f32_to_bf16(vsrc[e]);
+    }
+  }
+}
+
+extern "C" int bw_rope_kvwrite(float* qkv, void* q_out, const int32_t* positions, const int32_t* row_seq,
+                               const int32_t* block_table, int table_stride, const float* cos_table,
+                               const float* sin_table, void* k_cache, void* v_cache, int is_bf16, int rows,
+                               int heads, int kv_heads, int head_dim, int page_size, int write_cache,
+                               void* stream) {
+  if (rows <= 0) return 0;
+  if (head_dim % 2 || page_size <= 0) return -2;
+  RopeArgs a{qkv, positions, row_seq, block_table, cos_table, sin_table,
+             rows, heads, kv_heads, head_dim, page_size, table_stride, write_cache};
+  hipStream_t s = (hipStream_t)stream;
+  if (is_bf16)
+    hipLaunchKernelGGL(rope_kvwrite_bf16_kernel, dim3(rows), dim3(256), 0, s, a, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache);
+  else
+    hipLaunchKernelGGL(rope_kvwrite_f32_kernel, dim3(rows), dim3(256), 0, s, a, qkv, (float*)k_cache, (float*)v_cache);
+  return BW_LAUNCH_CHECK();
+}

@@ -1,0 +1,312 @@
+"""Python faces of the HIP kernels.  Each wrapper checks on the host that operand shapes,
+dtypes and strides are what its kernel and grid assume, then launches on torch's current
+stream.  There is no fallback: without the compiled library every call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+EPI_F32, EPI_BF16, EPI_ADD_F32, EPI_SWIGLU_BF16 = 0, 1, 2, 3
+ATT_PART = 64          # keys per partition of the bfloat16 attention fold
+HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
+
+_ERRORS = {
+    -2: "sizes or strides out of the kernel's range",
+    -3: "misaligned pointer or stride",
+    -4: f"head size not compiled in (supported: {HEAD_DIMS})",
+    -5: "page size not supported (a power of two from 4 to 64 is needed)",
+}
+
+_SIGS = {
+    "bw_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_add": [c_void_p, c_void_p, c_longlong, c_void_p],
+    "bw_swiglu_f32": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "bw_gather_rows_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_rope_kvwrite": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                        c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_f32": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
+                          c_void_p],
+    "bw_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    "bw_fingerprint": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+}
+
+_fns = {}
+
+
+def _fn(name: str):
+    f = _fns.get(name)
+    if f is None:
+        lib = _build.load()
+        f = getattr(lib, name)
+        f.argtypes = _SIGS[name]
+        f.restype = c_int
+        _fns[name] = f
+    return f
+
+
+def available() -> bool:
+    """True if the library is built or can be built here (no GPU needed to answer)."""
+    try:
+        _build.load()
+        return True
+    except _build.KernelLibraryError:
+        return False
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        why = _ERRORS.get(code, f"HIP error {code}")
+        raise RuntimeError(f"{what}: {why}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t: torch.Tensor, dtype, what: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{what} must live on the GPU (there is no CPU path)")
+    if t.dtype != dtype:
+        raise ValueError(f"{what} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what} must be contiguous")
+
+
+def _is_bf16(t: torch.Tensor, what: str) -> int:
+    if t.dtype == torch.bfloat16:
+        return 1
+    if t.dtype == torch.float32:
+        return 0
+    raise ValueError(f"{what} must be bfloat16 or float32, got {t.dtype}")
+
+
+# ------------------------------------------------------------------------------ row ops
+
+def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r, :] = float(table[tokens[r], :]); a negative token gives a zero row."""
+    _need(tokens, torch.int32, "tokens")
+    _need(out, torch.float32, "out")
+    rows = tokens.numel()
+    vocab, width = table.shape
+    if not table.is_cuda or not table.is_contiguous():
+        raise ValueError("embedding table must be a contiguous GPU tensor")
+    if out.shape[0] < rows or out.shape[1] != width:
+        raise ValueError(f"embed: out {tuple(out.shape)} does not fit {rows} rows of width {width}")
+    _check(_fn("bw_embed")(tokens.data_ptr(), table.data_ptr(), _is_bf16(table, "table"), out.data_ptr(), rows, width,
+                           vocab, _stream()), "embed")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, rows: int, eps: float) -> None:
+    """out[r] = (x[r] * 1/sqrt(mean(x[r]^2) + eps)) * weight; out float32 (reference order of
+    operations) or bfloat16 (32-bit arithmetic, one rounding)."""
+    _need(x, torch.float32, "x")
+    dim = x.shape[-1]
+    if weight.numel() != dim or not weight.is_cuda:
+        raise ValueError(f"rmsnorm: weight has {weight.numel()} elements, rows are {dim} wide")
+    if x.shape[0] < rows or out.shape[0] < rows or out.shape[-1] != dim or not out.is_contiguous() or not out.is_cuda:
+        raise ValueError("rmsnorm: out does not fit x")
+    _check(_fn("bw_rmsnorm")(x.data_ptr(), weight.data_ptr(), _is_bf16(weight, "weight"), out.data_ptr(),
+                             _is_bf16(out, "out"), rows, dim, out.stride(0), float(eps), _stream()), "rmsnorm")
+
+
+def add_(x: torch.Tensor, y: torch.Tensor, rows: int) -> None:
+    _need(x, torch.float32, "x")
+    _need(y, torch.float32, "y")
+    if x.shape[1:] != y.shape[1:] or x.shape[0] < rows or y.shape[0] < rows:
+        raise ValueError("add_: shapes differ")
+    _check(_fn("bw_add")(x.data_ptr(), y.data_ptr(), rows * x.stride(0), _stream()), "add")
+
+
+def swiglu_f32(gate_up: torch.Tensor, out: torch.Tensor, rows: int) -> None:
+    _need(gate_up, torch.float32, "gate_up")
+    _need(out, torch.float32, "out")
+    inter = out.shape[1]
+    if gate_up.shape[1] != 2 * inter or gate_up.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError("swiglu: gate_up must be [rows, 2*inter] for out [rows, inter]")
+    _check(_fn("bw_swiglu_f32")(gate_up.data_ptr(), out.data_ptr(), rows, inter, _stream()), "swiglu")
+
+
+def gather_rows(x: torch.Tensor, index: torch.Tensor, out: torch.Tensor, count: int) -> None:
+    _need(x, torch.float32, "x")
+    _need(index, torch.int32, "index")
+    _need(out, torch.float32, "out")
+    if out.shape[1] != x.shape[1] or out.shape[0] < count or index.numel() < count:
+        raise ValueError("gather_rows: out does not fit")
+    _check(_fn("bw_gather_rows_f32")(x.data_ptr(), index.data_ptr(), out.data_ptr(), count, x.shape[1], x.stride(0),
+                                     _stream()), "gather_rows")
+
+
+def rope_kvwrite(qkv: torch.Tensor, q_out: Optional[torch.Tensor], positions: torch.Tensor, row_seq: torch.Tensor,
+                 block_table: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, k_cache: torch.Tensor,
+                 v_cache: torch.Tensor, rows: int, heads: int, kv_heads: int, head_dim: int, page_size: int,
+                 write_cache: bool = True) -> None:
+    """Rotate q and k of every row at its position and store k, v in the row's page slot.
+    32-bit caches: q, k rotated in place in ``qkv``.  bfloat16 caches: q goes to ``q_out``."""
+    _need(qkv, torch.float32, "qkv")
+    _need(positions, torch.int32, "positions")
+    _need(row_seq, torch.int32, "row_seq")
+    _need(block_table, torch.int32, "block_table")
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    bf = _is_bf16(k_cache, "k_cache")
+    if v_cache.dtype != k_cache.dtype:
+        raise ValueError("k and v caches must have one dtype")
+    width = (heads + 2 * kv_heads) * head_dim
+    if qkv.shape[1] != width or qkv.shape[0] < rows or positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError(f"rope_kvwrite: qkv must be [>= {rows}, {width}]")
+    if cos.shape[1] != head_dim // 2 or sin.shape != cos.shape:
+        raise ValueError("rope_kvwrite: tables must be [positions, head_dim/2]")
+    page_elems = kv_heads * page_size * head_dim
+    if k_cache.numel() % page_elems or v_cache.numel() != k_cache.numel():
+        raise ValueError("rope_kvwrite: cache size is no multiple of a page")
+    if bf:
+        if q_out is None:
+            raise ValueError("rope_kvwrite: bfloat16 needs q_out")
+        _need(q_out, torch.bfloat16, "q_out")
+        if q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows:
+            raise ValueError("rope_kvwrite: q_out must be [rows, heads*head_dim]")
+    _check(_fn("bw_rope_kvwrite")(qkv.data_ptr(), q_out.data_ptr() if q_out is not None else 0, positions.data_ptr(),
+                                  row_seq.data_ptr(), block_table.data_ptr(), block_table.stride(0), cos.data_ptr(),
+                                  sin.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), bf, rows, heads, kv_heads,
+                                  head_dim, page_size, int(write_cache), _stream()), "rope_kvwrite")
+
+
+# ------------------------------------------------------------------------------ matrix products
+
+def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, accumulate: bool = False) -> None:
+    """out[:rows] (+)= x[:rows] @ w.T with one k-ascending fused multiply-add chain per output."""
+    _need(x, torch.float32, "x")
+    _need(out, torch.float32, "out")
+    if not w.is_cuda or not w.is_contiguous() or w.dim() != 2:
+        raise ValueError("gemm_f32: weight must be a contiguous [N, K] GPU tensor")
+    N, K = w.shape
+    if x.shape[1] != K or out.shape[1] != N or x.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError(f"gemm_f32: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
+    _check(_fn("bw_gemm_f32")(x.data_ptr(), w.data_ptr(), _is_bf16(w, "weight"), out.data_ptr(), rows, N, K,
+                              x.stride(0), out.stride(0), int(accumulate), _stream()), "gemm_f32")
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, epilogue: int) -> None:
+    """out[:rows] = epilogue(x[:rows] @ w.T) on the matrix cores; see gemm_bf16.hip for the
+    arithmetic.  EPI_SWIGLU_BF16 takes the stacked weight [2N, K] (gate rows, then up rows)."""
+    _need(x, torch.bfloat16, "x")
+    _need(w, torch.bfloat16, "weight")
+    if w.dim() != 2:
+        raise ValueError("gemm_bf16: weight must be [N, K]")
+    N, K = w.shape
+    if epilogue == EPI_SWIGLU_BF16:
+        if N % 2:
+            raise ValueError("gemm_bf16: SwiGLU needs a stacked weight with an even number of rows")
+        N //= 2
+    want = torch.bfloat16 if epilogue in (EPI_BF16, EPI_SWIGLU_BF16) else torch.float32
+    _need(out, want, "out")
+    if x.shape[1] != K or out.shape[1] != N or x.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError(f"gemm_bf16: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
+    if K % 8:
+        raise ValueError(f"gemm_bf16: inner size {K} must be a multiple of 8 (16-byte operand loads)")
+    _check(_fn("bw_gemm_bf16")(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, N, K, x.stride(0), out.stride(0),
+                               epilogue, _stream()), "gemm_bf16")
+
+
+# ------------------------------------------------------------------------------ attention
+
+def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, rows: int, heads: int,
+                  kv_heads: int, head_dim: int, page_size: int, window: int, scale: float) -> None:
+    """q: [rows, stride] float32 with head h at columns h*head_dim.. (the stacked q|k|v rows
+    serve as they are); caches [pages, kv_heads, page_size, head_dim] float32."""
+    _need(q, torch.float32, "q")
+    _need(out, torch.float32, "out")
+    _need(k_cache, torch.float32, "k_cache")
+    _need(v_cache, torch.float32, "v_cache")
+    _need(positions, torch.int32, "positions")
+    _need(row_seq, torch.int32, "row_seq")
+    _need(block_table, torch.int32, "block_table")
+    if head_dim not in HEAD_DIMS:
+        raise ValueError(f"attention: head size {head_dim} is not supported; supported: {HEAD_DIMS}")
+    if q.shape[0] < rows or q.shape[1] < heads * head_dim or out.shape[0] < rows or out.shape[1] != heads * head_dim:
+        raise ValueError("attention_f32: q or out too small")
+    if heads % kv_heads:
+        raise ValueError("attention: heads must be a multiple of kv_heads")
+    _check(_fn("bw_attention_f32")(q.data_ptr(), q.stride(0), positions.data_ptr(), row_seq.data_ptr(),
+                                   block_table.data_ptr(), block_table.stride(0), k_cache.data_ptr(),
+                                   v_cache.data_ptr(), out.data_ptr(), out.stride(0), rows, heads, kv_heads, head_dim,
+                                   page_size, int(window), float(scale), _stream()), "attention_f32")
+
+
+def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
+                   num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, heads: int,
+                   kv_heads: int, head_dim: int, page_size: int, window: int, scale: float, split: bool = False,
+                   max_parts: int = 0, part_o: Optional[torch.Tensor] = None,
+                   part_ml: Optional[torch.Tensor] = None) -> None:
+    """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
+    [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).  With
+    ``split`` (tiles of one token each) every (tile, partition) is a wave of its own and the
+    partials are folded by a second kernel; the bits equal the unsplit route."""
+    _need(q, torch.bfloat16, "q")
+    _need(out, torch.bfloat16, "out")
+    _need(k_cache, torch.bfloat16, "k_cache")
+    _need(v_cache, torch.bfloat16, "v_cache")
+    _need(positions, torch.int32, "positions")
+    _need(block_table, torch.int32, "block_table")
+    _need(tiles, torch.int32, "tiles")
+    if head_dim not in HEAD_DIMS:
+        raise ValueError(f"attention: head size {head_dim} is not supported; supported: {HEAD_DIMS}")
+    if heads % kv_heads:
+        raise ValueError("attention: heads must be a multiple of kv_heads")
+    if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or tiles.numel() < 4 * num_tiles:
+        raise ValueError("attention_bf16: q, out or tiles do not fit")
+    group = heads // kv_heads
+    hpt = min(group, 16)
+    items = num_tiles * kv_heads * ((group + hpt - 1) // hpt)
+    if split:
+        if part_o is None or part_ml is None or max_parts <= 0:
+            raise ValueError("attention_bf16: split needs scratch buffers")
+        _need(part_o, torch.float32, "part_o")
+        _need(part_ml, torch.float32, "part_ml")
+        if part_o.numel() < items * max_parts * head_dim * hpt or part_ml.numel() < items * max_parts * 2 * hpt:
+            raise ValueError("attention_bf16: scratch buffers too small")
+    _check(_fn("bw_attention_bf16")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
+                                    block_table.stride(0), tiles.data_ptr(), num_tiles, k_cache.data_ptr(),
+                                    v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads, kv_heads, head_dim,
+                                    page_size, int(window), float(scale), int(split), max_parts,
+                                    part_o.data_ptr() if part_o is not None else 0,
+                                    part_ml.data_ptr() if part_ml is not None else 0, _stream()), "attention_bf16")
+
+
+# ------------------------------------------------------------------------------ sampling
+
+def sample(logits: torch.Tensor, rows: int, temperature: torch.Tensor, uniform: torch.Tensor,
+           out: torch.Tensor) -> None:
+    """out[r] = first maximum of row r if temperature[r] <= 0, else the inverse-CDF draw at
+    uniform[r] from softmax(logits[r] / temperature[r])."""
+    _need(logits, torch.float32, "logits")
+    _need(temperature, torch.float32, "temperature")
+    _need(uniform, torch.float64, "uniform")
+    _need(out, torch.int32, "out")
+    if logits.shape[0] < rows or temperature.numel() < rows or uniform.numel() < rows or out.numel() < rows:
+        raise ValueError("sample: buffers shorter than the number of rows")
+    _check(_fn("bw_sample")(logits.data_ptr(), logits.shape[1], logits.stride(0), rows, temperature.data_ptr(),
+                            uniform.data_ptr(), out.data_ptr(), _stream()), "sample")
+
+
+def fingerprint(logits: torch.Tensor, rows: int, h_in: torch.Tensor, h_out: torch.Tensor) -> None:
+    """h_out[r] = the reference's logits hash chained from h_in[r] (int64 bit patterns)."""
+    _need(logits, torch.float32, "logits")
+    _need(h_in, torch.int64, "h_in")
+    _need(h_out, torch.int64, "h_out")
+    _check(_fn("bw_fingerprint")(logits.data_ptr(), logits.shape[1], logits.stride(0), rows, h_in.data_ptr(),
+                                 h_out.data_ptr(), _stream()), "fingerprint")

@@ -1,0 +1,151 @@
+// Token choice and logits fingerprints on the device, one workgroup per logits row.
+//
+// Greedy: the first maximum wins (the reference scans with a strict '>', src/engine.cpp:40-45).
+// Temperature: w[i] = expf((l[i] - max) / T) in 32-bit, sums in double, the token is the first
+// i whose running sum exceeds u * total, else the last i with positive weight
+// (src/engine.cpp:50-73).  The reference adds the weights one after the other; here each of
+// the 256 threads adds its own contiguous stretch of the vocabulary in order and the
+// stretches are joined in thread order, which moves the running sum by a few units of
+// 2^-53 and depends on nothing but the row itself.  u comes from the host's counter-based
+// generator keyed by (seed, position, stream).
+#include "common.h"
+#include "api.h"
+
+#define SMP_THREADS 256
+
+__global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __restrict__ logits, int vocab, int ld,
+                                                             const float* __restrict__ temperature,
+                                                             const double* __restrict__ uniform,
+                                                             int32_t* __restrict__ out) {
+  __shared__ float s_val[SMP_THREADS];
+  __shared__ int s_idx[SMP_THREADS];
+  __shared__ double s_sum[SMP_THREADS];
+  __shared__ int s_pick[SMP_THREADS];
+  __shared__ int s_lastpos[SMP_THREADS];
+  __shared__ double s_total;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* l = logits + (size_t)row * ld;
+  const int chunk = (vocab + SMP_THREADS - 1) / SMP_THREADS;
+  const int begin = tid * chunk < vocab ? tid * chunk : vocab;
+  const int end = begin + chunk < vocab ? begin + chunk : vocab;
+
+  // maximum and its first index
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int i = begin; i < end; ++i)
+    if (l[i] > best || best_i == 0x7fffffff) {  // first element of the stretch, or strictly greater
+      best = l[i];
+      best_i = i;
+    }
+  s_val[tid] = best;
+  s_idx[tid] = best_i;
+  __syncthreads();
+  for (int off = SMP_THREADS / 2; off >= 1; off >>= 1) {
+    if (tid < off) {
+      const float ov = s_val[tid + off];
+      const int oi = s_idx[tid + off];
+      if (oi != 0x7fffffff && (s_idx[tid] == 0x7fffffff || ov > s_val[tid] || (ov == s_val[tid] && oi < s_idx[tid]))) {
+        s_val[tid] = ov;
+        s_idx[tid] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  const float mx = s_val[0];
+  const float T = temperature[row];
+  if (T <= 0.0f) {
+    if (tid == 0) out[row] = s_idx[0];
+    return;
+  }
+
+  double part = 0.0;
+  int lastpos = -1;
+  for (int i = begin; i < end; ++i) {
+    const float w = expf((l[i] - mx) / T);
+    if (w > 0.0f) {
+      part += (double)w;
+      lastpos = i;
+    }
+  }
+  s_sum[tid] = part;
+  s_lastpos[tid] = lastpos;
+  s_pick[tid] = -1;
+  __syncthreads();
+  if (tid == 0) {  // exclusive prefix in thread order; s_sum[t] becomes the sum before stretch t
+    double run = 0.0;
+    int last = 0;
+    for (int t = 0; t < SMP_THREADS; ++t) {
+      const double p = s_sum[t];
+      s_sum[t] = run;
+      run += p;
+      if (s_lastpos[t] >= 0) last = s_lastpos[t];
+    }
+    s_lastpos[0] = last;
+    s_total = run;
+  }
+  __syncthreads();
+  const double total = s_total;
+  const double target = uniform[row] * total;
+  double cum = s_sum[tid];
+  if (cum <= target) {
+    for (int i = begin; i < end; ++i) {
+      const float w = expf((l[i] - mx) / T);
+      if (w <= 0.0f) continue;
+      cum += (double)w;
+      if (cum > target) {
+        s_pick[tid] = i;
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pick = s_lastpos[0];
+    for (int t = 0; t < SMP_THREADS; ++t)
+      if (s_pick[t] >= 0) {
+        pick = s_pick[t];
+        break;
+      }
+    out[row] = pick;
+  }
+}
+
+extern "C" int bw_sample(const float* logits, int vocab, int ld, int rows, const float* temperature,
+                         const double* uniform, int32_t* out, void* stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0 || ld < vocab) return -2;
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, (hipStream_t)stream, logits, vocab, ld,
+                     temperature, uniform, out);
+  return BW_LAUNCH_CHECK();
+}
+
+// Fingerprint chain of the reference (src/engine.cpp:18-29): h = (h ^ word) * 1099511628211
+// over the row's 8-byte words, single trailing bytes likewise, then the splitmix64 finaliser.
+// The chain is sequential by construction; one lane per row.
+__global__ void fingerprint_kernel(const float* __restrict__ logits, int vocab, int ld, int rows,
+                                   const uint64_t* __restrict__ h_in, uint64_t* __restrict__ h_out) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const uint32_t* p = reinterpret_cast<const uint32_t*>(logits + (size_t)row * ld);
+  uint64_t h = h_in[row];
+  int i = 0;
+  for (; i + 2 <= vocab; i += 2) {
+    const uint64_t wd = (uint64_t)p[i] | ((uint64_t)p[i + 1] << 32);
+    h = (h ^ wd) * 1099511628211ull;
+  }
+  if (i < vocab) {
+    const uint32_t t = p[i];
+    for (int b = 0; b < 4; ++b) h = (h ^ ((t >> (8 * b)) & 0xffu)) * 1099511628211ull;
+  }
+  h = (h ^ (h >> 30)) * 0xBF58476D1CE4E5B9ull;
+  h = (h ^ (h >> 27)) * 0x94D049BB133111EBull;
+  h_out[row] = h ^ (h >> 31);
+}
+
+extern "C" int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out,
+                              void* stream) {
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(fingerprint_kernel, dim3((rows + 63) / 64), dim3(64), 0, (hipStream_t)stream, logits, vocab, ld,
+                     rows, (const uint64_t*)h_in, (uint64_t*)h_out);
+  return BW_LAUNCH_CHECK();
+}

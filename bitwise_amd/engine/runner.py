@@ -1,0 +1,137 @@
+"""The step function: run one batch of (request, its next tokens) through the model, from
+the cache that earlier steps left, and return the logits at the wanted places.
+
+It runs only the tokens it is given.  Batches of nothing but single decoded tokens are
+replayed from HIP graphs captured per batch-size bucket (the launch sequence of a decode
+step is fixed; only the contents of the index arrays change); every other batch is launched
+kernel by kernel.  Both routes run the same kernels on the same data layout, so the logits
+of a position do not depend on the route.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..csrc.ops import ATT_PART
+from ..models.assembled import AssembledModel
+from .batch import AttentionPlan, Segment, StepContext
+from .storage import CacheStorage
+
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+
+
+class _StaticDecodeContext:
+    """Fixed device arrays for a decode batch of up to ``size`` requests, one row each."""
+
+    def __init__(self, size: int, num_groups: int, max_pages: int, max_parts: int, device: torch.device):
+        self.rows = self.nseq = self.num_wanted = size
+        self.device = device
+        self.max_pages = max_pages
+        self.tokens = torch.full((size,), -1, dtype=torch.int32, device=device)
+        self.positions = torch.full((size,), -1, dtype=torch.int32, device=device)
+        self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
+        self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
+        self.slots = torch.zeros(size, dtype=torch.int32, device=device)
+        self.block_tables = [torch.zeros((size, max_pages), dtype=torch.int32, device=device) for _ in range(num_groups)]
+        tiles = np.zeros((size, 4), np.int32)
+        tiles[:, 0] = tiles[:, 2] = np.arange(size)
+        tiles[:, 1] = 1
+        self._plan = AttentionPlan(None, 0, torch.from_numpy(tiles).to(device), size, max_parts)
+        self._host = np.empty((3 + num_groups * max_pages, size), np.int32)
+        self.segments: List[Segment] = []
+
+    def attention_plan(self, tokens_per_tile: int) -> AttentionPlan:
+        return self._plan
+
+    def fill(self, segments: Sequence[Segment]) -> None:
+        size, n = self.rows, len(segments)
+        self.segments = list(segments)
+        tok = np.full(size, -1, np.int32)
+        pos = np.full(size, -1, np.int32)
+        slot = np.zeros(size, np.int32)
+        for i, s in enumerate(segments):
+            tok[i], pos[i], slot[i] = s.tokens[0], s.pos0, s.slot
+        self.tokens.copy_(torch.from_numpy(tok))
+        self.positions.copy_(torch.from_numpy(pos))
+        self.slots.copy_(torch.from_numpy(slot))
+        for g, dev in enumerate(self.block_tables):
+            t = np.zeros((size, self.max_pages), np.int32)
+            for i, s in enumerate(segments):
+                row = np.asarray(s.tables[g], np.int32)
+                t[i, :len(row)] = np.maximum(row, 0)
+            dev.copy_(torch.from_numpy(t))
+
+
+class ModelRunner:
+    def __init__(self, model: AssembledModel, storage: CacheStorage, max_model_len: int, use_graphs: bool = True):
+        self.model, self.storage = model, storage
+        self.rt = model.rt
+        self.max_model_len = int(max_model_len)
+        self.use_graphs = bool(use_graphs) and model.graph_safe
+        self._graphs: Dict[int, tuple] = {}
+        self._graph_generation = -1
+
+    # ------------------------------------------------------------------ the step function
+    def step(self, segments: Sequence[Segment]) -> Optional[torch.Tensor]:
+        """Logits [wanted, vocab] (32-bit, on the device, valid until the next step) at the
+        wanted places in the order of the segments and of their ``want``; None if none."""
+        if not segments:
+            return None
+        rows = sum(len(s.tokens) for s in segments)
+        wanted = sum(len(s.want) for s in segments)
+        if rows > self.rt.max_rows:
+            raise ValueError(f"a step of {rows} tokens exceeds the engine's {self.rt.max_rows}")
+        if wanted > self.rt.max_logit_rows:
+            raise ValueError(f"logits wanted at {wanted} places, the engine allows {self.rt.max_logit_rows}")
+        for s in segments:
+            if not len(s.tokens):
+                raise ValueError("a request without tokens in a step")
+            if s.pos0 + len(s.tokens) > self.max_model_len:
+                raise ValueError(f"position {s.pos0 + len(s.tokens) - 1} is beyond the model length {self.max_model_len}")
+            need = (s.pos0 + len(s.tokens) + self.rt.page_size - 1) // self.rt.page_size
+            for t in s.tables:
+                if len(t) < need:
+                    raise ValueError("a request's block table does not cover its positions")
+        decode_only = all(len(s.tokens) == 1 and tuple(s.want) == (0,) for s in segments)
+        if self.use_graphs and decode_only and len(segments) <= GRAPH_BUCKETS[-1]:
+            return self._step_graph(segments)
+        ctx = StepContext(segments, len(self.model.group_specs), self.rt.device)
+        return self.model.forward(ctx)
+
+    # ------------------------------------------------------------------ graph replay
+    def _step_graph(self, segments: Sequence[Segment]) -> torch.Tensor:
+        n = len(segments)
+        bucket = next(b for b in GRAPH_BUCKETS if b >= n)
+        if bucket > self.rt.max_rows or bucket > self.rt.max_logit_rows:
+            ctx = StepContext(segments, len(self.model.group_specs), self.rt.device)
+            return self.model.forward(ctx)
+        if self._graph_generation != self.rt.scratch_generation:
+            self._graphs.clear()                      # a scratch tensor moved: old captures are stale
+        entry = self._graphs.get(bucket)
+        if entry is None:
+            entry = self._capture(bucket, segments)
+        ctx, graph, logits = entry
+        ctx.fill(segments)
+        graph.replay()
+        return logits[:n]
+
+    def _capture(self, bucket: int, segments: Sequence[Segment]):
+        rt = self.rt
+        max_pages = (self.max_model_len + rt.page_size - 1) // rt.page_size
+        max_parts = (self.max_model_len + ATT_PART - 1) // ATT_PART
+        ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, max_parts, rt.device)
+        ctx.fill(segments)
+        # One eager run first: it creates every scratch buffer the capture will use and it is
+        # the step's real work (writing the same cache slots twice with the same values is harmless).
+        self.model.forward(ctx)
+        torch.cuda.synchronize(rt.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx)
+        self._graph_generation = rt.scratch_generation
+        entry = (ctx, graph, logits)
+        self._graphs[bucket] = entry
+        return entry

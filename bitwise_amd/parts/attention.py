@@ -1,0 +1,109 @@
+"""Causal grouped-query attention over the paged cache (src/model.cpp:281-300).
+
+One stacked projection [q; k; v] (src/model.cpp:150-153), rotary encoding of q and k and the
+cache write in one kernel, attention over keys lo..p of the row's own sequence, output
+projection added into the residual stream.  The part knows its sizes and nothing else: which
+cache it reads, which block table belongs to it and where its rows sit arrive with the call.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import ops
+from .base import CacheSpec, Mixer, TensorSpec, lookup, register_mixer, POSITION_ENCODINGS
+from .linear import Linear
+
+# A decoded token's attention is cut into one wave per 64-key partition once its context is
+# at least this long (same bits either way; this only buys parallelism).
+SPLIT_MIN_CONTEXT = 256
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    """params: width, heads, kv_heads, head_dim, window (None = all keys), position (PartSpec
+    of the position encoding).  tensors: q_proj/k_proj/v_proj/o_proj .weight."""
+
+    graph_safe = True
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        p = params
+        self.width, self.heads, self.kv_heads, self.head_dim = int(p["width"]), int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        self.window: Optional[int] = p.get("window")
+        if self.heads % self.kv_heads:
+            raise ValueError(f"attention: {self.heads} heads are no multiple of {self.kv_heads} kv heads")
+        if self.head_dim not in ops.HEAD_DIMS:
+            raise ValueError(f"attention: head size {self.head_dim} is not supported by the kernels; "
+                             f"supported: {ops.HEAD_DIMS}")
+        self.q_dim, self.kv_dim = self.heads * self.head_dim, self.kv_heads * self.head_dim
+        self.scale = 1.0 / math.sqrt(float(self.head_dim))     # 1.0f / sqrtf(float(hd)), src/kernels.cpp:347
+        pos = p["position"]
+        self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+        self.qkv: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+        group = self.heads // self.kv_heads
+        self.heads_per_tile = min(group, 16)
+        self.tokens_per_tile = 16 // self.heads_per_tile
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        return {
+            "q_proj.weight": TensorSpec((self.q_dim, self.width)),
+            "k_proj.weight": TensorSpec((self.kv_dim, self.width)),
+            "v_proj.weight": TensorSpec((self.kv_dim, self.width)),
+            "o_proj.weight": TensorSpec((self.width, self.q_dim)),
+        }
+
+    def bind(self, tensors) -> None:
+        q, k, v = tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError("q, k and v projections must be stored in one dtype to be stacked")
+        self.qkv = Linear(torch.cat([q, k, v], dim=0), self.rt)
+        self.o = Linear(tensors["o_proj.weight"], self.rt)
+
+    def weight_bytes(self) -> int:
+        return self.qkv.nbytes() + self.o.nbytes()
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.kv_heads, self.head_dim, self.window)
+
+    def page_elements(self, page_size: int) -> int:
+        """Elements of one page of keys (and likewise of values) of one cache."""
+        return self.kv_heads * page_size * self.head_dim
+
+    def forward(self, ctx, call, h, residual) -> None:
+        rt, rows = self.rt, ctx.rows
+        table = ctx.block_tables[call.group]
+        window = int(self.window or 0)
+        qkv = rt.buffer("qkv", self.q_dim + 2 * self.kv_dim, torch.float32)
+        self.qkv.store(h, qkv, rows)
+        if rt.bf16:
+            q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
+            ops.rope_kvwrite(qkv, q, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
+                             call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
+                             rt.page_size, call.writes_cache)
+            out = rt.buffer("attn_out", self.q_dim, torch.bfloat16)
+            plan = ctx.attention_plan(self.tokens_per_tile)
+            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                      window, self.scale)
+            if plan.fold_count:
+                ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
+            if plan.split_count:
+                group = self.heads // self.kv_heads
+                columns = self.kv_heads * ((group + self.heads_per_tile - 1) // self.heads_per_tile) * self.heads_per_tile
+                cells = plan.split_count * plan.max_parts * columns
+                part_o = rt.scratch("attn_part_o", cells * self.head_dim, torch.float32)
+                part_ml = rt.scratch("attn_part_ml", cells * 2, torch.float32)
+                ops.attention_bf16(q, ctx.positions, table, plan.split_tiles, plan.split_count, *common,
+                                   split=True, max_parts=plan.max_parts, part_o=part_o, part_ml=part_ml)
+        else:
+            ops.rope_kvwrite(qkv, None, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
+                             call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
+                             rt.page_size, call.writes_cache)
+            out = rt.buffer("attn_out", self.q_dim, torch.float32)
+            ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
+                              self.heads, self.kv_heads, self.head_dim, rt.page_size, window, self.scale)
+        self.o.add_into(out, residual, rows)

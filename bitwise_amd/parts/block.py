@@ -1,0 +1,16 @@
+"""Arrangements of mixer, feed-forward and norms around the 32-bit residual stream."""
+
+from __future__ import annotations
+
+from .base import Block, register_block
+
+
+@register_block("prenorm")
+class PreNormBlock(Block):
+    """x += mixer(norm1(x)); x += feed_forward(norm2(x)) (src/model.cpp:281-305)."""
+
+    def forward(self, ctx, call, x) -> None:
+        h = self.mixer_norm.forward(ctx, x)
+        self.mixer.forward(ctx, call, h, x)
+        h = self.ffn_norm.forward(ctx, x)
+        self.feed_forward.forward(ctx, h, x)

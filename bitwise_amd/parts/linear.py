@@ -1,0 +1,52 @@
+"""A weight matrix [out, in] and the matrix product that fits its dtype and the mode.
+
+Reference: y[m][n] = sum_k x[m][k] * W[n][k], W as stored by the checkpoint, no bias
+(src/kernels.cpp:236-244).  bfloat16 weights run on the matrix cores in bfloat16 mode; a
+weight stored in 32-bit stays 32-bit and runs through the 32-bit kernel in either mode.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, runtime):
+        if weight.dim() != 2 or weight.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("a linear weight must be a bfloat16 or float32 matrix")
+        self.rt = runtime
+        self.weight = weight.to(runtime.device).contiguous()
+        self.out_features, self.in_features = self.weight.shape
+        self.mfma = runtime.bf16 and self.weight.dtype == torch.bfloat16
+        if self.mfma and self.in_features % 8:
+            raise ValueError(f"bfloat16 matrix product: inner size {self.in_features} must be a multiple of 8")
+
+    def nbytes(self) -> int:
+        return self.weight.numel() * self.weight.element_size()
+
+    def _x32(self, x: torch.Tensor, rows: int) -> torch.Tensor:
+        if x.dtype == torch.float32:
+            return x
+        buf = self.rt.buffer("linear_x32", x.shape[1], torch.float32)
+        buf[:rows].copy_(x[:rows])
+        return buf
+
+    def store(self, x: torch.Tensor, out: torch.Tensor, rows: int) -> None:
+        """out[:rows] = x[:rows] @ W.T (out float32, or bfloat16 on the matrix-core path)."""
+        if self.mfma:
+            ops.gemm_bf16(x, self.weight, out, rows, ops.EPI_BF16 if out.dtype == torch.bfloat16 else ops.EPI_F32)
+        elif out.dtype == torch.float32:
+            ops.gemm_f32(self._x32(x, rows), self.weight, out, rows)
+        else:
+            tmp = self.rt.buffer("linear_y32", self.out_features, torch.float32)
+            ops.gemm_f32(self._x32(x, rows), self.weight, tmp, rows)
+            out[:rows].copy_(tmp[:rows])
+
+    def add_into(self, x: torch.Tensor, residual: torch.Tensor, rows: int) -> None:
+        """residual[:rows] += x[:rows] @ W.T, the sum in 32-bit (src/model.cpp:300, :305)."""
+        if self.mfma:
+            ops.gemm_bf16(x, self.weight, residual, rows, ops.EPI_ADD_F32)
+        else:
+            ops.gemm_f32(self._x32(x, rows), self.weight, residual, rows, accumulate=True)

@@ -1,0 +1,96 @@
+"""Replaying given tokens through the engine's own step function and cache manager (the role
+of logits_chunked, tests/test_main.cpp:200-217, and of Model.logits, python/bindings.cpp:35-52,
+with requests that come, pause and end).  Nothing is sampled."""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from .cache.manager import CacheManager, GroupSpec, RequestCache
+from .engine.batch import Segment
+from .engine.runner import ModelRunner
+from .engine.storage import CacheStorage
+from .model import Model
+
+MAX_STEP_ROWS = 4096
+
+
+class Replayer:
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, use_graphs: bool = True,
+                 max_live: int = 64, model: Optional[Model] = None):
+        self.model = model if model is not None else Model.load(model_dir, dtype)
+        asm = self.model.assembled
+        rows = max(64, min(int(max_tokens), MAX_STEP_ROWS))
+        asm.rt.configure(max_rows=rows, page_size=block_size, max_logit_rows=rows)
+        pages = (int(max_tokens) + block_size - 1) // block_size
+        self.manager = CacheManager([GroupSpec(g.window) for g in asm.group_specs], pages, block_size, max_live,
+                                    prefix_caching=False, has_state=bool(asm.state_specs))
+        self.storage = CacheStorage(asm, pages, max_live)
+        max_len = min(asm.spec.max_positions, max(int(max_tokens), 1))
+        self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, use_graphs=use_graphs)
+        self.live: Dict[str, RequestCache] = {}
+
+    def step(self, entries: Sequence[dict], end: Sequence[str] = ()) -> Optional[np.ndarray]:
+        """Run one step; returns the wanted logits [wanted, vocab] or None."""
+        segments: List[Segment] = []
+        touched: List[RequestCache] = []
+        for e in entries:
+            rid, toks = str(e["id"]), list(e["tokens"])
+            rc = self.live.get(rid)
+            if rc is None:
+                rc = self.manager.open()
+                if rc is None:
+                    raise RuntimeError("more live requests than state slots")
+                self.storage.reset_slot(rc.slot)
+                self.live[rid] = rc
+            if not toks:
+                continue
+            if not self.manager.ensure(rc, rc.computed + len(toks)):
+                raise RuntimeError(f"out of cache pages at request {rid}: --max-tokens is too small for this trace")
+            want = [int(w) for w in e.get("want", [])]
+            if any(w < 0 or w >= len(toks) for w in want):
+                raise ValueError(f"request {rid}: 'want' names a place outside its tokens")
+            segments.append(Segment(toks, rc.computed, rc.tables, rc.slot, want))
+            touched.append(rc)
+        out = None
+        if segments:
+            out = self._run(segments)
+            for rc, seg in zip(touched, segments):
+                self.manager.advance(rc, (), rc.computed + len(seg.tokens))
+        for rid in end:
+            rc = self.live.pop(str(rid), None)
+            if rc is not None:
+                self.manager.close(rc)
+        return out
+
+    def _run(self, segments: List[Segment]) -> Optional[np.ndarray]:
+        limit = self.runner.rt.max_rows
+        if sum(len(s.tokens) for s in segments) <= limit:
+            lg = self.runner.step(segments)
+            return None if lg is None else lg.cpu().numpy()
+        # A step larger than the scratch buffers runs as several launches of the step
+        # function; the logits do not depend on the cut.
+        outs, batch, rows = [], [], 0
+
+        def flush():
+            nonlocal batch, rows
+            if batch:
+                lg = self.runner.step(batch)
+                if lg is not None:
+                    outs.append(lg.cpu().numpy())
+            batch, rows = [], 0
+
+        for s in segments:
+            off = 0
+            while off < len(s.tokens):
+                take = min(len(s.tokens) - off, limit - rows)
+                want = [w - off for w in s.want if off <= w < off + take]
+                batch.append(Segment(s.tokens[off:off + take], s.pos0 + off, s.tables, s.slot, want))
+                rows += take
+                off += take
+                if rows == limit:
+                    flush()
+        flush()
+        return np.concatenate(outs) if outs else None
