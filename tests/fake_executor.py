@@ -1,0 +1,69 @@
+"""A stand-in for the device in scheduler tests: a 'model' whose next token is a hash of the
+whole token sequence as read back from paged storage through the block tables.  If the
+scheduler or cache manager ever shares, reuses or loses a page wrongly, the sequence read
+back differs from the request's own tokens and the generated tokens change."""
+
+from __future__ import annotations
+
+from typing import Dict, List
+
+from bitwise_amd.cache.manager import GroupSpec
+
+_M64 = (1 << 64) - 1
+
+
+def _mix(z: int) -> int:
+    z &= _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+class FakeExecutor:
+    def __init__(self, page_size: int, vocab_size: int = 97, eos_token_id: int = 3, max_model_len: int = 1 << 20):
+        self.group_specs = [GroupSpec()]
+        self.has_state = False
+        self.vocab_size = vocab_size
+        self.eos_token_id = eos_token_id
+        self.max_model_len = max_model_len
+        self.page_size = page_size
+        self.pages: Dict[int, List[int]] = {}
+        self.steps = 0
+        self.rows_run = 0
+        self.reset_slots: List[int] = []
+
+    def reset_slot(self, slot: int) -> None:
+        self.reset_slots.append(slot)
+
+    def run(self, segments):
+        self.steps += 1
+        ps = self.page_size
+        for s in segments:                       # every row's token goes into its page slot first
+            for i, t in enumerate(s.tokens):
+                pos = s.pos0 + i
+                page = s.tables[0][pos // ps]
+                assert page >= 0
+                self.pages.setdefault(page, [None] * ps)[pos % ps] = t
+                self.rows_run += 1
+        out = []
+        for s in segments:
+            for w in s.want:
+                pos = s.pos0 + w
+                h = 1469598103934665603
+                for p in range(pos + 1):
+                    t = self.pages[s.tables[0][p // ps]][p % ps]
+                    assert t is not None, "read of a slot that was never written"
+                    h = _mix(h ^ (t + 1))
+                out.append(h)
+        return out
+
+    def sample(self, logits, temperatures, seeds, positions):
+        toks = []
+        for h, t, seed, pos in zip(logits, temperatures, seeds, positions):
+            if t > 0:
+                h = _mix(h ^ _mix(seed * 1000003 + pos))
+            toks.append(h % self.vocab_size)
+        return toks
+
+    def fingerprints(self, logits, previous):
+        return [_mix(p ^ h) for h, p in zip(logits, previous)]

@@ -1,0 +1,154 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice, under random
+orders of requests; the reference's own block-manager sequence; windowed groups."""
+
+import random
+
+import pytest
+
+from bitwise_amd.cache.manager import CacheManager, GroupSpec
+from bitwise_amd.cache.pages import PagePool, StateSlots, block_hash
+from plain_llama import block_hash as plain_block_hash
+
+
+def test_reference_block_manager_sequence():
+    """tests/test_main.cpp:171-197, step by step."""
+    m = PagePool(4, 16, prefix_caching=True)
+    assert m.available() == 4
+    a, b = m.allocate(), m.allocate()
+    assert a is not None and b is not None and a != b and (a, b) == (0, 1)      # low ids first
+    toks, other = list(range(16)), list(range(1, 17))
+    h = block_hash(0, toks)
+    m.register_full(a, h, toks)
+    assert m.lookup(h, other) is None                 # same hash, different tokens: never a hit
+    hit = m.lookup(h, toks)
+    assert hit == a and m.refcount(a) == 2
+    m.release(a)
+    m.release(a)                                       # now cached but unreferenced
+    assert m.available() == 3
+    assert m.lookup(h, toks) == a                      # revived from the evictable list
+    m.release(a)
+    c, d, e = m.allocate(), m.allocate(), m.allocate()
+    assert None not in (c, d, e) and m.evictions == 1  # free pages first, then the cached one
+    assert m.lookup(h, toks) is None
+    assert m.allocate() is None
+    m.check()
+
+
+def test_block_hash_matches_the_plain_formula_and_chains():
+    toks = [5, 17, 3, 0, 255, 2 ** 31 - 1, 7, 7]
+    assert block_hash(0, toks) == plain_block_hash(0, toks)
+    assert block_hash(123456789, toks) == plain_block_hash(123456789, toks)
+    assert block_hash(0, toks) != block_hash(1, toks) and block_hash(0, toks) != block_hash(0, toks[::-1])
+
+
+def test_double_release_is_an_error():
+    m = PagePool(2, 8)
+    p = m.allocate()
+    m.release(p)
+    with pytest.raises(RuntimeError, match="unreferenced"):
+        m.release(p)
+    s = StateSlots(2)
+    x = s.allocate()
+    s.release(x)
+    with pytest.raises(RuntimeError, match="free slot"):
+        s.release(x)
+
+
+@pytest.mark.parametrize("seed", range(25))
+def test_random_orders_lose_nothing(seed):
+    """Requests open, grow, share prefixes, get preempted and close in random order; after
+    every operation every page is free, cached or referenced exactly once per holder."""
+    rng = random.Random(seed)
+    ps = rng.choice([8, 16])
+    windows = rng.choice([[None], [None], [None, 24], [40]])
+    mgr = CacheManager([GroupSpec(w) for w in windows], num_pages=rng.randint(6, 20), page_size=ps, num_slots=5,
+                       prefix_caching=rng.random() < 0.7)
+    prefix = [rng.randrange(50) for _ in range(3 * ps)]
+    live = []
+    for _ in range(400):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            rc = mgr.open()
+            assert rc is not None
+            toks = (prefix if rng.random() < 0.6 else []) + [rng.randrange(50) for _ in range(rng.randint(1, 30))]
+            mgr.admit_prefix(rc, toks)
+            live.append((rc, toks))
+        elif op < 0.8 and live:
+            rc, toks = rng.choice(live)
+            n = rng.randint(1, 12)
+            target = min(rc.computed + n, len(toks))
+            if target == rc.computed:
+                toks.append(rng.randrange(50))
+                target += 1
+            if mgr.ensure(rc, target):
+                mgr.advance(rc, toks, target)
+            else:                                   # out of pages: recompute preemption of this request
+                mgr.release_pages(rc)
+                assert rc.computed == 0 and all(not t for t in rc.tables)
+        elif live:
+            rc, toks = live.pop(rng.randrange(len(live)))
+            mgr.close(rc)
+        mgr.check()
+        held = {}
+        for rc, _ in live:
+            for g, table in enumerate(rc.tables):
+                for page in table:
+                    if page >= 0:
+                        held[(g, page)] = held.get((g, page), 0) + 1
+        for (g, page), count in held.items():
+            assert mgr.pools[g].refcount(page) == count          # shared only through the prefix cache
+            if not mgr.prefix_caching:
+                assert count == 1
+        for g, pool in enumerate(mgr.pools):
+            referenced = sum(1 for page in range(pool.num_pages) if pool.refcount(page) > 0)
+            assert referenced == len([1 for (gg, _) in held if gg == g])
+            assert pool.available() == pool.num_pages - referenced
+    for rc, _ in live:
+        mgr.close(rc)
+    assert mgr.all_free()
+
+
+def test_window_pages_are_given_back_as_the_window_passes():
+    mgr = CacheManager([GroupSpec(None), GroupSpec(20)], num_pages=16, page_size=8, num_slots=2)
+    assert not mgr.prefix_caching                                  # two groups: no prefix reuse
+    rc = mgr.open()
+    toks = list(range(100))
+    assert mgr.ensure(rc, 30)
+    mgr.advance(rc, toks, 30)
+    # next query at position 30 reads keys 11..30 in the windowed group: page 0 (keys 0-7) is gone
+    assert rc.tables[1][0] == -1 and rc.tables[1][1] >= 0 and all(p >= 0 for p in rc.tables[0])
+    assert mgr.free_pages(1) == 16 - 3 and mgr.free_pages(0) == 16 - 4
+    for target in range(31, 101):
+        assert mgr.ensure(rc, target)
+        mgr.advance(rc, toks, target)
+        live = [p for p in rc.tables[1] if p >= 0]
+        assert len(live) <= 20 // 8 + 2                            # the window plus partial pages at both ends
+        first = (target - 20 + 1) // 8 if target >= 20 else 0
+        assert all(p == -1 for p in rc.tables[1][:first]) and all(p >= 0 for p in rc.tables[1][first:])
+    assert len([p for p in rc.tables[0] if p >= 0]) == 13
+    mgr.close(rc)
+    assert mgr.all_free()
+
+
+def test_prefix_reuse_rules():
+    mgr = CacheManager([GroupSpec(None)], num_pages=8, page_size=8, num_slots=3)
+    toks = list(range(24)) + [99]
+    a = mgr.open()
+    assert mgr.admit_prefix(a, toks) == 0
+    assert mgr.ensure(a, 25)
+    mgr.advance(a, toks, 25)
+    assert len(a.hashes) == 3                                       # only full pages are registered
+    b = mgr.open()
+    assert mgr.admit_prefix(b, toks) == 24 and b.tables[0] == a.tables[0][:3]
+    c = mgr.open()
+    assert mgr.admit_prefix(c, toks[:24]) == 16                    # the page of the last token is computed
+    assert mgr.admit_prefix(c, toks[:24]) == 16                    # asking again takes nothing more
+    assert mgr.pools[0].refcount(a.tables[0][0]) == 3
+    for rc in (a, b, c):
+        mgr.close(rc)
+    assert mgr.free_pages() == 8
+    d = mgr.open()                                                  # cached pages outlive their requests
+    assert mgr.admit_prefix(d, toks) == 24
+    mgr.close(d)
+    off = CacheManager([GroupSpec(None)], 8, 8, 2, prefix_caching=True, has_state=True)
+    assert not off.prefix_caching                                   # state outside the pages cannot be reused

@@ -1,0 +1,209 @@
+"""Trace replay on the GPU: the same requests whole, with the last 32 tokens one by one, in
+portions of changing size, and mixed with other requests so that pages are used again, in
+32-bit and in bfloat16, each compared with the plain implementation; and the cuttings
+compared with each other bit for bit, which is what the reference's own chunking test asks
+(tests/test_main.cpp:219-228)."""
+
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+import tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parents[1]
+
+# Largest allowed |engine - plain| relative to the largest |logit| of the request.  32-bit: a few
+# units of 2^-24 per accumulation.  bfloat16: activations are rounded to 8 bits of mantissa at the
+# same places in both, but probabilities are rounded against a partition's maximum in the engine and
+# against the row's maximum in the plain code, and accumulation orders differ.
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+
+
+def requests_for(cfg, seed, lengths):
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def plain_logits(folder, toks, dtype):
+    cfg, w = tiny.read_config(folder), tiny.read_weights(folder)
+    return pl.forward(cfg, w, toks, pl.round_bf16 if dtype == "bfloat16" else pl.identity).numpy()
+
+
+def replay(folder, dtype, name, steps, max_tokens, **kw):
+    """Run steps through a Replayer; returns {request: [len, vocab] logits} (every position wanted)."""
+    from bitwise_amd.replay import Replayer
+
+    rp = Replayer(str(folder), dtype, max_tokens, block_size=tiny.CONFIGS[name][3], **kw)
+    out = {}
+    for st in steps:
+        lg = rp.step(st["entries"], st.get("end", []))
+        row = 0
+        for e in st["entries"]:
+            for _ in e["want"]:
+                out.setdefault(e["id"], []).append(lg[row])
+                row += 1
+    assert rp.manager.all_free() or any(True for _ in rp.live)
+    return {k: np.stack(v) for k, v in out.items()}, rp
+
+
+def all_wanted(rid, toks):
+    return {"id": rid, "tokens": toks, "want": list(range(len(toks)))}
+
+
+def cut(toks, sizes):
+    out, pos = [], 0
+    for s in sizes:
+        out.append(toks[pos:pos + s])
+        pos += s
+    assert pos == len(toks)
+    return out
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, gpu):
+    tmp = tmp_path_factory.mktemp("models")
+    return {n: tiny.make_folder(tmp, n) for n in ("A", "B", "LONG")}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_cuttings_equal_plain_and_each_other(folders, name, dtype):
+    cfg = tiny.read_config(folders[name])
+    lengths = [100, 67, 41, 33]
+    reqs = requests_for(cfg, 11, lengths)
+    page = tiny.CONFIGS[name][3]
+    refs = {rid: plain_logits(folders[name], toks, dtype) for rid, toks in reqs.items()}
+
+    # 1. each request alone and whole
+    whole = {}
+    for rid, toks in reqs.items():
+        got, _ = replay(folders[name], dtype, name, [{"entries": [all_wanted(rid, toks)], "end": [rid]}], 128)
+        whole[rid] = got[rid]
+        scale = np.abs(refs[rid]).max()
+        err = np.abs(got[rid] - refs[rid]).max()
+        assert err <= TOL[dtype] * scale, f"{rid} whole: err {err:.3e} vs scale {scale:.3f}"
+
+    # 2. most of it in one step, the last 32 tokens one by one
+    for rid, toks in reqs.items():
+        n = len(toks)
+        steps = [{"entries": [all_wanted(rid, toks[:n - 32])]}]
+        steps += [{"entries": [{"id": rid, "tokens": [toks[i]], "want": [0]}]} for i in range(n - 32, n)]
+        for use_graphs in (True, False):
+            got, _ = replay(folders[name], dtype, name, steps, 128, use_graphs=use_graphs)
+            assert np.array_equal(got[rid], whole[rid]), f"{rid}: decoding differs from the whole prompt (graphs={use_graphs})"
+
+    # 3. portions of changing size, down to two tokens and one
+    sizes = {100: [3, 17, 1, 19, 2, 30, 2, 26], 67: [2, 2, 31, 1, 1, 30], 41: [40, 1], 33: [16, 16, 1]}
+    for rid, toks in reqs.items():
+        steps = [{"entries": [all_wanted(rid, part)]} for part in cut(toks, sizes[len(toks)])]
+        got, _ = replay(folders[name], dtype, name, steps, 128)
+        assert np.array_equal(got[rid], whole[rid]), f"{rid}: portions differ from the whole prompt"
+
+    # 4. mixed: up to four live requests, portions of some beside decoded tokens of others, and
+    # so few pages that finished requests' pages are used again
+    ids = list(reqs)
+    progress = {rid: 0 for rid in ids}
+    plan = {ids[0]: [30, 1, 1, 1, 20, 1, 1, 45], ids[1]: [2, 5, 1, 1, 1, 57], ids[2]: [41], ids[3]: [1, 1, 31]}
+    order = [[ids[0]], [ids[0], ids[1]], [ids[0], ids[1], ids[2]], [ids[1], ids[0]], [ids[0], ids[1]],
+             [ids[0], ids[1]], [ids[1], ids[0]], [ids[0]]]
+    steps, ended = [], set()
+    cursor = {rid: 0 for rid in ids}
+    for group in order:
+        entries, end = [], []
+        for rid in group:
+            part = plan[rid][cursor[rid]]
+            cursor[rid] += 1
+            toks = reqs[rid][progress[rid]:progress[rid] + part]
+            progress[rid] += part
+            entries.append(all_wanted(rid, toks))
+            if progress[rid] == len(reqs[rid]):
+                end.append(rid)
+                ended.add(rid)
+        steps.append({"entries": entries, "end": end})
+    # the fourth request arrives after the third has gone, into its pages
+    for part in plan[ids[3]]:
+        toks = reqs[ids[3]][progress[ids[3]]:progress[ids[3]] + part]
+        progress[ids[3]] += part
+        steps.append({"entries": [all_wanted(ids[3], toks)], "end": [ids[3]] if progress[ids[3]] == 33 else []})
+    assert all(progress[r] == len(reqs[r]) for r in ids)
+    max_tokens = 128 + 128 + 64            # a, b and one of c/d, each rounded up to 64: pages must come back
+    got, rp = replay(folders[name], dtype, name, steps, max_tokens)
+    assert rp.manager.all_free()
+    for rid in ids:
+        assert np.array_equal(got[rid], whole[rid]), f"{rid}: the mixed batch differs from the whole prompt"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_and_partition_edges(folders, dtype):
+    """Hundreds of keys: partitions of 64 keys, pages of 16, the split route of decoded tokens
+    (from 256 keys on) and graph replay, all against the plain implementation and each other."""
+    name = "LONG"
+    cfg = tiny.read_config(folders[name])
+    toks = requests_for(cfg, 3, [700])["r0"]
+    ref = plain_logits(folders[name], toks, dtype)
+    whole, _ = replay(folders[name], dtype, name, [{"entries": [all_wanted("x", toks)]}], 704)
+    scale = np.abs(ref).max()
+    err = np.abs(whole["x"] - ref).max(axis=1)
+    assert err.max() <= TOL[dtype] * scale, f"worst at position {err.argmax()}: {err.max():.3e} vs {scale:.3f}"
+    # prompt of 250 tokens, then one by one across the 256-key threshold and several partition edges
+    steps = [{"entries": [all_wanted("x", toks[:250])]}]
+    steps += [{"entries": [{"id": "x", "tokens": [toks[i]], "want": [0]}]} for i in range(250, 400)]
+    steps += [{"entries": [all_wanted("x", toks[400:447])]}, {"entries": [all_wanted("x", toks[447:449])]}]
+    steps += [{"entries": [{"id": "x", "tokens": [toks[i]], "want": [0]}]} for i in range(449, 700)]
+    for use_graphs in (True, False):
+        got, _ = replay(folders[name], dtype, name, steps, 704, use_graphs=use_graphs)
+        same = (got["x"] == whole["x"]).all(axis=1)
+        assert same.all(), f"first differing position {int(np.argmin(same))} (graphs={use_graphs})"
+
+
+def test_first_tokens_of_a_sequence(folders):
+    """Positions 0 and 1: one key, no rotation at position 0."""
+    for name in ("A", "B"):
+        for dtype in ("float32", "bfloat16"):
+            cfg = tiny.read_config(folders[name])
+            toks = requests_for(cfg, 5, [3])["r0"]
+            ref = plain_logits(folders[name], toks, dtype)
+            one, _ = replay(folders[name], dtype, name, [{"entries": [{"id": "a", "tokens": toks[:1], "want": [0]}]},
+                                                       {"entries": [{"id": "a", "tokens": toks[1:2], "want": [0]}]},
+                                                       {"entries": [{"id": "a", "tokens": toks[2:], "want": [0]}]}], 64)
+            assert np.abs(one["a"] - ref).max() <= TOL[dtype] * np.abs(ref).max()
+
+
+def test_trace_run_program(folders, tmp_path):
+    """bin/trace_run as a user calls it: JSON steps on standard input, <step>.f32 files, a
+    'done <step>' line after every step, exit 0; a request may pause and pages are reused."""
+    name, dtype = "B", "bfloat16"
+    cfg = tiny.read_config(folders[name])
+    reqs = requests_for(cfg, 21, [50, 20, 70])
+    a, b, c = reqs["r0"], reqs["r1"], reqs["r2"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b, "want": [19]}, {"id": "a", "tokens": a[30:32], "want": []}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "c", "tokens": c[:64], "want": [63]}], "end": []},                  # a pauses
+        {"step": 3, "entries": [{"id": "a", "tokens": a[32:33], "want": [0]}, {"id": "c", "tokens": c[64:], "want": [5]}], "end": ["c"]},
+        {"step": 4, "entries": [{"id": "a", "tokens": a[33:], "want": [16]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    env = dict(os.environ, PYTHONPATH=str(ROOT))
+    p = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folders[name]), "--dtype", dtype,
+                        "--out", str(out), "--max-tokens", "192", "--block-size", "8"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, env=env,
+                       timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3", "done", "4"]
+    V = cfg["vocab_size"]
+    ra, rb, rc = (plain_logits(folders[name], t, dtype) for t in (a, b, c))
+    want = {0: [ra[0], ra[29]], 1: [rb[19]], 2: [rc[63]], 3: [ra[32], rc[69]], 4: [ra[49]]}
+    for step, rows in want.items():
+        got = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, V)
+        assert got.shape[0] == len(rows)
+        for g, r in zip(got, rows):
+            assert np.abs(g - r).max() <= TOL[dtype] * np.abs(r).max()
