@@ -1,0 +1,149 @@
+"""The engine on the GPU: greedy and sampled generation through the entry point against the
+plain implementation, crowded batches against solo runs to the last bit, long decoding, and
+randomized scheduling traces (the reference's engine test and simulator,
+tests/test_main.cpp:241-302, sim/simulate.cpp)."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import bitwise_amd as bw
+import plain_llama as pl
+import tiny
+from bitwise_amd.sim import Simulator
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, gpu):
+    tmp = tmp_path_factory.mktemp("models")
+    return {n: tiny.make_folder(tmp, n) for n in ("A", "B")}
+
+
+def engine_config(name, dtype, **kw):
+    base = dict(num_blocks=64, block_size=tiny.CONFIGS[name][3], dtype=dtype)
+    base.update(kw)
+    return bw.EngineConfig(**base)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generation_equals_plain(folders, name, dtype):
+    """Greedy and temperature sampling through bw.generate: the tokens of the plain
+    implementation, which recomputes the whole sequence for every token."""
+    cfg, w = tiny.read_config(folders[name]), tiny.read_weights(folders[name])
+    model = bw.Model.load(folders[name], dtype)
+    rnd = pl.round_bf16 if dtype == "bfloat16" else pl.identity
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (1, 7, 19, 33)]
+    params = [bw.SamplingParams(max_new_tokens=16, ignore_eos=True),
+              bw.SamplingParams(max_new_tokens=12, temperature=0.8, seed=5, ignore_eos=True),
+              bw.SamplingParams(max_new_tokens=16), bw.SamplingParams(max_new_tokens=10, temperature=1.3, seed=9)]
+    results = bw.generate(model, prompts, params, engine_config(name, dtype, max_batched_tokens=24))
+    for p, sp, r in zip(prompts, params, results):
+        want = pl.generate(cfg, w, p, sp.max_new_tokens, sp.temperature, sp.seed, sp.ignore_eos, rnd)
+        assert r.tokens == want and r.finished
+    assert model.config.num_key_value_heads == cfg["num_key_value_heads"] and model.weight_bytes > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_crowded_engine_equals_solo_to_the_last_bit(folders, dtype):
+    """Six requests that share a 24-token prefix, sampled at temperature 0.8 with seeds 0-5, in
+    a pool so tight that prefixes are reused and at least one request is preempted and
+    recomputed: tokens and logits fingerprints equal each request run alone."""
+    name = "B"
+    cfg = tiny.read_config(folders[name])
+    model = bw.Model.load(folders[name], dtype)
+    g = torch.Generator().manual_seed(6)
+    shared = torch.randint(0, 500, (24,), generator=g).tolist()
+    prompts = [shared + torch.randint(0, 500, (n,), generator=g).tolist() for n in (0, 8, 16, 24, 32, 40)]
+    params = [bw.SamplingParams(temperature=0.8, seed=s, max_new_tokens=20, ignore_eos=True) for s in range(6)]
+    solo = []
+    for p, sp in zip(prompts, params):
+        (r,) = bw.generate(model, [p], sp, engine_config(name, dtype, prefix_caching=False, max_batched_tokens=256))
+        solo.append(r)
+    for tight in (dict(num_blocks=14, max_batched_tokens=32), dict(num_blocks=64, max_batched_tokens=24)):
+        eng = bw.Engine(model, None, engine_config(name, dtype, **tight))
+        ids = [eng.add_request(p, sp) for p, sp in zip(prompts, params)]
+        guard = 0
+        while not eng.idle():
+            eng.step()
+            guard += 1
+            assert guard < 5000, eng.debug_state()
+        for i, ref in zip(ids, solo):
+            assert eng.result(i).tokens == ref.tokens
+            assert eng.result(i).logits_fingerprint == ref.logits_fingerprint
+        assert eng.free_blocks == tight["num_blocks"]
+        assert eng.stats.prefix_hit_tokens > 0
+        if tight["num_blocks"] == 14:
+            assert eng.stats.preemptions > 0
+
+
+def test_long_decoding_with_and_without_graphs(folders):
+    """200 decoded tokens: graph replay and kernel-by-kernel launches give the same tokens and
+    fingerprints, and the tokens are those of the plain implementation."""
+    name, dtype = "A", "bfloat16"
+    cfg, w = tiny.read_config(folders[name]), tiny.read_weights(folders[name])
+    cfg_long = dict(cfg, max_position_embeddings=256)
+    folder = folders[name].parent / "tiny_A_long"
+    bw.write_random_model(folder, cfg_long, 0, 0.02)
+    model = bw.Model.load(folder, dtype)
+    prompt = [3, 14, 15, 92, 65]
+    sp = bw.SamplingParams(max_new_tokens=100, ignore_eos=True, temperature=0.9, seed=3)
+    outs = []
+    for graphs in (True, False):
+        (r,) = bw.generate(model, [prompt], sp, engine_config(name, dtype, use_graphs=graphs))
+        outs.append(r)
+    assert outs[0].tokens == outs[1].tokens and outs[0].logits_fingerprint == outs[1].logits_fingerprint
+    want = pl.generate(cfg_long, tiny.read_weights(folder), prompt, 100, 0.9, 3, True, pl.round_bf16)
+    assert outs[0].tokens == want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_randomized_traces(gpu, dtype):
+    """The reference's simulator (sim/simulate.cpp) on the real engine: 0 token or logit
+    mismatches, no hang, no leaked page, and the traces must reach preemption and prefix hits."""
+    from bitwise_amd.cli import TINY_SIM_CONFIG
+
+    model = bw.Model.random(TINY_SIM_CONFIG, 42, dtype, sigma=0.08)
+    out = Simulator(model, dtype, block_size=16).run(traces=12, seed=1)
+    assert out.violations() == 0, "\n".join(out.notes[:10])
+    assert out.requests_checked > 20 and out.preemptions > 0 and out.prefix_hits > 0
+
+
+def test_command_line(folders):
+    p = subprocess.run([sys.executable, "-m", "bitwise_amd", "generate", "--model", str(folders["A"]), "--dtype",
+                        "float32", "--prompt-tokens", "5,17,3", "--prompt-tokens", "9", "--max-new-tokens", "6",
+                        "--ignore-eos"], capture_output=True, text=True, cwd=str(ROOT), timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [json.loads(l) for l in p.stdout.strip().splitlines()]
+    cfg, w = tiny.read_config(folders["A"]), tiny.read_weights(folders["A"])
+    assert lines[0]["tokens"] == pl.generate(cfg, w, [5, 17, 3], 6, ignore_eos=True)
+    assert lines[1]["tokens"] == pl.generate(cfg, w, [9], 6, ignore_eos=True)
+    p = subprocess.run([sys.executable, "-m", "bitwise_amd", "generate", "--nonsense"], capture_output=True, text=True,
+                       cwd=str(ROOT), timeout=120)
+    assert p.returncode == 2
+
+
+def test_model_errors(folders, tmp_path):
+    with pytest.raises(bw.ConfigError, match="cannot open"):
+        bw.Model.load(tmp_path / "missing")
+    model = bw.Model.load(folders["A"], "float32")
+    with pytest.raises(ValueError, match="loaded as float32"):
+        bw.Engine(model, None, bw.EngineConfig(dtype="bfloat16"))
+    eng = bw.Engine(model, None, bw.EngineConfig(dtype="float32", num_blocks=4))
+    with pytest.raises(ValueError, match="never fit"):
+        eng.add_request(list(range(60)), bw.SamplingParams(max_new_tokens=8))
+    with pytest.raises(ValueError, match="model length"):
+        bw.Engine(model, None, bw.EngineConfig(dtype="float32", num_blocks=64)).add_request(
+            list(range(100)), bw.SamplingParams(max_new_tokens=60))
+    bad = dict(tiny.TINY_A, head_dim=24, hidden_size=96)
+    with pytest.raises(ValueError, match="head size 24 is not supported"):
+        bw.Model.random(bad, 0, "float32")

@@ -1,0 +1,402 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine's, with
+inputs built so that a fault shows: a far key among hundreds, a window's edge, a page's edge,
+poisoned memory that must not be read."""
+
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+from bitwise_amd.csrc import ops
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+
+
+def f32_round(fr: Fraction) -> np.float32:
+    """Round an exact rational to the nearest float32, ties to even."""
+    c = np.float32(float(fr))
+    best = c
+    for cand in (np.nextafter(c, np.float32(-np.inf)), np.nextafter(c, np.float32(np.inf))):
+        d_c, d_n = abs(Fraction(float(best)) - fr), abs(Fraction(float(cand)) - fr)
+        if d_n < d_c or (d_n == d_c and (cand.view(np.uint32) & 1) == 0):
+            best = cand
+    return best
+
+
+def fma32(a, b, c) -> np.float32:
+    return f32_round(Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c)))
+
+
+def chain_dot(x, w) -> np.float32:
+    """acc = fma(x[k], w[k], acc) for k ascending from 0.0f (src/kernels.cpp:236-244)."""
+    acc = np.float32(0.0)
+    for a, b in zip(x, w):
+        acc = fma32(a, b, acc)
+    return acc
+
+
+def canonical_sumsq(x) -> np.float32:
+    """16 chains lane = i % 16, then the fixed tree (src/kernels.cpp:57-64, tests/test_main.cpp:126-131)."""
+    lane = [np.float32(0.0)] * 16
+    for i, v in enumerate(x):
+        lane[i % 16] = fma32(v, v, lane[i % 16])
+    s8 = [np.float32(lane[i] + lane[i + 8]) for i in range(8)]
+    s4 = [np.float32(s8[i] + s8[i + 4]) for i in range(4)]
+    return np.float32(np.float32(s4[0] + s4[2]) + np.float32(s4[1] + s4[3]))
+
+
+# ----------------------------------------------------------------------------- matrix products
+
+def test_gemm_f32_is_the_scalar_chain_bit_for_bit(gpu):
+    g = torch.Generator().manual_seed(1)
+    for M, N, K in [(1, 1, 1), (2, 3, 33), (3, 17, 16), (5, 2, 70)]:
+        x, w = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g)
+        y = torch.zeros(M, N, device=gpu)
+        ops.gemm_f32(x.to(gpu), w.to(gpu), y, M)
+        want = np.array([[chain_dot(x[m].numpy(), w[n].numpy()) for n in range(N)] for m in range(M)], np.float32)
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32)), (M, N, K)
+
+
+def test_gemm_f32_grid_rows_and_accumulate(gpu):
+    """The reference's shape grid (tests/test_main.cpp:75-77) against float64, every row equal
+    to the same row computed alone (tests/test_main.cpp:95-120), bfloat16 weights widened."""
+    g = torch.Generator().manual_seed(2)
+    for M in (1, 2, 3, 4, 5, 7, 13, 50):
+        for N in (1, 15, 16, 17, 100, 300):
+            for K in (1, 16, 33, 64, 600):
+                x, w = torch.randn(M, K, generator=g).to(gpu), torch.randn(N, K, generator=g).to(gpu)
+                y = torch.full((M, N), 7.0, device=gpu)
+                ops.gemm_f32(x, w, y, M)
+                ref = x.double() @ w.double().T
+                assert (y.double() - ref).abs().max() <= 1e-6 * K ** 0.5 * ref.abs().max().clamp(min=1.0)
+    x, w = torch.randn(9, 1024, generator=g).to(gpu), torch.randn(200, 1024, generator=g).to(gpu)
+    wb = w.bfloat16()
+    batch, one = torch.zeros(9, 200, device=gpu), torch.zeros(1, 200, device=gpu)
+    for weight in (w, wb):
+        ops.gemm_f32(x, weight, batch, 9)
+        for r in range(9):
+            ops.gemm_f32(x[r:r + 1].contiguous(), weight, one, 1)
+            assert torch.equal(one[0], batch[r])
+    assert torch.allclose(batch.double(), x.double() @ wb.double().T, rtol=0, atol=1e-4)
+    before = batch.clone()
+    ops.gemm_f32(x, wb, batch, 9, accumulate=True)
+    assert torch.equal(batch, before + before)                     # y + acc, one addition per output
+
+
+def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
+    g = torch.Generator().manual_seed(3)
+    for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40)]:
+        x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+        w = torch.randn(N, K, generator=g).bfloat16().to(gpu)
+        y = torch.full((M, N), 3.0, device=gpu)
+        ops.gemm_bf16(x, w, y, M, ops.EPI_F32)
+        ref = x.double() @ w.double().T
+        assert (y.double() - ref).abs().max() <= 2e-6 * K ** 0.5 * ref.abs().max()
+        one = torch.zeros(1, N, device=gpu)
+        for r in range(0, M, max(1, M // 7)):                      # the skinny and the wide kernel agree bit for bit
+            ops.gemm_bf16(x[r:r + 1].contiguous(), w, one, 1, ops.EPI_F32)
+            assert torch.equal(one[0], y[r]), (M, N, K, r)
+        yb = torch.zeros(M, N, device=gpu, dtype=torch.bfloat16)
+        ops.gemm_bf16(x, w, yb, M, ops.EPI_BF16)
+        assert torch.equal(yb, y.bfloat16())
+        res = torch.randn(M, N, generator=g).to(gpu)
+        acc = res.clone()
+        ops.gemm_bf16(x, w, acc, M, ops.EPI_ADD_F32)
+        assert torch.equal(acc, res + y)
+    M, inter, K = 19, 56, 96
+    x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+    wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
+    h = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_bf16(x, wgu, h, M, ops.EPI_SWIGLU_BF16)
+    gate, up = x.double() @ wgu[:inter].double().T, x.double() @ wgu[inter:].double().T
+    want = pl.swiglu(gate.cpu(), up.cpu())
+    assert (h.cpu().double() - want).abs().max() <= 2 ** -8 * want.abs().max()     # one bfloat16 rounding
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ops.gemm_bf16(torch.zeros(2, 12, device=gpu, dtype=torch.bfloat16),
+                      torch.zeros(4, 12, device=gpu, dtype=torch.bfloat16), torch.zeros(2, 4, device=gpu), 2, ops.EPI_F32)
+
+
+# ----------------------------------------------------------------------------- row kernels
+
+def test_rmsnorm(gpu):
+    g = torch.Generator().manual_seed(4)
+    for rows, dim, eps in [(1, 1, 1e-5), (3, 33, 1e-6), (7, 96, 1e-5), (21, 100, 0.5), (5, 2048, 1e-5)]:
+        x, w = torch.randn(rows, dim, generator=g) * 3, torch.randn(dim, generator=g)
+        o32 = torch.zeros(rows, dim, device=gpu)
+        ob = torch.zeros(rows, dim, device=gpu, dtype=torch.bfloat16)
+        ops.rmsnorm(x.to(gpu), w.to(gpu), o32, rows, eps)
+        ops.rmsnorm(x.to(gpu), w.bfloat16().to(gpu), ob, rows, eps)
+        ref = pl.rmsnorm(x.double(), w, eps)
+        assert (o32.cpu().double() - ref).abs().max() <= 4e-7 * ref.abs().max()
+        refb = pl.rmsnorm(x.double(), w.bfloat16(), eps)
+        assert (ob.cpu().double() - refb).abs().max() <= 2 ** -8 * refb.abs().max()
+        if dim <= 100:                                             # the canonical order, bit for bit
+            for r in range(min(rows, 2)):
+                xr = x[r].numpy()
+                ss = canonical_sumsq(xr)
+                inv = np.float32(1.0) / np.sqrt(np.float32(ss / np.float32(dim) + np.float32(eps)), dtype=np.float32)
+                want = (xr * inv) * w.numpy()
+                assert np.array_equal(o32[r].cpu().numpy().view(np.uint32), want.astype(np.float32).view(np.uint32))
+    z = torch.zeros(2, 64, device=gpu)
+    out = torch.ones(2, 64, device=gpu)
+    ops.rmsnorm(z, torch.ones(64, device=gpu), out, 2, 1e-5)
+    assert torch.equal(out, z)                                     # x = 0 gives exactly 0
+
+
+def test_embed_gather_swiglu_add(gpu):
+    g = torch.Generator().manual_seed(5)
+    table = torch.randn(37, 24, generator=g).bfloat16().to(gpu)
+    toks = torch.tensor([5, 0, 36, -1, 5], dtype=torch.int32, device=gpu)
+    out = torch.full((5, 24), 9.0, device=gpu)
+    ops.embed(toks, table, out)
+    assert torch.equal(out[[0, 1, 2, 4]], table.float()[[5, 0, 36, 5]]) and torch.equal(out[3], torch.zeros(24, device=gpu))
+    table32 = torch.randn(37, 24, generator=g).to(gpu)
+    ops.embed(toks[:3].contiguous(), table32, out)
+    assert torch.equal(out[:3], table32[[5, 0, 36]])
+    x = torch.randn(11, 40, generator=g).to(gpu)
+    idx = torch.tensor([10, 0, 3, 3], dtype=torch.int32, device=gpu)
+    got = torch.zeros(4, 40, device=gpu)
+    ops.gather_rows(x, idx, got, 4)
+    assert torch.equal(got, x[[10, 0, 3, 3]])
+    gu = torch.randn(6, 2 * 28, generator=g).to(gpu) * 4
+    gu[0, 0], gu[0, 1], gu[0, 2] = 0.0, 40.0, -40.0
+    h = torch.zeros(6, 28, device=gpu)
+    ops.swiglu_f32(gu, h, 6)
+    want = pl.swiglu(gu[:, :28].double().cpu(), gu[:, 28:].double().cpu())
+    assert (h.cpu().double() - want).abs().max() <= 3e-7 * want.abs().max()
+    assert h[0, 0] == 0 and abs(h[0, 1].item() - 40.0 * gu[0, 29].item()) < 1e-4 and abs(h[0, 2].item()) < 1e-12
+    a, b = torch.randn(5, 16, generator=g).to(gpu), torch.randn(5, 16, generator=g).to(gpu)
+    s = a.clone()
+    ops.add_(s, b, 4)
+    assert torch.equal(s[:4], a[:4] + b[:4]) and torch.equal(s[4], a[4])
+
+
+def rope_tables(theta, hd, n, gpu):
+    inv = pl.rope_inv_freq(theta, hd)
+    ang = (np.arange(n, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float32).astype(np.float64)
+    return (torch.from_numpy(np.cos(ang).astype(np.float32)).to(gpu), torch.from_numpy(np.sin(ang).astype(np.float32)).to(gpu))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_rope_and_cache_write(gpu, bf16):
+    g = torch.Generator().manual_seed(6)
+    heads, kvh, hd, page, pages = 3, 2, 48, 8, 9
+    cos, sin = rope_tables(50000.0, hd, 80, gpu)
+    positions = [0, 1, 7, 8, 63, 70]
+    rows = len(positions)
+    width = (heads + 2 * kvh) * hd
+    qkv = torch.randn(rows, width, generator=g)
+    table = torch.tensor([[8, 2, 5, 0, 7, 1, 3, 6, 4], [4, 6, 3, 1, 7, 0, 5, 2, 8]], dtype=torch.int32, device=gpu)
+    row_seq = torch.tensor([0, 0, 1, 1, 0, 1], dtype=torch.int32, device=gpu)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    poison = 1e30
+    kc = torch.full((pages, kvh * page * hd), poison, dtype=dt, device=gpu)
+    vc = torch.full((pages, kvh * page * hd), poison, dtype=dt, device=gpu)
+    dev = qkv.to(gpu).clone()
+    q_out = torch.zeros(rows, heads * hd, dtype=torch.bfloat16, device=gpu) if bf16 else None
+    ops.rope_kvwrite(dev, q_out, torch.tensor(positions, dtype=torch.int32, device=gpu), row_seq, table, cos, sin,
+                     kc, vc, rows, heads, kvh, hd, page)
+    inv = pl.rope_inv_freq(50000.0, hd)
+    q_ref = pl.rope(qkv[:, :heads * hd].double().view(rows, heads, hd), positions, inv)
+    k_ref = pl.rope(qkv[:, heads * hd:(heads + kvh) * hd].double().view(rows, kvh, hd), positions, inv)
+    v_ref = qkv[:, (heads + kvh) * hd:].double().view(rows, kvh, hd)
+    tol = 2 ** -8 if bf16 else 2e-7
+    q_got = (q_out if bf16 else dev[:, :heads * hd]).cpu().double().view(rows, heads, hd)
+    assert (q_got - q_ref).abs().max() <= tol * q_ref.abs().max()
+    if bf16:
+        assert torch.equal(q_out[0], qkv[0, :heads * hd].bfloat16().to(gpu))          # position 0: no rotation
+    else:
+        assert torch.equal(dev[0, :(heads + kvh) * hd], qkv[0, :(heads + kvh) * hd].to(gpu))
+    kc4 = kc.view(pages, kvh, page, hd).cpu().double()
+    vc4 = (vc.view(pages, kvh, hd, page).transpose(2, 3) if bf16 else vc.view(pages, kvh, page, hd)).cpu().double()
+    written = set()
+    for r, p in enumerate(positions):
+        pg = int(table[int(row_seq[r]), p // page])
+        assert (kc4[pg, :, p % page] - k_ref[r]).abs().max() <= tol * k_ref.abs().max()
+        ref_v = v_ref[r].bfloat16().double() if bf16 else v_ref[r]
+        assert torch.equal(vc4[pg, :, p % page], ref_v)                              # v is stored untouched
+        written.add((pg, p % page))
+    for pg in range(pages):
+        for s in range(page):
+            if (pg, s) not in written:
+                assert (kc4[pg, :, s] == torch.tensor(poison).to(dt).double()).all()      # nothing else was touched
+
+
+# ----------------------------------------------------------------------------- attention
+
+def paged_setup(gpu, bf16, heads, kvh, hd, page, pages, n_keys, seed, poison=False):
+    """A sequence of n_keys keys and values scattered over pages by the reference's table
+    (i*7+3) % pages (tests/test_main.cpp:146-147); everything else is poison."""
+    g = torch.Generator().manual_seed(seed)
+    k, v = torch.randn(n_keys, kvh, hd, generator=g), torch.randn(n_keys, kvh, hd, generator=g)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    k, v = k.to(dt), v.to(dt)
+    fill = float("nan") if poison else 0.0
+    kc = torch.full((pages, kvh, page, hd), fill, dtype=dt)
+    vc = torch.full((pages, kvh, page, hd), fill, dtype=dt)
+    n_pages = (n_keys + page - 1) // page
+    table = [(i * 7 + 3) % pages for i in range(n_pages)]
+    assert len(set(table)) == n_pages
+    for j in range(n_keys):
+        kc[table[j // page], :, j % page] = k[j]
+        vc[table[j // page], :, j % page] = v[j]
+    if bf16:
+        vc = vc.transpose(2, 3).contiguous()
+    tab = torch.tensor([table], dtype=torch.int32, device=gpu)
+    return k, v, kc.reshape(pages, -1).to(gpu), vc.reshape(pages, -1).to(gpu), tab
+
+
+def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=0, split=False, tiles=None):
+    rows = len(positions)
+    pos = torch.tensor(positions, dtype=torch.int32, device=gpu)
+    scale = 1.0 / float(hd) ** 0.5
+    if not bf16:
+        out = torch.zeros(rows, heads * hd, device=gpu)
+        ops.attention_f32(q.to(gpu), pos, torch.zeros(rows, dtype=torch.int32, device=gpu), tab, kc, vc, out, rows,
+                          heads, kvh, hd, page, window, scale)
+        return out
+    out = torch.zeros(rows, heads * hd, device=gpu, dtype=torch.bfloat16)
+    if tiles is None:
+        tiles = [(r, 1, 0, 0) for r in range(rows)]
+    t = torch.tensor(tiles, dtype=torch.int32, device=gpu)
+    kw = {}
+    if split:
+        max_parts = max(positions) // ops.ATT_PART + 1
+        group = heads // kvh
+        cols = kvh * ((group + 15) // 16) * min(group, 16)
+        kw = dict(split=True, max_parts=max_parts, part_o=torch.empty(len(tiles) * max_parts * cols * hd, device=gpu),
+                  part_ml=torch.empty(len(tiles) * max_parts * cols * 2, device=gpu))
+    ops.attention_bf16(q.to(gpu), pos, tab, t, len(tiles), kc, vc, out, heads, kvh, hd, page, window, scale, **kw)
+    return out
+
+
+def plain_rows(q, k, v, positions, heads, window=None):
+    """Row r is the query at positions[r] over keys 0..positions[r] of the same sequence."""
+    hd = q.shape[-1] // heads
+    out = []
+    for r, p in enumerate(positions):
+        qq = torch.zeros(p + 1, heads, hd, dtype=F64)
+        qq[p] = q[r].double().view(heads, hd)
+        out.append(pl.attention(qq, k[:p + 1].double(), v[:p + 1].double(), window=window)[p].reshape(-1))
+    return torch.stack(out)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("heads,kvh,hd,page", [(4, 2, 16, 16), (3, 1, 32, 8), (5, 5, 80, 32), (2, 1, 128, 16), (6, 2, 64, 64)])
+def test_attention_batched_equals_alone_and_plain(gpu, bf16, heads, kvh, hd, page):
+    """The reference's invariance test (tests/test_main.cpp:137-169): positions 0, 5, 17, 300,
+    301, 302, 511 in one batch equal each row alone, bit for bit; everything outside the
+    sequence's written slots is NaN and must not be read."""
+    pages = 512 // page + 5
+    while pages % 7 == 0:
+        pages += 1                                                 # the table (i*7+3) % pages must not repeat
+    k, v, kc, vc, tab = paged_setup(gpu, bf16, heads, kvh, hd, page, pages, 512, seed=7, poison=True)
+    positions = [0, 5, 17, 300, 301, 302, 511]
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(len(positions), heads * hd, generator=g).to(torch.bfloat16 if bf16 else torch.float32)
+    batch = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page)
+    assert torch.isfinite(batch.float()).all()
+    for r, p in enumerate(positions):
+        alone = run_attention(gpu, bf16, q[r:r + 1], [p], tab, kc, vc, heads, kvh, hd, page)
+        assert torch.equal(alone[0], batch[r]), f"position {p}"
+    ref = plain_rows(q, k, v, positions, heads)
+    tol = 1.5e-2 if bf16 else 3e-6
+    assert (batch.cpu().double() - ref).abs().max() <= tol * ref.abs().max()
+    first = v[0].double().repeat_interleave(heads // kvh, dim=0).reshape(-1)
+    assert torch.equal(batch[0].cpu().double(), first)            # one key: the output is its value, exactly
+    if bf16:                                                      # one wave per partition gives the same bits
+        sp = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
+        assert torch.equal(sp, batch)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_attention_prompt_tiles_equal_single_rows(gpu, bf16):
+    """Rows of a prompt portion share a tile with consecutive positions; each must equal the
+    same query run as a single decoded token."""
+    heads, kvh, hd, page = 6, 2, 32, 16
+    k, v, kc, vc, tab = paged_setup(gpu, bf16, heads, kvh, hd, page, 40, 200, seed=9, poison=True)
+    positions = list(range(120, 147))
+    g = torch.Generator().manual_seed(10)
+    q = torch.randn(len(positions), heads * hd, generator=g).to(torch.bfloat16 if bf16 else torch.float32)
+    tpt = 16 // (heads // kvh)
+    tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+    portion = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, tiles=tiles)
+    single = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page)
+    assert torch.equal(portion, single)
+    ref = plain_rows(q, k, v, positions, heads)
+    assert (portion.cpu().double() - ref).abs().max() <= (1.5e-2 if bf16 else 3e-6) * ref.abs().max()
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_attention_finds_a_far_key_and_respects_the_window(gpu, bf16):
+    """One key among hundreds is made to stand out by scaling it and the query: the output must
+    be that key's value.  With a window, the key just outside must be invisible however
+    attractive it is, and the key just inside visible."""
+    heads, kvh, hd, page, n = 2, 1, 64, 16, 700
+    k, v, kc, vc, tab = paged_setup(gpu, bf16, heads, kvh, hd, page, 50, n, seed=11)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    g = torch.Generator().manual_seed(12)
+    for far in (3, 64, 333, 448):                                  # in a first page, at partition and page edges, mid
+        q = torch.randn(1, heads * hd, generator=g)
+        kk = k.clone()
+        kk[far, 0] = (q[0, :hd] * 4).to(dt)                        # head 0 of the query loves key `far`
+        kc2 = kc.clone().view(50, kvh, page, hd)
+        kc2[(far // page * 7 + 3) % 50, 0, far % page] = kk[far, 0].to(gpu)
+        out = run_attention(gpu, bf16, q.to(dt), [n - 1], tab, kc2.view(50, -1), vc, heads, kvh, hd, page)
+        assert (out[0, :hd].cpu().double() - v[far, 0].double()).abs().max() < 0.05, f"key {far} not found"
+        ref = plain_rows(q.to(dt), kk, v, [n - 1], heads)
+        assert (out.cpu().double() - ref).abs().max() <= (1.5e-2 if bf16 else 3e-6) * ref.abs().max()
+        # window of 100 keys: the query at position far+99 still sees it, the one at far+100 does not
+        for p, visible in ((far + 99, True), (far + 100, False)):
+            if p >= n:
+                continue
+            w = run_attention(gpu, bf16, q.to(dt), [p], tab, kc2.view(50, -1), vc, heads, kvh, hd, page, window=100)
+            hit = (w[0, :hd].cpu().double() - v[far, 0].double()).abs().max() < 0.05
+            assert hit == visible, f"key {far} from position {p}: visible={hit}"
+            refw = plain_rows(q.to(dt), kk, v, [p], heads, window=100)
+            assert (w.cpu().double() - refw).abs().max() <= (1.5e-2 if bf16 else 3e-6) * refw.abs().max()
+
+
+def test_attention_refuses_what_it_cannot_do(gpu):
+    z = torch.zeros(1, 40, device=gpu)
+    i32 = torch.zeros(1, dtype=torch.int32, device=gpu)
+    with pytest.raises(ValueError, match="head size 40"):
+        ops.attention_f32(z, i32, i32, i32.view(1, 1), z, z, z, 1, 1, 1, 40, 16, 0, 1.0)
+    zb = torch.zeros(1, 64, device=gpu, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="page size"):
+        ops.attention_bf16(zb, i32, i32.view(1, 1), torch.zeros(1, 4, dtype=torch.int32, device=gpu), 1,
+                           torch.zeros(1, 64 * 24, device=gpu, dtype=torch.bfloat16),
+                           torch.zeros(1, 64 * 24, device=gpu, dtype=torch.bfloat16), zb, 1, 1, 64, 24, 0, 1.0)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.rmsnorm(torch.zeros(1, 8), torch.ones(8), torch.zeros(1, 8), 1, 1e-5)
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def test_sampling_and_fingerprint(gpu):
+    g = torch.Generator().manual_seed(13)
+    V = 501
+    logits = (torch.randn(9, V, generator=g) * 3).to(gpu)
+    logits[0, 7] = logits[0, 400] = 50.0                           # a tie: the first maximum wins
+    logits[1, V - 1] = 60.0
+    temps = [0.0, 0.0, -1.0, 0.8, 0.8, 1.5, 0.3, 1.0, 1.0]
+    us = [0.0, 0.0, 0.0, 0.0, 1.0 - 2 ** -53, 0.37, 0.99, 0.5, 0.123456789]
+    out = torch.zeros(9, dtype=torch.int32, device=gpu)
+    ops.sample(logits, 9, torch.tensor(temps, device=gpu), torch.tensor(us, dtype=torch.float64, device=gpu), out)
+    got = out.cpu().tolist()
+    host = logits.cpu().numpy()
+    assert got[0] == 7 and got[1] == V - 1
+    for r in range(9):
+        want = pl.argmax_row(host[r]) if temps[r] <= 0 else pl.sample_row(host[r], temps[r], us[r])
+        assert got[r] == want, f"row {r}"
+    for Vv in (500, 501, 6):
+        rows = torch.randn(3, Vv, generator=g).to(gpu)
+        basis = [1469598103934665603, 12345, 2 ** 64 - 1]
+        h_in = torch.from_numpy(np.asarray(basis, np.uint64).view(np.int64)).to(gpu)
+        h_out = torch.zeros(3, dtype=torch.int64, device=gpu)
+        ops.fingerprint(rows, 3, h_in, h_out)
+        want = [pl.hash_floats(b, rows[i].cpu().numpy()) for i, b in enumerate(basis)]
+        assert h_out.cpu().numpy().view(np.uint64).tolist() == want

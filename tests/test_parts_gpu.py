@@ -1,0 +1,261 @@
+"""Each part alone against the plain implementation, a toy mixer with state of its own that
+is registered, built and stepped without touching the framework, and schedules that name a
+layer twice or let a layer read another layer's cache."""
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+import tiny
+from bitwise_amd.cache.manager import CacheManager, GroupSpec
+from bitwise_amd.engine.batch import Segment, StepContext
+from bitwise_amd.engine.runner import ModelRunner
+from bitwise_amd.engine.storage import CacheStorage
+from bitwise_amd.models.assembled import AssembledModel, CallBinding
+from bitwise_amd.parts import base
+from bitwise_amd.parts.base import LayerCall, LayerSpec, ModelSpec, PartSpec, StateSpec, TensorSpec
+from bitwise_amd.runtime import Runtime
+from bitwise_amd.weights.loader import random_tensors
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
+
+
+def rnd_for(mode):
+    return pl.round_bf16 if mode == "bfloat16" else pl.identity
+
+
+def one_request_ctx(rt, n, groups=1, pages=None):
+    pages = pages if pages is not None else list(range((n + rt.page_size - 1) // rt.page_size))
+    return StepContext([Segment([0] * n, 0, [pages] * groups, 0, [])], groups, rt.device)
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_norm_part(gpu, mode):
+    rt = Runtime(mode, gpu, max_rows=32, page_size=8)
+    part = base.NORMS["rmsnorm"]({"width": 72, "eps": 1e-3}, rt)
+    assert part.tensors() == {"weight": TensorSpec((72,), "norm")}
+    w = 1 + 0.1 * torch.randn(72)
+    part.bind({"weight": w.bfloat16()})
+    x = torch.zeros(32, 72, device=gpu)
+    x[:5] = torch.randn(5, 72, device=gpu) * 2
+    out = part.forward(one_request_ctx(rt, 5), x)
+    assert out.dtype == rt.act_dtype
+    ref = pl.rmsnorm(x[:5].double().cpu(), w.bfloat16(), 1e-3)
+    assert (out[:5].cpu().double() - ref).abs().max() <= (2 ** -8 if mode == "bfloat16" else 4e-7) * ref.abs().max()
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_feed_forward_part(gpu, mode):
+    rt = Runtime(mode, gpu, max_rows=64, page_size=8)
+    part = base.FEED_FORWARDS["swiglu"]({"width": 40, "inter": 88}, rt)
+    specs = part.tensors()
+    assert specs["down_proj.weight"].shape == (40, 88) and specs["gate_proj.weight"].shape == (88, 40)
+    w = dict(random_tensors(specs, 3, 0.3))
+    part.bind(w)
+    n = 21
+    h = torch.zeros(64, 40, device=gpu, dtype=rt.act_dtype)
+    h[:n] = torch.randn(n, 40, device=gpu).to(rt.act_dtype)
+    res = torch.randn(64, 40, device=gpu)
+    before = res.clone()
+    part.forward(one_request_ctx(rt, n), h, res)
+    hd = h[:n].cpu().double()
+    act = rnd_for(mode)(pl.swiglu(pl.linear(hd, w["gate_proj.weight"]), pl.linear(hd, w["up_proj.weight"])))
+    ref = before[:n].cpu().double() + pl.linear(act, w["down_proj.weight"])
+    assert (res[:n].cpu().double() - ref).abs().max() <= TOL[mode] * ref.abs().max()
+    assert torch.equal(res[n:], before[n:])                         # rows beyond the step are not touched
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kvh,hd,window", [(4, 2, 16, None), (3, 1, 32, None), (6, 3, 48, 10)])
+def test_attention_part(gpu, mode, heads, kvh, hd, window):
+    """The mixer alone: projections, rotation, cache write through a permuted block table,
+    attention (with a window as an option) and the output projection added to the residual."""
+    width, page = 56, 8
+    rt = Runtime(mode, gpu, max_rows=64, page_size=page)
+    pos_spec = PartSpec("rope", {"theta": 5000.0, "head_dim": hd, "max_positions": 64})
+    part = base.MIXERS["attention"]({"width": width, "heads": heads, "kv_heads": kvh, "head_dim": hd, "window": window,
+                                     "position": pos_spec}, rt)
+    w = dict(random_tensors(part.tensors(), 5, 0.2))
+    part.bind(w)
+    assert part.cache_spec().window == window and part.state_spec() is None
+    n = 37
+    pages = [6, 2, 5, 0, 4]
+    cache = torch.zeros(7, part.page_elements(page), device=gpu, dtype=rt.act_dtype)
+    call = CallBinding(0, 0, 0, 0, 0, True, k_cache=cache, v_cache=torch.zeros_like(cache))
+    h_all = torch.randn(n, width).to(rt.act_dtype)
+    res = torch.zeros(64, width, device=gpu)
+    # the first 30 positions as one portion, then 7 single tokens: the cache carries over
+    h = torch.zeros(64, width, device=gpu, dtype=rt.act_dtype)
+    h[:30] = h_all[:30].to(gpu)
+    ctx = StepContext([Segment([0] * 30, 0, [pages], 0, [])], 1, gpu)
+    part.forward(ctx, call, h, res)
+    got = [res[:30].cpu().clone()]
+    for p in range(30, n):
+        h[0] = h_all[p].to(gpu)
+        res.zero_()
+        part.forward(StepContext([Segment([0], p, [pages], 0, [])], 1, gpu), call, h, res)
+        got.append(res[:1].cpu().clone())
+    got = torch.cat(got).double()
+    x = h_all.double()
+    rnd = rnd_for(mode)
+    inv = pl.rope_inv_freq(5000.0, hd)
+    q = rnd(pl.rope(pl.linear(x, w["q_proj.weight"]).view(n, heads, hd), range(n), inv))
+    k = rnd(pl.rope(pl.linear(x, w["k_proj.weight"]).view(n, kvh, hd), range(n), inv))
+    v = rnd(pl.linear(x, w["v_proj.weight"]).view(n, kvh, hd))
+    ref = pl.linear(rnd(pl.attention(q, k, v, rnd, window)).reshape(n, -1), w["o_proj.weight"])
+    assert (got - ref).abs().max() <= TOL[mode] * ref.abs().max()
+
+
+# ----------------------------------------------------------------------------- a toy mixer with state
+
+@base.register_mixer("toy_running_mean")
+class RunningMean(base.Mixer):
+    """Adds gain * (mean of all rows of the request so far) to the residual.  Its per-request
+    state (count and running sum) lives in a slot, not in pages."""
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.width = params["width"]
+        self.gain = None
+
+    def tensors(self):
+        return {"gain": TensorSpec((self.width,), "norm")}
+
+    def bind(self, tensors):
+        self.gain = tensors["gain"].to(self.rt.device).float()
+
+    def state_spec(self):
+        return StateSpec((self.width + 1,), "float32")
+
+    def forward(self, ctx, call, h, residual):
+        for seg, r0 in zip(ctx.segments, ctx.seq_start):
+            n = len(seg.tokens)
+            st = call.state[seg.slot]
+            rows = h[r0:r0 + n].float()
+            sums = st[1:] + torch.cumsum(rows, 0)
+            counts = st[0] + torch.arange(1, n + 1, device=rows.device, dtype=torch.float32)
+            residual[r0:r0 + n] += self.gain * sums / counts[:, None]
+            st[0] += n
+            st[1:] = sums[-1]
+
+
+def toy_spec(width=32, vocab=50):
+    def layer(i, mixer):
+        pre = f"layers.{i}."
+        return LayerSpec("prenorm", mixer, PartSpec("swiglu", {"width": width, "inter": 48}, pre + "mlp."),
+                         PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm1."),
+                         PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm2."))
+    rope = PartSpec("rope", {"theta": 10000.0, "head_dim": 16, "max_positions": 128})
+    attn = PartSpec("attention", {"width": width, "heads": 2, "kv_heads": 1, "head_dim": 16, "window": None,
+                                  "position": rope}, "layers.1.attn.")
+    layers = [layer(0, PartSpec("toy_running_mean", {"width": width}, "layers.0.toy.")), layer(1, attn)]
+    # the toy layer runs twice (two states), the attention layer runs twice: the second call
+    # reads the cache the first one wrote
+    schedule = [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 1, writes_cache=False)]
+    return ModelSpec("ToyForTests", vocab, width, PartSpec("embedding", {"vocab": vocab, "width": width}, "embed."),
+                     layers, schedule, PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "norm."),
+                     PartSpec("lm_head", {"vocab": vocab, "width": width, "tied": True}, "head."), 128)
+
+
+def plain_toy(w, toks, rnd):
+    """The toy model with plain parts, whole sequence."""
+    n = len(toks)
+    x = pl.embed(toks, w["embed.weight"])
+
+    def mlp(x, pre):
+        hn = rnd(pl.rmsnorm(x, w[pre + "norm2.weight"], 1e-5))
+        a = rnd(pl.swiglu(pl.linear(hn, w[pre + "mlp.gate_proj.weight"]), pl.linear(hn, w[pre + "mlp.up_proj.weight"])))
+        return pl.linear(a, w[pre + "mlp.down_proj.weight"])
+
+    def toy(x):
+        hn = rnd(pl.rmsnorm(x, w["layers.0.norm1.weight"], 1e-5))
+        mean = torch.cumsum(hn, 0) / torch.arange(1, n + 1, dtype=F64)[:, None]
+        x = x + w["layers.0.toy.gain"].double() * mean
+        return x + mlp(x, "layers.0.")
+
+    kv = {}
+
+    def attn(x, write):
+        hn = rnd(pl.rmsnorm(x, w["layers.1.norm1.weight"], 1e-5))
+        inv = pl.rope_inv_freq(10000.0, 16)
+        q = rnd(pl.rope(pl.linear(hn, w["layers.1.attn.q_proj.weight"]).view(n, 2, 16), range(n), inv))
+        if write:
+            kv["k"] = rnd(pl.rope(pl.linear(hn, w["layers.1.attn.k_proj.weight"]).view(n, 1, 16), range(n), inv))
+            kv["v"] = rnd(pl.linear(hn, w["layers.1.attn.v_proj.weight"]).view(n, 1, 16))
+        a = rnd(pl.attention(q, kv["k"], kv["v"], rnd)).reshape(n, -1)
+        x = x + pl.linear(a, w["layers.1.attn.o_proj.weight"])
+        return x + mlp(x, "layers.1.")
+
+    x = attn(toy(attn(toy(x), True)), False)
+    return pl.linear(rnd(pl.rmsnorm(x, w["norm.weight"], 1e-5)), w["embed.weight"])
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_toy_mixer_with_state_and_a_schedule_that_repeats_and_shares(gpu, mode):
+    rt = Runtime(mode, gpu, max_rows=64, page_size=8)
+    model = AssembledModel(toy_spec(), rt)
+    assert len(model.state_specs) == 2 and len(model.group_specs) == 1 and model.group_caches == [[1]]
+    assert not model.graph_safe                                   # the toy part works on the host: no graph capture
+    specs = model.tensor_specs()
+    assert "layers.0.toy.gain" in specs and "head.weight" not in specs
+    w = dict(random_tensors(specs, 9, 0.2))
+    model.bind_tensors({k: v.to(gpu) for k, v in w.items()})
+    storage = CacheStorage(model, num_pages=12, num_slots=3)
+    manager = CacheManager([GroupSpec(None)], 12, 8, 3, prefix_caching=True, has_state=True)
+    assert not manager.prefix_caching                             # state outside the pages: no prefix reuse
+    runner = ModelRunner(model, storage, max_model_len=128, use_graphs=True)
+    a = [int(t) for t in torch.randint(0, 50, (23,), generator=torch.Generator().manual_seed(1))]
+    b = [int(t) for t in torch.randint(0, 50, (11,), generator=torch.Generator().manual_seed(2))]
+    rnd = rnd_for(mode)
+    ref = {"a": plain_toy(w, a, rnd).numpy(), "b": plain_toy(w, b, rnd).numpy()}
+    rcs = {"a": manager.open(), "b": manager.open()}
+    for rc in rcs.values():
+        storage.reset_slot(rc.slot)
+    got = {"a": [], "b": []}
+    cuts = [[("a", 9)], [("a", 1), ("b", 5)], [("b", 1), ("a", 2)], [("a", 11), ("b", 5)]]
+    prog = {"a": 0, "b": 0}
+    toks = {"a": a, "b": b}
+    for step in cuts:
+        segs = []
+        for rid, n in step:
+            rc = rcs[rid]
+            assert manager.ensure(rc, prog[rid] + n)
+            segs.append(Segment(toks[rid][prog[rid]:prog[rid] + n], prog[rid], rc.tables, rc.slot, list(range(n))))
+        lg = runner.step(segs).cpu().numpy()
+        row = 0
+        for rid, n in step:
+            got[rid].append(lg[row:row + n])
+            row += n
+            prog[rid] += n
+            manager.advance(rcs[rid], toks[rid], prog[rid])
+    for rid in ("a", "b"):
+        out = np.concatenate(got[rid])
+        assert out.shape == ref[rid].shape
+        assert np.abs(out - ref[rid]).max() <= (2e-2 if mode == "bfloat16" else 2e-5) * np.abs(ref[rid]).max()
+    # a slot that is taken again starts from zero state
+    manager.close(rcs["a"])
+    rc = manager.open()
+    storage.reset_slot(rc.slot)
+    assert manager.ensure(rc, len(b))
+    lg = runner.step([Segment(b, 0, rc.tables, rc.slot, list(range(len(b))))]).cpu().numpy()
+    assert np.abs(lg - ref["b"]).max() <= (2e-2 if mode == "bfloat16" else 2e-5) * np.abs(ref["b"]).max()
+
+
+def test_schedule_errors(gpu):
+    rt = Runtime("float32", gpu, max_rows=16, page_size=8)
+    spec = toy_spec()
+    spec.schedule = [LayerCall(1, 5, writes_cache=False)]
+    with pytest.raises(ValueError, match="before any call wrote it"):
+        AssembledModel(spec, rt)
+    spec.schedule = [LayerCall(1, 0), LayerCall(1, 0)]
+    with pytest.raises(ValueError, match="already has a writer"):
+        AssembledModel(spec, rt)
+    spec.schedule = [LayerCall(7, 0)]
+    with pytest.raises(ValueError, match="names layer 7"):
+        AssembledModel(spec, rt)
+    spec.layers[0].mixer.kind = "no_such_mixer"
+    with pytest.raises(KeyError, match="unknown mixer 'no_such_mixer'"):
+        AssembledModel(spec, rt)
