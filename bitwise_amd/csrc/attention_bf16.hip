@@ -19,6 +19,11 @@
 // product O^T = V^T P^T needs for its B operand; no LDS is used.  K pages are
 // [kv_head][slot][hd]; V pages are transposed, [kv_head][hd][slot], so that an A-operand
 // lane reads 4 consecutive keys of one d with one 8-byte load.
+//
+// Work shapes: in the fold kernel a wave owns up to QT tiles (QT*16 queries of one sequence
+// and kv head) and reuses every loaded K and V operand for all of them, prefetching the next
+// partition's keys while it works; in the split kernel a wave owns one tile and one
+// partition and issues all its loads at once.
 #include "common.h"
 #include "api.h"
 
@@ -28,88 +33,193 @@ struct AttnBf16Args {
   const bf16_t* q;            // [rows, q_stride]
   const int32_t* positions;   // [rows]; negative = padding row
   const int32_t* block_table; // [seqs, table_stride]
-  const int32_t* tiles;       // [tiles][4] = row0, tokens, seq, 0
+  const int32_t* tiles;       // [tiles][4] = row0, tokens, seq, 0; null: tile t is row t of sequence t
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   bf16_t* out;                // [rows, out_stride]
-  float* part_o;              // split mode: [items][max_parts][hd/4][4][hpt]
-  float* part_ml;             // split mode: [items][max_parts][2][hpt]
-  int heads, kv_heads, page_size, table_stride, q_stride, out_stride, window, hpt, nsub, max_parts;
+  float* part_o;              // split mode: [item][part][column][hd]
+  float* part_ml;             // split mode: [item][part][column][2]
+  int heads, kv_heads, page_size, table_stride, q_stride, out_stride, window, hpt, nsub, max_parts, num_tiles;
   float scale;
+};
+
+// What the lanes of a wave share for one group of tiles: sequence, kv head, key range.
+struct GroupCtx {
+  int lane, r, g, kvh, sub, kmax, kmin;
+  const int32_t* table;
 };
 
 template <int HD>
 struct TileCtx {
-  static constexpr int NT = HD / 16;          // 16-wide d tiles
   static constexpr int KS = (HD + 31) / 32;   // 32-deep k steps of the score product
-  int lane, r, g;
   int row_c, head_c, pos_c, lo_c;             // this lane's column (query): row, head, position, first visible key
-  int kvh, kmax, kmin;                        // tile-wide: kv head, last and first key any column sees
-  const int32_t* table;
   u32x4 qf[KS];
 };
 
-template <int HD>
-__device__ __forceinline__ bool tile_setup(const AttnBf16Args& a, int tile, int head_item, TileCtx<HD>& t) {
-  t.lane = threadIdx.x & 63;
-  t.r = t.lane & 15;
-  t.g = t.lane >> 4;
+template <int HD, int QT>
+__device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_tile, int head_item, GroupCtx& gc,
+                                            TileCtx<HD> (&tc)[QT]) {
+  gc.lane = threadIdx.x & 63;
+  gc.r = gc.lane & 15;
+  gc.g = gc.lane >> 4;
   const int group = a.heads / a.kv_heads;
-  t.kvh = head_item / a.nsub;
-  const int sub = head_item % a.nsub;
-  const int row0 = a.tiles[tile * 4 + 0], ntok = a.tiles[tile * 4 + 1], seq = a.tiles[tile * 4 + 2];
-  t.table = a.block_table + (size_t)seq * a.table_stride;
-  const int tok = t.r / a.hpt, hh = t.r % a.hpt;
-  const bool col_ok = tok < ntok && (sub * a.hpt + hh) < group && t.r < (16 / a.hpt) * a.hpt;
-  t.row_c = row0 + (col_ok ? tok : 0);
-  t.head_c = t.kvh * group + sub * a.hpt + (col_ok ? hh : 0);
-  t.pos_c = col_ok ? a.positions[t.row_c] : -1;
-  t.lo_c = (a.window > 0 && t.pos_c - a.window + 1 > 0) ? t.pos_c - a.window + 1 : 0;
-  int kmax = t.pos_c, kmin = t.pos_c >= 0 ? t.lo_c : 0x7fffffff;
+  gc.kvh = head_item / a.nsub;
+  gc.sub = head_item % a.nsub;
+  const int tok = gc.r / a.hpt, hh = gc.r % a.hpt;
+  const bool col_in = (gc.sub * a.hpt + hh) < group && gc.r < (16 / a.hpt) * a.hpt;
+  int seq = 0;
+  int kmax = -1, kmin = 0x7fffffff;
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const int tile = first_tile + t;
+    int row0 = tile, ntok = 1, tseq = tile;
+    if (tile >= a.num_tiles) ntok = 0;
+    else if (a.tiles != nullptr) {
+      row0 = a.tiles[tile * 4 + 0];
+      ntok = a.tiles[tile * 4 + 1];
+      tseq = a.tiles[tile * 4 + 2];
+    }
+    if (t == 0) seq = tseq;
+    const bool ok = col_in && tok < ntok;
+    tc[t].row_c = row0 + (ok ? tok : 0);
+    tc[t].head_c = gc.kvh * group + gc.sub * a.hpt + (ok ? hh : 0);
+    tc[t].pos_c = ok ? a.positions[tc[t].row_c] : -1;
+    tc[t].lo_c = (a.window > 0 && tc[t].pos_c - a.window + 1 > 0) ? tc[t].pos_c - a.window + 1 : 0;
+    kmax = max(kmax, tc[t].pos_c);
+    if (tc[t].pos_c >= 0) kmin = min(kmin, tc[t].lo_c);
+  }
 #pragma unroll
   for (int off = 8; off >= 1; off >>= 1) {
     kmax = max(kmax, __shfl_xor(kmax, off, BW_WAVE));
     kmin = min(kmin, __shfl_xor(kmin, off, BW_WAVE));
   }
-  t.kmax = kmax;
-  t.kmin = kmin;
+  gc.kmax = kmax;
+  gc.kmin = kmin;
+  gc.table = a.block_table + (size_t)seq * a.table_stride;
   if (kmax < 0) return false;
 #pragma unroll
-  for (int ks = 0; ks < TileCtx<HD>::KS; ++ks) {
-    const int d0 = 32 * ks + 8 * t.g;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (t.pos_c >= 0 && d0 < HD)
-      v = *reinterpret_cast<const u32x4*>(a.q + (size_t)t.row_c * a.q_stride + (size_t)t.head_c * HD + d0);
-    t.qf[ks] = v;
-  }
+  for (int t = 0; t < QT; ++t)
+#pragma unroll
+    for (int ks = 0; ks < TileCtx<HD>::KS; ++ks) {
+      const int d0 = 32 * ks + 8 * gc.g;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (tc[t].pos_c >= 0 && d0 < HD)
+        v = *reinterpret_cast<const u32x4*>(a.q + (size_t)tc[t].row_c * a.q_stride + (size_t)tc[t].head_c * HD + d0);
+      tc[t].qf[ks] = v;
+    }
   return true;
 }
 
-// One partition's partial for the tile: per column m_p, l_p (replicated over the 4 lane
-// groups) and O_p[dt][i] = element d = 16dt + 4g + i of the column.
 template <int HD>
-__device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const TileCtx<HD>& t, int part,
-                                                  float& m_p, float& l_p, f32x4 (&o_p)[HD / 16]) {
-  constexpr int NT = HD / 16, KS = (HD + 31) / 32;
+struct KFrags {
+  u32x4 k[4][(HD + 31) / 32];
+};
+// Keys of one partition as A operands: lane (r, g) feeds key 16u + r, elements 32ks + 8g .. +7.
+template <int HD>
+__device__ __forceinline__ void load_keys(const AttnBf16Args& a, const GroupCtx& gc, int part, KFrags<HD>& kf) {
+  constexpr int KS = (HD + 31) / 32;
   const int key0 = part * ATT_PART;
   const size_t kpage = (size_t)a.kv_heads * a.page_size * HD;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int key_r = key0 + 16 * u + gc.r;
+    const bool k_ok = key_r <= gc.kmax && key_r >= gc.kmin;
+    const bf16_t* kp = a.k_cache;
+    if (k_ok)
+      kp = a.k_cache + (size_t)gc.table[key_r / a.page_size] * kpage +
+           ((size_t)gc.kvh * a.page_size + key_r % a.page_size) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = 32 * ks + 8 * gc.g;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (k_ok && d0 < HD) v = *reinterpret_cast<const u32x4*>(kp + d0);
+      kf.k[u][ks] = v;
+    }
+  }
+}
+
+// Values of one partition as A operands of O^T = V^T P^T: lane (r, g) feeds d = 16dt + r and, for
+// the 32-key step w, keys 32w + 4g .. +3 and 32w + 16 + 4g .. +3 (the order in which the
+// probabilities sit in the score accumulators).  Keys no query of the group may see hold stale
+// data (never written, or given back): they are zeroed, so that 0 * garbage cannot make a NaN.
+template <int HD, int DT0, int NDT>
+__device__ __forceinline__ void load_values_range(const AttnBf16Args& a, const GroupCtx& gc, int part,
+                                                  u32x4 (&out)[NDT][2]) {
+  const int key0 = part * ATT_PART;
+  const size_t vpage = (size_t)a.kv_heads * HD * a.page_size;
+#pragma unroll
+  for (int w = 0; w < 2; ++w)
+#pragma unroll
+    for (int hseg = 0; hseg < 2; ++hseg) {
+      const int kA = key0 + 32 * w + 16 * hseg + 4 * gc.g;   // 4 consecutive keys
+      const bool ok = kA <= gc.kmax && kA + 3 >= gc.kmin;
+      const bf16_t* vp = a.v_cache;
+      if (ok) vp = a.v_cache + (size_t)gc.table[kA / a.page_size] * vpage + (size_t)gc.kvh * HD * a.page_size + kA % a.page_size;
+      uint32_t m0 = ok ? 0xffffffffu : 0u, m1 = m0;
+      const int over = kA + 3 - gc.kmax;                      // keys kA+4-over .. kA+3 are unwritten
+      if (over >= 1) m1 &= (over >= 2) ? 0u : 0x0000ffffu;
+      if (over >= 3) m0 &= (over >= 4) ? 0u : 0x0000ffffu;
+      const int under = gc.kmin - kA;                         // keys kA .. kA+under-1 are gone
+      if (under >= 1) m0 &= (under >= 2) ? 0u : 0xffff0000u;
+      if (under >= 3) m1 &= (under >= 4) ? 0u : 0xffff0000u;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        u32x2 v2 = {0u, 0u};
+        if (ok) v2 = *reinterpret_cast<const u32x2*>(vp + (size_t)(16 * (DT0 + dt) + gc.r) * a.page_size);
+        out[dt][w][2 * hseg] = v2[0] & m0;
+        out[dt][w][2 * hseg + 1] = v2[1] & m1;
+      }
+    }
+}
+
+// Head sizes up to 128 load a partition's values at once (and early); larger ones load them
+// 16 elements of d at a time where they are used, to stay within the register file.
+template <int HD>
+struct VFrags {
+  static constexpr bool EARLY = HD <= 128;
+  u32x4 v[EARLY ? HD / 16 : 1][2];
+};
+
+template <int HD>
+__device__ __forceinline__ void load_values(const AttnBf16Args& a, const GroupCtx& gc, int part, VFrags<HD>& vf) {
+  if constexpr (VFrags<HD>::EARLY) load_values_range<HD, 0, HD / 16>(a, gc, part, vf.v);
+}
+
+template <int HD, int DT>
+__device__ __forceinline__ void pv_step(const AttnBf16Args& a, const GroupCtx& gc, int part, const VFrags<HD>& vf,
+                                        const u32x4 (&pf)[2], f32x4 (&o_p)[HD / 16]) {
+  if constexpr (DT < HD / 16) {
+    o_p[DT] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if constexpr (VFrags<HD>::EARLY) {
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+        o_p[DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf.v[DT][w]), as_bf16x8(pf[w]), o_p[DT], 0, 0, 0);
+    } else {
+      u32x4 v[1][2];
+      load_values_range<HD, DT, 1>(a, gc, part, v);
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+        o_p[DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v[0][w]), as_bf16x8(pf[w]), o_p[DT], 0, 0, 0);
+    }
+    pv_step<HD, DT + 1>(a, gc, part, vf, pf, o_p);
+  }
+}
+
+// One partition's partial for one tile: per column m_p, l_p (replicated over the 4 lane
+// groups) and O_p[dt][i] = element d = 16dt + 4g + i of the column.
+template <int HD>
+__device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const GroupCtx& gc, const TileCtx<HD>& t,
+                                                  int part, const KFrags<HD>& kf, const VFrags<HD>& vf, float& m_p,
+                                                  float& l_p, f32x4 (&o_p)[HD / 16]) {
+  constexpr int KS = (HD + 31) / 32;
+  const int key0 = part * ATT_PART;
   f32x4 st[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     st[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int key_r = key0 + 16 * u + t.r;           // the key this lane feeds as an A row
-    const bool k_ok = key_r <= t.kmax && key_r >= t.kmin;
-    const bf16_t* kp = nullptr;
-    if (k_ok)
-      kp = a.k_cache + (size_t)t.table[key_r / a.page_size] * kpage +
-           ((size_t)t.kvh * a.page_size + key_r % a.page_size) * HD;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d0 = 32 * ks + 8 * t.g;
-      u32x4 kf = {0u, 0u, 0u, 0u};
-      if (k_ok && d0 < HD) kf = *reinterpret_cast<const u32x4*>(kp + d0);
-      st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(t.qf[ks]), st[u], 0, 0, 0);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+      st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf.k[u][ks]), as_bf16x8(t.qf[ks]), st[u], 0, 0, 0);
   }
   // scale, mask, column maximum
   float mx = -INFINITY;
@@ -118,7 +228,7 @@ __device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const T
   for (int u = 0; u < 4; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = key0 + 16 * u + 4 * t.g + i;
+      const int key = key0 + 16 * u + 4 * gc.g + i;
       vis[u][i] = key <= t.pos_c && key >= t.lo_c;
       const float s = st[u][i] * a.scale;
       st[u][i] = s;
@@ -147,36 +257,14 @@ __device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const T
   lsum += __shfl_xor(lsum, 32, BW_WAVE);
   l_p = lsum;
   // O_p^T = V^T P^T, keys ascending in steps of 32
-  const size_t vpage = (size_t)a.kv_heads * HD * a.page_size;
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    o_p[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int d = 16 * dt + t.r;
-#pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      u32x4 vf;
-#pragma unroll
-      for (int hseg = 0; hseg < 2; ++hseg) {
-        const int kA = key0 + 32 * w + 16 * hseg + 4 * t.g;   // 4 consecutive keys
-        u32x2 v2 = {0u, 0u};
-        if (kA <= t.kmax && kA + 3 >= t.kmin) {
-          const bf16_t* vp = a.v_cache + (size_t)t.table[kA / a.page_size] * vpage +
-                             ((size_t)t.kvh * HD + d) * a.page_size + kA % a.page_size;
-          v2 = *reinterpret_cast<const u32x2*>(vp);
-          // keys beyond the last written one (or before the window) hold stale data: zero them
-          const int over = kA + 3 - t.kmax;                  // keys kA+4-over .. kA+3 are unwritten
-          if (over >= 1) v2[1] &= (over >= 2) ? 0u : 0x0000ffffu;
-          if (over >= 3) v2[0] &= (over >= 4) ? 0u : 0x0000ffffu;
-          const int under = t.kmin - kA;                     // keys kA .. kA+under-1 are gone
-          if (under >= 1) v2[0] &= (under >= 2) ? 0u : 0xffff0000u;
-          if (under >= 3) v2[1] &= (under >= 4) ? 0u : 0xffff0000u;
-        }
-        vf[2 * hseg] = v2[0];
-        vf[2 * hseg + 1] = v2[1];
-      }
-      o_p[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[w]), o_p[dt], 0, 0, 0);
-    }
-  }
+  pv_step<HD, 0>(a, gc, part, vf, pf, o_p);
+}
+
+// The fold step, element by element; the combine kernel runs the same statements.
+__device__ __forceinline__ void fold_scalars(float m, float m_p, float& mn, float& fa, float& fb) {
+  mn = fmaxf(m, m_p);
+  fa = fast_exp(m - mn);
+  fb = fast_exp(m_p - mn);
 }
 
 template <int NT>
@@ -189,8 +277,8 @@ __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m
     for (int dt = 0; dt < NT; ++dt) o[dt] = o_p[dt];
     return;
   }
-  const float mn = fmaxf(m, m_p);
-  const float fa = fast_exp(m - mn), fb = fast_exp(m_p - mn);
+  float mn, fa, fb;
+  fold_scalars(m, m_p, mn, fa, fb);
   l = fmaf(l, fa, l_p * fb);
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt)
@@ -199,88 +287,155 @@ __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m
   m = mn;
 }
 
-template <int HD>
-__device__ __forceinline__ void finish(const AttnBf16Args& a, const TileCtx<HD>& t, float l, const f32x4 (&o)[HD / 16]) {
-  if (t.pos_c < 0) return;
-  const float inv = 1.0f / l;
-  bf16_t* dst = a.out + (size_t)t.row_c * a.out_stride + (size_t)t.head_c * HD;
-#pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) {
-    u32x2 pk = {pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv), pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv)};
-    *reinterpret_cast<u32x2*>(dst + 16 * dt + 4 * t.g) = pk;
-  }
-}
-
-// Route 1: one wave folds all partitions of its tile.
-template <int HD>
+// Route 1: one wave folds all partitions of its group of QT tiles.
+template <int HD, int QT>
 __global__ __launch_bounds__(64) void attention_fold_kernel(AttnBf16Args a) {
   constexpr int NT = HD / 16;
-  TileCtx<HD> t;
-  if (!tile_setup<HD>(a, blockIdx.x, blockIdx.y, t)) return;
-  float m = -INFINITY, l = 0.0f;
-  f32x4 o[NT];
+  GroupCtx gc;
+  TileCtx<HD> tc[QT];
+  if (!group_setup<HD, QT>(a, blockIdx.x * QT, blockIdx.y, gc, tc)) return;
+  float m[QT], l[QT];
+  f32x4 o[QT][NT];
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int part = t.kmin / ATT_PART; part <= t.kmax / ATT_PART; ++part) {
-    float m_p, l_p;
-    f32x4 o_p[NT];
-    partition_partial<HD>(a, t, part, m_p, l_p, o_p);
-    fold<NT>(m, l, o, m_p, l_p, o_p);
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) o[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
-  finish<HD>(a, t, l, o);
+  const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
+  constexpr bool PREFETCH = HD <= 128;      // the next partition's keys are loaded while this one is worked on
+  KFrags<HD> kf, kf_next;
+  VFrags<HD> vf;
+  if constexpr (PREFETCH) load_keys<HD>(a, gc, first, kf);
+  for (int part = first; part <= last; ++part) {
+    if constexpr (!PREFETCH) load_keys<HD>(a, gc, part, kf);
+    load_values<HD>(a, gc, part, vf);
+    if constexpr (PREFETCH) {
+      if (part < last) load_keys<HD>(a, gc, part + 1, kf_next);
+    }
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      float m_p, l_p;
+      f32x4 o_p[NT];
+      partition_partial<HD>(a, gc, tc[t], part, kf, vf, m_p, l_p, o_p);
+      fold<NT>(m[t], l[t], o[t], m_p, l_p, o_p);
+    }
+    if constexpr (PREFETCH) kf = kf_next;
+  }
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    if (tc[t].pos_c < 0) continue;
+    const float inv = 1.0f / l[t];
+    bf16_t* dst = a.out + (size_t)tc[t].row_c * a.out_stride + (size_t)tc[t].head_c * HD;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      u32x2 pk = {pack_bf16x2(o[t][dt][0] * inv, o[t][dt][1] * inv), pack_bf16x2(o[t][dt][2] * inv, o[t][dt][3] * inv)};
+      *reinterpret_cast<u32x2*>(dst + 16 * dt + 4 * gc.g) = pk;
+    }
+  }
 }
 
 // Route 2a: one wave per (tile, partition) stores the partial.  Tiles of this route hold one
 // token, so the live columns are the first hpt (one per head of the group); only those are
-// stored: O as [register][lane group][column], m and l as [column].
+// stored, each as m, l and hd contiguous 32-bit values.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_split_kernel(AttnBf16Args a) {
   constexpr int NT = HD / 16;
-  TileCtx<HD> t;
-  if (!tile_setup<HD>(a, blockIdx.x, blockIdx.y, t)) return;
+  GroupCtx gc;
+  TileCtx<HD> tc[1];
+  if (!group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc)) return;
   const int part = blockIdx.z;
-  if (part < t.kmin / ATT_PART || part > t.kmax / ATT_PART) return;
+  if (part < gc.kmin / ATT_PART || part > gc.kmax / ATT_PART) return;
+  KFrags<HD> kf;
+  VFrags<HD> vf;
+  load_keys<HD>(a, gc, part, kf);
+  load_values<HD>(a, gc, part, vf);
   float m_p, l_p;
   f32x4 o_p[NT];
-  partition_partial<HD>(a, t, part, m_p, l_p, o_p);
-  if (t.r >= a.hpt) return;
-  const size_t item = ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * a.max_parts + part;
-  if (t.g == 0) {
-    a.part_ml[(item * 2 + 0) * a.hpt + t.r] = m_p;
-    a.part_ml[(item * 2 + 1) * a.hpt + t.r] = l_p;
+  partition_partial<HD>(a, gc, tc[0], part, kf, vf, m_p, l_p, o_p);
+  if (gc.r >= a.hpt) return;
+  const size_t cell = (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * a.max_parts + part) * a.hpt + gc.r;
+  if (gc.g == 0) {
+    a.part_ml[cell * 2 + 0] = m_p;
+    a.part_ml[cell * 2 + 1] = l_p;
   }
-  float* po = a.part_o + item * (size_t)(HD * a.hpt);
+  float* po = a.part_o + cell * HD;
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) po[((dt * 4 + i) * 4 + t.g) * a.hpt + t.r] = o_p[dt][i];
+  for (int dt = 0; dt < NT; ++dt) *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * gc.g) = o_p[dt];
 }
 
-// Route 2b: the same left fold, reading the stored partials in partition order.
+// Route 2b: the same left fold, one wave per query (tile, kv head, column), lane l owning
+// elements l, l+64, ... of the output; the partials are read in partition order.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_combine_kernel(AttnBf16Args a) {
-  constexpr int NT = HD / 16;
-  TileCtx<HD> t;
-  if (!tile_setup<HD>(a, blockIdx.x, blockIdx.y, t)) return;
-  float m = -INFINITY, l = 0.0f;
-  f32x4 o[NT];
+  constexpr int DPL = (HD + 63) / 64;
+  const int lane = threadIdx.x, tile = blockIdx.x, head_item = blockIdx.y, col = blockIdx.z;
+  const int group = a.heads / a.kv_heads;
+  const int kvh = head_item / a.nsub, sub = head_item % a.nsub;
+  if (sub * a.hpt + col >= group) return;
+  const int row = a.tiles != nullptr ? a.tiles[tile * 4] : tile;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int first = lo / ATT_PART, last = pos / ATT_PART;
+  const size_t cell0 = (((size_t)tile * gridDim.y + head_item) * a.max_parts) * a.hpt + col;
+  float m = -INFINITY, l = 0.0f, o[DPL];
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  if (t.r < a.hpt) {
-    for (int part = t.kmin / ATT_PART; part <= t.kmax / ATT_PART; ++part) {
-      const size_t item = ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * a.max_parts + part;
-      const float m_p = a.part_ml[(item * 2 + 0) * a.hpt + t.r];
-      const float l_p = a.part_ml[(item * 2 + 1) * a.hpt + t.r];
-      const float* po = a.part_o + item * (size_t)(HD * a.hpt);
-      f32x4 o_p[NT];
+  for (int t = 0; t < DPL; ++t) o[t] = 0.0f;
+  constexpr int UN = 4;
+  for (int p0 = first; p0 <= last; p0 += UN) {
+    float mp[UN], lp[UN], op[UN][DPL];
 #pragma unroll
-      for (int dt = 0; dt < NT; ++dt)
+    for (int j = 0; j < UN; ++j) {
+      const int p = p0 + j;
+      const size_t cell = cell0 + (size_t)(p <= last ? p : last) * a.hpt;
+      mp[j] = a.part_ml[cell * 2 + 0];
+      lp[j] = a.part_ml[cell * 2 + 1];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o_p[dt][i] = po[((dt * 4 + i) * 4 + t.g) * a.hpt + t.r];
-      fold<NT>(m, l, o, m_p, l_p, o_p);
+      for (int t = 0; t < DPL; ++t) {
+        const int d = lane + 64 * t;
+        op[j][t] = d < HD ? a.part_o[cell * HD + d] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      if (p0 + j > last || mp[j] == -INFINITY) continue;
+      if (m == -INFINITY) {
+        m = mp[j];
+        l = lp[j];
+#pragma unroll
+        for (int t = 0; t < DPL; ++t) o[t] = op[j][t];
+        continue;
+      }
+      float mn, fa, fb;
+      fold_scalars(m, mp[j], mn, fa, fb);
+      l = fmaf(l, fa, lp[j] * fb);
+#pragma unroll
+      for (int t = 0; t < DPL; ++t) o[t] = fmaf(o[t], fa, op[j][t] * fb);
+      m = mn;
     }
   }
-  finish<HD>(a, t, l, o);
+  const float inv = 1.0f / l;
+  bf16_t* dst = a.out + (size_t)row * a.out_stride + (size_t)(kvh * group + sub * a.hpt + col) * HD;
+#pragma unroll
+  for (int t = 0; t < DPL; ++t) {
+    const int d = lane + 64 * t;
+    if (d < HD) dst[d] = f32_to_bf16(o[t] * inv);
+  }
+}
+
+template <int HD>
+static void launch_attention(const AttnBf16Args& a, int split, hipStream_t s) {
+  const dim3 block(64);
+  const int items = a.kv_heads * a.nsub;
+  if (split) {
+    hipLaunchKernelGGL(attention_split_kernel<HD>, dim3(a.num_tiles, items, a.max_parts), block, 0, s, a);
+    hipLaunchKernelGGL(attention_combine_kernel<HD>, dim3(a.num_tiles, items, a.hpt), block, 0, s, a);
+  } else {
+    constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
+    hipLaunchKernelGGL((attention_fold_kernel<HD, QT>), dim3((a.num_tiles + QT - 1) / QT, items), block, 0, s, a);
+  }
 }
 
 extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
@@ -302,20 +457,12 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   a.hpt = group < 16 ? group : 16;
   a.nsub = (group + a.hpt - 1) / a.hpt;
   a.max_parts = max_parts;
+  a.num_tiles = num_tiles;
   a.scale = scale;
   if (kv_heads * a.nsub > 65535 || max_parts > 65535) return -2;
   if (split && (max_parts <= 0 || !part_o || !part_ml)) return -2;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(num_tiles, kv_heads * a.nsub), block(64);
-#define BW_CASE(HD)                                                                                   \
-  case HD:                                                                                            \
-    if (split) {                                                                                      \
-      hipLaunchKernelGGL(attention_split_kernel<HD>, dim3(grid.x, grid.y, max_parts), block, 0, s, a); \
-      hipLaunchKernelGGL(attention_combine_kernel<HD>, grid, block, 0, s, a);                         \
-    } else {                                                                                          \
-      hipLaunchKernelGGL(attention_fold_kernel<HD>, grid, block, 0, s, a);                            \
-    }                                                                                                 \
-    break;
+#define BW_CASE(HD) case HD: launch_attention<HD>(a, split, s); break;
   switch (head_dim) {
     BW_CASE(16) BW_CASE(32) BW_CASE(48) BW_CASE(64) BW_CASE(80) BW_CASE(96) BW_CASE(112) BW_CASE(128)
     BW_CASE(160) BW_CASE(192) BW_CASE(224) BW_CASE(256)

@@ -70,21 +70,56 @@ __global__ void rmsnorm_f32_kernel(const float* __restrict__ x, const WT* __rest
 
 // ------------------------------------------------------------------------- RMSNorm, bfloat16 out
 
-// One wave per row; lane l sums x[i]^2 over i = l, l+64, ... by fused multiply-adds, the
-// lanes are joined by xor butterflies (32, 16, ..., 1).  All in 32-bit; one rounding at the
-// store.  A row's result depends on that row alone.
+// One wave per row.  Rows whose width is a multiple of 4 are read as 16-byte vectors: lane l
+// takes vectors l, l+64, ... and runs one fused multiply-add chain over its elements in
+// ascending order; other widths take elements l, l+64, ...  The lanes are joined by xor
+// butterflies (32, 16, ..., 1).  All in 32-bit; one rounding at the store.  The order depends
+// on the width alone, so a row's result depends on that row alone.
 template <typename WT>
-__global__ void rmsnorm_bf16_kernel(const float* __restrict__ x, const WT* __restrict__ w,
-                                    bf16_t* __restrict__ y, int rows, int dim, int ldy, float eps) {
+__global__ __launch_bounds__(256) void rmsnorm_bf16_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                           bf16_t* __restrict__ y, int rows, int dim, int ldy,
+                                                           float eps) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= rows) return;
   const float* xr = x + (size_t)row * dim;
+  bf16_t* yr = y + (size_t)row * ldy;
   float acc = 0.0f;
+  if ((dim & 3) == 0 && (ldy & 3) == 0) {
+    const int nvec = dim >> 2;
+    const f32x4* xv = reinterpret_cast<const f32x4*>(xr);
+    constexpr int UN = 8;
+    for (int c0 = 0; c0 < nvec; c0 += 64 * UN) {
+      f32x4 v[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j) {
+        const int c = c0 + 64 * j + lane;
+        v[j] = c < nvec ? xv[c] : (f32x4){0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = fmaf(v[j][e], v[j][e], acc);
+    }
+    acc = wave_sum(acc);
+    const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+    for (int c = lane; c < nvec; c += 64) {
+      const f32x4 v = xv[c];
+      float wv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if constexpr (sizeof(WT) == 2) wv[e] = bf16_to_f32(w[4 * c + e]);
+        else wv[e] = w[4 * c + e];
+      }
+      u32x2 pk = {pack_bf16x2((v[0] * inv) * wv[0], (v[1] * inv) * wv[1]),
+                  pack_bf16x2((v[2] * inv) * wv[2], (v[3] * inv) * wv[3])};
+      *reinterpret_cast<u32x2*>(yr + 4 * c) = pk;
+    }
+    return;
+  }
   for (int i = lane; i < dim; i += 64) acc = fmaf(xr[i], xr[i], acc);
   acc = wave_sum(acc);
   const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
-  bf16_t* yr = y + (size_t)row * ldy;
   for (int i = lane; i < dim; i += 64) {
     float wi;
     if constexpr (sizeof(WT) == 2) wi = bf16_to_f32(w[i]);

@@ -15,6 +15,12 @@ from . import build as _build
 
 EPI_F32, EPI_BF16, EPI_ADD_F32, EPI_SWIGLU_BF16 = 0, 1, 2, 3
 ATT_PART = 64          # keys per partition of the bfloat16 attention fold
+
+
+def fold_group_tiles(head_dim: int) -> int:
+    """Tiles (of 16 query columns) one wave of the fold kernel owns; a wave's tiles must belong
+    to one sequence, so the host pads every sequence's tile list to a multiple of this."""
+    return 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
 HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
 
 _ERRORS = {
@@ -247,13 +253,15 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
                                    page_size, int(window), float(scale), _stream()), "attention_f32")
 
 
-def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
-                   num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, heads: int,
+def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
+                   tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, heads: int,
                    kv_heads: int, head_dim: int, page_size: int, window: int, scale: float, split: bool = False,
                    max_parts: int = 0, part_o: Optional[torch.Tensor] = None,
                    part_ml: Optional[torch.Tensor] = None) -> None:
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
-    [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).  With
+    [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0), or None for
+    "tile t is row t of sequence t" (split route only).  Without ``split`` the tiles of a
+    sequence must come in runs padded to ``fold_group_tiles(head_dim)`` (empty tiles allowed).  With
     ``split`` (tiles of one token each) every (tile, partition) is a wave of its own and the
     partials are folded by a second kernel; the bits equal the unsplit route."""
     _need(q, torch.bfloat16, "q")
@@ -262,12 +270,16 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     _need(v_cache, torch.bfloat16, "v_cache")
     _need(positions, torch.int32, "positions")
     _need(block_table, torch.int32, "block_table")
-    _need(tiles, torch.int32, "tiles")
+    if tiles is not None:
+        _need(tiles, torch.int32, "tiles")
+    elif not split:
+        raise ValueError("attention_bf16: implicit tiles are for the split route only")
     if head_dim not in HEAD_DIMS:
         raise ValueError(f"attention: head size {head_dim} is not supported; supported: {HEAD_DIMS}")
     if heads % kv_heads:
         raise ValueError("attention: heads must be a multiple of kv_heads")
-    if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or tiles.numel() < 4 * num_tiles:
+    if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or (
+            tiles is not None and tiles.numel() < 4 * num_tiles):
         raise ValueError("attention_bf16: q, out or tiles do not fit")
     group = heads // kv_heads
     hpt = min(group, 16)
@@ -280,7 +292,8 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
         if part_o.numel() < items * max_parts * head_dim * hpt or part_ml.numel() < items * max_parts * 2 * hpt:
             raise ValueError("attention_bf16: scratch buffers too small")
     _check(_fn("bw_attention_bf16")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
-                                    block_table.stride(0), tiles.data_ptr(), num_tiles, k_cache.data_ptr(),
+                                    block_table.stride(0), tiles.data_ptr() if tiles is not None else 0, num_tiles,
+                                    k_cache.data_ptr(),
                                     v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads, kv_heads, head_dim,
                                     page_size, int(window), float(scale), int(split), max_parts,
                                     part_o.data_ptr() if part_o is not None else 0,

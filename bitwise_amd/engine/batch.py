@@ -74,12 +74,14 @@ class StepContext:
         self.tokens, self.positions, self.row_seq, self.want_rows, self.slots = view[:5]
         self.block_tables = [view[5 + g].view(nseq, widths[g]) for g in range(num_groups)]
         self.host_positions = positions
-        self._plans: Dict[int, AttentionPlan] = {}
+        self._plans: Dict[tuple, AttentionPlan] = {}
 
-    def attention_plan(self, tokens_per_tile: int) -> AttentionPlan:
-        """Tiles of up to ``tokens_per_tile`` consecutive rows of one request.  Single decoded
-        tokens with a long context go the split route (a wave per 64-key partition)."""
-        plan = self._plans.get(tokens_per_tile)
+    def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
+        """Tiles of up to ``tokens_per_tile`` consecutive rows of one request; every request's
+        run of tiles is padded with empty tiles to a multiple of ``group_tiles`` (the tiles one
+        wave owns must belong to one request).  Single decoded tokens with a long context go
+        the split route (a wave per 64-key partition)."""
+        plan = self._plans.get((tokens_per_tile, group_tiles))
         if plan is not None:
             return plan
         fold, split = [], []
@@ -92,9 +94,11 @@ class StepContext:
                 continue
             for off in range(0, n, tokens_per_tile):
                 fold.append((r0 + off, min(tokens_per_tile, n - off), i, 0))
+            while len(fold) % group_tiles:
+                fold.append((r0, 0, i, 0))
         both = np.asarray(fold + split, np.int32).reshape(-1, 4)
         dev = torch.from_numpy(both).to(self.device)
         plan = AttentionPlan(dev[:len(fold)].contiguous() if fold else None, len(fold),
                              dev[len(fold):].contiguous() if split else None, len(split), max_parts)
-        self._plans[tokens_per_tile] = plan
+        self._plans[(tokens_per_tile, group_tiles)] = plan
         return plan

@@ -36,14 +36,11 @@ class _StaticDecodeContext:
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self.slots = torch.zeros(size, dtype=torch.int32, device=device)
         self.block_tables = [torch.zeros((size, max_pages), dtype=torch.int32, device=device) for _ in range(num_groups)]
-        tiles = np.zeros((size, 4), np.int32)
-        tiles[:, 0] = tiles[:, 2] = np.arange(size)
-        tiles[:, 1] = 1
-        self._plan = AttentionPlan(None, 0, torch.from_numpy(tiles).to(device), size, max_parts)
+        self._plan = AttentionPlan(None, 0, None, size, max_parts)      # implicit tiles: tile t = row t of request t
         self._host = np.empty((3 + num_groups * max_pages, size), np.int32)
         self.segments: List[Segment] = []
 
-    def attention_plan(self, tokens_per_tile: int) -> AttentionPlan:
+    def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
         return self._plan
 
     def fill(self, segments: Sequence[Segment]) -> None:

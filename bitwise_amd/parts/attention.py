@@ -86,7 +86,7 @@ class Attention(Mixer):
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              rt.page_size, call.writes_cache)
             out = rt.buffer("attn_out", self.q_dim, torch.bfloat16)
-            plan = ctx.attention_plan(self.tokens_per_tile)
+            plan = ctx.attention_plan(self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
             common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
                       window, self.scale)
             if plan.fold_count:
