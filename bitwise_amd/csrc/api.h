@@ -29,8 +29,15 @@ int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, con
 int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                       int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                       const void* v_cache, void* out, int out_stride, int heads, int kv_heads, int head_dim,
-                      int page_size, int window, float scale, int split, int max_parts, float* part_o,
-                      float* part_ml, void* stream);
+                      int page_size, int window, float scale, int decode, void* stream);
+int bw_decode_gemm_supported(int M, int K, int norm);
+int bw_decode_gemm_bf16(const void* a_rows, int lda, int a_is_f32, const void* norm_w, int norm_w_is_bf16, float eps,
+                        const void* w, void* out, int ldo, int M, int N, int K, int epilogue, void* stream);
+int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps,
+                          const void* w_qkv, void* q_out, const int32_t* positions, const int32_t* row_seq,
+                          const int32_t* block_table, int table_stride, const float* cos_table,
+                          const float* sin_table, void* k_cache, void* v_cache, int M, int heads, int kv_heads,
+                          int head_dim, int K, int page_size, int write_cache, void* stream);
 int bw_sample(const float* logits, int vocab, int ld, int rows, const float* temperature, const double* uniform,
               int32_t* out, void* stream);
 int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out, void* stream);

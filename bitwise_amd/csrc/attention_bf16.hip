@@ -10,9 +10,9 @@
 //   m' = max(m, m_t); a = exp(m - m'); b = exp(m_t - m'); l = fma(l, a, l_t*b); O = fma(O, a, O_t*b)
 // (the first partition a query sees initialises the state; a partition it cannot see is
 // skipped).  out = O * (1/l).  The fold kernel walks the partitions inside one wave; the
-// split kernel computes one partition per wave and the combine kernel performs the same fold
-// from memory, so both routes give the same bits, and a query's result depends on nothing
-// but its own row, its position and the cache contents at positions it may see.
+// decode kernel gives every partition a wave of its own and performs the same fold from LDS
+// in partition order, so both routes give the same bits, and a query's result depends on
+// nothing but its own row, its position and the cache contents at positions it may see.
 //
 // Layout: S^T = K Q^T is computed (keys are MFMA rows, queries are columns), so the
 // probabilities come out of the accumulator in exactly the lane layout that the second
@@ -22,8 +22,9 @@
 //
 // Work shapes: in the fold kernel a wave owns up to QT tiles (QT*16 queries of one sequence
 // and kv head) and reuses every loaded K and V operand for all of them, prefetching the next
-// partition's keys while it works; in the split kernel a wave owns one tile and one
-// partition and issues all its loads at once.
+// partition's keys while it works; in the decode kernel a workgroup owns one tile (one token,
+// the heads of one kv head) and each of its waves one partition at a time, all loads of a
+// partition issued at once.
 #include "common.h"
 #include "api.h"
 
@@ -37,9 +38,7 @@ struct AttnBf16Args {
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   bf16_t* out;                // [rows, out_stride]
-  float* part_o;              // split mode: [item][part][column][hd]
-  float* part_ml;             // split mode: [item][part][column][2]
-  int heads, kv_heads, page_size, table_stride, q_stride, out_stride, window, hpt, nsub, max_parts, num_tiles;
+  int heads, kv_heads, page_size, table_stride, q_stride, out_stride, window, hpt, nsub, num_tiles;
   float scale;
 };
 
@@ -124,10 +123,11 @@ __device__ __forceinline__ void load_keys(const AttnBf16Args& a, const GroupCtx&
   for (int u = 0; u < 4; ++u) {
     const int key_r = key0 + 16 * u + gc.r;
     const bool k_ok = key_r <= gc.kmax && key_r >= gc.kmin;
-    const bf16_t* kp = a.k_cache;
-    if (k_ok)
-      kp = a.k_cache + (size_t)gc.table[key_r / a.page_size] * kpage +
-           ((size_t)gc.kvh * a.page_size + key_r % a.page_size) * HD;
+    // the table entry is read whether or not the key is live (index clamped into the row), so
+    // that this load does not have to wait for the positions
+    const int pidx = key_r / a.page_size;
+    const int page = gc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
+    const bf16_t* kp = a.k_cache + (size_t)page * kpage + ((size_t)gc.kvh * a.page_size + key_r % a.page_size) * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = 32 * ks + 8 * gc.g;
@@ -153,8 +153,9 @@ __device__ __forceinline__ void load_values_range(const AttnBf16Args& a, const G
     for (int hseg = 0; hseg < 2; ++hseg) {
       const int kA = key0 + 32 * w + 16 * hseg + 4 * gc.g;   // 4 consecutive keys
       const bool ok = kA <= gc.kmax && kA + 3 >= gc.kmin;
-      const bf16_t* vp = a.v_cache;
-      if (ok) vp = a.v_cache + (size_t)gc.table[kA / a.page_size] * vpage + (size_t)gc.kvh * HD * a.page_size + kA % a.page_size;
+      const int pidx = kA / a.page_size;
+      const int page = gc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
+      const bf16_t* vp = a.v_cache + (size_t)page * vpage + (size_t)gc.kvh * HD * a.page_size + kA % a.page_size;
       uint32_t m0 = ok ? 0xffffffffu : 0u, m1 = m0;
       const int over = kA + 3 - gc.kmax;                      // keys kA+4-over .. kA+3 are unwritten
       if (over >= 1) m1 &= (over >= 2) ? 0u : 0x0000ffffu;
@@ -336,113 +337,122 @@ __global__ __launch_bounds__(64) void attention_fold_kernel(AttnBf16Args a) {
   }
 }
 
-// Route 2a: one wave per (tile, partition) stores the partial.  Tiles of this route hold one
-// token, so the live columns are the first hpt (one per head of the group); only those are
-// stored, each as m, l and hd contiguous 32-bit values.
-template <int HD>
-__global__ __launch_bounds__(64) void attention_split_kernel(AttnBf16Args a) {
+// Route 2, for tiles of one token (decoded tokens): the workgroup's W waves deal the
+// partitions among themselves (wave w takes partitions w, w+W, ..., prefetching the next one's
+// keys), park every partition's partial in LDS, and after one barrier the threads fold the
+// partials in partition order (thread t owns output elements t, t + threads, ... of the tile's
+// live columns).  The statements are those of fold(), so the bits equal route 1; the waves
+// only buy memory parallelism.  LDS holds ``pcap`` partitions; longer contexts take passes.
+template <int HD, int W>
+__global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a, int pcap) {
   constexpr int NT = HD / 16;
+  constexpr int THREADS = 64 * W;
+  constexpr int EPT = (16 * HD + THREADS - 1) / THREADS;   // output elements per thread at most (16 live columns)
+  constexpr int CELL = HD + 2;                              // m, l, then hd values
+  constexpr bool PREFETCH = HD <= 64;
+  extern __shared__ float parts[];                          // [pcap][hpt][CELL]
   GroupCtx gc;
   TileCtx<HD> tc[1];
-  if (!group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc)) return;
-  const int part = blockIdx.z;
-  if (part < gc.kmin / ATT_PART || part > gc.kmax / ATT_PART) return;
-  KFrags<HD> kf;
-  VFrags<HD> vf;
-  load_keys<HD>(a, gc, part, kf);
-  load_values<HD>(a, gc, part, vf);
-  float m_p, l_p;
-  f32x4 o_p[NT];
-  partition_partial<HD>(a, gc, tc[0], part, kf, vf, m_p, l_p, o_p);
-  if (gc.r >= a.hpt) return;
-  const size_t cell = (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * a.max_parts + part) * a.hpt + gc.r;
-  if (gc.g == 0) {
-    a.part_ml[cell * 2 + 0] = m_p;
-    a.part_ml[cell * 2 + 1] = l_p;
-  }
-  float* po = a.part_o + cell * HD;
+  if (!group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc)) return;   // uniform over the workgroup
+  const int wave = threadIdx.x >> 6;
+  const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
+  const int elems = a.hpt * HD;
+  float m[EPT], l[EPT], o[EPT];
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * gc.g) = o_p[dt];
-}
-
-// Route 2b: the same left fold, one wave per query (tile, kv head, column), lane l owning
-// elements l, l+64, ... of the output; the partials are read in partition order.
-template <int HD>
-__global__ __launch_bounds__(64) void attention_combine_kernel(AttnBf16Args a) {
-  constexpr int DPL = (HD + 63) / 64;
-  const int lane = threadIdx.x, tile = blockIdx.x, head_item = blockIdx.y, col = blockIdx.z;
+  for (int j = 0; j < EPT; ++j) {
+    m[j] = -INFINITY;
+    l[j] = 0.0f;
+    o[j] = 0.0f;
+  }
+  for (int pass0 = first; pass0 <= last; pass0 += pcap) {
+    const int pass_last = (last - pass0) < pcap ? last : pass0 + pcap - 1;
+    KFrags<HD> kf, kf_next;
+    VFrags<HD> vf;
+    int part = pass0 + wave;
+    if constexpr (PREFETCH) {
+      if (part <= pass_last) load_keys<HD>(a, gc, part, kf);
+    }
+    for (; part <= pass_last; part += W) {
+      if constexpr (!PREFETCH) load_keys<HD>(a, gc, part, kf);
+      load_values<HD>(a, gc, part, vf);
+      if constexpr (PREFETCH) {
+        if (part + W <= pass_last) load_keys<HD>(a, gc, part + W, kf_next);
+      }
+      float m_p, l_p;
+      f32x4 o_p[NT];
+      partition_partial<HD>(a, gc, tc[0], part, kf, vf, m_p, l_p, o_p);
+      if (gc.r < a.hpt) {
+        float* cell = parts + ((size_t)(part - pass0) * a.hpt + gc.r) * CELL;
+        if (gc.g == 0) {
+          cell[0] = m_p;
+          cell[1] = l_p;
+        }
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) cell[2 + 16 * dt + 4 * gc.g + i] = o_p[dt][i];
+      }
+      if constexpr (PREFETCH) kf = kf_next;
+    }
+    __syncthreads();
+    const int count = pass_last - pass0 + 1;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = threadIdx.x + j * THREADS;
+      if (e >= elems) continue;
+      const int col = e / HD, d = e % HD;
+      for (int wv = 0; wv < count; ++wv) {
+        const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
+        const float m_p = cell[0], l_p = cell[1], o_p = cell[2 + d];
+        if (m_p == -INFINITY) continue;
+        if (m[j] == -INFINITY) {
+          m[j] = m_p;
+          l[j] = l_p;
+          o[j] = o_p;
+          continue;
+        }
+        float mn, fa, fb;
+        fold_scalars(m[j], m_p, mn, fa, fb);
+        l[j] = fmaf(l[j], fa, l_p * fb);
+        o[j] = fmaf(o[j], fa, o_p * fb);
+        m[j] = mn;
+      }
+    }
+    __syncthreads();
+  }
+  // columns of a one-token tile: column c is head sub*hpt + c of the kv head's group
   const int group = a.heads / a.kv_heads;
-  const int kvh = head_item / a.nsub, sub = head_item % a.nsub;
-  if (sub * a.hpt + col >= group) return;
-  const int row = a.tiles != nullptr ? a.tiles[tile * 4] : tile;
-  const int pos = a.positions[row];
-  if (pos < 0) return;
-  const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
-  const int first = lo / ATT_PART, last = pos / ATT_PART;
-  const size_t cell0 = (((size_t)tile * gridDim.y + head_item) * a.max_parts) * a.hpt + col;
-  float m = -INFINITY, l = 0.0f, o[DPL];
+  const int row = a.tiles != nullptr ? a.tiles[blockIdx.x * 4] : blockIdx.x;
 #pragma unroll
-  for (int t = 0; t < DPL; ++t) o[t] = 0.0f;
-  constexpr int UN = 4;
-  for (int p0 = first; p0 <= last; p0 += UN) {
-    float mp[UN], lp[UN], op[UN][DPL];
-#pragma unroll
-    for (int j = 0; j < UN; ++j) {
-      const int p = p0 + j;
-      const size_t cell = cell0 + (size_t)(p <= last ? p : last) * a.hpt;
-      mp[j] = a.part_ml[cell * 2 + 0];
-      lp[j] = a.part_ml[cell * 2 + 1];
-#pragma unroll
-      for (int t = 0; t < DPL; ++t) {
-        const int d = lane + 64 * t;
-        op[j][t] = d < HD ? a.part_o[cell * HD + d] : 0.0f;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < UN; ++j) {
-      if (p0 + j > last || mp[j] == -INFINITY) continue;
-      if (m == -INFINITY) {
-        m = mp[j];
-        l = lp[j];
-#pragma unroll
-        for (int t = 0; t < DPL; ++t) o[t] = op[j][t];
-        continue;
-      }
-      float mn, fa, fb;
-      fold_scalars(m, mp[j], mn, fa, fb);
-      l = fmaf(l, fa, lp[j] * fb);
-#pragma unroll
-      for (int t = 0; t < DPL; ++t) o[t] = fmaf(o[t], fa, op[j][t] * fb);
-      m = mn;
-    }
-  }
-  const float inv = 1.0f / l;
-  bf16_t* dst = a.out + (size_t)row * a.out_stride + (size_t)(kvh * group + sub * a.hpt + col) * HD;
-#pragma unroll
-  for (int t = 0; t < DPL; ++t) {
-    const int d = lane + 64 * t;
-    if (d < HD) dst[d] = f32_to_bf16(o[t] * inv);
+  for (int j = 0; j < EPT; ++j) {
+    const int e = threadIdx.x + j * THREADS;
+    if (e >= elems) continue;
+    const int col = e / HD, d = e % HD;
+    if (gc.sub * a.hpt + col >= group) continue;
+    const float inv = 1.0f / l[j];
+    a.out[(size_t)row * a.out_stride + (size_t)(gc.kvh * group + gc.sub * a.hpt + col) * HD + d] = f32_to_bf16(o[j] * inv);
   }
 }
 
 template <int HD>
-static void launch_attention(const AttnBf16Args& a, int split, hipStream_t s) {
-  const dim3 block(64);
+static void launch_attention(const AttnBf16Args& a, int decode, hipStream_t s) {
   const int items = a.kv_heads * a.nsub;
-  if (split) {
-    hipLaunchKernelGGL(attention_split_kernel<HD>, dim3(a.num_tiles, items, a.max_parts), block, 0, s, a);
-    hipLaunchKernelGGL(attention_combine_kernel<HD>, dim3(a.num_tiles, items, a.hpt), block, 0, s, a);
+  if (decode) {
+    constexpr int W = 8;
+    const size_t cell = (size_t)a.hpt * (HD + 2) * sizeof(float);
+    int pcap = (int)((48 * 1024) / cell);          // partitions whose partials fit 48 KB of LDS
+    pcap = pcap < W ? W : (pcap > 256 ? 256 : pcap);
+    hipLaunchKernelGGL((attention_decode_kernel<HD, W>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a, pcap);
   } else {
     constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
-    hipLaunchKernelGGL((attention_fold_kernel<HD, QT>), dim3((a.num_tiles + QT - 1) / QT, items), block, 0, s, a);
+    hipLaunchKernelGGL((attention_fold_kernel<HD, QT>), dim3((a.num_tiles + QT - 1) / QT, items), dim3(64), 0, s, a);
   }
 }
 
 extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                                  int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                                  const void* v_cache, void* out, int out_stride, int heads, int kv_heads,
-                                 int head_dim, int page_size, int window, float scale, int split, int max_parts,
-                                 float* part_o, float* part_ml, void* stream) {
+                                 int head_dim, int page_size, int window, float scale, int decode, void* stream) {
   if (num_tiles <= 0) return 0;
   if (kv_heads <= 0 || heads % kv_heads) return -2;
   if (page_size < 4 || (page_size & (page_size - 1)) || page_size > ATT_PART) return -5;  // 4-key loads stay inside a page
@@ -451,18 +461,15 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   AttnBf16Args a;
   a.q = (const bf16_t*)q; a.positions = positions; a.block_table = block_table; a.tiles = tiles;
   a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache; a.out = (bf16_t*)out;
-  a.part_o = part_o; a.part_ml = part_ml;
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size; a.table_stride = table_stride;
   a.q_stride = q_stride; a.out_stride = out_stride; a.window = window;
   a.hpt = group < 16 ? group : 16;
   a.nsub = (group + a.hpt - 1) / a.hpt;
-  a.max_parts = max_parts;
   a.num_tiles = num_tiles;
   a.scale = scale;
-  if (kv_heads * a.nsub > 65535 || max_parts > 65535) return -2;
-  if (split && (max_parts <= 0 || !part_o || !part_ml)) return -2;
+  if (kv_heads * a.nsub > 65535) return -2;
   hipStream_t s = (hipStream_t)stream;
-#define BW_CASE(HD) case HD: launch_attention<HD>(a, split, s); break;
+#define BW_CASE(HD) case HD: launch_attention<HD>(a, decode, s); break;
   switch (head_dim) {
     BW_CASE(16) BW_CASE(32) BW_CASE(48) BW_CASE(64) BW_CASE(80) BW_CASE(96) BW_CASE(112) BW_CASE(128)
     BW_CASE(160) BW_CASE(192) BW_CASE(224) BW_CASE(256)

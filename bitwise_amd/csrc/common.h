@@ -51,5 +51,70 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Sum of squares of one row given as 16-byte vectors: lane l owns vectors l, l+64, ... and runs
+// one fused multiply-add chain over their elements in ascending order; the lanes are joined by
+// the xor butterflies of wave_sum.  Every kernel that needs a row's sum of squares in bfloat16
+// mode calls this, so the bits agree.
+__device__ __forceinline__ float row_sumsq_vec(const f32x4* __restrict__ xv, int nvec, int lane) {
+  float acc = 0.0f;
+  constexpr int UN = 8;
+  for (int c0 = 0; c0 < nvec; c0 += 64 * UN) {
+    f32x4 v[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      const int c = c0 + 64 * j + lane;
+      v[j] = c < nvec ? xv[c] : (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = fmaf(v[j][e], v[j][e], acc);
+  }
+  return wave_sum(acc);
+}
+
+// Load 4 norm weights (bfloat16 or 32-bit) starting at element 4c as floats.
+__device__ __forceinline__ f32x4 load_norm_w4(const void* __restrict__ w, int is_bf16, int c) {
+  if (is_bf16) {
+    const u32x2 p = reinterpret_cast<const u32x2*>(w)[c];
+    return (f32x4){__uint_as_float(p[0] << 16), __uint_as_float(p[0] & 0xffff0000u), __uint_as_float(p[1] << 16),
+                   __uint_as_float(p[1] & 0xffff0000u)};
+  }
+  return reinterpret_cast<const f32x4*>(w)[c];
+}
+
+// RMSNorm of one row of at most 2048 elements (a multiple of 4) by one wave, with every load
+// issued before anything is computed: the row's vectors stay in registers between the sum of
+// squares and the scaling.  Same order and statements as row_sumsq_vec and the store loop of
+// rmsnorm_bf16_kernel.  ``store(c, packed)`` receives vector c as four bfloat16 in 8 bytes.
+template <typename Store>
+__device__ __forceinline__ void rmsnorm_row_small(const f32x4* __restrict__ xv, const void* __restrict__ w,
+                                                  int w_is_bf16, int nvec, int dim, float eps, int lane, Store store) {
+  constexpr int UN = 8;
+  f32x4 v[UN], wv[UN];
+#pragma unroll
+  for (int j = 0; j < UN; ++j) {
+    const int c = 64 * j + lane;
+    v[j] = c < nvec ? xv[c] : (f32x4){0.f, 0.f, 0.f, 0.f};
+    wv[j] = c < nvec ? load_norm_w4(w, w_is_bf16, c) : (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < UN; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = fmaf(v[j][e], v[j][e], acc);
+  acc = wave_sum(acc);
+  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+#pragma unroll
+  for (int j = 0; j < UN; ++j) {
+    const int c = 64 * j + lane;
+    if (c < nvec) {
+      u32x2 pk = {pack_bf16x2((v[j][0] * inv) * wv[j][0], (v[j][1] * inv) * wv[j][1]),
+                  pack_bf16x2((v[j][2] * inv) * wv[j][2], (v[j][3] * inv) * wv[j][3])};
+      store(c, pk);
+    }
+  }
+}
+
 // The launch wrappers return hipGetLastError() as int; 0 is success.
 #define BW_LAUNCH_CHECK() ((int)hipGetLastError())

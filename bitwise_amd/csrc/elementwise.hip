@@ -88,29 +88,16 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16_kernel(const float* __restri
   if ((dim & 3) == 0 && (ldy & 3) == 0) {
     const int nvec = dim >> 2;
     const f32x4* xv = reinterpret_cast<const f32x4*>(xr);
-    constexpr int UN = 8;
-    for (int c0 = 0; c0 < nvec; c0 += 64 * UN) {
-      f32x4 v[UN];
-#pragma unroll
-      for (int j = 0; j < UN; ++j) {
-        const int c = c0 + 64 * j + lane;
-        v[j] = c < nvec ? xv[c] : (f32x4){0.f, 0.f, 0.f, 0.f};
-      }
-#pragma unroll
-      for (int j = 0; j < UN; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = fmaf(v[j][e], v[j][e], acc);
+    if (dim <= 2048) {      // the whole row fits the wave's registers: one round of loads
+      rmsnorm_row_small(xv, w, sizeof(WT) == 2, nvec, dim, eps, lane,
+                        [&](int c, u32x2 pk) { *reinterpret_cast<u32x2*>(yr + 4 * c) = pk; });
+      return;
     }
-    acc = wave_sum(acc);
+    acc = row_sumsq_vec(xv, nvec, lane);
     const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
     for (int c = lane; c < nvec; c += 64) {
       const f32x4 v = xv[c];
-      float wv[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if constexpr (sizeof(WT) == 2) wv[e] = bf16_to_f32(w[4 * c + e]);
-        else wv[e] = w[4 * c + e];
-      }
+      const f32x4 wv = load_norm_w4(w, sizeof(WT) == 2, c);
       u32x2 pk = {pack_bf16x2((v[0] * inv) * wv[0], (v[1] * inv) * wv[1]),
                   pack_bf16x2((v[2] * inv) * wv[2], (v[3] * inv) * wv[3])};
       *reinterpret_cast<u32x2*>(yr + 4 * c) = pk;

@@ -1,0 +1,334 @@
+// The matrix product of decode steps (up to 16 rows, bfloat16 mode), with the work around it
+// fused in: optionally RMSNorm in front (the rows arrive as the 32-bit residual stream), and
+// behind it a plain store, the residual add, SwiGLU, or rotary encoding plus the cache write
+// (for the stacked q|k|v product).  A decode step is bound by kernel count and by how many
+// weight bytes are in flight, not by arithmetic; this kernel keeps the rows in LDS, so that
+// every outstanding memory request of a wave is a weight load, and replaces up to three
+// launches by one.
+//
+// The arithmetic is that of the separate kernels, statement for statement, so a row's bits
+// do not depend on which route ran it:
+//   * RMSNorm: the sum of squares in the order of rmsnorm_bf16_kernel (lane l owns 16-byte
+//     vectors l, l+64, ...; xor butterflies), inv = 1/sqrt(ss/dim + eps), bf16((x*inv)*w);
+//   * product: K in segments of 2048; per segment every 16x16 block of outputs is one
+//     v_mfma_f32_16x16x32_bf16 chain over k ascending from zero; segments added left to right;
+//   * rotary: o1 = x1*c - x2*s, o2 = x2*c + x1*s on the 32-bit products, one rounding when
+//     q goes to its buffer and k, v to their page slots (v transposed).
+//
+// Shape: a workgroup is SPW strips of 16 output columns times S segments, one wave each (for
+// q|k|v with rotary: the strips of one head).  Every wave first puts D steps of its weights in
+// flight, then all waves bring the rows into LDS as bfloat16 (normalising them on the way if
+// asked; rows padded by 16 bytes so that operand reads hit distinct banks), and then each
+// runs its chain with A operands from LDS and B operands from its ring.  Segment results of
+// a strip meet in LDS and are added in segment order.
+#include "common.h"
+#include "api.h"
+
+enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI_ROPE_KV = 4 };
+
+#define DEC_SEG 2048
+
+struct DecodeGemmArgs {
+  const void* a;           // NORM: float [M, lda] residual rows; else bf16 [M, lda]
+  const void* norm_w;      // [K] (NORM only)
+  const bf16_t* w;         // [N (or 2N for SwiGLU), K]
+  void* out;               // F32/ADD: float [M, ldo]; BF16/SWIGLU: bf16 [M, ldo]; ROPE_KV: q bf16 [M, heads*hd]
+  int M, N, K, lda, ldo, S, norm_w_is_bf16;
+  float eps;
+  // rotary + cache write
+  const int32_t* positions;
+  const int32_t* row_seq;
+  const int32_t* block_table;
+  const float* cos_table;
+  const float* sin_table;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  int heads, kv_heads, head_dim, page_size, table_stride, write_cache;
+};
+
+template <int EPI, bool NORM, int D>
+__global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
+  constexpr int NB = (EPI == DEPI_SWIGLU_BF16) ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int K = a.K, M = a.M, S = a.S;
+  const int lds_row = K + 8;                      // bf16 elements; +16 bytes keeps operand reads conflict-free
+  bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int strip = wave / S, seg = wave % S;     // the S waves of a strip are neighbours
+  const int n0 = (blockIdx.x * (nwaves / S) + strip) * 16;
+  const bool n_ok = n0 + r < a.N;
+  const int k_begin = seg * DEC_SEG;
+  const int k_end = (K - k_begin) < DEC_SEG ? K : k_begin + DEC_SEG;
+  const bf16_t* wp[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) wp[b] = a.w + ((size_t)b * a.N + (n_ok ? n0 + r : 0)) * K + 8 * g;
+
+  // 1. weight loads in flight first: they depend on nothing
+  u32x4 bq[D][NB];
+  auto issue = [&](int d, int k) {
+    const int ks = k < k_end ? k : k_begin;       // past the end: re-read the first step, never used
+#pragma unroll
+    for (int b = 0; b < NB; ++b) bq[d][b] = *reinterpret_cast<const u32x4*>(wp[b] + ks);
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) issue(d, k_begin + 32 * d);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // rotary epilogue: this thread's (row, pair) items and what they need are fetched now, so that
+  // the position -> table/angle chain runs while the weights stream (at most 2 items a thread)
+  int r_pos[2] = {-1, -1}, r_page[2] = {0, 0};
+  float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
+  if constexpr (EPI == DEPI_ROPE_KV) {
+    const int half = a.head_dim >> 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * blockDim.x;
+      if (e < M * half) {
+        const int m = e / half, i = e % half;
+        const int pos = a.positions[m];
+        r_pos[j] = pos;
+        if (pos >= 0) {
+          r_cos[j] = a.cos_table[(size_t)pos * half + i];
+          r_sin[j] = a.sin_table[(size_t)pos * half + i];
+          r_page[j] = a.block_table[(size_t)a.row_seq[m] * a.table_stride + pos / a.page_size];
+        }
+      }
+    }
+  }
+
+  // 2. the M rows into LDS as bfloat16
+  if constexpr (NORM) {
+    const int nvec = K >> 2;
+    for (int m = wave; m < M; m += nwaves) {     // rows dealt to the waves round robin
+      bf16_t* dst = xs + (size_t)m * lds_row;
+      rmsnorm_row_small(reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda), a.norm_w,
+                        a.norm_w_is_bf16, nvec, K, a.eps, lane,
+                        [&](int c, u32x2 pk) { *reinterpret_cast<u32x2*>(dst + 4 * c) = pk; });
+    }
+  } else {
+    const int cpr = K >> 3;                       // 16-byte chunks per row
+    const int total = M * cpr;
+    constexpr int UN = 8;
+    for (int base = 0; base < total; base += UN * blockDim.x) {
+      u32x4 v[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j) {
+        const int idx = base + j * blockDim.x + threadIdx.x;
+        if (idx < total)
+          v[j] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.a + (size_t)(idx / cpr) * a.lda + (idx % cpr) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < UN; ++j) {
+        const int idx = base + j * blockDim.x + threadIdx.x;
+        if (idx < total) *reinterpret_cast<u32x4*>(xs + (size_t)(idx / cpr) * lds_row + (idx % cpr) * 8) = v[j];
+      }
+    }
+  }
+  __syncthreads();
+
+  // 3. the product: A from LDS (rows past M read row 0; their results are thrown away), B from the ring
+  const bf16_t* ap = xs + (size_t)(r < M ? r : 0) * lds_row + 8 * g;
+  f32x4 acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  constexpr int PA = 4;                            // A operands are read from LDS this many steps ahead
+  static_assert(D % PA == 0, "the A look-ahead must divide the ring depth");
+  u32x4 aq[PA];
+  auto fetch_a = [&](int slot, int k) { aq[slot] = *reinterpret_cast<const u32x4*>(ap + (k < k_end ? k : k_begin)); };
+#pragma unroll
+  for (int j = 0; j < PA; ++j) fetch_a(j, k_begin + 32 * j);
+  for (int k0 = k_begin; k0 < k_end; k0 += 32 * D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int k = k0 + 32 * d;
+      const bool live = k < k_end;
+      const u32x4 af = aq[d % PA];
+      u32x4 bc[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) bc[b] = live ? bq[d][b] : zero;
+      issue(d, k + 32 * D);
+      fetch_a(d % PA, k + 32 * PA);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(bc[b]), acc[b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // 4. segments of a strip meet in LDS and are added in segment order by the strip's first wave
+  if (S > 1) {
+    __syncthreads();                               // every wave is done reading the rows
+    float* red = reinterpret_cast<float*>(smem);   // [wave][NB][4][64]
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) red[((wave * NB + b) * 4 + q) * 64 + lane] = acc[b][q];
+    __syncthreads();
+    if (seg != 0) return;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float y = acc[b][q];
+        for (int s = 1; s < S; ++s) y += red[(((wave + s) * NB + b) * 4 + q) * 64 + lane];
+        acc[b][q] = y;
+      }
+  }
+
+  // 5. epilogue
+  if constexpr (EPI != DEPI_ROPE_KV) {
+    if (!n_ok) return;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = 4 * g + q;
+      if (m >= M) continue;
+      const size_t o = (size_t)m * a.ldo + n0 + r;
+      const float v = acc[0][q];
+      if constexpr (EPI == DEPI_F32) ((float*)a.out)[o] = v;
+      else if constexpr (EPI == DEPI_BF16) ((bf16_t*)a.out)[o] = f32_to_bf16(v);
+      else if constexpr (EPI == DEPI_ADD_F32) ((float*)a.out)[o] += v;
+      else {
+        const float uv = acc[NB - 1][q];
+        ((bf16_t*)a.out)[o] = f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * uv);
+      }
+    }
+  } else {
+    // The workgroup's strips are one head (S is 1 here): blockIdx.x < heads is a q head, then the
+    // k heads, then the v heads.  The 32-bit products go through LDS so that the rotary pairs
+    // (i, i + hd/2), which sit in different strips, meet.
+    const int hd = a.head_dim, half = hd >> 1;
+    __syncthreads();                               // every wave is done reading the rows
+    float* os = reinterpret_cast<float*>(smem);    // [M][hd]
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = 4 * g + q;
+      if (m < M) os[m * hd + 16 * wave + r] = acc[0][q];
+    }
+    __syncthreads();
+    const int head = blockIdx.x;
+    const int q_dim = a.heads * hd;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * blockDim.x;
+      if (e >= M * half) continue;
+      const int m = e / half, i = e % half;
+      const int pos = r_pos[j];
+      if (pos < 0) continue;
+      const float x1 = os[m * hd + i], x2 = os[m * hd + i + half];
+      if (head < a.heads + a.kv_heads) {
+        const float c = r_cos[j], s = r_sin[j];
+        const float o1 = x1 * c - x2 * s;
+        const float o2 = x2 * c + x1 * s;
+        if (head < a.heads) {
+          bf16_t* dst = (bf16_t*)a.out + (size_t)m * q_dim + (size_t)head * hd;
+          dst[i] = f32_to_bf16(o1);
+          dst[i + half] = f32_to_bf16(o2);
+        } else if (a.write_cache) {
+          bf16_t* dst = a.k_cache + (((size_t)r_page[j] * a.kv_heads + (head - a.heads)) * a.page_size + pos % a.page_size) * hd;
+          dst[i] = f32_to_bf16(o1);
+          dst[i + half] = f32_to_bf16(o2);
+        }
+      } else if (a.write_cache) {
+        bf16_t* dst = a.v_cache + ((size_t)r_page[j] * a.kv_heads + (head - a.heads - a.kv_heads)) * hd * a.page_size + pos % a.page_size;
+        dst[(size_t)i * a.page_size] = f32_to_bf16(x1);
+        dst[(size_t)(i + half) * a.page_size] = f32_to_bf16(x2);
+      }
+    }
+  }
+}
+
+static const size_t kMaxLds = 160 * 1024 - 1024;
+
+template <int EPI, bool NORM, int D>
+static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hipStream_t s) {
+  static bool raised = false;
+  size_t lds = (size_t)a.M * (a.K + 8) * sizeof(bf16_t);
+  const size_t red = (size_t)waves * 2 * 4 * 64 * sizeof(float);
+  if (a.S > 1 && red > lds) lds = red;
+  if (lds > kMaxLds) return -2;
+  if (!raised) {   // more than 64 KB of dynamic LDS has to be asked for once
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, NORM, D>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds) != hipSuccess)
+      return (int)hipGetLastError();
+    raised = true;
+  }
+  hipLaunchKernelGGL((decode_gemm_kernel<EPI, NORM, D>), dim3(blocks), dim3(64 * waves), lds, s, a);
+  return BW_LAUNCH_CHECK();
+}
+
+// Can the rows (M of them, K wide) live in LDS, and do the waves of a strip fit a workgroup?
+static int check_decode_gemm(const DecodeGemmArgs& a, bool norm) {
+  if (a.M <= 0 || a.M > 16 || a.N <= 0 || a.K <= 0 || (a.K % 32)) return -2;
+  if (a.S > 4) return -2;
+  if ((size_t)a.M * (a.K + 8) * sizeof(bf16_t) > kMaxLds) return -2;
+  if (norm && (a.K > 2048 || (a.lda % 4))) return -2;
+  if (!norm && (a.lda % 8)) return -2;
+  if (a.lda < a.K) return -2;
+  return 0;
+}
+
+extern "C" int bw_decode_gemm_supported(int M, int K, int norm) {
+  DecodeGemmArgs a{};
+  a.M = M; a.N = 16; a.K = K; a.lda = K; a.S = (K + DEC_SEG - 1) / DEC_SEG;
+  return check_decode_gemm(a, norm != 0) == 0;
+}
+
+extern "C" int bw_decode_gemm_bf16(const void* a_rows, int lda, int a_is_f32, const void* norm_w, int norm_w_is_bf16,
+                                   float eps, const void* w, void* out, int ldo, int M, int N, int K, int epilogue,
+                                   void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  DecodeGemmArgs a{};
+  a.a = a_rows; a.norm_w = norm_w; a.w = (const bf16_t*)w; a.out = out;
+  a.M = M; a.N = N; a.K = K; a.lda = lda; a.ldo = ldo; a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
+  a.S = (K + DEC_SEG - 1) / DEC_SEG;
+  const bool norm = a_is_f32 != 0;
+  const int bad = check_decode_gemm(a, norm);
+  if (bad) return bad;
+  if (ldo < N) return -2;
+  if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
+  const int spw = a.S == 1 ? 4 : (a.S == 2 ? 2 : 1);     // strips per workgroup; waves = spw * S <= 4
+  const int waves = spw * a.S;
+  const int strips = (N + 15) / 16;
+  const int blocks = (strips + spw - 1) / spw;
+  hipStream_t s = (hipStream_t)stream;
+#define BW_DEC(EPIV, DV)                                                        \
+  case EPIV:                                                                    \
+    return norm ? launch_decode_gemm<EPIV, true, DV>(a, waves, blocks, s)       \
+                : launch_decode_gemm<EPIV, false, DV>(a, waves, blocks, s);
+  switch (epilogue) {
+    BW_DEC(DEPI_F32, 32)
+    BW_DEC(DEPI_BF16, 32)
+    BW_DEC(DEPI_ADD_F32, 32)
+    BW_DEC(DEPI_SWIGLU_BF16, 20)
+  }
+#undef BW_DEC
+  return -2;
+}
+
+extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps,
+                                     const void* w_qkv, void* q_out, const int32_t* positions,
+                                     const int32_t* row_seq, const int32_t* block_table, int table_stride,
+                                     const float* cos_table, const float* sin_table, void* k_cache, void* v_cache,
+                                     int M, int heads, int kv_heads, int head_dim, int K, int page_size,
+                                     int write_cache, void* stream) {
+  if (M <= 0) return 0;
+  if (head_dim % 16 || head_dim < 16 || head_dim > 64 || page_size <= 0) return -4;   // one wave per strip, four at most
+  DecodeGemmArgs a{};
+  a.a = x; a.norm_w = norm_w; a.w = (const bf16_t*)w_qkv; a.out = q_out;
+  a.M = M; a.N = (heads + 2 * kv_heads) * head_dim; a.K = K; a.lda = ldx; a.ldo = heads * head_dim;
+  a.S = 1;
+  a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
+  a.positions = positions; a.row_seq = row_seq; a.block_table = block_table; a.cos_table = cos_table;
+  a.sin_table = sin_table; a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache;
+  a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.page_size = page_size;
+  a.table_stride = table_stride; a.write_cache = write_cache;
+  if (K > DEC_SEG) return -2;
+  const int bad = check_decode_gemm(a, true);
+  if (bad) return bad;
+  if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
+  if ((size_t)M * head_dim * sizeof(float) > (size_t)M * (K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
+  return launch_decode_gemm<DEPI_ROPE_KV, true, 32>(a, head_dim / 16, heads + 2 * kv_heads, (hipStream_t)stream);
+}

@@ -43,8 +43,13 @@ _SIGS = {
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p,
-                          c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "bw_decode_gemm_supported": [c_int, c_int, c_int],
+    "bw_decode_gemm_bf16": [c_void_p, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
+                            c_int, c_int, c_void_p],
+    "bw_norm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                              c_int, c_int, c_int, c_void_p],
     "bw_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_fingerprint": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
 }
@@ -227,6 +232,88 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
                                epilogue, _stream()), "gemm_bf16")
 
 
+# ------------------------------------------------------------------------------ decode fusions
+
+_decode_ok = {}
+
+
+def decode_gemm_supported(rows: int, inner: int, norm: bool) -> bool:
+    """Whether the decode product kernel (rows kept in LDS) takes this many rows of this width."""
+    key = (rows, inner, norm)
+    if key not in _decode_ok:
+        _decode_ok[key] = bool(_fn("bw_decode_gemm_supported")(rows, inner, int(norm)))
+    return _decode_ok[key]
+
+
+def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor) -> bool:
+    """Whether RMSNorm + product can run as one kernel for this step."""
+    K = weight.shape[1]
+    return (weight.dtype == torch.bfloat16 and x.dtype == torch.float32 and x.shape[1] == K
+            and x.stride(0) % 4 == 0 and decode_gemm_supported(rows, K, True))
+
+
+def _decode_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, epilogue: int,
+                 norm_weight: Optional[torch.Tensor], eps: float) -> None:
+    N, K = w.shape
+    if epilogue == EPI_SWIGLU_BF16:
+        N //= 2
+    _check(_fn("bw_decode_gemm_bf16")(a.data_ptr(), a.stride(0), int(norm_weight is not None),
+                                      norm_weight.data_ptr() if norm_weight is not None else 0,
+                                      _is_bf16(norm_weight, "norm weight") if norm_weight is not None else 0,
+                                      float(eps), w.data_ptr(), out.data_ptr(), out.stride(0), rows, N, K, epilogue,
+                                      _stream()), "decode_gemm_bf16")
+
+
+def norm_gemm_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+                   rows: int, epilogue: int) -> None:
+    """out[:rows] = epilogue(rmsnorm(x[:rows]) @ w.T) in one kernel; the bits of rmsnorm followed
+    by gemm_bf16.  epilogue as for gemm_bf16 (EPI_SWIGLU_BF16 takes the stacked weight [2N, K])."""
+    _need(x, torch.float32, "x")
+    _need(w, torch.bfloat16, "weight")
+    N, K = w.shape
+    if epilogue == EPI_SWIGLU_BF16:
+        N //= 2
+    _need(out, torch.bfloat16 if epilogue in (EPI_BF16, EPI_SWIGLU_BF16) else torch.float32, "out")
+    if not can_fuse_norm(rows, w, x) or norm_weight.numel() != K or not norm_weight.is_cuda:
+        raise ValueError(f"norm_gemm_bf16: {rows} rows of width {x.shape[1]} against weight {tuple(w.shape)} cannot be fused")
+    if out.shape[1] != N or out.shape[0] < rows or x.shape[0] < rows:
+        raise ValueError("norm_gemm_bf16: out does not fit")
+    _decode_gemm(x, w, out, rows, epilogue, norm_weight, eps)
+
+
+def norm_qkv_rope_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor, q_out: torch.Tensor,
+                       positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor, cos: torch.Tensor,
+                       sin: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, rows: int, heads: int,
+                       kv_heads: int, head_dim: int, page_size: int, write_cache: bool = True) -> None:
+    """RMSNorm, the stacked q|k|v product, rotation and the cache write in one kernel (one
+    workgroup per head); the bits of rmsnorm, gemm_bf16 and rope_kvwrite run one after the other."""
+    _need(x, torch.float32, "x")
+    _need(w_qkv, torch.bfloat16, "qkv weight")
+    _need(q_out, torch.bfloat16, "q_out")
+    _need(k_cache, torch.bfloat16, "k_cache")
+    _need(v_cache, torch.bfloat16, "v_cache")
+    _need(positions, torch.int32, "positions")
+    _need(row_seq, torch.int32, "row_seq")
+    _need(block_table, torch.int32, "block_table")
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    N, K = w_qkv.shape
+    if N != (heads + 2 * kv_heads) * head_dim or head_dim > 64 or head_dim % 16:
+        raise ValueError("norm_qkv_rope_bf16: weight is not [q|k|v] heads of at most 64 elements")
+    if not can_fuse_norm(rows, w_qkv, x) or norm_weight.numel() != K:
+        raise ValueError("norm_qkv_rope_bf16: this step cannot be fused")
+    if q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows or positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("norm_qkv_rope_bf16: buffers too small")
+    if cos.shape[1] != head_dim // 2 or sin.shape != cos.shape:
+        raise ValueError("norm_qkv_rope_bf16: tables must be [positions, head_dim/2]")
+    _check(_fn("bw_norm_qkv_rope_bf16")(x.data_ptr(), x.stride(0), norm_weight.data_ptr(),
+                                        _is_bf16(norm_weight, "norm weight"), float(eps), w_qkv.data_ptr(),
+                                        q_out.data_ptr(), positions.data_ptr(), row_seq.data_ptr(),
+                                        block_table.data_ptr(), block_table.stride(0), cos.data_ptr(), sin.data_ptr(),
+                                        k_cache.data_ptr(), v_cache.data_ptr(), rows, heads, kv_heads, head_dim, K,
+                                        page_size, int(write_cache), _stream()), "norm_qkv_rope_bf16")
+
+
 # ------------------------------------------------------------------------------ attention
 
 def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
@@ -254,16 +341,17 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
 
 
 def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
-                   tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, heads: int,
-                   kv_heads: int, head_dim: int, page_size: int, window: int, scale: float, split: bool = False,
-                   max_parts: int = 0, part_o: Optional[torch.Tensor] = None,
-                   part_ml: Optional[torch.Tensor] = None) -> None:
+                   tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   out: torch.Tensor, heads: int, kv_heads: int, head_dim: int, page_size: int, window: int,
+                   scale: float, decode: bool = False) -> None:
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
-    [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0), or None for
-    "tile t is row t of sequence t" (split route only).  Without ``split`` the tiles of a
-    sequence must come in runs padded to ``fold_group_tiles(head_dim)`` (empty tiles allowed).  With
-    ``split`` (tiles of one token each) every (tile, partition) is a wave of its own and the
-    partials are folded by a second kernel; the bits equal the unsplit route."""
+    [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).
+
+    ``decode`` False: one wave folds all partitions of up to ``fold_group_tiles(head_dim)`` tiles;
+    the tiles of a sequence must come in runs padded to that number (empty tiles allowed).
+    ``decode`` True (tiles of one token each; ``tiles`` None means "tile t is row t of sequence
+    t"): a workgroup per tile whose waves take one 64-key partition each and fold through LDS
+    in partition order.  The bits are the same either way."""
     _need(q, torch.bfloat16, "q")
     _need(out, torch.bfloat16, "out")
     _need(k_cache, torch.bfloat16, "k_cache")
@@ -272,8 +360,8 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     _need(block_table, torch.int32, "block_table")
     if tiles is not None:
         _need(tiles, torch.int32, "tiles")
-    elif not split:
-        raise ValueError("attention_bf16: implicit tiles are for the split route only")
+    elif not decode:
+        raise ValueError("attention_bf16: implicit tiles are for decoded tokens only")
     if head_dim not in HEAD_DIMS:
         raise ValueError(f"attention: head size {head_dim} is not supported; supported: {HEAD_DIMS}")
     if heads % kv_heads:
@@ -281,23 +369,13 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or (
             tiles is not None and tiles.numel() < 4 * num_tiles):
         raise ValueError("attention_bf16: q, out or tiles do not fit")
-    group = heads // kv_heads
-    hpt = min(group, 16)
-    items = num_tiles * kv_heads * ((group + hpt - 1) // hpt)
-    if split:
-        if part_o is None or part_ml is None or max_parts <= 0:
-            raise ValueError("attention_bf16: split needs scratch buffers")
-        _need(part_o, torch.float32, "part_o")
-        _need(part_ml, torch.float32, "part_ml")
-        if part_o.numel() < items * max_parts * head_dim * hpt or part_ml.numel() < items * max_parts * 2 * hpt:
-            raise ValueError("attention_bf16: scratch buffers too small")
+    if tiles is None and (positions.numel() < num_tiles or block_table.shape[0] < num_tiles):
+        raise ValueError("attention_bf16: fewer rows or block tables than implicit tiles")
     _check(_fn("bw_attention_bf16")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
                                     block_table.stride(0), tiles.data_ptr() if tiles is not None else 0, num_tiles,
-                                    k_cache.data_ptr(),
-                                    v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads, kv_heads, head_dim,
-                                    page_size, int(window), float(scale), int(split), max_parts,
-                                    part_o.data_ptr() if part_o is not None else 0,
-                                    part_ml.data_ptr() if part_ml is not None else 0, _stream()), "attention_bf16")
+                                    k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
+                                    kv_heads, head_dim, page_size, int(window), float(scale), int(decode), _stream()),
+           "attention_bf16")
 
 
 # ------------------------------------------------------------------------------ sampling

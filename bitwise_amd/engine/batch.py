@@ -11,8 +11,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..csrc.ops import ATT_PART
-from ..parts.attention import SPLIT_MIN_CONTEXT
+from ..parts.attention import DECODE_MIN_CONTEXT
 
 
 @dataclass
@@ -29,9 +28,8 @@ class Segment:
 class AttentionPlan:
     fold_tiles: Optional[torch.Tensor]
     fold_count: int
-    split_tiles: Optional[torch.Tensor]
-    split_count: int
-    max_parts: int
+    decode_tiles: Optional[torch.Tensor]      # None with a positive count: tile t is row t of request t
+    decode_count: int
 
 
 class StepContext:
@@ -80,17 +78,15 @@ class StepContext:
         """Tiles of up to ``tokens_per_tile`` consecutive rows of one request; every request's
         run of tiles is padded with empty tiles to a multiple of ``group_tiles`` (the tiles one
         wave owns must belong to one request).  Single decoded tokens with a long context go
-        the split route (a wave per 64-key partition)."""
+        to the decode kernel (a wave per 64-key partition)."""
         plan = self._plans.get((tokens_per_tile, group_tiles))
         if plan is not None:
             return plan
         fold, split = [], []
-        max_parts = 0
         for i, s in enumerate(self.segments):
             n, r0 = len(s.tokens), self.seq_start[i]
-            if n == 1 and s.pos0 + 1 >= SPLIT_MIN_CONTEXT:
+            if n == 1 and s.pos0 + 1 >= DECODE_MIN_CONTEXT:
                 split.append((r0, 1, i, 0))
-                max_parts = max(max_parts, s.pos0 // ATT_PART + 1)
                 continue
             for off in range(0, n, tokens_per_tile):
                 fold.append((r0 + off, min(tokens_per_tile, n - off), i, 0))
@@ -99,6 +95,6 @@ class StepContext:
         both = np.asarray(fold + split, np.int32).reshape(-1, 4)
         dev = torch.from_numpy(both).to(self.device)
         plan = AttentionPlan(dev[:len(fold)].contiguous() if fold else None, len(fold),
-                             dev[len(fold):].contiguous() if split else None, len(split), max_parts)
+                             dev[len(fold):].contiguous() if split else None, len(split))
         self._plans[(tokens_per_tile, group_tiles)] = plan
         return plan

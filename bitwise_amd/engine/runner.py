@@ -15,7 +15,6 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..csrc.ops import ATT_PART
 from ..models.assembled import AssembledModel
 from .batch import AttentionPlan, Segment, StepContext
 from .storage import CacheStorage
@@ -26,7 +25,7 @@ GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 class _StaticDecodeContext:
     """Fixed device arrays for a decode batch of up to ``size`` requests, one row each."""
 
-    def __init__(self, size: int, num_groups: int, max_pages: int, max_parts: int, device: torch.device):
+    def __init__(self, size: int, num_groups: int, max_pages: int, device: torch.device):
         self.rows = self.nseq = self.num_wanted = size
         self.device = device
         self.max_pages = max_pages
@@ -36,8 +35,7 @@ class _StaticDecodeContext:
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self.slots = torch.zeros(size, dtype=torch.int32, device=device)
         self.block_tables = [torch.zeros((size, max_pages), dtype=torch.int32, device=device) for _ in range(num_groups)]
-        self._plan = AttentionPlan(None, 0, None, size, max_parts)      # implicit tiles: tile t = row t of request t
-        self._host = np.empty((3 + num_groups * max_pages, size), np.int32)
+        self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
         self.segments: List[Segment] = []
 
     def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
@@ -118,8 +116,7 @@ class ModelRunner:
     def _capture(self, bucket: int, segments: Sequence[Segment]):
         rt = self.rt
         max_pages = (self.max_model_len + rt.page_size - 1) // rt.page_size
-        max_parts = (self.max_model_len + ATT_PART - 1) // ATT_PART
-        ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, max_parts, rt.device)
+        ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, rt.device)
         ctx.fill(segments)
         # One eager run first: it creates every scratch buffer the capture will use and it is
         # the step's real work (writing the same cache slots twice with the same values is harmless).

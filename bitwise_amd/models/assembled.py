@@ -136,5 +136,8 @@ class AssembledModel:
             return None
         last = self.rt.buffer("wanted_rows", self.spec.width, torch.float32, rows=self.rt.max_logit_rows)
         ops.gather_rows(x, ctx.want_rows, last, count)
-        normed = self.final_norm.forward(ctx, last, out_name="final_normed", rows=count)
-        return self.lm_head.forward(ctx, normed, count)[:count]
+        logits = self.lm_head.forward_with_norm(ctx, last, self.final_norm, count)
+        if logits is None:
+            normed = self.final_norm.forward(ctx, last, out_name="final_normed", rows=count)
+            logits = self.lm_head.forward(ctx, normed, count)
+        return logits[:count]

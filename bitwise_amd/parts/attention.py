@@ -17,9 +17,9 @@ from ..csrc import ops
 from .base import CacheSpec, Mixer, TensorSpec, lookup, register_mixer, POSITION_ENCODINGS
 from .linear import Linear
 
-# A decoded token's attention is cut into one wave per 64-key partition once its context is
-# at least this long (same bits either way; this only buys parallelism).
-SPLIT_MIN_CONTEXT = 256
+# A decoded token's attention goes to the kernel that gives every 64-key partition a wave of its
+# own once its context is at least this long (same bits either way; this only buys parallelism).
+DECODE_MIN_CONTEXT = 128
 
 
 @register_mixer("attention")
@@ -74,6 +74,21 @@ class Attention(Mixer):
         """Elements of one page of keys (and likewise of values) of one cache."""
         return self.kv_heads * page_size * self.head_dim
 
+    def forward_with_norm(self, ctx, call, x, norm, residual) -> bool:
+        """Decode steps of few rows: norm, q|k|v product, rotation and cache write are one kernel."""
+        from .norm import RMSNorm
+        rt = self.rt
+        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma and self.head_dim <= 64
+                and ops.can_fuse_norm(ctx.rows, self.qkv.weight, x)):
+            return False
+        q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
+        ops.norm_qkv_rope_bf16(x, norm.weight, norm.eps, self.qkv.weight, q, ctx.positions, ctx.row_seq,
+                               ctx.block_tables[call.group], self.position.cos, self.position.sin, call.k_cache,
+                               call.v_cache, ctx.rows, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                               call.writes_cache)
+        self._attend(ctx, call, q, residual)
+        return True
+
     def forward(self, ctx, call, h, residual) -> None:
         rt, rows = self.rt, ctx.rows
         table = ctx.block_tables[call.group]
@@ -85,20 +100,7 @@ class Attention(Mixer):
             ops.rope_kvwrite(qkv, q, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              rt.page_size, call.writes_cache)
-            out = rt.buffer("attn_out", self.q_dim, torch.bfloat16)
-            plan = ctx.attention_plan(self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
-            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
-                      window, self.scale)
-            if plan.fold_count:
-                ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
-            if plan.split_count:
-                group = self.heads // self.kv_heads
-                columns = self.kv_heads * ((group + self.heads_per_tile - 1) // self.heads_per_tile) * self.heads_per_tile
-                cells = plan.split_count * plan.max_parts * columns
-                part_o = rt.scratch("attn_part_o", cells * self.head_dim, torch.float32)
-                part_ml = rt.scratch("attn_part_ml", cells * 2, torch.float32)
-                ops.attention_bf16(q, ctx.positions, table, plan.split_tiles, plan.split_count, *common,
-                                   split=True, max_parts=plan.max_parts, part_o=part_o, part_ml=part_ml)
+            self._attend(ctx, call, q, residual)
         else:
             ops.rope_kvwrite(qkv, None, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
@@ -106,4 +108,19 @@ class Attention(Mixer):
             out = rt.buffer("attn_out", self.q_dim, torch.float32)
             ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
                               self.heads, self.kv_heads, self.head_dim, rt.page_size, window, self.scale)
+            self.o.add_into(out, residual, rows)
+
+    def _attend(self, ctx, call, q, residual) -> None:
+        """bfloat16 attention over the cache for rotated queries ``q``, then the output projection."""
+        rt, rows = self.rt, ctx.rows
+        table = ctx.block_tables[call.group]
+        window = int(self.window or 0)
+        out = rt.buffer("attn_out", self.q_dim, torch.bfloat16)
+        plan = ctx.attention_plan(self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
+        common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                  window, self.scale)
+        if plan.fold_count:
+            ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
+        if plan.decode_count:
+            ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True)
         self.o.add_into(out, residual, rows)

@@ -137,9 +137,19 @@ class Mixer(Part):
         """
         raise NotImplementedError
 
+    def forward_with_norm(self, ctx, call, x, norm, residual) -> bool:
+        """Optional: run ``norm`` and the mixer as fused kernels on the un-normed rows ``x``.
+        Return False (and do nothing) if this step cannot be fused; the block then calls the
+        norm and ``forward`` one after the other.  The result must be the same bits."""
+        return False
+
 
 class FeedForward(Part):
     graph_safe = False
+
+    def forward_with_norm(self, ctx, x, norm, residual) -> bool:
+        """As Mixer.forward_with_norm."""
+        return False
 
     def forward(self, ctx, h, residual) -> None:
         """h: normed rows; adds the feed-forward's output into ``residual`` in place."""

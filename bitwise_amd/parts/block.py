@@ -10,7 +10,9 @@ class PreNormBlock(Block):
     """x += mixer(norm1(x)); x += feed_forward(norm2(x)) (src/model.cpp:281-305)."""
 
     def forward(self, ctx, call, x) -> None:
-        h = self.mixer_norm.forward(ctx, x)
-        self.mixer.forward(ctx, call, h, x)
-        h = self.ffn_norm.forward(ctx, x)
-        self.feed_forward.forward(ctx, h, x)
+        if not self.mixer.forward_with_norm(ctx, call, x, self.mixer_norm, x):
+            h = self.mixer_norm.forward(ctx, x)
+            self.mixer.forward(ctx, call, h, x)
+        if not self.feed_forward.forward_with_norm(ctx, x, self.ffn_norm, x):
+            h = self.ffn_norm.forward(ctx, x)
+            self.feed_forward.forward(ctx, h, x)

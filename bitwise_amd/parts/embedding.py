@@ -55,6 +55,17 @@ class LMHead(Part):
     def weight_bytes(self) -> int:
         return self.linear.nbytes()
 
+    def forward_with_norm(self, ctx, x: torch.Tensor, norm, count: int):
+        """Few wanted rows: the final norm and the head product are one kernel.  Returns the
+        logits buffer, or None if this step cannot be fused."""
+        from .norm import RMSNorm
+        if not (self.rt.bf16 and isinstance(norm, RMSNorm) and self.linear.mfma
+                and ops.can_fuse_norm(count, self.linear.weight, x)):
+            return None
+        logits = self.rt.buffer("logits", self.vocab, torch.float32, rows=self.rt.max_logit_rows)
+        ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.linear.weight, logits, count, ops.EPI_F32)
+        return logits
+
     def forward(self, ctx, normed: torch.Tensor, count: int) -> torch.Tensor:
         logits = self.rt.buffer("logits", self.vocab, torch.float32, rows=self.rt.max_logit_rows)
         self.linear.store(normed, logits, count)

@@ -88,7 +88,8 @@ def test_gemm_f32_grid_rows_and_accumulate(gpu):
 
 def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     g = torch.Generator().manual_seed(3)
-    for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40)]:
+    for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
+                    (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144)]:      # several 2048-segments of K
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = torch.randn(N, K, generator=g).bfloat16().to(gpu)
         y = torch.full((M, N), 3.0, device=gpu)
@@ -262,14 +263,8 @@ def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, wi
     if tiles is None:
         tiles = [(r, 1, 0, 0) for r in range(rows)]
     t = torch.tensor(tiles, dtype=torch.int32, device=gpu)
-    kw = {}
-    if split:
-        max_parts = max(positions) // ops.ATT_PART + 1
-        group = heads // kvh
-        cols = kvh * ((group + 15) // 16) * min(group, 16)
-        kw = dict(split=True, max_parts=max_parts, part_o=torch.empty(len(tiles) * max_parts * cols * hd, device=gpu),
-                  part_ml=torch.empty(len(tiles) * max_parts * cols * 2, device=gpu))
-    ops.attention_bf16(q.to(gpu), pos, tab, t, len(tiles), kc, vc, out, heads, kvh, hd, page, window, scale, **kw)
+    ops.attention_bf16(q.to(gpu), pos, tab, t, len(tiles), kc, vc, out, heads, kvh, hd, page, window, scale,
+                       decode=split)
     return out
 
 
@@ -307,7 +302,7 @@ def test_attention_batched_equals_alone_and_plain(gpu, bf16, heads, kvh, hd, pag
     assert (batch.cpu().double() - ref).abs().max() <= tol * ref.abs().max()
     first = v[0].double().repeat_interleave(heads // kvh, dim=0).reshape(-1)
     assert torch.equal(batch[0].cpu().double(), first)            # one key: the output is its value, exactly
-    if bf16:                                                      # one wave per partition gives the same bits
+    if bf16:                                                      # a wave per partition gives the same bits
         sp = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
         assert torch.equal(sp, batch)
 
@@ -400,3 +395,58 @@ def test_sampling_and_fingerprint(gpu):
         ops.fingerprint(rows, 3, h_in, h_out)
         want = [pl.hash_floats(b, rows[i].cpu().numpy()) for i, b in enumerate(basis)]
         assert h_out.cpu().numpy().view(np.uint64).tolist() == want
+
+
+# ----------------------------------------------------------------------------- decode fusions
+
+def test_fused_norm_products_equal_the_separate_kernels(gpu):
+    """RMSNorm fused into the product (and rotation plus cache write into the q|k|v product)
+    must give the bits of the kernels run one after the other."""
+    g = torch.Generator().manual_seed(14)
+    for M, K, N in [(1, 64, 48), (5, 96, 500), (8, 2048, 6144), (16, 224, 112), (13, 1024, 72)]:
+        x = (torch.randn(M, K, generator=g) * 2).to(gpu)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().to(gpu)
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
+        h = torch.zeros(M, K, device=gpu, dtype=torch.bfloat16)
+        ops.rmsnorm(x, nw, h, M, 1e-5)
+        sep = torch.zeros(M, N, device=gpu)
+        ops.gemm_bf16(h, w, sep, M, ops.EPI_F32)
+        fused = torch.full((M, N), 5.0, device=gpu)
+        ops.norm_gemm_bf16(x, nw, 1e-5, w, fused, M, ops.EPI_F32)
+        assert torch.equal(fused, sep), (M, K, N)
+        if N % 2 == 0:
+            sep_s = torch.zeros(M, N // 2, device=gpu, dtype=torch.bfloat16)
+            ops.gemm_bf16(h, w, sep_s, M, ops.EPI_SWIGLU_BF16)
+            fused_s = torch.zeros(M, N // 2, device=gpu, dtype=torch.bfloat16)
+            ops.norm_gemm_bf16(x, nw.float(), 1e-5, w, fused_s, M, ops.EPI_SWIGLU_BF16)
+            assert torch.equal(fused_s, sep_s), (M, K, N)
+    assert not ops.can_fuse_norm(17, w, x) and not ops.can_fuse_norm(4, torch.zeros(8, 4096, dtype=torch.bfloat16), x)
+
+    for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 96), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 160)]:
+        M, pages = 7, 12
+        cos, sin = rope_tables(10000.0, hd, 100, gpu)
+        x = (torch.randn(M, K, generator=g) * 2).to(gpu)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().to(gpu)
+        w = (torch.randn((heads + 2 * kvh) * hd, K, generator=g) * 0.05).bfloat16().to(gpu)
+        positions = torch.tensor([0, 1, 17, 63, 64, -1, 95], dtype=torch.int32, device=gpu)
+        row_seq = torch.tensor([0, 1, 0, 1, 0, 0, 1], dtype=torch.int32, device=gpu)
+        table = torch.tensor([[(i * 5 + 1) % pages for i in range(12)], [(i * 7 + 2) % pages for i in range(12)]],
+                             dtype=torch.int32, device=gpu)
+        outs = []
+        for fused in (False, True):
+            kc = torch.full((pages, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+            vc = torch.full((pages, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+            q = torch.zeros(M, heads * hd, dtype=torch.bfloat16, device=gpu)
+            if fused:
+                ops.norm_qkv_rope_bf16(x, nw, 1e-6, w, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh,
+                                       hd, page)
+            else:
+                h = torch.zeros(M, K, device=gpu, dtype=torch.bfloat16)
+                ops.rmsnorm(x, nw, h, M, 1e-6)
+                qkv = torch.zeros(M, w.shape[0], device=gpu)
+                ops.gemm_bf16(h, w, qkv, M, ops.EPI_F32)
+                ops.rope_kvwrite(qkv, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh, hd, page)
+            outs.append((q, kc, vc))
+        live = [0, 1, 2, 3, 4, 6]                                  # the row with position -1 is padding
+        assert torch.equal(outs[0][0][live], outs[1][0][live])
+        assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2])
