@@ -23,18 +23,25 @@ GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 
 class _StaticDecodeContext:
-    """Fixed device arrays for a decode batch of up to ``size`` requests, one row each."""
+    """Fixed device arrays for a decode batch of up to ``size`` requests, one row each.  All of
+    them are views of one device buffer that a step refreshes with a single copy from pinned
+    host memory."""
 
     def __init__(self, size: int, num_groups: int, max_pages: int, device: torch.device):
         self.rows = self.nseq = self.num_wanted = size
         self.device = device
         self.max_pages = max_pages
-        self.tokens = torch.full((size,), -1, dtype=torch.int32, device=device)
-        self.positions = torch.full((size,), -1, dtype=torch.int32, device=device)
+        words = 3 * size + num_groups * size * max_pages
+        self._host = torch.zeros(words, dtype=torch.int32, pin_memory=True)
+        self._host_np = self._host.numpy()
+        self._dev = torch.zeros(words, dtype=torch.int32, device=device)
+        self.tokens = self._dev[0:size]
+        self.positions = self._dev[size:2 * size]
+        self.slots = self._dev[2 * size:3 * size]
+        self.block_tables = [self._dev[3 * size + g * size * max_pages:3 * size + (g + 1) * size * max_pages].view(size, max_pages)
+                             for g in range(num_groups)]
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
-        self.slots = torch.zeros(size, dtype=torch.int32, device=device)
-        self.block_tables = [torch.zeros((size, max_pages), dtype=torch.int32, device=device) for _ in range(num_groups)]
         self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
         self.segments: List[Segment] = []
 
@@ -44,20 +51,20 @@ class _StaticDecodeContext:
     def fill(self, segments: Sequence[Segment]) -> None:
         size, n = self.rows, len(segments)
         self.segments = list(segments)
-        tok = np.full(size, -1, np.int32)
-        pos = np.full(size, -1, np.int32)
-        slot = np.zeros(size, np.int32)
+        h = self._host_np
+        h[0:size] = -1                      # padding rows: token -1, position -1
+        h[size:2 * size] = -1
+        h[2 * size:3 * size] = 0
         for i, s in enumerate(segments):
-            tok[i], pos[i], slot[i] = s.tokens[0], s.pos0, s.slot
-        self.tokens.copy_(torch.from_numpy(tok))
-        self.positions.copy_(torch.from_numpy(pos))
-        self.slots.copy_(torch.from_numpy(slot))
-        for g, dev in enumerate(self.block_tables):
-            t = np.zeros((size, self.max_pages), np.int32)
+            h[i], h[size + i], h[2 * size + i] = s.tokens[0], s.pos0, s.slot
+        base = 3 * size
+        for g in range(len(self.block_tables)):
+            t = h[base + g * size * self.max_pages:base + (g + 1) * size * self.max_pages].reshape(size, self.max_pages)
             for i, s in enumerate(segments):
-                row = np.asarray(s.tables[g], np.int32)
-                t[i, :len(row)] = np.maximum(row, 0)
-            dev.copy_(torch.from_numpy(t))
+                row = s.tables[g]
+                t[i, :len(row)] = row
+            np.maximum(t[:n], 0, out=t[:n])  # pages given back (-1) are never read
+        self._dev.copy_(self._host, non_blocking=True)
 
 
 class ModelRunner:
