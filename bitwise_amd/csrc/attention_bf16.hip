@@ -29,6 +29,8 @@
 #include "api.h"
 
 #define ATT_PART 64
+#define FOLD_QT(HD) 1
+#define FOLD_NW(HD) ((HD) <= 192 ? 8 : 4)  // waves per workgroup of the fold kernel
 
 struct AttnBf16Args {
   const bf16_t* q;            // [rows, q_stride]
@@ -38,8 +40,8 @@ struct AttnBf16Args {
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   bf16_t* out;                // [rows, out_stride]
-  int heads, kv_heads, page_size, table_stride, q_stride, out_stride, window, hpt, nsub, num_tiles;
-  float scale;
+  int heads, kv_heads, page_size, page_shift, num_pages, table_stride, q_stride, out_stride, window, hpt, nsub, num_tiles;
+  float scale_log2;           // softmax scale times log2(e)
 };
 
 // What the lanes of a wave share for one group of tiles: sequence, kv head, key range.
@@ -52,6 +54,7 @@ template <int HD>
 struct TileCtx {
   static constexpr int KS = (HD + 31) / 32;   // 32-deep k steps of the score product
   int row_c, head_c, pos_c, lo_c;             // this lane's column (query): row, head, position, first visible key
+  int all_hi, all_lo;                         // keys all_lo..all_hi are visible to every column (all_hi < all_lo: to none)
   u32x4 qf[KS];
 };
 
@@ -86,6 +89,15 @@ __device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_til
     tc[t].lo_c = (a.window > 0 && tc[t].pos_c - a.window + 1 > 0) ? tc[t].pos_c - a.window + 1 : 0;
     kmax = max(kmax, tc[t].pos_c);
     if (tc[t].pos_c >= 0) kmin = min(kmin, tc[t].lo_c);
+    // columns without a query do not count: what they compute is finite and never stored
+    int hi = tc[t].pos_c >= 0 ? tc[t].pos_c : 0x7fffffff, lo = tc[t].pos_c >= 0 ? tc[t].lo_c : -1;
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) {
+      hi = min(hi, __shfl_xor(hi, off, BW_WAVE));
+      lo = max(lo, __shfl_xor(lo, off, BW_WAVE));
+    }
+    tc[t].all_hi = hi;
+    tc[t].all_lo = lo;
   }
 #pragma unroll
   for (int off = 8; off >= 1; off >>= 1) {
@@ -109,66 +121,107 @@ __device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_til
   return true;
 }
 
+// ---- operands from the pages straight into registers (the decode kernel)
+//
+// Every load is unconditional and its address is always inside the cache (table index clamped
+// into the row, page clamped into the pool), so that no load waits for a branch and the table
+// lookups of a partition can be issued a partition ahead of the loads that need them.  Keys
+// need no masking: a key no query sees gets probability 0 whatever its score.  Values do: 0
+// times stale data (never written, or given back) could be NaN, so in a partition that is not
+// wholly live the stale keys' values are zeroed before the product.
+struct PartPages {
+  int k[4], v[4];
+};
+
+__device__ __forceinline__ void load_pages(const AttnBf16Args& a, const GroupCtx& gc, int part, PartPages& pg) {
+  const int key0 = part * ATT_PART;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int pk = (key0 + 16 * u + gc.r) >> a.page_shift, pv = (key0 + 16 * u + 4 * gc.g) >> a.page_shift;
+    pg.k[u] = gc.table[pk < a.table_stride ? pk : a.table_stride - 1];
+    pg.v[u] = gc.table[pv < a.table_stride ? pv : a.table_stride - 1];
+  }
+}
+
+__device__ __forceinline__ size_t clamp_page(const AttnBf16Args& a, int page) {
+  return (size_t)min((unsigned)page, (unsigned)(a.num_pages - 1));
+}
+
 template <int HD>
 struct KFrags {
   u32x4 k[4][(HD + 31) / 32];
 };
 // Keys of one partition as A operands: lane (r, g) feeds key 16u + r, elements 32ks + 8g .. +7.
 template <int HD>
-__device__ __forceinline__ void load_keys(const AttnBf16Args& a, const GroupCtx& gc, int part, KFrags<HD>& kf) {
+__device__ __forceinline__ void load_keys(const AttnBf16Args& a, const GroupCtx& gc, int part, const PartPages& pg,
+                                          KFrags<HD>& kf) {
   constexpr int KS = (HD + 31) / 32;
-  const int key0 = part * ATT_PART;
   const size_t kpage = (size_t)a.kv_heads * a.page_size * HD;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    const int key_r = key0 + 16 * u + gc.r;
-    const bool k_ok = key_r <= gc.kmax && key_r >= gc.kmin;
-    // the table entry is read whether or not the key is live (index clamped into the row), so
-    // that this load does not have to wait for the positions
-    const int pidx = key_r / a.page_size;
-    const int page = gc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
-    const bf16_t* kp = a.k_cache + (size_t)page * kpage + ((size_t)gc.kvh * a.page_size + key_r % a.page_size) * HD;
+    const int slot = (16 * u + gc.r) & (a.page_size - 1);
+    const bf16_t* kp = a.k_cache + clamp_page(a, pg.k[u]) * kpage + ((size_t)gc.kvh * a.page_size + slot) * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = 32 * ks + 8 * gc.g;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (k_ok && d0 < HD) v = *reinterpret_cast<const u32x4*>(kp + d0);
-      kf.k[u][ks] = v;
+      if constexpr (HD % 32 != 0) {                 // the last step is half empty: zero against a zero query
+        const u32x4 v = *reinterpret_cast<const u32x4*>(kp + (d0 < HD ? d0 : 0));
+        kf.k[u][ks] = d0 < HD ? v : (u32x4){0u, 0u, 0u, 0u};
+      } else {
+        kf.k[u][ks] = *reinterpret_cast<const u32x4*>(kp + d0);
+      }
     }
   }
 }
 
 // Values of one partition as A operands of O^T = V^T P^T: lane (r, g) feeds d = 16dt + r and, for
 // the 32-key step w, keys 32w + 4g .. +3 and 32w + 16 + 4g .. +3 (the order in which the
-// probabilities sit in the score accumulators).  Keys no query of the group may see hold stale
-// data (never written, or given back): they are zeroed, so that 0 * garbage cannot make a NaN.
+// probabilities sit in the score accumulators).
 template <int HD, int DT0, int NDT>
-__device__ __forceinline__ void load_values_range(const AttnBf16Args& a, const GroupCtx& gc, int part,
+__device__ __forceinline__ void load_values_range(const AttnBf16Args& a, const GroupCtx& gc, const PartPages& pg,
                                                   u32x4 (&out)[NDT][2]) {
-  const int key0 = part * ATT_PART;
   const size_t vpage = (size_t)a.kv_heads * HD * a.page_size;
 #pragma unroll
   for (int w = 0; w < 2; ++w)
 #pragma unroll
     for (int hseg = 0; hseg < 2; ++hseg) {
-      const int kA = key0 + 32 * w + 16 * hseg + 4 * gc.g;   // 4 consecutive keys
-      const bool ok = kA <= gc.kmax && kA + 3 >= gc.kmin;
-      const int pidx = kA / a.page_size;
-      const int page = gc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
-      const bf16_t* vp = a.v_cache + (size_t)page * vpage + (size_t)gc.kvh * HD * a.page_size + kA % a.page_size;
-      uint32_t m0 = ok ? 0xffffffffu : 0u, m1 = m0;
-      const int over = kA + 3 - gc.kmax;                      // keys kA+4-over .. kA+3 are unwritten
-      if (over >= 1) m1 &= (over >= 2) ? 0u : 0x0000ffffu;
-      if (over >= 3) m0 &= (over >= 4) ? 0u : 0x0000ffffu;
-      const int under = gc.kmin - kA;                         // keys kA .. kA+under-1 are gone
-      if (under >= 1) m0 &= (under >= 2) ? 0u : 0xffff0000u;
-      if (under >= 3) m1 &= (under >= 4) ? 0u : 0xffff0000u;
+      const int slot = (32 * w + 16 * hseg + 4 * gc.g) & (a.page_size - 1);
+      const bf16_t* vp = a.v_cache + clamp_page(a, pg.v[2 * w + hseg]) * vpage + (size_t)gc.kvh * HD * a.page_size + slot;
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
-        u32x2 v2 = {0u, 0u};
-        if (ok) v2 = *reinterpret_cast<const u32x2*>(vp + (size_t)(16 * (DT0 + dt) + gc.r) * a.page_size);
-        out[dt][w][2 * hseg] = v2[0] & m0;
-        out[dt][w][2 * hseg + 1] = v2[1] & m1;
+        const u32x2 v2 = *reinterpret_cast<const u32x2*>(vp + (size_t)(16 * (DT0 + dt) + gc.r) * a.page_size);
+        out[dt][w][2 * hseg] = v2[0];
+        out[dt][w][2 * hseg + 1] = v2[1];
+      }
+    }
+}
+
+// Zero the values of keys outside kmin..kmax (four keys of one d in two words: m0 the first two).
+__device__ __forceinline__ void stale_masks(int kA, int kmin, int kmax, uint32_t& m0, uint32_t& m1) {
+  m0 = (kA <= kmax && kA + 3 >= kmin) ? 0xffffffffu : 0u;
+  m1 = m0;
+  const int over = kA + 3 - kmax;                        // keys kA+4-over .. kA+3 are unwritten
+  if (over >= 1) m1 &= (over >= 2) ? 0u : 0x0000ffffu;
+  if (over >= 3) m0 &= (over >= 4) ? 0u : 0x0000ffffu;
+  const int under = kmin - kA;                           // keys kA .. kA+under-1 are gone
+  if (under >= 1) m0 &= (under >= 2) ? 0u : 0xffff0000u;
+  if (under >= 3) m1 &= (under >= 4) ? 0u : 0xffff0000u;
+}
+
+template <int NDT>
+__device__ __forceinline__ void mask_values(const GroupCtx& gc, int part, u32x4 (&v)[NDT][2]) {
+  const int key0 = part * ATT_PART;
+  if (key0 >= gc.kmin && key0 + ATT_PART - 1 <= gc.kmax) return;   // wholly live
+#pragma unroll
+  for (int w = 0; w < 2; ++w)
+#pragma unroll
+    for (int hseg = 0; hseg < 2; ++hseg) {
+      uint32_t m0, m1;
+      stale_masks(key0 + 32 * w + 16 * hseg + 4 * gc.g, gc.kmin, gc.kmax, m0, m1);
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        v[dt][w][2 * hseg] &= m0;
+        v[dt][w][2 * hseg + 1] &= m1;
       }
     }
 }
@@ -182,13 +235,13 @@ struct VFrags {
 };
 
 template <int HD>
-__device__ __forceinline__ void load_values(const AttnBf16Args& a, const GroupCtx& gc, int part, VFrags<HD>& vf) {
-  if constexpr (VFrags<HD>::EARLY) load_values_range<HD, 0, HD / 16>(a, gc, part, vf.v);
+__device__ __forceinline__ void load_values(const AttnBf16Args& a, const GroupCtx& gc, const PartPages& pg, VFrags<HD>& vf) {
+  if constexpr (VFrags<HD>::EARLY) load_values_range<HD, 0, HD / 16>(a, gc, pg, vf.v);
 }
 
 template <int HD, int DT>
-__device__ __forceinline__ void pv_step(const AttnBf16Args& a, const GroupCtx& gc, int part, const VFrags<HD>& vf,
-                                        const u32x4 (&pf)[2], f32x4 (&o_p)[HD / 16]) {
+__device__ __forceinline__ void pv_step(const AttnBf16Args& a, const GroupCtx& gc, int part, const PartPages& pg,
+                                        const VFrags<HD>& vf, const u32x4 (&pf)[2], f32x4 (&o_p)[HD / 16]) {
   if constexpr (DT < HD / 16) {
     o_p[DT] = (f32x4){0.f, 0.f, 0.f, 0.f};
     if constexpr (VFrags<HD>::EARLY) {
@@ -197,23 +250,107 @@ __device__ __forceinline__ void pv_step(const AttnBf16Args& a, const GroupCtx& g
         o_p[DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf.v[DT][w]), as_bf16x8(pf[w]), o_p[DT], 0, 0, 0);
     } else {
       u32x4 v[1][2];
-      load_values_range<HD, DT, 1>(a, gc, part, v);
+      load_values_range<HD, DT, 1>(a, gc, pg, v);
+      mask_values<1>(gc, part, v);
 #pragma unroll
       for (int w = 0; w < 2; ++w)
         o_p[DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v[0][w]), as_bf16x8(pf[w]), o_p[DT], 0, 0, 0);
     }
-    pv_step<HD, DT + 1>(a, gc, part, vf, pf, o_p);
+    pv_step<HD, DT + 1>(a, gc, part, pg, vf, pf, o_p);
   }
 }
 
-// One partition's partial for one tile: per column m_p, l_p (replicated over the 4 lane
-// groups) and O_p[dt][i] = element d = 16dt + 4g + i of the column.
+// Maximum without the canonicalising move that fmaxf costs; the operands are never NaN.
+__device__ __forceinline__ float max2_raw(float x, float y) {
+  float d;
+  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y));
+  return d;
+}
+__device__ __forceinline__ float max3_raw(float x, float y, float z) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(y), "v"(z));
+  return d;
+}
+
+// Maximum over the lanes l, l^16, l^32, l^48 (the four lane groups that share a column) with the
+// register-to-register lane swaps of gfx950; no trip through LDS.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  typedef __attribute__((ext_vector_type(2))) unsigned u2;
+  const u2 h = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = max2_raw(__uint_as_float(h[0]), __uint_as_float(h[1]));
+  const u2 q = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return max2_raw(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
+// Scores of one tile against one partition -> probabilities as the B operand of the second
+// product, and the column's maximum.  ``st`` holds the raw dot products.  Everything is in the
+// base-2 domain: c = scale * log2(e), m_p = max_j(dot_j) * c, p_j = bf16(exp2(fma(dot_j, c, -m_p))).
+template <int HD>
+__device__ __forceinline__ void softmax_partition(const AttnBf16Args& a, const GroupCtx& gc, const TileCtx<HD>& t,
+                                                  int key0, const f32x4 (&st)[4], float& m_p, u32x4 (&pf)[2]) {
+  float mx = -INFINITY;
+  if (key0 >= t.all_lo && key0 + ATT_PART - 1 <= t.all_hi) {
+    // every key of the partition is visible to every column: the same statements without the masks
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      mx = max3_raw(mx, st[u][0], st[u][1]);
+      mx = max3_raw(mx, st[u][2], st[u][3]);
+    }
+    mx = max_over_lane_groups(mx);
+    mx = mx * a.scale_log2;
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const int u = 2 * w + (e >> 2), i = e & 3;
+        pf[w][e >> 1] = pack_bf16x2(__builtin_amdgcn_exp2f(fmaf(st[u][i], a.scale_log2, -mx)),
+                                    __builtin_amdgcn_exp2f(fmaf(st[u][i + 1], a.scale_log2, -mx)));
+      }
+  } else {
+    bool vis[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 16 * u + 4 * gc.g + i;
+        vis[u][i] = key <= t.pos_c && key >= t.lo_c;
+      }
+      mx = max3_raw(mx, vis[u][0] ? st[u][0] : -INFINITY, vis[u][1] ? st[u][1] : -INFINITY);
+      mx = max3_raw(mx, vis[u][2] ? st[u][2] : -INFINITY, vis[u][3] ? st[u][3] : -INFINITY);
+    }
+    mx = max_over_lane_groups(mx);
+    mx = mx * a.scale_log2;
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const int u = 2 * w + (e >> 2), i = e & 3;
+        const float p0 = vis[u][i] ? __builtin_amdgcn_exp2f(fmaf(st[u][i], a.scale_log2, -mx)) : 0.0f;
+        const float p1 = vis[u][i + 1] ? __builtin_amdgcn_exp2f(fmaf(st[u][i + 1], a.scale_log2, -mx)) : 0.0f;
+        pf[w][e >> 1] = pack_bf16x2(p0, p1);
+      }
+  }
+  m_p = mx;
+}
+
+// l_p = sum of the rounded probabilities of each column, on the matrix core against rows of ones
+// (every accumulator row holds the column's sum, so no lane exchange is needed).
+__device__ __forceinline__ float probability_sum(const u32x4 (&pf)[2]) {
+  const u32x4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(pf[0]), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(pf[1]), acc, 0, 0, 0);
+  return acc[0];
+}
+
+// One partition's partial for one tile from operands in registers: per column m_p, l_p
+// (replicated over the 4 lane groups) and O_p[dt][i] = element d = 16dt + 4g + i of the column.
+// ``pg`` holds the partition's pages (head sizes over 128 load their values here).
 template <int HD>
 __device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const GroupCtx& gc, const TileCtx<HD>& t,
-                                                  int part, const KFrags<HD>& kf, const VFrags<HD>& vf, float& m_p,
-                                                  float& l_p, f32x4 (&o_p)[HD / 16]) {
+                                                  int part, const PartPages& pg, const KFrags<HD>& kf, VFrags<HD>& vf,
+                                                  float& m_p, float& l_p, f32x4 (&o_p)[HD / 16]) {
   constexpr int KS = (HD + 31) / 32;
-  const int key0 = part * ATT_PART;
   f32x4 st[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
@@ -222,62 +359,28 @@ __device__ __forceinline__ void partition_partial(const AttnBf16Args& a, const G
     for (int ks = 0; ks < KS; ++ks)
       st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf.k[u][ks]), as_bf16x8(t.qf[ks]), st[u], 0, 0, 0);
   }
-  // scale, mask, column maximum
-  float mx = -INFINITY;
-  bool vis[4][4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = key0 + 16 * u + 4 * gc.g + i;
-      vis[u][i] = key <= t.pos_c && key >= t.lo_c;
-      const float s = st[u][i] * a.scale;
-      st[u][i] = s;
-      if (vis[u][i]) mx = fmaxf(mx, s);
-    }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, BW_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, BW_WAVE));
-  m_p = mx;
-  // probabilities, rounded to bfloat16 once; their sum in fixed order
-  float lsum = 0.0f;
   u32x4 pf[2];
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    float p[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int u = 2 * w + (e >> 2), i = e & 3;
-      const float pe = vis[u][i] ? fast_exp(st[u][i] - mx) : 0.0f;
-      const bf16_t pb = f32_to_bf16(pe);
-      p[e] = bf16_to_f32(pb);
-      lsum += p[e];
-    }
-    pf[w] = (u32x4){pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
-  }
-  lsum += __shfl_xor(lsum, 16, BW_WAVE);
-  lsum += __shfl_xor(lsum, 32, BW_WAVE);
-  l_p = lsum;
+  softmax_partition<HD>(a, gc, t, part * ATT_PART, st, m_p, pf);
+  l_p = probability_sum(pf);
   // O_p^T = V^T P^T, keys ascending in steps of 32
-  pv_step<HD, 0>(a, gc, part, vf, pf, o_p);
+  if constexpr (VFrags<HD>::EARLY) mask_values<HD / 16>(gc, part, vf.v);
+  pv_step<HD, 0>(a, gc, part, pg, vf, pf, o_p);
 }
 
-// The fold step, element by element; the combine kernel runs the same statements.
+// The fold step, without branches.  A state that has seen nothing is m = -inf, l = 0, O = 0, and a
+// partial of a partition the query sees nothing of is m_p = -inf, l_p = 0, O_p = 0: with the
+// factors below the first leaves the partial as it is (0 * 0 + x) and the second leaves the
+// state as it is (x * 1 + 0 * 0).  Only when both are -inf the difference would be NaN, so the
+// reference point is moved to 0 then.  The decode kernel's fold from LDS runs the same statements.
 __device__ __forceinline__ void fold_scalars(float m, float m_p, float& mn, float& fa, float& fb) {
-  mn = fmaxf(m, m_p);
-  fa = fast_exp(m - mn);
-  fb = fast_exp(m_p - mn);
+  mn = max2_raw(m, m_p);
+  const float ref = mn == -INFINITY ? 0.0f : mn;
+  fa = __builtin_amdgcn_exp2f(m - ref);
+  fb = __builtin_amdgcn_exp2f(m_p - ref);
 }
 
 template <int NT>
 __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m_p, float l_p, const f32x4 (&o_p)[NT]) {
-  if (m_p == -INFINITY) return;       // the query sees no key of this partition
-  if (m == -INFINITY) {               // first partition it sees
-    m = m_p;
-    l = l_p;
-#pragma unroll
-    for (int dt = 0; dt < NT; ++dt) o[dt] = o_p[dt];
-    return;
-  }
   float mn, fa, fb;
   fold_scalars(m, m_p, mn, fa, fb);
   l = fmaf(l, fa, l_p * fb);
@@ -288,13 +391,164 @@ __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m
   m = mn;
 }
 
-// Route 1: one wave folds all partitions of its group of QT tiles.
-template <int HD, int QT>
-__global__ __launch_bounds__(64) void attention_fold_kernel(AttnBf16Args a) {
-  constexpr int NT = HD / 16;
+// Route 1, for prompt portions.  A workgroup of 4 waves owns FoldShape::GROUP consecutive tiles
+// of one sequence and one kv head (the host pads every sequence's tile list to a multiple of
+// that), wave w the tiles w*QT .. w*QT+QT-1.  The workgroup walks the partitions any of its
+// queries may see; the threads together copy a partition's keys and values from the pages into
+// LDS (the next partition's loads fly while this one is worked on), and every wave whose queries
+// see the partition takes its operands from there and folds it into its own state.  Workgroups
+// are handed out from the last tiles to the first: in a prompt the last queries see the most
+// keys, and the long workgroups should start first.
+template <int HD>
+struct FoldShape {
+  static constexpr int NW = FOLD_NW(HD);
+  static constexpr int QT = FOLD_QT(HD);
+  static constexpr int GROUP = NW * QT;
+  static constexpr int NBUF = HD <= 128 ? 2 : 1;
+  static constexpr int WAVES = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);   // waves per SIMD the register budget is set for
+  static constexpr int KSTR = HD * 2 + 16;          // bytes from key to key in LDS (16 of padding against bank conflicts)
+  static constexpr int VSTR = ATT_PART * 2 + 16;    // bytes from d to d
+  static constexpr int KBYTES = ATT_PART * KSTR;
+  static constexpr int BYTES = KBYTES + HD * VSTR;  // one partition
+  static constexpr int KJ = (ATT_PART * (HD / 8) + 64 * NW - 1) / (64 * NW);   // 16-byte key chunks per thread
+  static constexpr int VJ = (HD * (ATT_PART / 4) + 64 * NW - 1) / (64 * NW);   // 8-byte value chunks per thread
+};
+
+template <int HD>
+struct Staged {
+  u32x4 k[FoldShape<HD>::KJ];
+  u32x2 v[FoldShape<HD>::VJ];
+};
+
+// What the workgroup shares: sequence, kv head, the range of keys any of its queries sees.
+struct WorkgroupCtx {
+  const int32_t* table;
+  int kvh, kmin, kmax;
+};
+
+// What a thread's chunks of a partition look like does not change from partition to partition
+// (a partition starts at a multiple of the page size): which of the partition's pages, and
+// where in the page.
+template <int HD>
+struct StagePlan {
+  int k_key[FoldShape<HD>::KJ], k_off[FoldShape<HD>::KJ];   // key within the partition (64: no chunk); offset in the page
+  int v_key[FoldShape<HD>::VJ], v_off[FoldShape<HD>::VJ], v_d[FoldShape<HD>::VJ];
+};
+
+template <int HD>
+__device__ __forceinline__ void stage_plan(const AttnBf16Args& a, int kvh, StagePlan<HD>& sp) {
+  using S = FoldShape<HD>;
+  constexpr int SEG = HD / 8, THREADS = 64 * S::NW;
+#pragma unroll
+  for (int j = 0; j < S::KJ; ++j) {
+    const int c = (int)threadIdx.x + THREADS * j;
+    const int key = c / SEG, seg = c % SEG;
+    sp.k_key[j] = c < ATT_PART * SEG ? key : ATT_PART;
+    sp.k_off[j] = (kvh * a.page_size + (key & (a.page_size - 1))) * HD + seg * 8;   // inside the page for any c
+  }
+  // values: a chunk is 4 consecutive keys of one d; consecutive threads take consecutive chunks of a page
+  const int cshift = a.page_shift - 2;
+#pragma unroll
+  for (int j = 0; j < S::VJ; ++j) {
+    const int c = (int)threadIdx.x + THREADS * j;
+    const int within = c & ((1 << cshift) - 1), rowi = c >> cshift;
+    const int d = rowi % HD, key = ((rowi / HD) << a.page_shift) + 4 * within;
+    sp.v_key[j] = key < ATT_PART ? key : ATT_PART;
+    sp.v_off[j] = (kvh * HD + d) * a.page_size + (key & (a.page_size - 1));
+    sp.v_d[j] = d;
+  }
+}
+
+template <int HD>
+struct StagePages {
+  int k[FoldShape<HD>::KJ], v[FoldShape<HD>::VJ];
+};
+
+// The pages of a partition's chunks; the index is clamped into the table's row, so this may be
+// asked for a partition past the last one.
+template <int HD>
+__device__ __forceinline__ void stage_pages(const AttnBf16Args& a, const WorkgroupCtx& wc, const StagePlan<HD>& sp,
+                                            int part, StagePages<HD>& pg) {
+  using S = FoldShape<HD>;
+  const int page0 = (part * ATT_PART) >> a.page_shift;
+#pragma unroll
+  for (int j = 0; j < S::KJ; ++j) {
+    const int pidx = page0 + (sp.k_key[j] >> a.page_shift);
+    pg.k[j] = wc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
+  }
+#pragma unroll
+  for (int j = 0; j < S::VJ; ++j) {
+    const int pidx = page0 + (sp.v_key[j] >> a.page_shift);
+    pg.v[j] = wc.table[pidx < a.table_stride ? pidx : a.table_stride - 1];
+  }
+}
+
+// Unconditional loads from addresses that are always inside the cache; see the operand loaders above.
+template <int HD>
+__device__ __forceinline__ void stage_load(const AttnBf16Args& a, const StagePlan<HD>& sp, const StagePages<HD>& pg,
+                                           Staged<HD>& sg) {
+  using S = FoldShape<HD>;
+  const size_t kpage = (size_t)a.kv_heads * a.page_size * HD;   // values: the same number of elements
+#pragma unroll
+  for (int j = 0; j < S::KJ; ++j)
+    sg.k[j] = *reinterpret_cast<const u32x4*>(a.k_cache + clamp_page(a, pg.k[j]) * kpage + sp.k_off[j]);
+#pragma unroll
+  for (int j = 0; j < S::VJ; ++j)
+    sg.v[j] = *reinterpret_cast<const u32x2*>(a.v_cache + clamp_page(a, pg.v[j]) * kpage + sp.v_off[j]);
+}
+
+// Staged partition -> LDS; in a partition that is not wholly live the stale keys' values are zeroed.
+template <int HD>
+__device__ __forceinline__ void stage_store(const WorkgroupCtx& wc, const StagePlan<HD>& sp, int part,
+                                            const Staged<HD>& sg, unsigned char* buf) {
+  using S = FoldShape<HD>;
+  const int key0 = part * ATT_PART;
+  const bool inner = key0 >= wc.kmin && key0 + ATT_PART - 1 <= wc.kmax;
+#pragma unroll
+  for (int j = 0; j < S::KJ; ++j)
+    if (sp.k_key[j] < ATT_PART)
+      *reinterpret_cast<u32x4*>(buf + sp.k_key[j] * S::KSTR + (sp.k_off[j] % HD) * 2) = sg.k[j];
+#pragma unroll
+  for (int j = 0; j < S::VJ; ++j) {
+    u32x2 v2 = sg.v[j];
+    if (!inner) {
+      uint32_t m0, m1;
+      stale_masks(key0 + sp.v_key[j], wc.kmin, wc.kmax, m0, m1);
+      v2 = (u32x2){v2[0] & m0, v2[1] & m1};
+    }
+    if (sp.v_key[j] < ATT_PART)
+      *reinterpret_cast<u32x2*>(buf + S::KBYTES + sp.v_d[j] * S::VSTR + sp.v_key[j] * 2) = v2;
+  }
+}
+
+template <int HD>
+__global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves_per_eu(FoldShape<HD>::WAVES, FoldShape<HD>::WAVES))) void attention_fold_kernel(AttnBf16Args a) {
+  using S = FoldShape<HD>;
+  constexpr int NT = HD / 16, KS = (HD + 31) / 32, QT = S::QT, NW = S::NW;
+  extern __shared__ __align__(16) unsigned char lds[];
+  __shared__ int ranges[2 * NW];
+  const int wave = threadIdx.x >> 6;
+  const int first_tile = (int)(gridDim.x - 1 - blockIdx.x) * S::GROUP;
   GroupCtx gc;
   TileCtx<HD> tc[QT];
-  if (!group_setup<HD, QT>(a, blockIdx.x * QT, blockIdx.y, gc, tc)) return;
+  const bool live = group_setup<HD, QT>(a, first_tile + wave * QT, blockIdx.y, gc, tc);
+  if (gc.lane == 0) {
+    ranges[2 * wave] = live ? gc.kmin : 0x7fffffff;
+    ranges[2 * wave + 1] = live ? gc.kmax : -1;
+  }
+  __syncthreads();
+  WorkgroupCtx wc;
+  wc.kmin = 0x7fffffff;
+  wc.kmax = -1;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    wc.kmin = min(wc.kmin, ranges[2 * w]);
+    wc.kmax = max(wc.kmax, ranges[2 * w + 1]);
+  }
+  if (wc.kmax < 0) return;                       // the same for every thread of the workgroup
+  wc.kvh = gc.kvh;
+  wc.table = a.block_table + (size_t)(a.tiles != nullptr ? a.tiles[first_tile * 4 + 2] : first_tile) * a.table_stride;
+  const int my_first = live ? gc.kmin / ATT_PART : 1, my_last = live ? gc.kmax / ATT_PART : 0;
   float m[QT], l[QT];
   f32x4 o[QT][NT];
 #pragma unroll
@@ -304,26 +558,70 @@ __global__ __launch_bounds__(64) void attention_fold_kernel(AttnBf16Args a) {
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) o[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
-  const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
-  constexpr bool PREFETCH = HD <= 128;      // the next partition's keys are loaded while this one is worked on
-  KFrags<HD> kf, kf_next;
-  VFrags<HD> vf;
-  if constexpr (PREFETCH) load_keys<HD>(a, gc, first, kf);
+  const int first = wc.kmin / ATT_PART, last = wc.kmax / ATT_PART;
+  StagePlan<HD> sp;
+  stage_plan<HD>(a, wc.kvh, sp);
+  StagePages<HD> pg;
+  stage_pages<HD>(a, wc, sp, first, pg);
+  Staged<HD> sg;
+  stage_load<HD>(a, sp, pg, sg);
+  stage_pages<HD>(a, wc, sp, first + 1, pg);
+  int b = 0;
   for (int part = first; part <= last; ++part) {
-    if constexpr (!PREFETCH) load_keys<HD>(a, gc, part, kf);
-    load_values<HD>(a, gc, part, vf);
-    if constexpr (PREFETCH) {
-      if (part < last) load_keys<HD>(a, gc, part + 1, kf_next);
+    unsigned char* buf = lds + b * S::BYTES;
+    if constexpr (S::NBUF == 1) __syncthreads();   // everyone is done with the partition before
+    stage_store<HD>(wc, sp, part, sg, buf);
+    __syncthreads();
+    if (part < last) {
+      stage_load<HD>(a, sp, pg, sg);
+      stage_pages<HD>(a, wc, sp, part + 2, pg);
     }
+    if (part >= my_first && part <= my_last) {
+      // scores of all the wave's tiles; a key operand is read once and used for each of them
+      f32x4 st[QT][4];
 #pragma unroll
-    for (int t = 0; t < QT; ++t) {
-      float m_p, l_p;
-      f32x4 o_p[NT];
-      partition_partial<HD>(a, gc, tc[t], part, kf, vf, m_p, l_p, o_p);
-      fold<NT>(m[t], l[t], o[t], m_p, l_p, o_p);
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int t = 0; t < QT; ++t) st[t][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = 32 * ks + 8 * gc.g;
+          u32x4 kfrag = {0u, 0u, 0u, 0u};
+          if (d0 < HD) kfrag = *reinterpret_cast<const u32x4*>(buf + (16 * u + gc.r) * S::KSTR + d0 * 2);
+#pragma unroll
+          for (int t = 0; t < QT; ++t)
+            st[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kfrag), as_bf16x8(tc[t].qf[ks]), st[t][u], 0, 0, 0);
+        }
+      }
+      float m_p[QT], l_p[QT];
+      u32x4 pf[QT][2];
+#pragma unroll
+      for (int t = 0; t < QT; ++t) {
+        softmax_partition<HD>(a, gc, tc[t], part * ATT_PART, st[t], m_p[t], pf[t]);
+        l_p[t] = probability_sum(pf[t]);
+      }
+      f32x4 o_p[QT][NT];
+      const unsigned char* vb = buf + S::KBYTES;
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt) {
+#pragma unroll
+        for (int t = 0; t < QT; ++t) o_p[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const unsigned char* vrow = vb + (16 * dt + gc.r) * S::VSTR + (32 * w + 4 * gc.g) * 2;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow), hi = *reinterpret_cast<const u32x2*>(vrow + 32);
+          const u32x4 vfrag = {lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+          for (int t = 0; t < QT; ++t)
+            o_p[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vfrag), as_bf16x8(pf[t][w]), o_p[t][dt], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < QT; ++t) fold<NT>(m[t], l[t], o[t], m_p[t], l_p[t], o_p[t]);
     }
-    if constexpr (PREFETCH) kf = kf_next;
+    if constexpr (S::NBUF == 2) b ^= 1;
   }
+  if (!live) return;
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     if (tc[t].pos_c < 0) continue;
@@ -367,20 +665,31 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
   for (int pass0 = first; pass0 <= last; pass0 += pcap) {
     const int pass_last = (last - pass0) < pcap ? last : pass0 + pcap - 1;
     KFrags<HD> kf, kf_next;
-    VFrags<HD> vf;
+    VFrags<HD> vf, vf_next;
+    PartPages pg, pg_now;
     int part = pass0 + wave;
+    load_pages(a, gc, part, pg);
     if constexpr (PREFETCH) {
-      if (part <= pass_last) load_keys<HD>(a, gc, part, kf);
+      load_keys<HD>(a, gc, part, pg, kf);
+      load_values<HD>(a, gc, pg, vf);
+      load_pages(a, gc, part + W, pg);
     }
     for (; part <= pass_last; part += W) {
-      if constexpr (!PREFETCH) load_keys<HD>(a, gc, part, kf);
-      load_values<HD>(a, gc, part, vf);
       if constexpr (PREFETCH) {
-        if (part + W <= pass_last) load_keys<HD>(a, gc, part + W, kf_next);
+        if (part + W <= pass_last) {
+          load_keys<HD>(a, gc, part + W, pg, kf_next);
+          load_values<HD>(a, gc, pg, vf_next);
+          load_pages(a, gc, part + 2 * W, pg);
+        }
+      } else {
+        pg_now = pg;
+        load_keys<HD>(a, gc, part, pg_now, kf);
+        load_values<HD>(a, gc, pg_now, vf);
+        load_pages(a, gc, part + W, pg);
       }
       float m_p, l_p;
       f32x4 o_p[NT];
-      partition_partial<HD>(a, gc, tc[0], part, kf, vf, m_p, l_p, o_p);
+      partition_partial<HD>(a, gc, tc[0], part, PREFETCH ? pg : pg_now, kf, vf, m_p, l_p, o_p);
       if (gc.r < a.hpt) {
         float* cell = parts + ((size_t)(part - pass0) * a.hpt + gc.r) * CELL;
         if (gc.g == 0) {
@@ -392,7 +701,10 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
 #pragma unroll
           for (int i = 0; i < 4; ++i) cell[2 + 16 * dt + 4 * gc.g + i] = o_p[dt][i];
       }
-      if constexpr (PREFETCH) kf = kf_next;
+      if constexpr (PREFETCH) {
+        kf = kf_next;
+        vf = vf_next;
+      }
     }
     __syncthreads();
     const int count = pass_last - pass0 + 1;
@@ -404,13 +716,6 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
       for (int wv = 0; wv < count; ++wv) {
         const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
         const float m_p = cell[0], l_p = cell[1], o_p = cell[2 + d];
-        if (m_p == -INFINITY) continue;
-        if (m[j] == -INFINITY) {
-          m[j] = m_p;
-          l[j] = l_p;
-          o[j] = o_p;
-          continue;
-        }
         float mn, fa, fb;
         fold_scalars(m[j], m_p, mn, fa, fb);
         l[j] = fmaf(l[j], fa, l_p * fb);
@@ -444,16 +749,26 @@ static void launch_attention(const AttnBf16Args& a, int decode, hipStream_t s) {
     pcap = pcap < W ? W : (pcap > 256 ? 256 : pcap);
     hipLaunchKernelGGL((attention_decode_kernel<HD, W>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a, pcap);
   } else {
-    constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
-    hipLaunchKernelGGL((attention_fold_kernel<HD, QT>), dim3((a.num_tiles + QT - 1) / QT, items), dim3(64), 0, s, a);
+    using S = FoldShape<HD>;
+    constexpr int lds_bytes = S::NBUF * S::BYTES;
+    static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
+    if (!allowed && lds_bytes > 48 * 1024) {
+      (void)hipFuncSetAttribute((const void*)attention_fold_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      allowed = true;
+    }
+    hipLaunchKernelGGL((attention_fold_kernel<HD>), dim3((a.num_tiles + S::GROUP - 1) / S::GROUP, items), dim3(64 * S::NW),
+                       lds_bytes, s, a);
   }
 }
 
+extern "C" int bw_attention_fold_group_tiles(int head_dim) { return FOLD_NW(head_dim) * FOLD_QT(head_dim); }
+
 extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                                  int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
-                                 const void* v_cache, void* out, int out_stride, int heads, int kv_heads,
-                                 int head_dim, int page_size, int window, float scale, int decode, void* stream) {
+                                 const void* v_cache, int num_pages, void* out, int out_stride, int heads,
+                                 int kv_heads, int head_dim, int page_size, int window, float scale, int decode, void* stream) {
   if (num_tiles <= 0) return 0;
+  if (num_pages <= 0) return -2;
   if (kv_heads <= 0 || heads % kv_heads) return -2;
   if (page_size < 4 || (page_size & (page_size - 1)) || page_size > ATT_PART) return -5;  // 4-key loads stay inside a page
   if ((q_stride % 8) || (out_stride % 4)) return -3;
@@ -462,11 +777,14 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   a.q = (const bf16_t*)q; a.positions = positions; a.block_table = block_table; a.tiles = tiles;
   a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache; a.out = (bf16_t*)out;
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size; a.table_stride = table_stride;
+  a.page_shift = __builtin_ctz((unsigned)page_size);
+  a.num_pages = num_pages;
   a.q_stride = q_stride; a.out_stride = out_stride; a.window = window;
   a.hpt = group < 16 ? group : 16;
   a.nsub = (group + a.hpt - 1) / a.hpt;
   a.num_tiles = num_tiles;
-  a.scale = scale;
+  if (!(scale > 0.0f)) return -2;                // the maximum is taken before the scaling
+  a.scale_log2 = scale * 1.44269504088896340736f;
   if (kv_heads * a.nsub > 65535) return -2;
   hipStream_t s = (hipStream_t)stream;
 #define BW_CASE(HD) case HD: launch_attention<HD>(a, decode, s); break;

@@ -16,17 +16,17 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// Round to nearest even; NaN stays NaN.
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t b = __float_as_uint(f);
-  if ((b & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((b >> 16) | 0x40);
-  b += 0x7fffu + ((b >> 16) & 1u);
-  return (bf16_t)(b >> 16);
-}
+// Round to nearest even with the hardware conversion (v_cvt_pk_bf16_f32); NaN stays NaN.
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  const bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, r);
 }
+
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return (bf16_t)(pack_bf16x2(f, 0.0f) & 0xffffu); }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;

@@ -20,7 +20,7 @@ ATT_PART = 64          # keys per partition of the bfloat16 attention fold
 def fold_group_tiles(head_dim: int) -> int:
     """Tiles (of 16 query columns) one wave of the fold kernel owns; a wave's tiles must belong
     to one sequence, so the host pads every sequence's tile list to a multiple of this."""
-    return 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
+    return int(_fn("bw_attention_fold_group_tiles")(int(head_dim)))
 HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
 
 _ERRORS = {
@@ -42,8 +42,9 @@ _SIGS = {
     "bw_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
-    "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "bw_attention_fold_group_tiles": [c_int],
     "bw_decode_gemm_supported": [c_int, c_int, c_int],
     "bw_decode_gemm_bf16": [c_void_p, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_void_p],
@@ -347,7 +348,10 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
     [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).
 
-    ``decode`` False: one wave folds all partitions of up to ``fold_group_tiles(head_dim)`` tiles;
+    k_cache and v_cache are [pages, kv_heads*page_size*head_dim]: page numbers from the table
+    are clamped into the pool, so a stale table entry can cost nothing worse than a wasted load.
+
+    ``decode`` False: a workgroup folds all partitions for ``fold_group_tiles(head_dim)`` tiles;
     the tiles of a sequence must come in runs padded to that number (empty tiles allowed).
     ``decode`` True (tiles of one token each; ``tiles`` None means "tile t is row t of sequence
     t"): a workgroup per tile whose waves take one 64-key partition each and fold through LDS
@@ -371,10 +375,13 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
         raise ValueError("attention_bf16: q, out or tiles do not fit")
     if tiles is None and (positions.numel() < num_tiles or block_table.shape[0] < num_tiles):
         raise ValueError("attention_bf16: fewer rows or block tables than implicit tiles")
+    page_elems = kv_heads * page_size * head_dim
+    if k_cache.dim() != 2 or k_cache.shape[1] != page_elems or v_cache.shape != k_cache.shape:
+        raise ValueError(f"attention_bf16: caches must be [pages, {page_elems}]")
     _check(_fn("bw_attention_bf16")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
                                     block_table.stride(0), tiles.data_ptr() if tiles is not None else 0, num_tiles,
-                                    k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
-                                    kv_heads, head_dim, page_size, int(window), float(scale), int(decode), _stream()),
+                                    k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], out.data_ptr(),
+                                    out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode), _stream()),
            "attention_bf16")
 
 
