@@ -96,18 +96,18 @@ __device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_til
       hi = min(hi, __shfl_xor(hi, off, BW_WAVE));
       lo = max(lo, __shfl_xor(lo, off, BW_WAVE));
     }
-    tc[t].all_hi = hi;
-    tc[t].all_lo = lo;
+    tc[t].all_hi = __builtin_amdgcn_readfirstlane(hi);   // the same in every lane: say so, branches on them are scalar then
+    tc[t].all_lo = __builtin_amdgcn_readfirstlane(lo);
   }
 #pragma unroll
   for (int off = 8; off >= 1; off >>= 1) {
     kmax = max(kmax, __shfl_xor(kmax, off, BW_WAVE));
     kmin = min(kmin, __shfl_xor(kmin, off, BW_WAVE));
   }
-  gc.kmax = kmax;
-  gc.kmin = kmin;
+  gc.kmax = __builtin_amdgcn_readfirstlane(kmax);
+  gc.kmin = __builtin_amdgcn_readfirstlane(kmin);
   gc.table = a.block_table + (size_t)seq * a.table_stride;
-  if (kmax < 0) return false;
+  if (gc.kmax < 0) return false;
 #pragma unroll
   for (int t = 0; t < QT; ++t)
 #pragma unroll
@@ -260,17 +260,12 @@ __device__ __forceinline__ void pv_step(const AttnBf16Args& a, const GroupCtx& g
   }
 }
 
-// Maximum without the canonicalising move that fmaxf costs; the operands are never NaN.
-__device__ __forceinline__ float max2_raw(float x, float y) {
-  float d;
-  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y));
-  return d;
-}
-__device__ __forceinline__ float max3_raw(float x, float y, float z) {
-  float d;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(y), "v"(z));
-  return d;
-}
+// Maximum without the canonicalising moves that fmaxf costs (the operands are never NaN): the
+// median of x, y and +inf.  A builtin and not inline assembly on purpose: the operands often come
+// straight out of a matrix instruction, and the compiler inserts the wait states that such a
+// read needs only for instructions it knows.
+__device__ __forceinline__ float max2_raw(float x, float y) { return __builtin_amdgcn_fmed3f(x, y, INFINITY); }
+__device__ __forceinline__ float max3_raw(float x, float y, float z) { return max2_raw(max2_raw(x, y), z); }
 
 // Maximum over the lanes l, l^16, l^32, l^48 (the four lane groups that share a column) with the
 // register-to-register lane swaps of gfx950; no trip through LDS.
@@ -527,7 +522,7 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
   constexpr int NT = HD / 16, KS = (HD + 31) / 32, QT = S::QT, NW = S::NW;
   extern __shared__ __align__(16) unsigned char lds[];
   __shared__ int ranges[2 * NW];
-  const int wave = threadIdx.x >> 6;
+  const int wave = wave_index();
   const int first_tile = (int)(gridDim.x - 1 - blockIdx.x) * S::GROUP;
   GroupCtx gc;
   TileCtx<HD> tc[QT];
@@ -545,6 +540,8 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
     wc.kmin = min(wc.kmin, ranges[2 * w]);
     wc.kmax = max(wc.kmax, ranges[2 * w + 1]);
   }
+  wc.kmin = __builtin_amdgcn_readfirstlane(wc.kmin);
+  wc.kmax = __builtin_amdgcn_readfirstlane(wc.kmax);
   if (wc.kmax < 0) return;                       // the same for every thread of the workgroup
   wc.kvh = gc.kvh;
   wc.table = a.block_table + (size_t)(a.tiles != nullptr ? a.tiles[first_tile * 4 + 2] : first_tile) * a.table_stride;
@@ -652,7 +649,7 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
   GroupCtx gc;
   TileCtx<HD> tc[1];
   if (!group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc)) return;   // uniform over the workgroup
-  const int wave = threadIdx.x >> 6;
+  const int wave = wave_index();
   const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
   const int elems = a.hpt * HD;
   float m[EPT], l[EPT], o[EPT];

@@ -14,6 +14,12 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define BW_WAVE 64
 
+// The wave's number in its workgroup as a scalar: the compiler cannot see that threadIdx.x >> 6 is
+// the same for all lanes, and everything derived from it (segments, strips, loop bounds) would
+// be computed per lane and branched on per lane.  A branch around a matrix instruction must be
+// scalar in particular: the matrix cores ignore the execution mask.
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
 // Round to nearest even with the hardware conversion (v_cvt_pk_bf16_f32); NaN stays NaN.
@@ -73,47 +79,93 @@ __device__ __forceinline__ float row_sumsq_vec(const f32x4* __restrict__ xv, int
   return wave_sum(acc);
 }
 
-// Load 4 norm weights (bfloat16 or 32-bit) starting at element 4c as floats.
-__device__ __forceinline__ f32x4 load_norm_w4(const void* __restrict__ w, int is_bf16, int c) {
+// 4 norm weights (bfloat16 or 32-bit) starting at element 4c: the load leaves the bits as they
+// come (8 or 16 bytes), the conversion to floats is a separate step, so that a caller can issue
+// all its loads before anything waits for one.
+__device__ __forceinline__ u32x4 load_norm_w_raw(const void* __restrict__ w, int is_bf16, int c) {
   if (is_bf16) {
     const u32x2 p = reinterpret_cast<const u32x2*>(w)[c];
-    return (f32x4){__uint_as_float(p[0] << 16), __uint_as_float(p[0] & 0xffff0000u), __uint_as_float(p[1] << 16),
-                   __uint_as_float(p[1] & 0xffff0000u)};
+    return (u32x4){p[0], p[1], 0u, 0u};
   }
-  return reinterpret_cast<const f32x4*>(w)[c];
+  return reinterpret_cast<const u32x4*>(w)[c];
 }
 
-// RMSNorm of one row of at most 2048 elements (a multiple of 4) by one wave, with every load
-// issued before anything is computed: the row's vectors stay in registers between the sum of
-// squares and the scaling.  Same order and statements as row_sumsq_vec and the store loop of
-// rmsnorm_bf16_kernel.  ``store(c, packed)`` receives vector c as four bfloat16 in 8 bytes.
+__device__ __forceinline__ f32x4 norm_w_floats(u32x4 raw, int is_bf16) {
+  if (is_bf16)
+    return (f32x4){__uint_as_float(raw[0] << 16), __uint_as_float(raw[0] & 0xffff0000u), __uint_as_float(raw[1] << 16),
+                   __uint_as_float(raw[1] & 0xffff0000u)};
+  return (f32x4){__uint_as_float(raw[0]), __uint_as_float(raw[1]), __uint_as_float(raw[2]), __uint_as_float(raw[3])};
+}
+
+__device__ __forceinline__ f32x4 load_norm_w4(const void* __restrict__ w, int is_bf16, int c) {
+  return norm_w_floats(load_norm_w_raw(w, is_bf16, c), is_bf16);
+}
+
+// RMSNorm of up to R rows of at most 2048 elements (a multiple of 4) by one wave, in two phases:
+// every load is issued in the first (vector indices past the row are clamped, missing rows read
+// the first row, so nothing is conditional), everything is computed in the second.  Between
+// them the caller may put other loads in flight: memory results are waited for in issue order,
+// so what is issued later does not hold the reductions up.  rows[0] must be a row; rows[j]
+// null skips row j.  The order is that of row_sumsq_vec and of the store loop of
+// rmsnorm_bf16_kernel: lane l owns vectors l, l+64, ...; ``store(j, c, packed)`` receives vector
+// c of row j as four bfloat16 in 8 bytes.
+template <int R>
+struct NormRows {
+  f32x4 v[R][8];
+  u32x4 w[8];
+};
+
+template <int R>
+__device__ __forceinline__ void norm_rows_load(NormRows<R>& nr, const f32x4* const (&rows)[R], const void* __restrict__ w,
+                                               int w_is_bf16, int nvec, int lane) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = 64 * j + lane < nvec ? 64 * j + lane : nvec - 1;
+    nr.w[j] = load_norm_w_raw(w, w_is_bf16, c);
+#pragma unroll
+    for (int i = 0; i < R; ++i) nr.v[i][j] = (rows[i] != nullptr ? rows[i] : rows[0])[c];
+  }
+}
+
+template <int R, typename Store>
+__device__ __forceinline__ void norm_rows_finish(const NormRows<R>& nr, const f32x4* const (&rows)[R], int w_is_bf16,
+                                                 int nvec, int dim, float eps, int lane, Store store) {
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (rows[i] == nullptr) continue;
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool in = 64 * j + lane < nvec;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x = in ? nr.v[i][j][e] : 0.0f;
+        acc = fmaf(x, x, acc);
+      }
+    }
+    acc = wave_sum(acc);
+    const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = 64 * j + lane;
+      if (c < nvec) {
+        const f32x4 wv = norm_w_floats(nr.w[j], w_is_bf16);
+        u32x2 pk = {pack_bf16x2((nr.v[i][j][0] * inv) * wv[0], (nr.v[i][j][1] * inv) * wv[1]),
+                    pack_bf16x2((nr.v[i][j][2] * inv) * wv[2], (nr.v[i][j][3] * inv) * wv[3])};
+        store(i, c, pk);
+      }
+    }
+  }
+}
+
+// One row at once: the whole of rmsnorm_bf16_kernel for rows that fit a wave's registers.
 template <typename Store>
 __device__ __forceinline__ void rmsnorm_row_small(const f32x4* __restrict__ xv, const void* __restrict__ w,
                                                   int w_is_bf16, int nvec, int dim, float eps, int lane, Store store) {
-  constexpr int UN = 8;
-  f32x4 v[UN], wv[UN];
-#pragma unroll
-  for (int j = 0; j < UN; ++j) {
-    const int c = 64 * j + lane;
-    v[j] = c < nvec ? xv[c] : (f32x4){0.f, 0.f, 0.f, 0.f};
-    wv[j] = c < nvec ? load_norm_w4(w, w_is_bf16, c) : (f32x4){0.f, 0.f, 0.f, 0.f};
-  }
-  float acc = 0.0f;
-#pragma unroll
-  for (int j = 0; j < UN; ++j)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc = fmaf(v[j][e], v[j][e], acc);
-  acc = wave_sum(acc);
-  const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
-#pragma unroll
-  for (int j = 0; j < UN; ++j) {
-    const int c = 64 * j + lane;
-    if (c < nvec) {
-      u32x2 pk = {pack_bf16x2((v[j][0] * inv) * wv[j][0], (v[j][1] * inv) * wv[j][1]),
-                  pack_bf16x2((v[j][2] * inv) * wv[j][2], (v[j][3] * inv) * wv[j][3])};
-      store(c, pk);
-    }
-  }
+  NormRows<1> nr;
+  const f32x4* rows[1] = {xv};
+  norm_rows_load<1>(nr, rows, w, w_is_bf16, nvec, lane);
+  norm_rows_finish<1>(nr, rows, w_is_bf16, nvec, dim, eps, lane, [&](int, int c, u32x2 pk) { store(c, pk); });
 }
 
 // The launch wrappers return hipGetLastError() as int; 0 is success.

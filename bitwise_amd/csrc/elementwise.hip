@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16_kernel(const float* __restri
                                                            bf16_t* __restrict__ y, int rows, int dim, int ldy,
                                                            float eps) {
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int row = blockIdx.x * (blockDim.x >> 6) + wave_index();
   if (row >= rows) return;
   const float* xr = x + (size_t)row * dim;
   bf16_t* yr = y + (size_t)row * ldy;

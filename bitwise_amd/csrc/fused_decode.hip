@@ -44,67 +44,120 @@ struct DecodeGemmArgs {
   bf16_t* k_cache;
   bf16_t* v_cache;
   int heads, kv_heads, head_dim, page_size, table_stride, write_cache;
+  int pairs;               // rotary: 16-wide pairs of strips a head is cut into (0: a workgroup is a whole head)
 };
 
 template <int EPI, bool NORM, int D>
 __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   constexpr int NB = (EPI == DEPI_SWIGLU_BF16) ? 2 : 1;
+  constexpr bool FULL = D * 32 >= DEC_SEG;        // the ring holds a whole segment: nothing is refilled
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int K = a.K, M = a.M, S = a.S;
   const int lds_row = K + 8;                      // bf16 elements; +16 bytes keeps operand reads conflict-free
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row]
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int strip = wave / S, seg = wave % S;     // the S waves of a strip are neighbours
-  const int n0 = (blockIdx.x * (nwaves / S) + strip) * 16;
+  // rotary: a workgroup is a head (its strips in order), or, when half a head is a multiple of
+  // 16, one strip of the first half and its partner in the second (workgroup p of the head:
+  // strips p and p + pairs), so that twice as many workgroups share the stream
+  int rope_head = 0, rope_base = 0, rope_lw = 0;
+  int n0 = (blockIdx.x * (nwaves / S) + strip) * 16;
+  if constexpr (EPI == DEPI_ROPE_KV) {
+    if (a.pairs > 0) {
+      rope_head = blockIdx.x / a.pairs;
+      rope_base = 16 * (blockIdx.x % a.pairs);
+      rope_lw = 32;
+      n0 = rope_head * a.head_dim + rope_base + wave * (a.head_dim >> 1);
+    } else {
+      rope_head = blockIdx.x;
+      rope_lw = a.head_dim;
+    }
+  }
   const bool n_ok = n0 + r < a.N;
   const int k_begin = seg * DEC_SEG;
   const int k_end = (K - k_begin) < DEC_SEG ? K : k_begin + DEC_SEG;
-  const bf16_t* wp[NB];
+  // weights through buffer descriptors that cover the strip's rows (rows past N read as zeros):
+  // one per-lane offset for the whole kernel, the step's offset in a scalar register
+  const int w_rows = min(16, a.N - n0);
+  __amdgpu_buffer_rsrc_t rs_w[NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) wp[b] = a.w + ((size_t)b * a.N + (n_ok ? n0 + r : 0)) * K + 8 * g;
+  for (int b = 0; b < NB; ++b)
+    rs_w[b] = __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + ((size_t)b * a.N + n0) * K), 0,
+                                                (int)((size_t)(w_rows > 0 ? w_rows : 0) * K * 2), 0x00020000);
+  const int voff_w = (r * K + 8 * g) * 2;
 
-  // 1. weight loads in flight first: they depend on nothing
+  // 1. Loads go out in the order in which their results are needed, because results are waited
+  // for in issue order: first the rows to normalise (their first batch) and the positions, then
+  // the weights, which stay in flight while the rows are normalised.
+  constexpr int RB = 4;                            // rows a wave normalises at a time
+  const int nvec = K >> 2;
+  NormRows<RB> nr;
+  const f32x4* nrows[RB];
+  if constexpr (NORM) {
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      const int m = wave + i * nwaves;             // rows are dealt to the waves round robin
+      nrows[i] = m < M ? reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda) : nullptr;
+    }
+    if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
+  }
+  int r_pos[2] = {-1, -1}, r_seq[2] = {0, 0};
+  if constexpr (EPI == DEPI_ROPE_KV) {
+    const int lh = rope_lw >> 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * blockDim.x;
+      if (e < M * lh) {
+        r_pos[j] = a.positions[e / lh];
+        r_seq[j] = a.row_seq[e / lh];
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
   u32x4 bq[D][NB];
   auto issue = [&](int d, int k) {
     const int ks = k < k_end ? k : k_begin;       // past the end: re-read the first step, never used
 #pragma unroll
-    for (int b = 0; b < NB; ++b) bq[d][b] = *reinterpret_cast<const u32x4*>(wp[b] + ks);
+    for (int b = 0; b < NB; ++b) bq[d][b] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[b], voff_w, ks * 2, 0);
   };
 #pragma unroll
   for (int d = 0; d < D; ++d) issue(d, k_begin + 32 * d);
   __builtin_amdgcn_sched_barrier(0);
 
-  // rotary epilogue: this thread's (row, pair) items and what they need are fetched now, so that
-  // the position -> table/angle chain runs while the weights stream (at most 2 items a thread)
-  int r_pos[2] = {-1, -1}, r_page[2] = {0, 0};
+  // rotary epilogue: what this thread's (row, pair) items need is asked for now and used after the
+  // product (at most 2 items a thread)
+  int r_page[2] = {0, 0};
   float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
   if constexpr (EPI == DEPI_ROPE_KV) {
-    const int half = a.head_dim >> 1;
+    const int half = a.head_dim >> 1, lh = rope_lw >> 1;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int e = threadIdx.x + j * blockDim.x;
-      if (e < M * half) {
-        const int m = e / half, i = e % half;
-        const int pos = a.positions[m];
-        r_pos[j] = pos;
-        if (pos >= 0) {
-          r_cos[j] = a.cos_table[(size_t)pos * half + i];
-          r_sin[j] = a.sin_table[(size_t)pos * half + i];
-          r_page[j] = a.block_table[(size_t)a.row_seq[m] * a.table_stride + pos / a.page_size];
-        }
+      const int pos = r_pos[j];
+      if (e < M * lh && pos >= 0) {
+        const int i = rope_base + e % lh;
+        r_cos[j] = a.cos_table[(size_t)pos * half + i];
+        r_sin[j] = a.sin_table[(size_t)pos * half + i];
+        r_page[j] = a.block_table[(size_t)r_seq[j] * a.table_stride + pos / a.page_size];
       }
     }
   }
 
   // 2. the M rows into LDS as bfloat16
   if constexpr (NORM) {
-    const int nvec = K >> 2;
-    for (int m = wave; m < M; m += nwaves) {     // rows dealt to the waves round robin
-      bf16_t* dst = xs + (size_t)m * lds_row;
-      rmsnorm_row_small(reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda), a.norm_w,
-                        a.norm_w_is_bf16, nvec, K, a.eps, lane,
-                        [&](int c, u32x2 pk) { *reinterpret_cast<u32x2*>(dst + 4 * c) = pk; });
+    for (int m0 = wave; m0 < M;) {
+      norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
+        *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
+      });
+      m0 += RB * nwaves;
+      if (m0 >= M) break;
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        const int m = m0 + i * nwaves;
+        nrows[i] = m < M ? reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda) : nullptr;
+      }
+      norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
     }
   } else {
     const int cpr = K >> 3;                       // 16-byte chunks per row
@@ -132,7 +185,6 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   f32x4 acc[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  const u32x4 zero = {0u, 0u, 0u, 0u};
   constexpr int PA = 4;                            // A operands are read from LDS this many steps ahead
   static_assert(D % PA == 0, "the A look-ahead must divide the ring depth");
   u32x4 aq[PA];
@@ -143,17 +195,18 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int k = k0 + 32 * d;
-      const bool live = k < k_end;
       const u32x4 af = aq[d % PA];
       u32x4 bc[NB];
 #pragma unroll
-      for (int b = 0; b < NB; ++b) bc[b] = live ? bq[d][b] : zero;
-      issue(d, k + 32 * D);
+      for (int b = 0; b < NB; ++b) bc[b] = bq[d][b];
+      if constexpr (!FULL) issue(d, k + 32 * D);
       fetch_a(d % PA, k + 32 * PA);
       __builtin_amdgcn_sched_barrier(0);
+      if (k < k_end) {                             // scalar: a step past the segment's end is skipped
 #pragma unroll
-      for (int b = 0; b < NB; ++b)
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(bc[b]), acc[b], 0, 0, 0);
+        for (int b = 0; b < NB; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(bc[b]), acc[b], 0, 0, 0);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -196,28 +249,28 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
       }
     }
   } else {
-    // The workgroup's strips are one head (S is 1 here): blockIdx.x < heads is a q head, then the
-    // k heads, then the v heads.  The 32-bit products go through LDS so that the rotary pairs
-    // (i, i + hd/2), which sit in different strips, meet.
-    const int hd = a.head_dim, half = hd >> 1;
+    // The workgroup's strips are one head or one pair of strips of it (S is 1 here); heads come
+    // in the order q heads, k heads, v heads.  The 32-bit products go through LDS so that the
+    // rotary pairs (i, i + hd/2), which sit in different strips, meet.
+    const int hd = a.head_dim, half = hd >> 1, lw = rope_lw, lh = lw >> 1;
     __syncthreads();                               // every wave is done reading the rows
-    float* os = reinterpret_cast<float*>(smem);    // [M][hd]
+    float* os = reinterpret_cast<float*>(smem);    // [M][lw]
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = 4 * g + q;
-      if (m < M) os[m * hd + 16 * wave + r] = acc[0][q];
+      if (m < M) os[m * lw + 16 * wave + r] = acc[0][q];
     }
     __syncthreads();
-    const int head = blockIdx.x;
+    const int head = rope_head;
     const int q_dim = a.heads * hd;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int e = threadIdx.x + j * blockDim.x;
-      if (e >= M * half) continue;
-      const int m = e / half, i = e % half;
+      if (e >= M * lh) continue;
+      const int m = e / lh, il = e % lh, i = rope_base + il;
       const int pos = r_pos[j];
       if (pos < 0) continue;
-      const float x1 = os[m * hd + i], x2 = os[m * hd + i + half];
+      const float x1 = os[m * lw + il], x2 = os[m * lw + il + lh];
       if (head < a.heads + a.kv_heads) {
         const float c = r_cos[j], s = r_sin[j];
         const float o1 = x1 * c - x2 * s;
@@ -315,7 +368,9 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
                                      int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                                      int write_cache, void* stream) {
   if (M <= 0) return 0;
-  if (head_dim % 16 || head_dim < 16 || head_dim > 64 || page_size <= 0) return -4;   // one wave per strip, four at most
+  if (head_dim % 16 || head_dim < 16 || page_size <= 0) return -4;
+  const int pairs = (head_dim % 32 == 0) ? head_dim / 32 : 0;
+  if (!pairs && head_dim > 64) return -4;            // a whole head per workgroup: one wave per strip, four at most
   DecodeGemmArgs a{};
   a.a = x; a.norm_w = norm_w; a.w = (const bf16_t*)w_qkv; a.out = q_out;
   a.M = M; a.N = (heads + 2 * kv_heads) * head_dim; a.K = K; a.lda = ldx; a.ldo = heads * head_dim;
@@ -325,10 +380,13 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
   a.sin_table = sin_table; a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache;
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.page_size = page_size;
   a.table_stride = table_stride; a.write_cache = write_cache;
+  a.pairs = pairs;
   if (K > DEC_SEG) return -2;
   const int bad = check_decode_gemm(a, true);
   if (bad) return bad;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
-  if ((size_t)M * head_dim * sizeof(float) > (size_t)M * (K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
-  return launch_decode_gemm<DEPI_ROPE_KV, true, 32>(a, head_dim / 16, heads + 2 * kv_heads, (hipStream_t)stream);
+  if ((size_t)(pairs ? 32 : head_dim) * sizeof(float) > (size_t)(K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
+  const int all_heads = heads + 2 * kv_heads;
+  if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, true, 64>(a, 2, all_heads * pairs, (hipStream_t)stream);
+  return launch_decode_gemm<DEPI_ROPE_KV, true, 64>(a, head_dim / 16, all_heads, (hipStream_t)stream);
 }

@@ -36,28 +36,44 @@ __device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o,
 
 // ------------------------------------------------------------------------------ skinny
 
-// TAIL: K is no multiple of 32, so the last step of the last segment is partly zero-filled,
-// lane by lane.  Without TAIL nothing in the main loop depends on the lane: rows of W past N
-// and rows of x past M are read from row 0 instead and their results thrown away, ring
-// refills past the segment's end re-read its first step and are never used, and a segment
-// whose step count is no multiple of D runs a few extra steps on zeros (adding exact zeros
-// to an accumulator does not change its bits).
-template <int WM, int EPI, int D, bool TAIL>
+// One wave per (strip of CW output columns, segment of K).  All its loads go through buffer
+// descriptors with one per-lane offset fixed for the whole kernel and the step's offset in a
+// scalar register, and every decision about a step (is it inside the segment?) is scalar too:
+// the loop spends no vector instruction on addresses or masks.  Rows of W past N and rows of x
+// past M lie outside their descriptors and read as zeros.  A ring of D operand registers keeps
+// D steps of weights in flight (D = 64 holds a whole segment: nothing is refilled); the few rows
+// of x come from cache a few steps ahead.
+//
+// CW = 8 halves the strip (lanes 8..15 repeat the columns of lanes 0..7 and their results are
+// dropped): twice as many workgroups, for products with too few columns to give every compute
+// unit a 16-column strip.  TAIL: K is no multiple of 32, so the last step of the last segment
+// is zero-filled lane by lane past K.
+template <int WM, int EPI, int D, bool TAIL, int CW>
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                void* __restrict__ out, int M, int N, int K, int ldx,
                                                                int ldo, int S) {
   constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
+  constexpr int DA = D < 32 ? D : 32;             // look-ahead of the x operands (they come from cache)
+  constexpr bool FULL = D * 32 >= GEMM_SEG;
+  static_assert(D % DA == 0, "the x look-ahead must divide the ring depth");
   extern __shared__ float red[];   // [S][NB][WM][4][64] when S > 1
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const bool n_ok = n0 + r < N;
-  const bf16_t* wp[NB];
+  const int c = r % CW;
+  const int n0 = blockIdx.x * CW;
+  const bool n_ok = r < CW && n0 + c < N;
+  const int w_rows = min(CW, N - n0);
+  __amdgpu_buffer_rsrc_t rs_w[NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) wp[b] = w + ((size_t)b * N + (n_ok ? n0 + r : 0)) * K + 8 * g;
-  const bf16_t* xp[WM];
+  for (int b = 0; b < NB; ++b)
+    rs_w[b] = __builtin_amdgcn_make_buffer_rsrc((void*)(w + ((size_t)b * N + n0) * K), 0, (int)((size_t)w_rows * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x =
+      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
+  // in a half strip the lanes 8..15 point outside the descriptor: they read zeros and ask memory for nothing
+  const int voff_w = r < CW ? (c * K + 8 * g) * 2 : 0x7ffffff0;
+  int voff_x[WM];
 #pragma unroll
-  for (int i = 0; i < WM; ++i) xp[i] = x + (size_t)(16 * i + r < M ? 16 * i + r : 0) * ldx + 8 * g;
+  for (int i = 0; i < WM; ++i) voff_x[i] = ((16 * i + r) * ldx + 8 * g) * 2;
   const u32x4 zero = {0u, 0u, 0u, 0u};
   f32x4 acc[NB][WM];
   for (int s = wave; s < S; s += nwaves) {
@@ -67,38 +83,51 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
     for (int b = 0; b < NB; ++b)
 #pragma unroll
       for (int i = 0; i < WM; ++i) acc[b][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    u32x4 bq[D][NB], aq[D][WM];
-    auto issue = [&](int d, int k) {
-      // k is the same for all lanes; past the end the slot is filled from the segment's first step
+    u32x4 bq[D][NB], aq[DA][WM];
+    // k is the same for all lanes; past the end the slot is filled from the segment's first step
+    auto issue_w = [&](int d, int k) {
       const int ks = k < k_end ? k : k_begin;
 #pragma unroll
-      for (int b = 0; b < NB; ++b) bq[d][b] = *reinterpret_cast<const u32x4*>(wp[b] + ks);
+      for (int b = 0; b < NB; ++b) bq[d][b] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[b], voff_w, ks * 2, 0);
+    };
+    auto issue_x = [&](int d, int k) {
+      const int ks = k < k_end ? k : k_begin;
 #pragma unroll
-      for (int i = 0; i < WM; ++i) aq[d][i] = *reinterpret_cast<const u32x4*>(xp[i] + ks);
+      for (int i = 0; i < WM; ++i) aq[d][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff_x[i], ks * 2, 0);
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) issue(d, k_begin + 32 * d);
+    for (int d = 0; d < DA; ++d) issue_x(d, k_begin + 32 * d);
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue_w(d, k_begin + 32 * d);
     __builtin_amdgcn_sched_barrier(0);
     for (int k0 = k_begin; k0 < k_end; k0 += 32 * D) {
 #pragma unroll
       for (int d = 0; d < D; ++d) {
         const int k = k0 + 32 * d;
         u32x4 bc[NB], ac[WM];
-        bool live = k < k_end;
-        if constexpr (TAIL) live = k + 8 * g < k_end && (k + 8 * g + 8 <= K);
 #pragma unroll
-        for (int b = 0; b < NB; ++b) bc[b] = live ? bq[d][b] : zero;
+        for (int b = 0; b < NB; ++b) bc[b] = bq[d][b];
 #pragma unroll
-        for (int i = 0; i < WM; ++i) ac[i] = live ? aq[d][i] : zero;
-        issue(d, k + 32 * D);
+        for (int i = 0; i < WM; ++i) ac[i] = aq[d % DA][i];
+        if constexpr (TAIL) {
+          const bool live = k + 8 * g + 8 <= K;
+#pragma unroll
+          for (int b = 0; b < NB; ++b) bc[b] = live ? bc[b] : zero;
+#pragma unroll
+          for (int i = 0; i < WM; ++i) ac[i] = live ? ac[i] : zero;
+        }
+        issue_x(d % DA, k + 32 * DA);
+        if constexpr (!FULL) issue_w(d, k + 32 * D);
         // keep the refill where it is written: the scheduler would otherwise sink every load
         // to just before its use and the ring would hold nothing in flight
         __builtin_amdgcn_sched_barrier(0);
+        if (k < k_end) {                           // scalar: a step past the segment's end is skipped
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
+          for (int b = 0; b < NB; ++b)
 #pragma unroll
-          for (int i = 0; i < WM; ++i)
-            acc[b][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ac[i]), as_bf16x8(bc[b]), acc[b][i], 0, 0, 0);
+            for (int i = 0; i < WM; ++i)
+              acc[b][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ac[i]), as_bf16x8(bc[b]), acc[b][i], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -131,7 +160,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = 16 * i + 4 * g + q;
-      if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n0 + r, acc[0][i][q], acc[NB - 1][i][q]);
+      if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[0][i][q], acc[NB - 1][i][q]);
     }
 }
 
@@ -143,7 +172,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #define WIDE_LDS_ROW 72   // bf16 elements per LDS row: 64 of data + 8 of padding (144 bytes)
 
 template <int EPI, bool MULTI>
-__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, int M, int N, int K, int ldx,
                                                              int ldo, int m_tiles, int n_tiles) {
   // In SwiGLU mode a block covers 64 output columns: B rows 0-63 are gate rows, 64-127 up rows.
@@ -161,23 +190,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const bf16_t* __res
   const int m0 = (bid % m_tiles) * WIDE_BM;
   const int n0 = (bid / m_tiles) * COLS;
 
-  // this thread's share of the global -> LDS copies: rows lr + 32j, 16-byte chunk lc
+  // This thread's share of the global -> LDS copies: rows lr + 32j, 16-byte chunk lc.  The loads
+  // go through buffer descriptors that cover exactly the block's rows of x and of W, so a row
+  // past M or N reads as zeros by itself and one 32-bit offset per operand is all a thread keeps.
   const int lr = tid >> 3, lc = tid & 7;
-  const bf16_t* ga[4];
-  const bf16_t* gb[4];
-  bool ga_ok[4], gb_ok[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = lr + 32 * j;
-    ga_ok[j] = m0 + row < M;
-    ga[j] = x + (size_t)(ga_ok[j] ? m0 + row : 0) * ldx + lc * 8;
-    int wrow;
-    if constexpr (EPI == EPI_SWIGLU_BF16) wrow = (row < 64) ? n0 + row : N + n0 + row - 64;
-    else wrow = n0 + row;
-    const int ncol = (EPI == EPI_SWIGLU_BF16) ? n0 + (row & 63) : n0 + row;
-    gb_ok[j] = ncol < N;
-    gb[j] = w + (size_t)(gb_ok[j] ? wrow : 0) * K + lc * 8;
-  }
+  const int a_rows = min(WIDE_BM, M - m0);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+  const int b_rows = min(COLS, N - n0);              // gate rows and up rows alike in SwiGLU mode
+  const __amdgpu_buffer_rsrc_t rs_b0 =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_b1 = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(w + ((size_t)N + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int voff_a = (lr * ldx + lc * 8) * 2, voff_b = (lr * K + lc * 8) * 2;
   // LDS rows of this wave's four B tiles
   int brow[4];
 #pragma unroll
@@ -195,31 +220,35 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const bf16_t* __res
       if constexpr (MULTI) tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
+  // Tiles travel global -> registers -> LDS.  A tile is asked for two steps before it is used
+  // and parked in one of two register sets meanwhile, so that a load has about two steps of
+  // matrix work to arrive in; it is written to LDS (two buffers) one step before its use.
+  // Loads are unconditional; a chunk past K (it would read the next row) is zeroed when it is
+  // written to LDS.
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  u32x4 ra[4], rb[4];
-  auto fetch = [&](int k0) {
-    const bool in = k0 + lc * 8 < K;
+  u32x4 ra[2][4], rb[2][4];
+  auto fetch = [&](int set, int k0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      ra[j] = (in && ga_ok[j]) ? *reinterpret_cast<const u32x4*>(ga[j] + k0) : zero;
-      rb[j] = (in && gb_ok[j]) ? *reinterpret_cast<const u32x4*>(gb[j] + k0) : zero;
+      ra[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, voff_a, (32 * j * ldx + k0) * 2, 0);
+      if constexpr (EPI == EPI_SWIGLU_BF16)
+        rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(j < 2 ? rs_b0 : rs_b1, voff_b, (32 * (j & 1) * K + k0) * 2, 0);
+      else
+        rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_b0, voff_b, (32 * j * K + k0) * 2, 0);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int set, int buf, int k0) {
+    if (k0 + WIDE_BK > K && k0 + lc * 8 >= K) {       // only in a last step that K does not fill
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ra[set][j] = rb[set][j] = zero;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[j];
-      *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[j];
+      *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set][j];
+      *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set][j];
     }
   };
-
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  int buf = 0;
-  for (int k0 = 0; k0 < K; k0 += WIDE_BK) {
-    const bool more = k0 + WIDE_BK < K;
-    if (more) fetch(k0 + WIDE_BK);
+  auto step = [&](int k0, int buf) {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       u32x4 fa[4], fb[4];
@@ -248,9 +277,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const bf16_t* __res
           }
       }
     }
-    if (more) stash(buf ^ 1);
+  };
+
+  fetch(0, 0);
+  fetch(1, WIDE_BK);
+  stash(0, 0, 0);
+  __syncthreads();
+  // steps in pairs, so that register sets and buffers are named at compile time
+  for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
+    fetch(0, k0 + 2 * WIDE_BK);
+    step(k0, 0);
+    stash(1, 1, k0 + WIDE_BK);
     __syncthreads();
-    buf ^= 1;
+    if (k0 + WIDE_BK >= K) break;
+    fetch(1, k0 + 3 * WIDE_BK);
+    step(k0 + WIDE_BK, 1);
+    stash(0, 0, k0 + 2 * WIDE_BK);
+    __syncthreads();
   }
 
 #pragma unroll
@@ -290,19 +333,25 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
   if (M <= 64) {
     const int wm = (M + 15) / 16;
     const int waves = S < 4 ? S : 4;      // one wave per SIMD: the operand ring may use up to 512 registers
-    dim3 grid((N + 15) / 16), block(64 * waves);
+    // few columns: half strips, so that there are at least as many workgroups as compute units
+    const bool half = (N + 15) / 16 < 256 && wm == 1;
+    dim3 grid(half ? (N + 7) / 8 : (N + 15) / 16), block(64 * waves);
     const size_t lds = S > 1 ? (size_t)S * NB * wm * 4 * 64 * sizeof(float) : 0;
     if (lds > 64 * 1024) return -2;
-#define BW_SKINNY(WMV, DV)                                                                                         \
+    if ((size_t)2 * N * K * 2 >= ((size_t)1 << 31) || (size_t)M * ldx * 2 >= ((size_t)1 << 31)) return -2;
+#define BW_SKINNY(WMV, DV, CWV)                                                                                    \
   if (K % 32)                                                                                                      \
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, true>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S); \
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, true, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S); \
   else                                                                                                             \
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, false>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S);
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, false, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S);
     switch (wm) {
-      case 1: BW_SKINNY(1, (NB == 2 ? 12 : 16)) break;
-      case 2: BW_SKINNY(2, (NB == 2 ? 8 : 12)) break;
-      case 3: BW_SKINNY(3, 8) break;
-      default: BW_SKINNY(4, 8) break;
+      case 1:
+        if (half) { BW_SKINNY(1, 16, 8) }
+        else { BW_SKINNY(1, 16, 16) }
+        break;
+      case 2: BW_SKINNY(2, (NB == 2 ? 8 : 16), 16) break;
+      case 3: BW_SKINNY(3, 8, 16) break;
+      default: BW_SKINNY(4, 8, 16) break;
     }
 #undef BW_SKINNY
   } else {

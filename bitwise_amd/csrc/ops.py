@@ -246,6 +246,12 @@ def decode_gemm_supported(rows: int, inner: int, norm: bool) -> bool:
     return _decode_ok[key]
 
 
+def qkv_rope_head_dim_ok(head_dim: int) -> bool:
+    """Head sizes the fused norm + q|k|v + rotation kernel takes: multiples of 32 (a workgroup
+    is a pair of 16-column strips half a head apart) and 16 or 48 (a workgroup is a head)."""
+    return head_dim % 16 == 0 and head_dim >= 16 and (head_dim % 32 == 0 or head_dim <= 64)
+
+
 def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor) -> bool:
     """Whether RMSNorm + product can run as one kernel for this step."""
     K = weight.shape[1]
@@ -299,8 +305,8 @@ def norm_qkv_rope_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w
     _need(cos, torch.float32, "cos table")
     _need(sin, torch.float32, "sin table")
     N, K = w_qkv.shape
-    if N != (heads + 2 * kv_heads) * head_dim or head_dim > 64 or head_dim % 16:
-        raise ValueError("norm_qkv_rope_bf16: weight is not [q|k|v] heads of at most 64 elements")
+    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_head_dim_ok(head_dim):
+        raise ValueError("norm_qkv_rope_bf16: weight is not [q|k|v] heads of a supported size")
     if not can_fuse_norm(rows, w_qkv, x) or norm_weight.numel() != K:
         raise ValueError("norm_qkv_rope_bf16: this step cannot be fused")
     if q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows or positions.numel() < rows or row_seq.numel() < rows:

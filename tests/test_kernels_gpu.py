@@ -422,7 +422,8 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
             assert torch.equal(fused_s, sep_s), (M, K, N)
     assert not ops.can_fuse_norm(17, w, x) and not ops.can_fuse_norm(4, torch.zeros(8, 4096, dtype=torch.bfloat16), x)
 
-    for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 96), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 160)]:
+    for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 96), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 160),
+                                     (2, 1, 128, 16, 256), (3, 3, 96, 16, 128)]:
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
