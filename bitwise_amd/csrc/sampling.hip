@@ -29,14 +29,29 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
   const int begin = tid * chunk < vocab ? tid * chunk : vocab;
   const int end = begin + chunk < vocab ? begin + chunk : vocab;
 
-  // maximum and its first index
+  // maximum and its first index: every thread scans an interleaved share of the row in ascending
+  // order (16-byte loads where the row allows), the shares are joined below with ties going to
+  // the smaller index, so the first maximum of the whole row wins whatever the split
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = begin; i < end; ++i)
-    if (l[i] > best || best_i == 0x7fffffff) {  // first element of the stretch, or strictly greater
-      best = l[i];
-      best_i = i;
+  if ((vocab & 3) == 0 && (ld & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
+    const f32x4* lv = reinterpret_cast<const f32x4*>(l);
+    for (int v = tid; v < (vocab >> 2); v += SMP_THREADS) {
+      const f32x4 x = lv[v];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (x[e] > best || best_i == 0x7fffffff) {  // the share's first element, or strictly greater
+          best = x[e];
+          best_i = 4 * v + e;
+        }
     }
+  } else {
+    for (int i = tid; i < vocab; i += SMP_THREADS)
+      if (l[i] > best || best_i == 0x7fffffff) {
+        best = l[i];
+        best_i = i;
+      }
+  }
   s_val[tid] = best;
   s_idx[tid] = best_i;
   __syncthreads();

@@ -14,6 +14,8 @@ import time
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence as Seq
 
+import numpy as np
+
 from ..cache.manager import CacheManager, GroupSpec
 from ..config.engine import EngineConfig, SamplingParams
 from ..sampling.rng import FINGERPRINT_BASIS
@@ -81,10 +83,20 @@ class GpuExecutor:
     def reset_slot(self, slot: int) -> None:
         self.storage.reset_slot(slot)
 
-    def run(self, segments: Seq[Segment]):
-        return self.runner.step(segments)
+    fused_sampling = True      # run() takes the sampling parameters and may sample inside the step
+
+    def run(self, segments: Seq[Segment], sampling=None):
+        """``sampling`` = (temperatures, seeds, positions) of the rows that will be sampled."""
+        if sampling is not None:
+            temps, seeds, positions = sampling
+            sampling = (np.asarray(temps, np.float32), self.sampler.uniforms(temps, seeds, positions))
+        return self.runner.step(segments, sampling)
 
     def sample(self, logits, temperatures, seeds, positions) -> List[int]:
+        done = self.runner.last_sampled
+        if done is not None and done.numel() == len(temperatures):      # the step's graph has sampled already
+            self.runner.last_sampled = None
+            return done.cpu().tolist()
         return self.sampler.sample(logits, temperatures, seeds, positions)
 
     def fingerprints(self, logits, previous) -> List[int]:
@@ -202,12 +214,16 @@ class Engine:
             else:
                 self._stats.prefill_tokens += w.n
         t0 = self.now()
-        logits = self.exec.run(segments)
+        draw = ([w.seq.params.temperature for w in sampled], [w.seq.params.seed for w in sampled],
+                [len(w.seq.tokens) for w in sampled])
+        if sampled and getattr(self.exec, "fused_sampling", False):
+            logits = self.exec.run(segments, draw)
+        else:
+            logits = self.exec.run(segments)
         new_tokens: List[int] = []
         prints: List[int] = []
         if sampled:
-            new_tokens = self.exec.sample(logits, [w.seq.params.temperature for w in sampled],
-                                          [w.seq.params.seed for w in sampled], [len(w.seq.tokens) for w in sampled])
+            new_tokens = self.exec.sample(logits, *draw)
             if self.cfg.fingerprint_logits:
                 prints = self.exec.fingerprints(logits, [self._results[w.seq.id].logits_fingerprint for w in sampled])
         self._stats.forward_seconds += self.now() - t0

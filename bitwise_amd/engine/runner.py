@@ -15,6 +15,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
+from ..csrc import ops
 from ..models.assembled import AssembledModel
 from .batch import AttentionPlan, Segment, StepContext
 from .storage import CacheStorage
@@ -23,15 +24,18 @@ GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 
 class _StaticDecodeContext:
-    """Fixed device arrays for a decode batch of up to ``size`` requests, one row each.  All of
-    them are views of one device buffer that a step refreshes with a single copy from pinned
-    host memory."""
+    """Fixed device arrays for a decode batch of up to ``size`` requests, one row each: the
+    step's index arrays and, for sampling inside the graph, each row's temperature and
+    uniform.  All of them are views of one device buffer that a step refreshes with a single
+    copy from pinned host memory."""
 
     def __init__(self, size: int, num_groups: int, max_pages: int, device: torch.device):
         self.rows = self.nseq = self.num_wanted = size
         self.device = device
         self.max_pages = max_pages
-        words = 3 * size + num_groups * size * max_pages
+        off_temp = 3 * size + num_groups * size * max_pages
+        off_uni = off_temp + size + ((off_temp + size) & 1)        # 64-bit values start at an even word
+        words = off_uni + 2 * size
         self._host = torch.zeros(words, dtype=torch.int32, pin_memory=True)
         self._host_np = self._host.numpy()
         self._dev = torch.zeros(words, dtype=torch.int32, device=device)
@@ -40,6 +44,11 @@ class _StaticDecodeContext:
         self.slots = self._dev[2 * size:3 * size]
         self.block_tables = [self._dev[3 * size + g * size * max_pages:3 * size + (g + 1) * size * max_pages].view(size, max_pages)
                              for g in range(num_groups)]
+        self.temps = self._dev[off_temp:off_temp + size].view(torch.float32)
+        self.unis = self._dev[off_uni:off_uni + 2 * size].view(torch.float64)
+        self._host_temps = self._host_np[off_temp:off_temp + size].view(np.float32)
+        self._host_unis = self._host_np[off_uni:off_uni + 2 * size].view(np.float64)
+        self.sampled = torch.zeros(size, dtype=torch.int32, device=device)
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
@@ -48,8 +57,14 @@ class _StaticDecodeContext:
     def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
         return self._plan
 
-    def fill(self, segments: Sequence[Segment]) -> None:
+    def fill(self, segments: Sequence[Segment], sampling=None) -> None:
+        """``sampling``: (temperatures, uniforms) of the rows, or None (greedy everywhere)."""
         size, n = self.rows, len(segments)
+        self._host_temps[:] = 0.0
+        self._host_unis[:] = 0.0
+        if sampling is not None:
+            self._host_temps[:n] = sampling[0]
+            self._host_unis[:n] = sampling[1]
         self.segments = list(segments)
         h = self._host_np
         h[0:size] = -1                      # padding rows: token -1, position -1
@@ -75,11 +90,17 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs: Dict[int, tuple] = {}
         self._graph_generation = -1
+        self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
 
     # ------------------------------------------------------------------ the step function
-    def step(self, segments: Sequence[Segment]) -> Optional[torch.Tensor]:
+    def step(self, segments: Sequence[Segment], sampling=None) -> Optional[torch.Tensor]:
         """Logits [wanted, vocab] (32-bit, on the device, valid until the next step) at the
-        wanted places in the order of the segments and of their ``want``; None if none."""
+        wanted places in the order of the segments and of their ``want``; None if none.
+
+        ``sampling`` = (temperatures, uniforms), one per wanted place: a step that is replayed
+        from a graph then also samples inside the graph (the same kernel a separate call
+        would run) and leaves the tokens in ``last_sampled``; any other step leaves None there."""
+        self.last_sampled = None
         if not segments:
             return None
         rows = sum(len(s.tokens) for s in segments)
@@ -99,12 +120,12 @@ class ModelRunner:
                     raise ValueError("a request's block table does not cover its positions")
         decode_only = all(len(s.tokens) == 1 and tuple(s.want) == (0,) for s in segments)
         if self.use_graphs and decode_only and len(segments) <= GRAPH_BUCKETS[-1]:
-            return self._step_graph(segments)
+            return self._step_graph(segments, sampling)
         ctx = StepContext(segments, len(self.model.group_specs), self.rt.device)
         return self.model.forward(ctx)
 
     # ------------------------------------------------------------------ graph replay
-    def _step_graph(self, segments: Sequence[Segment]) -> torch.Tensor:
+    def _step_graph(self, segments: Sequence[Segment], sampling=None) -> torch.Tensor:
         n = len(segments)
         bucket = next(b for b in GRAPH_BUCKETS if b >= n)
         if bucket > self.rt.max_rows or bucket > self.rt.max_logit_rows:
@@ -116,8 +137,10 @@ class ModelRunner:
         if entry is None:
             entry = self._capture(bucket, segments)
         ctx, graph, logits = entry
-        ctx.fill(segments)
+        ctx.fill(segments, sampling)
         graph.replay()
+        if sampling is not None:
+            self.last_sampled = ctx.sampled[:n]
         return logits[:n]
 
     def _capture(self, bucket: int, segments: Sequence[Segment]):
@@ -132,6 +155,7 @@ class ModelRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
+            ops.sample(logits, bucket, ctx.temps, ctx.unis, ctx.sampled)
         self._graph_generation = rt.scratch_generation
         entry = (ctx, graph, logits)
         self._graphs[bucket] = entry

@@ -35,12 +35,17 @@ class Sampler:
         if rows > self.max_rows or logits.shape[0] < rows:
             raise ValueError("more rows to sample than the sampler was made for")
         temps = np.asarray(temperatures, np.float32)
-        unis = np.asarray([counter_uniform(s, p, STREAM_SAMPLE) if t > 0 else 0.0
-                           for t, s, p in zip(temperatures, seeds, positions)], np.float64)
+        unis = self.uniforms(temperatures, seeds, positions)
         self._temp[:rows].copy_(torch.from_numpy(temps))
         self._uni[:rows].copy_(torch.from_numpy(unis))
         ops.sample(logits, rows, self._temp, self._uni, self._out)
         return self._out[:rows].cpu().tolist()
+
+    @staticmethod
+    def uniforms(temperatures: Sequence[float], seeds: Sequence[int], positions: Sequence[int]) -> np.ndarray:
+        """The uniform of each row's draw (0 where the row is greedy)."""
+        return np.asarray([counter_uniform(s, p, STREAM_SAMPLE) if t > 0 else 0.0
+                           for t, s, p in zip(temperatures, seeds, positions)], np.float64)
 
     def fingerprints(self, logits: torch.Tensor, previous: Sequence[int]) -> List[int]:
         """previous[r] chained over row r of ``logits`` (unsigned 64-bit values)."""
