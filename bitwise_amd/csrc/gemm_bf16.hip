@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #define WIDE_BK 64
 #define WIDE_LDS_ROW 72   // bf16 elements per LDS row: 64 of data + 8 of padding (144 bytes)
 
-template <int EPI, bool MULTI>
+template <int EPI, bool MULTI, bool FAST>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, int M, int N, int K, int ldx,
                                                              int ldo, int m_tiles, int n_tiles) {
@@ -238,14 +238,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
   };
   auto stash = [&](int set, int buf, int k0) {
-    if (k0 + WIDE_BK > K && k0 + lc * 8 >= K) {       // only in a last step that K does not fill
+    // the loaded registers are only ever read here: writing zeros into them instead would make
+    // the compiler wait for every load in flight first
+    if (k0 + WIDE_BK > K) {                           // a last step that K does not fill
+      const bool in = k0 + lc * 8 < K;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) ra[set][j] = rb[set][j] = zero;
-    }
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = in ? ra[set][j] : zero;
+        *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = in ? rb[set][j] : zero;
+      }
+    } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set][j];
-      *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set][j];
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set][j];
+        *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set][j];
+      }
     }
   };
   auto step = [&](int k0, int buf) {
@@ -283,6 +290,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   fetch(1, WIDE_BK);
   stash(0, 0, 0);
   __syncthreads();
+  if constexpr (FAST) {
+    // K is a multiple of 128 and one segment: every step is whole, and a step's body is one
+    // straight run of instructions that the scheduler is told how to interleave, so that the
+    // LDS traffic and the global loads hide behind the matrix instructions of the same wave:
+    //   8 operand reads (first half of the step);
+    //   8 x [2 matrix instructions, 1 operand read (second half), 1 global load (the tile after next)];
+    //   8 x [2 matrix instructions, 1 LDS write (the next tile, loaded a step ago)].
+    auto fast_step = [&](int k0, int set_fetch, int buf) {
+      fetch(set_fetch, k0 + 2 * WIDE_BK);             // past K: outside the descriptors, zeros, never used
+      u32x4 fa[2][4], fb[2][4];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          fa[kk][i] = *reinterpret_cast<const u32x4*>(&lds_a[buf][(64 * wy + 16 * i + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          fb[kk][j] = *reinterpret_cast<const u32x4*>(&lds_b[buf][(brow[j] + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<u32x4*>(&lds_a[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set_fetch ^ 1][j];
+        *reinterpret_cast<u32x4*>(&lds_b[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set_fetch ^ 1][j];
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
+      __syncthreads();
+    };
+    for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
+      fast_step(k0, 0, 0);
+      fast_step(k0 + WIDE_BK, 1, 1);
+    }
+  } else
   // steps in pairs, so that register sets and buffers are named at compile time
   for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
     fetch(0, k0 + 2 * WIDE_BK);
@@ -359,9 +416,11 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
     if (S > 1)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+    else if (K % (2 * WIDE_BK) == 0)
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
     else
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
   }
   return BW_LAUNCH_CHECK();
 }
