@@ -31,9 +31,9 @@ int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, con
                       const void* v_cache, int num_pages, void* out, int out_stride, int heads, int kv_heads,
                       int head_dim, int page_size, int window, float scale, int decode, void* stream);
 int bw_attention_fold_group_tiles(int head_dim);
-int bw_decode_gemm_supported(int M, int K, int norm);
-int bw_decode_gemm_bf16(const void* a_rows, int lda, int a_is_f32, const void* norm_w, int norm_w_is_bf16, float eps,
-                        const void* w, void* out, int ldo, int M, int N, int K, int epilogue, void* stream);
+int bw_norm_gemm_supported(int M, int K);
+int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps, const void* w,
+                      void* out, int ldo, int M, int N, int K, int epilogue, void* stream);
 int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps,
                           const void* w_qkv, void* q_out, const int32_t* positions, const int32_t* row_seq,
                           const int32_t* block_table, int table_stride, const float* cos_table,

@@ -1,26 +1,26 @@
-// The matrix product of decode steps (up to 16 rows, bfloat16 mode), with the work around it
-// fused in: optionally RMSNorm in front (the rows arrive as the 32-bit residual stream), and
-// behind it a plain store, the residual add, SwiGLU, or rotary encoding plus the cache write
-// (for the stacked q|k|v product).  A decode step is bound by kernel count and by how many
-// weight bytes are in flight, not by arithmetic; this kernel keeps the rows in LDS, so that
-// every outstanding memory request of a wave is a weight load, and replaces up to three
-// launches by one.
+// Decode steps of up to 16 rows in bfloat16 mode: RMSNorm fused into the matrix product that
+// follows it (the rows arrive as the 32-bit residual stream), and behind the product a plain
+// store, a residual add, SwiGLU, or rotary encoding plus the cache write (for the stacked
+// q|k|v product).  A decode step is bound by kernel count and by how many weight bytes are in
+// flight, not by arithmetic; this kernel keeps the normalised rows in LDS, so that every
+// outstanding memory request of a wave is a weight load, and replaces up to three launches.
 //
 // The arithmetic is that of the separate kernels, statement for statement, so a row's bits
 // do not depend on which route ran it:
 //   * RMSNorm: the sum of squares in the order of rmsnorm_bf16_kernel (lane l owns 16-byte
 //     vectors l, l+64, ...; xor butterflies), inv = 1/sqrt(ss/dim + eps), bf16((x*inv)*w);
-//   * product: K in segments of 2048; per segment every 16x16 block of outputs is one
-//     v_mfma_f32_16x16x32_bf16 chain over k ascending from zero; segments added left to right;
+//   * product: K is at most one segment (2048) here; every 16x16 block of outputs is one
+//     v_mfma_f32_16x16x32_bf16 chain over k ascending from zero;
 //   * rotary: o1 = x1*c - x2*s, o2 = x2*c + x1*s on the 32-bit products, one rounding when
 //     q goes to its buffer and k, v to their page slots (v transposed).
 //
-// Shape: a workgroup is SPW strips of 16 output columns times S segments, one wave each (for
-// q|k|v with rotary: the strips of one head).  Every wave first puts D steps of its weights in
-// flight, then all waves bring the rows into LDS as bfloat16 (normalising them on the way if
-// asked; rows padded by 16 bytes so that operand reads hit distinct banks), and then each
-// runs its chain with A operands from LDS and B operands from its ring.  Segment results of
-// a strip meet in LDS and are added in segment order.
+// Shape: a workgroup is a few strips of 16 output columns, one wave each (for q|k|v with
+// rotary: the strips of one head, or one strip and its rotary partner).  Loads go out in the
+// order their results are needed, because memory results are waited for in issue order: the
+// rows to normalise and the positions first, then D steps of the wave's weights, which stay in
+// flight while the rows are normalised into LDS (rows padded by 16 bytes so that operand reads
+// hit distinct banks).  Then each wave runs its chain with A operands from LDS and B operands
+// from its ring of registers.
 #include "common.h"
 #include "api.h"
 
@@ -29,11 +29,11 @@ enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI
 #define DEC_SEG 2048
 
 struct DecodeGemmArgs {
-  const void* a;           // NORM: float [M, lda] residual rows; else bf16 [M, lda]
-  const void* norm_w;      // [K] (NORM only)
+  const float* a;          // [M, lda] rows of the 32-bit residual stream
+  const void* norm_w;      // [K]
   const bf16_t* w;         // [N (or 2N for SwiGLU), K]
   void* out;               // F32/ADD: float [M, ldo]; BF16/SWIGLU: bf16 [M, ldo]; ROPE_KV: q bf16 [M, heads*hd]
-  int M, N, K, lda, ldo, S, norm_w_is_bf16;
+  int M, N, K, lda, ldo, norm_w_is_bf16;
   float eps;
   // rotary + cache write
   const int32_t* positions;
@@ -47,22 +47,21 @@ struct DecodeGemmArgs {
   int pairs;               // rotary: 16-wide pairs of strips a head is cut into (0: a workgroup is a whole head)
 };
 
-template <int EPI, bool NORM, int D>
+template <int EPI, int D>
 __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   constexpr int NB = (EPI == DEPI_SWIGLU_BF16) ? 2 : 1;
   constexpr bool FULL = D * 32 >= DEC_SEG;        // the ring holds a whole segment: nothing is refilled
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int K = a.K, M = a.M, S = a.S;
+  const int K = a.K, M = a.M;
   const int lds_row = K + 8;                      // bf16 elements; +16 bytes keeps operand reads conflict-free
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row]
   const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int strip = wave / S, seg = wave % S;     // the S waves of a strip are neighbours
   // rotary: a workgroup is a head (its strips in order), or, when half a head is a multiple of
   // 16, one strip of the first half and its partner in the second (workgroup p of the head:
   // strips p and p + pairs), so that twice as many workgroups share the stream
   int rope_head = 0, rope_base = 0, rope_lw = 0;
-  int n0 = (blockIdx.x * (nwaves / S) + strip) * 16;
+  int n0 = (blockIdx.x * nwaves + wave) * 16;
   if constexpr (EPI == DEPI_ROPE_KV) {
     if (a.pairs > 0) {
       rope_head = blockIdx.x / a.pairs;
@@ -75,8 +74,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     }
   }
   const bool n_ok = n0 + r < a.N;
-  const int k_begin = seg * DEC_SEG;
-  const int k_end = (K - k_begin) < DEC_SEG ? K : k_begin + DEC_SEG;
+  const int k_begin = 0, k_end = K;
   // weights through buffer descriptors that cover the strip's rows (rows past N read as zeros):
   // one per-lane offset for the whole kernel, the step's offset in a scalar register
   const int w_rows = min(16, a.N - n0);
@@ -94,14 +92,12 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   const int nvec = K >> 2;
   NormRows<RB> nr;
   const f32x4* nrows[RB];
-  if constexpr (NORM) {
 #pragma unroll
-    for (int i = 0; i < RB; ++i) {
-      const int m = wave + i * nwaves;             // rows are dealt to the waves round robin
-      nrows[i] = m < M ? reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda) : nullptr;
-    }
-    if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
+  for (int i = 0; i < RB; ++i) {
+    const int m = wave + i * nwaves;               // rows are dealt to the waves round robin
+    nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
   }
+  if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
   int r_pos[2] = {-1, -1}, r_seq[2] = {0, 0};
   if constexpr (EPI == DEPI_ROPE_KV) {
     const int lh = rope_lw >> 1;
@@ -144,39 +140,19 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     }
   }
 
-  // 2. the M rows into LDS as bfloat16
-  if constexpr (NORM) {
-    for (int m0 = wave; m0 < M;) {
-      norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
-        *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
-      });
-      m0 += RB * nwaves;
-      if (m0 >= M) break;
+  // 2. the M rows into LDS as bfloat16, normalised
+  for (int m0 = wave; m0 < M;) {
+    norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
+      *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
+    });
+    m0 += RB * nwaves;
+    if (m0 >= M) break;
 #pragma unroll
-      for (int i = 0; i < RB; ++i) {
-        const int m = m0 + i * nwaves;
-        nrows[i] = m < M ? reinterpret_cast<const f32x4*>((const float*)a.a + (size_t)m * a.lda) : nullptr;
-      }
-      norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
+    for (int i = 0; i < RB; ++i) {
+      const int m = m0 + i * nwaves;
+      nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
     }
-  } else {
-    const int cpr = K >> 3;                       // 16-byte chunks per row
-    const int total = M * cpr;
-    constexpr int UN = 8;
-    for (int base = 0; base < total; base += UN * blockDim.x) {
-      u32x4 v[UN];
-#pragma unroll
-      for (int j = 0; j < UN; ++j) {
-        const int idx = base + j * blockDim.x + threadIdx.x;
-        if (idx < total)
-          v[j] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.a + (size_t)(idx / cpr) * a.lda + (idx % cpr) * 8);
-      }
-#pragma unroll
-      for (int j = 0; j < UN; ++j) {
-        const int idx = base + j * blockDim.x + threadIdx.x;
-        if (idx < total) *reinterpret_cast<u32x4*>(xs + (size_t)(idx / cpr) * lds_row + (idx % cpr) * 8) = v[j];
-      }
-    }
+    norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
   }
   __syncthreads();
 
@@ -211,27 +187,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     }
   }
 
-  // 4. segments of a strip meet in LDS and are added in segment order by the strip's first wave
-  if (S > 1) {
-    __syncthreads();                               // every wave is done reading the rows
-    float* red = reinterpret_cast<float*>(smem);   // [wave][NB][4][64]
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) red[((wave * NB + b) * 4 + q) * 64 + lane] = acc[b][q];
-    __syncthreads();
-    if (seg != 0) return;
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        float y = acc[b][q];
-        for (int s = 1; s < S; ++s) y += red[(((wave + s) * NB + b) * 4 + q) * 64 + lane];
-        acc[b][q] = y;
-      }
-  }
-
-  // 5. epilogue
+  // 4. epilogue
   if constexpr (EPI != DEPI_ROPE_KV) {
     if (!n_ok) return;
 #pragma unroll
@@ -295,69 +251,55 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
 
 static const size_t kMaxLds = 160 * 1024 - 1024;
 
-template <int EPI, bool NORM, int D>
+template <int EPI, int D>
 static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hipStream_t s) {
   static bool raised = false;
-  size_t lds = (size_t)a.M * (a.K + 8) * sizeof(bf16_t);
-  const size_t red = (size_t)waves * 2 * 4 * 64 * sizeof(float);
-  if (a.S > 1 && red > lds) lds = red;
+  const size_t lds = (size_t)a.M * (a.K + 8) * sizeof(bf16_t);
   if (lds > kMaxLds) return -2;
   if (!raised) {   // more than 64 KB of dynamic LDS has to be asked for once
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, NORM, D>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, D>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds) != hipSuccess)
       return (int)hipGetLastError();
     raised = true;
   }
-  hipLaunchKernelGGL((decode_gemm_kernel<EPI, NORM, D>), dim3(blocks), dim3(64 * waves), lds, s, a);
+  hipLaunchKernelGGL((decode_gemm_kernel<EPI, D>), dim3(blocks), dim3(64 * waves), lds, s, a);
   return BW_LAUNCH_CHECK();
 }
 
 // Can the rows (M of them, K wide) live in LDS, and do the waves of a strip fit a workgroup?
-static int check_decode_gemm(const DecodeGemmArgs& a, bool norm) {
+static int check_decode_gemm(const DecodeGemmArgs& a) {
   if (a.M <= 0 || a.M > 16 || a.N <= 0 || a.K <= 0 || (a.K % 32)) return -2;
-  if (a.S > 4) return -2;
+  if (a.K > DEC_SEG || (a.lda % 4) || a.lda < a.K) return -2;      // a row is normalised from a wave's registers
   if ((size_t)a.M * (a.K + 8) * sizeof(bf16_t) > kMaxLds) return -2;
-  if (norm && (a.K > 2048 || (a.lda % 4))) return -2;
-  if (!norm && (a.lda % 8)) return -2;
-  if (a.lda < a.K) return -2;
   return 0;
 }
 
-extern "C" int bw_decode_gemm_supported(int M, int K, int norm) {
+extern "C" int bw_norm_gemm_supported(int M, int K) {
   DecodeGemmArgs a{};
-  a.M = M; a.N = 16; a.K = K; a.lda = K; a.S = (K + DEC_SEG - 1) / DEC_SEG;
-  return check_decode_gemm(a, norm != 0) == 0;
+  a.M = M; a.N = 16; a.K = K; a.lda = K;
+  return check_decode_gemm(a) == 0;
 }
 
-extern "C" int bw_decode_gemm_bf16(const void* a_rows, int lda, int a_is_f32, const void* norm_w, int norm_w_is_bf16,
-                                   float eps, const void* w, void* out, int ldo, int M, int N, int K, int epilogue,
-                                   void* stream) {
+extern "C" int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps,
+                                 const void* w, void* out, int ldo, int M, int N, int K, int epilogue, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   DecodeGemmArgs a{};
-  a.a = a_rows; a.norm_w = norm_w; a.w = (const bf16_t*)w; a.out = out;
-  a.M = M; a.N = N; a.K = K; a.lda = lda; a.ldo = ldo; a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
-  a.S = (K + DEC_SEG - 1) / DEC_SEG;
-  const bool norm = a_is_f32 != 0;
-  const int bad = check_decode_gemm(a, norm);
+  a.a = x; a.norm_w = norm_w; a.w = (const bf16_t*)w; a.out = out;
+  a.M = M; a.N = N; a.K = K; a.lda = ldx; a.ldo = ldo; a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
+  const int bad = check_decode_gemm(a);
   if (bad) return bad;
   if (ldo < N) return -2;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
-  const int spw = a.S == 1 ? 4 : (a.S == 2 ? 2 : 1);     // strips per workgroup; waves = spw * S <= 4
-  const int waves = spw * a.S;
+  const int waves = 4;                                   // strips per workgroup
   const int strips = (N + 15) / 16;
-  const int blocks = (strips + spw - 1) / spw;
+  const int blocks = (strips + waves - 1) / waves;
   hipStream_t s = (hipStream_t)stream;
-#define BW_DEC(EPIV, DV)                                                        \
-  case EPIV:                                                                    \
-    return norm ? launch_decode_gemm<EPIV, true, DV>(a, waves, blocks, s)       \
-                : launch_decode_gemm<EPIV, false, DV>(a, waves, blocks, s);
   switch (epilogue) {
-    BW_DEC(DEPI_F32, 32)
-    BW_DEC(DEPI_BF16, 32)
-    BW_DEC(DEPI_ADD_F32, 32)
-    BW_DEC(DEPI_SWIGLU_BF16, 20)
+    case DEPI_F32: return launch_decode_gemm<DEPI_F32, 32>(a, waves, blocks, s);
+    case DEPI_BF16: return launch_decode_gemm<DEPI_BF16, 32>(a, waves, blocks, s);
+    case DEPI_ADD_F32: return launch_decode_gemm<DEPI_ADD_F32, 32>(a, waves, blocks, s);
+    case DEPI_SWIGLU_BF16: return launch_decode_gemm<DEPI_SWIGLU_BF16, 20>(a, waves, blocks, s);
   }
-#undef BW_DEC
   return -2;
 }
 
@@ -374,19 +316,17 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
   DecodeGemmArgs a{};
   a.a = x; a.norm_w = norm_w; a.w = (const bf16_t*)w_qkv; a.out = q_out;
   a.M = M; a.N = (heads + 2 * kv_heads) * head_dim; a.K = K; a.lda = ldx; a.ldo = heads * head_dim;
-  a.S = 1;
   a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
   a.positions = positions; a.row_seq = row_seq; a.block_table = block_table; a.cos_table = cos_table;
   a.sin_table = sin_table; a.k_cache = (bf16_t*)k_cache; a.v_cache = (bf16_t*)v_cache;
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.page_size = page_size;
   a.table_stride = table_stride; a.write_cache = write_cache;
   a.pairs = pairs;
-  if (K > DEC_SEG) return -2;
-  const int bad = check_decode_gemm(a, true);
+  const int bad = check_decode_gemm(a);
   if (bad) return bad;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
   if ((size_t)(pairs ? 32 : head_dim) * sizeof(float) > (size_t)(K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
   const int all_heads = heads + 2 * kv_heads;
-  if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, true, 64>(a, 2, all_heads * pairs, (hipStream_t)stream);
-  return launch_decode_gemm<DEPI_ROPE_KV, true, 64>(a, head_dim / 16, all_heads, (hipStream_t)stream);
+  if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, 64>(a, 2, all_heads * pairs, (hipStream_t)stream);
+  return launch_decode_gemm<DEPI_ROPE_KV, 64>(a, head_dim / 16, all_heads, (hipStream_t)stream);
 }

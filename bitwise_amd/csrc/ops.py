@@ -45,9 +45,9 @@ _SIGS = {
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "bw_attention_fold_group_tiles": [c_int],
-    "bw_decode_gemm_supported": [c_int, c_int, c_int],
-    "bw_decode_gemm_bf16": [c_void_p, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
-                            c_int, c_int, c_void_p],
+    "bw_norm_gemm_supported": [c_int, c_int],
+    "bw_norm_gemm_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_int, c_void_p],
     "bw_norm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                               c_int, c_int, c_int, c_void_p],
@@ -238,11 +238,11 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
 _decode_ok = {}
 
 
-def decode_gemm_supported(rows: int, inner: int, norm: bool) -> bool:
-    """Whether the decode product kernel (rows kept in LDS) takes this many rows of this width."""
-    key = (rows, inner, norm)
+def norm_gemm_supported(rows: int, inner: int) -> bool:
+    """Whether the fused RMSNorm + product kernel (rows kept in LDS) takes this many rows of this width."""
+    key = (rows, inner)
     if key not in _decode_ok:
-        _decode_ok[key] = bool(_fn("bw_decode_gemm_supported")(rows, inner, int(norm)))
+        _decode_ok[key] = bool(_fn("bw_norm_gemm_supported")(rows, inner))
     return _decode_ok[key]
 
 
@@ -256,19 +256,7 @@ def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor) -> bool:
     """Whether RMSNorm + product can run as one kernel for this step."""
     K = weight.shape[1]
     return (weight.dtype == torch.bfloat16 and x.dtype == torch.float32 and x.shape[1] == K
-            and x.stride(0) % 4 == 0 and decode_gemm_supported(rows, K, True))
-
-
-def _decode_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, epilogue: int,
-                 norm_weight: Optional[torch.Tensor], eps: float) -> None:
-    N, K = w.shape
-    if epilogue == EPI_SWIGLU_BF16:
-        N //= 2
-    _check(_fn("bw_decode_gemm_bf16")(a.data_ptr(), a.stride(0), int(norm_weight is not None),
-                                      norm_weight.data_ptr() if norm_weight is not None else 0,
-                                      _is_bf16(norm_weight, "norm weight") if norm_weight is not None else 0,
-                                      float(eps), w.data_ptr(), out.data_ptr(), out.stride(0), rows, N, K, epilogue,
-                                      _stream()), "decode_gemm_bf16")
+            and x.stride(0) % 4 == 0 and norm_gemm_supported(rows, K))
 
 
 def norm_gemm_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
@@ -285,7 +273,9 @@ def norm_gemm_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: to
         raise ValueError(f"norm_gemm_bf16: {rows} rows of width {x.shape[1]} against weight {tuple(w.shape)} cannot be fused")
     if out.shape[1] != N or out.shape[0] < rows or x.shape[0] < rows:
         raise ValueError("norm_gemm_bf16: out does not fit")
-    _decode_gemm(x, w, out, rows, epilogue, norm_weight, eps)
+    _check(_fn("bw_norm_gemm_bf16")(x.data_ptr(), x.stride(0), norm_weight.data_ptr(), _is_bf16(norm_weight, "norm weight"),
+                                    float(eps), w.data_ptr(), out.data_ptr(), out.stride(0), rows, N, K, epilogue,
+                                    _stream()), "norm_gemm_bf16")
 
 
 def norm_qkv_rope_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor, q_out: torch.Tensor,
