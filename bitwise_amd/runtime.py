@@ -29,9 +29,8 @@ class Runtime:
             raise RuntimeError("bitwise_amd runs on the GPU only; there is no CPU path")
         self.act_dtype = torch.bfloat16 if mode == "bfloat16" else torch.float32
         self._buffers: Dict[Any, torch.Tensor] = {}
-        self._scratch: Dict[str, torch.Tensor] = {}
         self._shared: Dict[Any, Any] = {}
-        self.scratch_generation = 0      # bumped when a scratch tensor moves (captured graphs go stale)
+        self.scratch_generation = 0      # bumped when the buffers are dropped (captured graphs go stale)
         self.configure(max_rows, page_size, max_logit_rows)
 
     def configure(self, max_rows: int, page_size: int, max_logit_rows: int | None = None) -> None:
@@ -40,7 +39,6 @@ class Runtime:
         self.page_size = int(page_size)
         self.max_logit_rows = int(max_logit_rows if max_logit_rows is not None else max_rows)
         self._buffers.clear()
-        self._scratch.clear()
         self.scratch_generation += 1
 
     @property
@@ -54,15 +52,6 @@ class Runtime:
         if buf is None:
             buf = torch.zeros((rows if rows is not None else self.max_rows, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf
-
-    def scratch(self, name: str, numel: int, dtype: torch.dtype) -> torch.Tensor:
-        """A flat scratch tensor of at least ``numel`` elements; it grows (and moves) on demand."""
-        buf = self._scratch.get(name)
-        if buf is None or buf.numel() < numel or buf.dtype != dtype:
-            buf = torch.empty(max(int(numel), 1024), dtype=dtype, device=self.device)
-            self._scratch[name] = buf
-            self.scratch_generation += 1
         return buf
 
     def shared(self, key: Any, make: Callable[[], Any]) -> Any:
