@@ -22,6 +22,10 @@ int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, i
                 int accumulate, void* stream);
 int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, int epilogue,
                  void* stream);
+int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out, const int32_t* positions,
+                          const int32_t* row_seq, const int32_t* block_table, int table_stride, const float* cos_table,
+                          const float* sin_table, void* k_cache, void* v_cache, int M, int heads, int kv_heads,
+                          int head_dim, int K, int page_size, int write_cache, void* stream);
 int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
                      const int32_t* block_table, int table_stride, const float* k_cache, const float* v_cache,
                      float* out, int out_stride, int rows, int heads, int kv_heads, int head_dim, int page_size,

@@ -22,7 +22,20 @@
 #include "common.h"
 #include "api.h"
 
-enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3 };
+enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3, EPI_QKV_ROPE = 4 };
+
+// What the rotary epilogue of the stacked q|k|v product needs (wide kernel, heads of 64): the
+// statements of rope_kvwrite_bf16_kernel on the 32-bit products while they are still in registers.
+struct QkvRopeArgs {
+  const int32_t* positions;    // [rows]; negative = padding row
+  const int32_t* row_seq;      // [rows] -> row of the block table
+  const int32_t* block_table;
+  const float* cos_table;      // [max_pos, 32]
+  const float* sin_table;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  int heads, kv_heads, page_size, table_stride, write_cache;
+};
 
 #define GEMM_SEG 2048
 
@@ -31,7 +44,7 @@ __device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o,
   if constexpr (EPI == EPI_F32) ((float*)out)[o] = v;
   else if constexpr (EPI == EPI_BF16) ((bf16_t*)out)[o] = f32_to_bf16(v);
   else if constexpr (EPI == EPI_ADD_F32) ((float*)out)[o] += v;
-  else ((bf16_t*)out)[o] = f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * u);
+  else if constexpr (EPI == EPI_SWIGLU_BF16) ((bf16_t*)out)[o] = f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * u);
 }
 
 // ------------------------------------------------------------------------------ skinny
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 template <int EPI, bool MULTI, bool FAST>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, int M, int N, int K, int ldx,
-                                                             int ldo, int m_tiles, int n_tiles) {
+                                                             int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
   // In SwiGLU mode a block covers 64 output columns: B rows 0-63 are gate rows, 64-127 up rows.
   constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][WIDE_BM * WIDE_LDS_ROW];
@@ -359,7 +372,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int q = 0; q < 4; ++q) {
       const int m = m0 + 64 * wy + 16 * i + 4 * g + q;
       if (m >= M) continue;
-      if constexpr (EPI == EPI_SWIGLU_BF16) {
+      if constexpr (EPI == EPI_QKV_ROPE) {
+        // the wave's 64 columns are one head: tiles j and j + 2 hold the rotary pairs (d, d + 32) in
+        // the same lane; q heads go to the q buffer, k heads rotated and v heads as they are to
+        // this row's page slot (v transposed)
+        const int head = (n0 >> 6) + wx;
+        const int pos = rp.positions[m];
+        if (head >= rp.heads + 2 * rp.kv_heads || pos < 0) continue;
+        const int q_dim = rp.heads * 64;
+        size_t page = 0;
+        if (head >= rp.heads) page = (size_t)rp.block_table[(size_t)rp.row_seq[m] * rp.table_stride + pos / rp.page_size];
+        const int slot = pos % rp.page_size;
+        if (head < rp.heads + rp.kv_heads) {
+          bf16_t* dst = head < rp.heads ? (bf16_t*)out + (size_t)m * q_dim + (size_t)head * 64
+                                        : rp.k_cache + ((page * rp.kv_heads + (head - rp.heads)) * rp.page_size + slot) * 64;
+          if (head < rp.heads || rp.write_cache) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int d = 16 * j + r;
+              const float c = rp.cos_table[(size_t)pos * 32 + d], s = rp.sin_table[(size_t)pos * 32 + d];
+              const float x1 = acc[i][j][q], x2 = acc[i][j + 2][q];
+              const float o1 = x1 * c - x2 * s;
+              const float o2 = x2 * c + x1 * s;
+              dst[d] = f32_to_bf16(o1);
+              dst[d + 32] = f32_to_bf16(o2);
+            }
+          }
+        } else if (rp.write_cache) {
+          bf16_t* dst = rp.v_cache + (page * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size + slot;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
+        }
+      } else if constexpr (EPI == EPI_SWIGLU_BF16) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int n = n0 + 32 * wx + 16 * j + r;
@@ -384,10 +428,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <int EPI>
 static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo,
-                            hipStream_t s) {
+                            hipStream_t s, const QkvRopeArgs& rp = QkvRopeArgs{}) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
   constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
   if (M <= 64) {
+    if constexpr (EPI == EPI_QKV_ROPE) return -2;       // the rotary epilogue belongs to the wide kernel
     const int wm = (M + 15) / 16;
     const int waves = S < 4 ? S : 4;      // one wave per SIMD: the operand ring may use up to 512 registers
     // few columns: half strips, so that there are at least as many workgroups as compute units
@@ -416,11 +461,11 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
     if (S > 1)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else if (K % (2 * WIDE_BK) == 0)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
   }
   return BW_LAUNCH_CHECK();
 }
@@ -440,4 +485,23 @@ extern "C" int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int 
     case EPI_SWIGLU_BF16: return launch_gemm_bf16<EPI_SWIGLU_BF16>(xp, wp, out, M, N, K, ldx, ldo, s);
   }
   return -2;
+}
+
+// The stacked q|k|v product of a prompt portion with rotation and cache write in its epilogue
+// (heads of 64 elements, more than 64 rows, K of one segment): q rotated to q_out [M, heads*64],
+// k rotated and v to their page slots.  The bits of gemm_bf16 (32-bit store) + rope_kvwrite.
+extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out, const int32_t* positions,
+                                     const int32_t* row_seq, const int32_t* block_table, int table_stride,
+                                     const float* cos_table, const float* sin_table, void* k_cache, void* v_cache,
+                                     int M, int heads, int kv_heads, int head_dim, int K, int page_size,
+                                     int write_cache, void* stream) {
+  if (M <= 0) return 0;
+  if (head_dim != 64) return -4;
+  if (M <= 64 || K <= 0 || K > GEMM_SEG || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_qkv)) & 15) return -3;
+  QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                 heads, kv_heads, page_size, table_stride, write_cache};
+  const int N = (heads + 2 * kv_heads) * 64;
+  return launch_gemm_bf16<EPI_QKV_ROPE>((const bf16_t*)x, (const bf16_t*)w_qkv, q_out, M, N, K, ldx, heads * 64,
+                                        (hipStream_t)stream, rp);
 }

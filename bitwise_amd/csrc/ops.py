@@ -40,6 +40,8 @@ _SIGS = {
                         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_f32": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
@@ -379,6 +381,41 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
                                     k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], out.data_ptr(),
                                     out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode), _stream()),
            "attention_bf16")
+
+
+def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int) -> bool:
+    """Whether the q|k|v product of a prompt portion can take rotation and cache write into its epilogue."""
+    return rows > 64 and head_dim == 64 and inner <= 2048 and inner % 8 == 0
+
+
+def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                       row_seq: torch.Tensor, block_table: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor, rows: int, heads: int, kv_heads: int,
+                       head_dim: int, page_size: int, write_cache: bool = True) -> None:
+    """The stacked q|k|v product of more than 64 rows with rotation and cache write in its epilogue
+    (heads of 64); the bits of gemm_bf16 into a 32-bit buffer followed by rope_kvwrite."""
+    _need(x, torch.bfloat16, "x")
+    _need(w_qkv, torch.bfloat16, "qkv weight")
+    _need(q_out, torch.bfloat16, "q_out")
+    _need(k_cache, torch.bfloat16, "k_cache")
+    _need(v_cache, torch.bfloat16, "v_cache")
+    _need(positions, torch.int32, "positions")
+    _need(row_seq, torch.int32, "row_seq")
+    _need(block_table, torch.int32, "block_table")
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    N, K = w_qkv.shape
+    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_gemm_ok(rows, head_dim, K):
+        raise ValueError("gemm_qkv_rope_bf16: not a [q|k|v] weight of 64-element heads, or too few rows")
+    if x.shape[1] != K or x.shape[0] < rows or q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows:
+        raise ValueError("gemm_qkv_rope_bf16: buffers do not fit")
+    if positions.numel() < rows or row_seq.numel() < rows or cos.shape[1] != head_dim // 2 or sin.shape != cos.shape:
+        raise ValueError("gemm_qkv_rope_bf16: positions or rotary tables do not fit")
+    _check(_fn("bw_gemm_qkv_rope_bf16")(x.data_ptr(), x.stride(0), w_qkv.data_ptr(), q_out.data_ptr(),
+                                        positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
+                                        block_table.stride(0), cos.data_ptr(), sin.data_ptr(), k_cache.data_ptr(),
+                                        v_cache.data_ptr(), rows, heads, kv_heads, head_dim, K, page_size,
+                                        int(write_cache), _stream()), "gemm_qkv_rope_bf16")
 
 
 # ------------------------------------------------------------------------------ sampling

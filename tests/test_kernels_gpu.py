@@ -452,3 +452,39 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
         live = [0, 1, 2, 3, 4, 6]                                  # the row with position -1 is padding
         assert torch.equal(outs[0][0][live], outs[1][0][live])
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2])
+
+
+def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu):
+    """More than 64 rows and heads of 64: the wide product rotates and writes the cache in its
+    epilogue; q, the key pages and the value pages must be the bits of product + rope_kvwrite.
+    Rows of two requests, a padding row, positions across page edges, a ragged last tile."""
+    g = torch.Generator().manual_seed(21)
+    for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32)]:
+        hd, pages = 64, 40
+        cos, sin = rope_tables(10000.0, hd, 400, gpu)
+        h = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+        w = (torch.randn((heads + 2 * kvh) * hd, K, generator=g) * 0.05).bfloat16().to(gpu)
+        pos = [(r if r < M // 2 else r - M // 2 + 3) for r in range(M)]
+        pos[7] = -1
+        positions = torch.tensor(pos, dtype=torch.int32, device=gpu)
+        row_seq = torch.tensor([0 if r < M // 2 else 1 for r in range(M)], dtype=torch.int32, device=gpu)
+        per = (M + page - 1) // page + 2
+        table = torch.tensor([[(i * 3 + 1) % pages for i in range(per)], [(i * 3 + 2) % pages for i in range(per)]],
+                             dtype=torch.int32, device=gpu)
+        outs = []
+        for fused in (False, True):
+            kc = torch.full((pages, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+            vc = torch.full((pages, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+            q = torch.zeros(M, heads * hd, dtype=torch.bfloat16, device=gpu)
+            if fused:
+                assert ops.qkv_rope_gemm_ok(M, hd, K)
+                ops.gemm_qkv_rope_bf16(h, w, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh, hd, page)
+            else:
+                qkv = torch.zeros(M, w.shape[0], device=gpu)
+                ops.gemm_bf16(h, w, qkv, M, ops.EPI_F32)
+                ops.rope_kvwrite(qkv, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh, hd, page)
+            outs.append((q, kc, vc))
+        live = [r for r in range(M) if pos[r] >= 0]
+        assert torch.equal(outs[0][0][live], outs[1][0][live]), (heads, kvh, K, M)
+        assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), (heads, kvh, K, M)
+    assert not ops.qkv_rope_gemm_ok(64, 64, 256) and not ops.qkv_rope_gemm_ok(200, 128, 256)
