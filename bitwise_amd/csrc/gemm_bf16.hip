@@ -5,8 +5,9 @@
 // (a property of the weight, never of the batch).  Within a segment each 16x16 block of
 // outputs is one accumulator that runs v_mfma_f32_16x16x32_bf16 over k ascending in steps
 // of 32 from zero; within an instruction lane group g holds k = kk+8g..kk+8g+7.  Segment
-// results are added in 32-bit left to right: y = ((p0 + p1) + p2) + ...  An output's bits
-// therefore depend only on its own row of x and row of W.
+// results are added in 32-bit left to right: y = ((p0 + p1) + p2) + ..., and where the product
+// is added into a residual the chain starts there: y = ((res + p0) + p1) + ...  An output's bits
+// therefore depend only on its own row of x and row of W (and its own residual).
 //
 // Two kernels run this arithmetic.  The skinny one (up to 64 rows: decode) gives every
 // 16-column strip of W and every segment a wave of its own, which streams its 16 x 2048
@@ -163,6 +164,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float y = red[((b * WM + i) * 4 + q) * 64 + lane];
+          if constexpr (EPI == EPI_ADD_F32) {          // the chain of additions starts at the residual
+            const int m = 16 * i + 4 * g + q;
+            if (n_ok && m < M) y = ((const float*)out)[(size_t)m * ldo + n0 + c] + y;
+          }
           for (int s = 1; s < S; ++s) y += red[(((s * NB + b) * WM + i) * 4 + q) * 64 + lane];
           acc[b][i][q] = y;
         }
@@ -173,7 +178,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = 16 * i + 4 * g + q;
-      if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[0][i][q], acc[NB - 1][i][q]);
+      if (m >= M) continue;
+      if (EPI == EPI_ADD_F32 && S > 1) ((float*)out)[(size_t)m * ldo + n0 + c] = acc[0][i][q];   // the residual is in already
+      else epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[0][i][q], acc[NB - 1][i][q]);
     }
 }
 
@@ -224,13 +231,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     else brow[j] = 64 * wx + 16 * j;
   }
 
-  f32x4 acc[4][4], tot[MULTI ? 4 : 1][MULTI ? 4 : 1];
+  constexpr bool TOT = MULTI && !FAST;             // the fast path joins segments in the output itself
+  f32x4 acc[4][4], tot[TOT ? 4 : 1][TOT ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      if constexpr (MULTI) tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if constexpr (TOT) tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
   // Tiles travel global -> registers -> LDS.  A tile is asked for two steps before it is used
@@ -284,7 +292,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
     }
-    if constexpr (MULTI) {
+    if constexpr (TOT) {
       const int kn = k0 + WIDE_BK;
       if (kn % GEMM_SEG == 0 || kn >= K) {          // a segment ends: join it to the total, left to right
         const bool first = k0 < GEMM_SEG;
@@ -292,7 +300,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            tot[i][j] = first ? acc[i][j] : tot[i][j] + acc[i][j];
+            if constexpr (EPI == EPI_ADD_F32) {
+              if (first) {                          // the chain of additions starts at the residual
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 64 * wx + 16 * j + r;
+                  tot[i][j][q] = (m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;
+                }
+              }
+              tot[i][j] = tot[i][j] + acc[i][j];
+            } else {
+              tot[i][j] = first ? acc[i][j] : tot[i][j] + acc[i][j];
+            }
             acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
           }
       }
@@ -351,6 +370,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
       fast_step(k0, 0, 0);
       fast_step(k0 + WIDE_BK, 1, 1);
+      if constexpr (MULTI) {                         // residual add over several segments
+        const int kn = k0 + 2 * WIDE_BK;
+        if (kn % GEMM_SEG == 0 && kn < K) {          // a segment ends before the last: add it into the output now
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 64 * wx + 16 * j + r;
+                if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] += acc[i][j][q];
+              }
+              acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+        }
+      }
     }
   } else
   // steps in pairs, so that register sets and buffers are named at compile time
@@ -408,8 +443,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int j = 0; j < 2; ++j) {
           const int n = n0 + 32 * wx + 16 * j + r;
           if (n >= N) continue;
-          const float gv = MULTI ? tot[MULTI ? i : 0][MULTI ? j : 0][q] : acc[i][j][q];
-          const float uv = MULTI ? tot[MULTI ? i : 0][MULTI ? j + 2 : 0][q] : acc[i][j + 2][q];
+          const float gv = TOT ? tot[TOT ? i : 0][TOT ? j : 0][q] : acc[i][j][q];
+          const float uv = TOT ? tot[TOT ? i : 0][TOT ? j + 2 : 0][q] : acc[i][j + 2][q];
           epilogue_store<EPI>(out, (size_t)m * ldo + n, gv, uv);
         }
       } else {
@@ -417,8 +452,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int j = 0; j < 4; ++j) {
           const int n = n0 + 64 * wx + 16 * j + r;
           if (n >= N) continue;
-          const float v = MULTI ? tot[MULTI ? i : 0][MULTI ? j : 0][q] : acc[i][j][q];
-          epilogue_store<EPI>(out, (size_t)m * ldo + n, v, v);
+          const float v = TOT ? tot[TOT ? i : 0][TOT ? j : 0][q] : acc[i][j][q];
+          if (EPI == EPI_ADD_F32 && TOT) ((float*)out)[(size_t)m * ldo + n] = v;     // the residual is in already
+          else epilogue_store<EPI>(out, (size_t)m * ldo + n, v, v);
         }
       }
     }
@@ -460,7 +496,9 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
-    if (S > 1)
+    if (S > 1 && EPI == EPI_ADD_F32 && K % (2 * WIDE_BK) == 0)
+      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, EPI == EPI_ADD_F32>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
+    else if (S > 1)
       hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else if (K % (2 * WIDE_BK) == 0)
       hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);

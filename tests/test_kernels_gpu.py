@@ -90,7 +90,8 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     g = torch.Generator().manual_seed(3)
     for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
-                    (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144)]:      # several 2048-segments of K
+                    (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
+                    (129, 96, 6144)]:                                     # several 2048-segments of K
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = torch.randn(N, K, generator=g).bfloat16().to(gpu)
         y = torch.full((M, N), 3.0, device=gpu)
@@ -107,7 +108,12 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
         res = torch.randn(M, N, generator=g).to(gpu)
         acc = res.clone()
         ops.gemm_bf16(x, w, acc, M, ops.EPI_ADD_F32)
-        assert torch.equal(acc, res + y)
+        want = res.clone()                                         # the chain of segment sums starts at the residual
+        for k0 in range(0, K, 2048):
+            part = torch.zeros(M, N, device=gpu)
+            ops.gemm_bf16(x[:, k0:k0 + 2048].contiguous(), w[:, k0:k0 + 2048].contiguous(), part, M, ops.EPI_F32)
+            want = want + part
+        assert torch.equal(acc, want), (M, N, K)
     M, inter, K = 19, 56, 96
     x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
