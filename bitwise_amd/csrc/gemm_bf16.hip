@@ -231,7 +231,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     else brow[j] = 64 * wx + 16 * j;
   }
 
-  constexpr bool TOT = MULTI && !FAST;             // the fast path joins segments in the output itself
+  static_assert(!(MULTI && FAST), "the fast path is for one segment");
+  constexpr bool TOT = MULTI;
   f32x4 acc[4][4], tot[TOT ? 4 : 1][TOT ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -323,13 +324,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   stash(0, 0, 0);
   __syncthreads();
   if constexpr (FAST) {
-    // K is a multiple of 128 and one segment: every step is whole, and a step's body is one
-    // straight run of instructions that the scheduler is told how to interleave, so that the
-    // LDS traffic and the global loads hide behind the matrix instructions of the same wave:
+    // K is a multiple of 128: every step is whole, and a step's body is one straight run of
+    // instructions that the scheduler is told how to interleave, so that the LDS traffic and the
+    // global loads hide behind the matrix instructions of the same wave:
     //   8 operand reads (first half of the step);
     //   8 x [2 matrix instructions, 1 operand read (second half), 1 global load (the tile after next)];
     //   8 x [2 matrix instructions, 1 LDS write (the next tile, loaded a step ago)].
+    // (What then bounds the kernel is how many bytes of tile loads a compute unit can keep in
+    // flight: about 45 KB, which at the latency of the L2 is a little more than the 64 KB a step
+    // of two resident workgroups asks for.)
     auto fast_step = [&](int k0, int set_fetch, int buf) {
+      const int set_stash = set_fetch ^ 1;
       fetch(set_fetch, k0 + 2 * WIDE_BK);             // past K: outside the descriptors, zeros, never used
       u32x4 fa[2][4], fb[2][4];
 #pragma unroll
@@ -350,8 +355,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        *reinterpret_cast<u32x4*>(&lds_a[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set_fetch ^ 1][j];
-        *reinterpret_cast<u32x4*>(&lds_b[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set_fetch ^ 1][j];
+        *reinterpret_cast<u32x4*>(&lds_a[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set_stash][j];
+        *reinterpret_cast<u32x4*>(&lds_b[buf ^ 1][(lr + 32 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set_stash][j];
       }
       __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
@@ -370,22 +375,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
       fast_step(k0, 0, 0);
       fast_step(k0 + WIDE_BK, 1, 1);
-      if constexpr (MULTI) {                         // residual add over several segments
-        const int kn = k0 + 2 * WIDE_BK;
-        if (kn % GEMM_SEG == 0 && kn < K) {          // a segment ends before the last: add it into the output now
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 64 * wx + 16 * j + r;
-                if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] += acc[i][j][q];
-              }
-              acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            }
-        }
-      }
     }
   } else
   // steps in pairs, so that register sets and buffers are named at compile time
@@ -460,6 +449,126 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// The same tiles worked by eight waves (each 64 x 32 outputs), for products whose grid is too
+// small to give every compute unit two workgroups of four: two waves per SIMD inside one
+// workgroup, so that one wave's LDS traffic hides behind the other's matrix instructions.
+// K in whole double steps; epilogues store / bf16 / residual add (several segments: added into
+// the output segment by segment, the chain starting at the residual).
+template <int EPI>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_wide8_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
+    int ldo, int m_tiles, int n_tiles) {
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][WIDE_BM * WIDE_LDS_ROW];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][WIDE_BN * WIDE_LDS_ROW];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int wy = wave >> 2, wx = wave & 3;
+  int bid = blockIdx.x;
+  const int nblocks = m_tiles * n_tiles;
+  if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;
+  const int m0 = (bid % m_tiles) * WIDE_BM;
+  const int n0 = (bid / m_tiles) * WIDE_BN;
+  const int lr = tid >> 3, lc = tid & 7;             // rows lr, lr + 64; 16-byte chunk lc
+  const int a_rows = min(WIDE_BM, M - m0), b_rows = min(WIDE_BN, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_b =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int voff_a = (lr * ldx + lc * 8) * 2, voff_b = (lr * K + lc * 8) * 2;
+
+  f32x4 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  u32x4 ra[2][2], rb[2][2];
+  auto fetch = [&](int set, int k0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      ra[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, voff_a, (64 * j * ldx + k0) * 2, 0);
+      rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_b, voff_b, (64 * j * K + k0) * 2, 0);
+    }
+  };
+  auto stash = [&](int set, int buf) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 64 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set][j];
+      *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 64 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set][j];
+    }
+  };
+  auto fast_step = [&](int k0, int set_fetch, int buf) {
+    fetch(set_fetch, k0 + 2 * WIDE_BK);               // past K: outside the descriptors, zeros, never used
+    u32x4 fa[2][4], fb[2][2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        fa[kk][i] = *reinterpret_cast<const u32x4*>(&lds_a[buf][(64 * wy + 16 * i + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        fb[kk][j] = *reinterpret_cast<const u32x4*>(&lds_b[buf][(32 * wx + 16 * j + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
+    stash(set_fetch ^ 1, buf ^ 1);
+    // 8 operand reads; 4 x [2 matrix instructions, 1 operand read, 1 global load]; 4 x [2 matrix instructions, 1 LDS write]
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    __syncthreads();
+  };
+  fetch(0, 0);
+  fetch(1, WIDE_BK);
+  stash(0, 0);
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
+    fast_step(k0, 0, 0);
+    fast_step(k0 + WIDE_BK, 1, 1);
+    if constexpr (EPI == EPI_ADD_F32) {
+      const int kn = k0 + 2 * WIDE_BK;
+      if (kn % GEMM_SEG == 0 && kn < K) {            // a segment ends before the last: add it into the output now
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 32 * wx + 16 * j + r;
+              if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] += acc[i][j][q];
+            }
+            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = m0 + 64 * wy + 16 * i + 4 * g + q;
+      if (m >= M) continue;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int n = n0 + 32 * wx + 16 * j + r;
+        if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j][q]);
+      }
+    }
+}
+
 // ------------------------------------------------------------------------------ launch
 
 template <int EPI>
@@ -496,9 +605,15 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
-    if (S > 1 && EPI == EPI_ADD_F32 && K % (2 * WIDE_BK) == 0)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, EPI == EPI_ADD_F32>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
-    else if (S > 1)
+    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_ADD_F32) {
+      // too few tiles for two workgroups of four waves per compute unit: eight waves a tile
+      // (and every residual add over several segments: it joins them in the output itself)
+      if (K % (2 * WIDE_BK) == 0 && ((S == 1 && m_tiles * n_tiles <= 256) || (S > 1 && EPI == EPI_ADD_F32))) {
+        hipLaunchKernelGGL((gemm_bf16_wide8_kernel<EPI>), grid, dim3(512), 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+        return BW_LAUNCH_CHECK();
+      }
+    }
+    if (S > 1)
       hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else if (K % (2 * WIDE_BK) == 0)
       hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);

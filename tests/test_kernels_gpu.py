@@ -90,6 +90,7 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     g = torch.Generator().manual_seed(3)
     for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
+                    (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
                     (129, 96, 6144)]:                                     # several 2048-segments of K
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
