@@ -120,9 +120,15 @@ def main() -> int:
 
     def decode_point(batch: int, steps: int, warmup: int):
         torch.cuda.empty_cache()
-        eng = make_engine(bw, model, batch, steps + warmup, dtype)
-        fill(eng, bw, torch, batch, vocab, steps + warmup + 4, seed=batch)
+        # Requests admitted early decode while the later ones are still being prefilled (one prompt a
+        # step): every request gets enough new tokens to outlast the prefills, the warm-up and the
+        # timed steps, so that each timed step has all ``batch`` rows.
+        new_tokens = steps + warmup + batch + 8
+        eng = make_engine(bw, model, batch, new_tokens, dtype)
+        fill(eng, bw, torch, batch, vocab, new_tokens, seed=batch)
+        assert len(eng.sched.running) == batch
         secs = time_decode(eng, torch, steps, warmup)
+        assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
         kv_token = eng.exec.storage.bytes_per_token()
         del eng
         return secs, kv_token
@@ -130,7 +136,9 @@ def main() -> int:
     secs, kv_token = decode_point(args.batch, args.steps, args.warmup)
     ms_step = secs / args.steps * 1e3
     value = args.batch * args.steps / secs
-    avg_ctx = CONTEXT + args.warmup + (args.steps + 1) / 2          # keys a decoded token reads, on average
+    # keys a decoded token reads, on average: the prompt, what the request decoded while later
+    # prompts were prefilled, the warm-up, and half the timed steps
+    avg_ctx = CONTEXT + (args.batch - 1) / 2 + args.warmup + (args.steps + 1) / 2
     step_bytes = model.weight_bytes + args.batch * avg_ctx * kv_token
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
     points = {}
