@@ -495,3 +495,29 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
         assert torch.equal(outs[0][0][live], outs[1][0][live]), (heads, kvh, K, M)
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), (heads, kvh, K, M)
     assert not ops.qkv_rope_gemm_ok(64, 64, 256) and not ops.qkv_rope_gemm_ok(200, 128, 256)
+
+
+def test_decode_attention_beyond_one_pass_of_partials(gpu):
+    """A context so long that the decode kernel's partials do not fit LDS at once (several
+    passes over the partitions): still the bits of the fold kernel, and the plain result."""
+    heads, kvh, hd, page = 2, 1, 64, 64
+    n = 12600                                                      # 197 partitions of 64 keys; one pass holds 186
+    pages = n // page + 4
+    while pages % 7 == 0:
+        pages += 1
+    k, v, kc, vc, tab = paged_setup(gpu, True, heads, kvh, hd, page, pages, n, seed=31, poison=True)
+    g = torch.Generator().manual_seed(32)
+    positions = [n - 1, 11903, 11904, 5000]                        # at the pass edge, and a short one
+    q = torch.randn(len(positions), heads * hd, generator=g).bfloat16()
+    fold = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page)
+    split = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
+    assert torch.isfinite(split.float()).all()
+    assert torch.equal(split, fold)
+    for r, p in enumerate(positions):                              # softmax(q k^T / sqrt(hd)) v for this one row, in float64
+        for h in range(heads):
+            qh = q[r].double().view(heads, hd)[h]
+            kk, vv = k[:p + 1, h // (heads // kvh)].double(), v[:p + 1, h // (heads // kvh)].double()
+            w = torch.softmax(kk @ qh / hd ** 0.5, dim=0)
+            want = w @ vv
+            got = split[r].cpu().double().view(heads, hd)[h]
+            assert (got - want).abs().max() <= 1.5e-2 * want.abs().max().clamp(min=0.05), (p, h)
