@@ -1,35 +1,39 @@
 // bfloat16 causal attention over the paged cache on the matrix cores.
 //
 // Arithmetic (one definition for prompt portions and decoded tokens alike): the keys of a
-// sequence are cut at absolute positions into partitions of 64.  For a query (one column of
-// a 16-column tile) and a partition t the partial result is
-//   s_j = (q . k_j) * scale           32-bit, from v_mfma_f32_16x16x32_bf16 over d ascending
-//   m_t = max_j s_j                   over the partition's keys the query may see
-//   p_j = bf16(exp(s_j - m_t)),  l_t = sum_j p_j (fixed order),  O_t = sum_j p_j * v_j (MFMA, keys ascending)
-// and the partials are folded strictly left to right over t:
-//   m' = max(m, m_t); a = exp(m - m'); b = exp(m_t - m'); l = fma(l, a, l_t*b); O = fma(O, a, O_t*b)
-// (the first partition a query sees initialises the state; a partition it cannot see is
-// skipped).  out = O * (1/l).  The fold kernel walks the partitions inside one wave; the
-// decode kernel gives every partition a wave of its own and performs the same fold from LDS
-// in partition order, so both routes give the same bits, and a query's result depends on
-// nothing but its own row, its position and the cache contents at positions it may see.
+// sequence are cut at absolute positions into partitions of 64.  Everything is in the base-2
+// domain with c = scale * log2(e).  For a query (one column of a 16-column tile) and a
+// partition t the partial result is
+//   d_j = q . k_j                      32-bit, from v_mfma_f32_16x16x32_bf16 over the head's elements ascending
+//   m_t = (max_j d_j) * c              over the partition's keys the query may see
+//   p_j = bf16(exp2(fma(d_j, c, -m_t))), 0 for a key it may not see
+//   l_t = sum_j p_j                    on the matrix core against rows of ones
+//   O_t = sum_j p_j * v_j              by MFMA, keys ascending in steps of 32
+// and the partials are folded strictly left to right over t, without branches:
+//   m' = max(m, m_t); a = exp2(m - m'); b = exp2(m_t - m'); l = fma(l, a, l_t*b); O = fma(O, a, O_t*b)
+// from the state m = -inf, l = 0, O = 0.  out = O * (1/l).  The fold kernel and the decode
+// kernel call the same device functions for the partial and run the same statements for the
+// fold, so both give the same bits, and a query's result depends on nothing but its own row,
+// its position and the cache contents at positions it may see.
 //
 // Layout: S^T = K Q^T is computed (keys are MFMA rows, queries are columns), so the
 // probabilities come out of the accumulator in exactly the lane layout that the second
-// product O^T = V^T P^T needs for its B operand; no LDS is used.  K pages are
-// [kv_head][slot][hd]; V pages are transposed, [kv_head][hd][slot], so that an A-operand
-// lane reads 4 consecutive keys of one d with one 8-byte load.
+// product O^T = V^T P^T needs for its B operand.  K pages are [kv_head][slot][hd]; V pages are
+// transposed, [kv_head][hd][slot], so that an A-operand lane reads 4 consecutive keys of one
+// element with one 8-byte load.
 //
-// Work shapes: in the fold kernel a wave owns up to QT tiles (QT*16 queries of one sequence
-// and kv head) and reuses every loaded K and V operand for all of them, prefetching the next
-// partition's keys while it works; in the decode kernel a workgroup owns one tile (one token,
-// the heads of one kv head) and each of its waves one partition at a time, all loads of a
-// partition issued at once.
+// Work shapes: the fold kernel (prompt portions) gives a workgroup of up to 8 waves as many
+// tiles of one sequence and kv head, a tile a wave; the threads together stage each partition's
+// keys and values once in LDS (the next partition's loads fly meanwhile), and every wave whose
+// queries see the partition folds it into its own state.  The decode kernel (tiles of one
+// token) gives a workgroup one tile and each of its 8 waves one partition at a time, operands
+// straight from the pages into registers; the partials meet in LDS and are folded there in
+// partition order.
 #include "common.h"
 #include "api.h"
 
 #define ATT_PART 64
-#define FOLD_QT(HD) 1
+#define FOLD_QT(HD) 1                      // tiles per wave of the fold kernel
 #define FOLD_NW(HD) ((HD) <= 192 ? 8 : 4)  // waves per workgroup of the fold kernel
 
 struct AttnBf16Args {
@@ -386,7 +390,7 @@ __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m
   m = mn;
 }
 
-// Route 1, for prompt portions.  A workgroup of 4 waves owns FoldShape::GROUP consecutive tiles
+// Route 1, for prompt portions.  A workgroup of FoldShape::NW waves owns FoldShape::GROUP consecutive tiles
 // of one sequence and one kv head (the host pads every sequence's tile list to a multiple of
 // that), wave w the tiles w*QT .. w*QT+QT-1.  The workgroup walks the partitions any of its
 // queries may see; the threads together copy a partition's keys and values from the pages into
