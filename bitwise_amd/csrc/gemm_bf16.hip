@@ -75,6 +75,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
   const int r = lane & 15, g = lane >> 4;
   const int c = r % CW;
   const int n0 = blockIdx.x * CW;
+  // blockIdx.y: which block of 16*WM rows
+  x += (size_t)blockIdx.y * (16 * WM) * ldx;
+  M -= blockIdx.y * (16 * WM);
+  if constexpr (EPI == EPI_F32 || EPI == EPI_ADD_F32) out = (float*)out + (size_t)blockIdx.y * (16 * WM) * ldo;
+  else out = (bf16_t*)out + (size_t)blockIdx.y * (16 * WM) * ldo;
   const bool n_ok = r < CW && n0 + c < N;
   const int w_rows = min(CW, N - n0);
   __amdgpu_buffer_rsrc_t rs_w[NB];
@@ -578,11 +583,16 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
   constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
   if (M <= 64) {
     if constexpr (EPI == EPI_QKV_ROPE) return -2;       // the rotary epilogue belongs to the wide kernel
-    const int wm = (M + 15) / 16;
+    const int row_blocks = (M + 15) / 16, strips = (N + 15) / 16;
+    // Few columns and more than 16 rows: a workgroup per block of 16 rows (the strips of W are then
+    // fetched once per block of rows, from cache after the first, by four times the waves).  Many
+    // columns: one wave takes all rows of its strip.
+    const bool split_rows = row_blocks > 1 && strips < 256;
+    const int wm = split_rows ? 1 : row_blocks;
     const int waves = S < 4 ? S : 4;      // one wave per SIMD: the operand ring may use up to 512 registers
     // few columns: half strips, so that there are at least as many workgroups as compute units
-    const bool half = (N + 15) / 16 < 256 && wm == 1;
-    dim3 grid(half ? (N + 7) / 8 : (N + 15) / 16), block(64 * waves);
+    const bool half = strips < 256 && row_blocks == 1;
+    dim3 grid(half ? (N + 7) / 8 : strips, split_rows ? row_blocks : 1), block(64 * waves);
     const size_t lds = S > 1 ? (size_t)S * NB * wm * 4 * 64 * sizeof(float) : 0;
     if (lds > 64 * 1024) return -2;
     if ((size_t)2 * N * K * 2 >= ((size_t)1 << 31) || (size_t)M * ldx * 2 >= ((size_t)1 << 31)) return -2;
