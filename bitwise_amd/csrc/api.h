@@ -33,7 +33,10 @@ int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, con
 int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                       int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                       const void* v_cache, int num_pages, void* out, int out_stride, int heads, int kv_heads,
-                      int head_dim, int page_size, int window, float scale, int decode, void* stream);
+                      int head_dim, int page_size, int window, float scale, int decode, float* scratch,
+                      long long scratch_floats, int32_t* counters, int num_counters, void* stream);
+int bw_attention_decode_scratch(int num_tiles, int heads, int kv_heads, int head_dim, int table_stride,
+                                int page_size, long long* scratch_floats, int* counters);
 int bw_attention_fold_group_tiles(int head_dim);
 int bw_norm_gemm_supported(int M, int K);
 int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps, const void* w,

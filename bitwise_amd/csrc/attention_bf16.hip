@@ -642,17 +642,72 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
 // partials in partition order (thread t owns output elements t, t + threads, ... of the tile's
 // live columns).  The statements are those of fold(), so the bits equal route 1; the waves
 // only buy memory parallelism.  LDS holds ``pcap`` partitions; longer contexts take passes.
+//
+// SPLIT, for so few tiles that a workgroup each would leave most compute units idle: gridDim.z
+// workgroups share a tile; workgroup z takes the partitions of rounds z, z + gridDim.z, ... (a
+// round = W partitions) and writes their partials to ``scratch`` in device memory instead; each
+// workgroup then counts itself in, and the one that finds all others counted in folds all
+// partials, again in partition order from the first: the same statements on the same values.
+// The counter is back at zero when the kernel ends.
 template <int HD, int W>
-__global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a, int pcap) {
+__device__ __forceinline__ void decode_fold_pass(const AttnBf16Args& a, const float* parts, int count,
+                                                 float (&m)[(16 * HD + 64 * W - 1) / (64 * W)],
+                                                 float (&l)[(16 * HD + 64 * W - 1) / (64 * W)],
+                                                 float (&o)[(16 * HD + 64 * W - 1) / (64 * W)]) {
+  constexpr int THREADS = 64 * W, EPT = (16 * HD + THREADS - 1) / THREADS, CELL = HD + 2;
+  const int elems = a.hpt * HD;
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = threadIdx.x + j * THREADS;
+    if (e >= elems) continue;
+    const int col = e / HD, d = e % HD;
+    for (int wv = 0; wv < count; ++wv) {
+      const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
+      const float m_p = cell[0], l_p = cell[1], o_p = cell[2 + d];
+      float mn, fa, fb;
+      fold_scalars(m[j], m_p, mn, fa, fb);
+      l[j] = fmaf(l[j], fa, l_p * fb);
+      o[j] = fmaf(o[j], fa, o_p * fb);
+      m[j] = mn;
+    }
+  }
+}
+
+// DEVICE: the cells lie in device memory and another workgroup, maybe on another die with its own
+// L2, will read them in this same kernel: device-scope stores (they write through).
+template <int HD, bool DEVICE>
+__device__ __forceinline__ void store_partial(const AttnBf16Args& a, const GroupCtx& gc, float* cells, float m_p,
+                                              float l_p, const f32x4 (&o_p)[HD / 16]) {
+  if (gc.r >= a.hpt) return;
+  float* cell = cells + (size_t)gc.r * (HD + 2);    // a partition's cells: [hpt][m, l, hd values]
+  auto put = [&](int i, float v) {
+    if constexpr (DEVICE) __hip_atomic_store(cell + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else cell[i] = v;
+  };
+  if (gc.g == 0) {
+    put(0, m_p);
+    put(1, l_p);
+  }
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(2 + 16 * dt + 4 * gc.g + i, o_p[dt][i]);
+}
+
+template <int HD, int W, bool SPLIT>
+__global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a, int pcap, float* __restrict__ scratch,
+                                                                  int* __restrict__ counters, int max_parts) {
   constexpr int NT = HD / 16;
   constexpr int THREADS = 64 * W;
   constexpr int EPT = (16 * HD + THREADS - 1) / THREADS;   // output elements per thread at most (16 live columns)
   constexpr int CELL = HD + 2;                              // m, l, then hd values
-  constexpr bool PREFETCH = HD <= 64;
+  constexpr bool PREFETCH = HD <= 64 && !SPLIT;
   extern __shared__ float parts[];                          // [pcap][hpt][CELL]
+  __shared__ int is_last;
   GroupCtx gc;
   TileCtx<HD> tc[1];
-  if (!group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc)) return;   // uniform over the workgroup
+  const bool live = group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc);   // uniform over the workgroup
+  if (!SPLIT && !live) return;
   const int wave = wave_index();
   const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
   const int elems = a.hpt * HD;
@@ -663,68 +718,80 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
     l[j] = 0.0f;
     o[j] = 0.0f;
   }
-  for (int pass0 = first; pass0 <= last; pass0 += pcap) {
-    const int pass_last = (last - pass0) < pcap ? last : pass0 + pcap - 1;
-    KFrags<HD> kf, kf_next;
-    VFrags<HD> vf, vf_next;
-    PartPages pg, pg_now;
-    int part = pass0 + wave;
-    load_pages(a, gc, part, pg);
-    if constexpr (PREFETCH) {
-      load_keys<HD>(a, gc, part, pg, kf);
-      load_values<HD>(a, gc, pg, vf);
-      load_pages(a, gc, part + W, pg);
+  if constexpr (SPLIT) {
+    const int item = blockIdx.x * gridDim.y + blockIdx.y;
+    float* mine = scratch + (size_t)item * max_parts * a.hpt * CELL;
+    if (live) {
+      PartPages pg;
+      KFrags<HD> kf;
+      VFrags<HD> vf;
+      for (int part = first + blockIdx.z * W + wave; part <= last; part += W * gridDim.z) {
+        load_pages(a, gc, part, pg);
+        load_keys<HD>(a, gc, part, pg, kf);
+        load_values<HD>(a, gc, pg, vf);
+        float m_p, l_p;
+        f32x4 o_p[NT];
+        partition_partial<HD>(a, gc, tc[0], part, pg, kf, vf, m_p, l_p, o_p);
+        store_partial<HD, true>(a, gc, mine + (size_t)(part - first) * a.hpt * CELL, m_p, l_p, o_p);
+      }
     }
-    for (; part <= pass_last; part += W) {
+    // The barrier waits for every thread's stores (device-scope ones: they are in memory then, no
+    // cache has to be written back) before the workgroup counts itself in, and orders the last
+    // workgroup's loads (device scope again) behind its count.
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = atomicAdd(&counters[item], 1) == (int)gridDim.z - 1;
+    __syncthreads();
+    if (!is_last) return;
+    if (threadIdx.x == 0) counters[item] = 0;
+    if (!live) return;
+    for (int pass0 = first; pass0 <= last; pass0 += pcap) {
+      const int count = (last - pass0) < pcap ? last - pass0 + 1 : pcap;
+      const float* src = mine + (size_t)(pass0 - first) * a.hpt * CELL;
+      for (int i = threadIdx.x; i < count * a.hpt * CELL; i += THREADS)
+        parts[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      decode_fold_pass<HD, W>(a, parts, count, m, l, o);
+      __syncthreads();
+    }
+  } else {
+    for (int pass0 = first; pass0 <= last; pass0 += pcap) {
+      const int pass_last = (last - pass0) < pcap ? last : pass0 + pcap - 1;
+      KFrags<HD> kf, kf_next;
+      VFrags<HD> vf, vf_next;
+      PartPages pg, pg_now;
+      int part = pass0 + wave;
+      load_pages(a, gc, part, pg);
       if constexpr (PREFETCH) {
-        if (part + W <= pass_last) {
-          load_keys<HD>(a, gc, part + W, pg, kf_next);
-          load_values<HD>(a, gc, pg, vf_next);
-          load_pages(a, gc, part + 2 * W, pg);
-        }
-      } else {
-        pg_now = pg;
-        load_keys<HD>(a, gc, part, pg_now, kf);
-        load_values<HD>(a, gc, pg_now, vf);
+        load_keys<HD>(a, gc, part, pg, kf);
+        load_values<HD>(a, gc, pg, vf);
         load_pages(a, gc, part + W, pg);
       }
-      float m_p, l_p;
-      f32x4 o_p[NT];
-      partition_partial<HD>(a, gc, tc[0], part, PREFETCH ? pg : pg_now, kf, vf, m_p, l_p, o_p);
-      if (gc.r < a.hpt) {
-        float* cell = parts + ((size_t)(part - pass0) * a.hpt + gc.r) * CELL;
-        if (gc.g == 0) {
-          cell[0] = m_p;
-          cell[1] = l_p;
+      for (; part <= pass_last; part += W) {
+        if constexpr (PREFETCH) {
+          if (part + W <= pass_last) {
+            load_keys<HD>(a, gc, part + W, pg, kf_next);
+            load_values<HD>(a, gc, pg, vf_next);
+            load_pages(a, gc, part + 2 * W, pg);
+          }
+        } else {
+          pg_now = pg;
+          load_keys<HD>(a, gc, part, pg_now, kf);
+          load_values<HD>(a, gc, pg_now, vf);
+          load_pages(a, gc, part + W, pg);
         }
-#pragma unroll
-        for (int dt = 0; dt < NT; ++dt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) cell[2 + 16 * dt + 4 * gc.g + i] = o_p[dt][i];
+        float m_p, l_p;
+        f32x4 o_p[NT];
+        partition_partial<HD>(a, gc, tc[0], part, PREFETCH ? pg : pg_now, kf, vf, m_p, l_p, o_p);
+        store_partial<HD, false>(a, gc, parts + (size_t)(part - pass0) * a.hpt * CELL, m_p, l_p, o_p);
+        if constexpr (PREFETCH) {
+          kf = kf_next;
+          vf = vf_next;
+        }
       }
-      if constexpr (PREFETCH) {
-        kf = kf_next;
-        vf = vf_next;
-      }
+      __syncthreads();
+      decode_fold_pass<HD, W>(a, parts, pass_last - pass0 + 1, m, l, o);
+      __syncthreads();
     }
-    __syncthreads();
-    const int count = pass_last - pass0 + 1;
-#pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-      const int e = threadIdx.x + j * THREADS;
-      if (e >= elems) continue;
-      const int col = e / HD, d = e % HD;
-      for (int wv = 0; wv < count; ++wv) {
-        const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
-        const float m_p = cell[0], l_p = cell[1], o_p = cell[2 + d];
-        float mn, fa, fb;
-        fold_scalars(m[j], m_p, mn, fa, fb);
-        l[j] = fmaf(l[j], fa, l_p * fb);
-        o[j] = fmaf(o[j], fa, o_p * fb);
-        m[j] = mn;
-      }
-    }
-    __syncthreads();
   }
   // columns of a one-token tile: column c is head sub*hpt + c of the kv head's group
   const int group = a.heads / a.kv_heads;
@@ -740,15 +807,40 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
   }
 }
 
+#define DECODE_W 8
+
+// How a decode launch over ``num_tiles`` tiles is split: workgroups per tile (1 = no split) and
+// the partitions a tile's scratch must hold.  Depends on nothing that changes from step to step.
+static void decode_split_shape(int num_tiles, int items, int table_stride, int page_size, int& nsplit, int& max_parts) {
+  max_parts = (table_stride * page_size + ATT_PART - 1) / ATT_PART + 1;
+  const int rounds = (max_parts + DECODE_W - 1) / DECODE_W;
+  const int wgs = num_tiles * items;
+  nsplit = wgs >= 128 ? 1 : 256 / wgs;
+  if (nsplit > rounds) nsplit = rounds;
+  if (nsplit < 1) nsplit = 1;
+}
+
 template <int HD>
-static void launch_attention(const AttnBf16Args& a, int decode, hipStream_t s) {
+static int launch_attention(const AttnBf16Args& a, int decode, float* scratch, size_t scratch_floats, int* counters,
+                            int num_counters, hipStream_t s) {
   const int items = a.kv_heads * a.nsub;
   if (decode) {
-    constexpr int W = 8;
+    constexpr int W = DECODE_W;
     const size_t cell = (size_t)a.hpt * (HD + 2) * sizeof(float);
     int pcap = (int)((48 * 1024) / cell);          // partitions whose partials fit 48 KB of LDS
     pcap = pcap < W ? W : (pcap > 256 ? 256 : pcap);
-    hipLaunchKernelGGL((attention_decode_kernel<HD, W>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a, pcap);
+    int nsplit, max_parts;
+    decode_split_shape(a.num_tiles, items, a.table_stride, a.page_size, nsplit, max_parts);
+    if (scratch == nullptr || counters == nullptr) nsplit = 1;
+    if (nsplit > 1) {
+      if (scratch_floats < (size_t)a.num_tiles * items * max_parts * a.hpt * (HD + 2) || num_counters < a.num_tiles * items)
+        return -6;
+      hipLaunchKernelGGL((attention_decode_kernel<HD, W, true>), dim3(a.num_tiles, items, nsplit), dim3(64 * W), pcap * cell, s,
+                         a, pcap, scratch, counters, max_parts);
+    } else {
+      hipLaunchKernelGGL((attention_decode_kernel<HD, W, false>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a,
+                         pcap, nullptr, nullptr, 0);
+    }
   } else {
     using S = FoldShape<HD>;
     constexpr int lds_bytes = S::NBUF * S::BYTES;
@@ -760,14 +852,35 @@ static void launch_attention(const AttnBf16Args& a, int decode, hipStream_t s) {
     hipLaunchKernelGGL((attention_fold_kernel<HD>), dim3((a.num_tiles + S::GROUP - 1) / S::GROUP, items), dim3(64 * S::NW),
                        lds_bytes, s, a);
   }
+  return 0;
 }
 
 extern "C" int bw_attention_fold_group_tiles(int head_dim) { return FOLD_NW(head_dim) * FOLD_QT(head_dim); }
 
+// What a split decode launch needs beside its inputs: floats of scratch and counters (int32, zero
+// before the first launch; every launch leaves them zero).  Both 0: the launch is not split.
+extern "C" int bw_attention_decode_scratch(int num_tiles, int heads, int kv_heads, int head_dim, int table_stride,
+                                           int page_size, long long* scratch_floats, int* counters) {
+  *scratch_floats = 0;
+  *counters = 0;
+  if (num_tiles <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0) return -2;
+  const int group = heads / kv_heads;
+  const int hpt = group < 16 ? group : 16, nsub = (group + hpt - 1) / hpt;
+  int nsplit, max_parts;
+  decode_split_shape(num_tiles, kv_heads * nsub, table_stride, page_size, nsplit, max_parts);
+  if (nsplit > 1) {
+    *scratch_floats = (long long)num_tiles * kv_heads * nsub * max_parts * hpt * (head_dim + 2);
+    *counters = num_tiles * kv_heads * nsub;
+  }
+  return 0;
+}
+
 extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                                  int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                                  const void* v_cache, int num_pages, void* out, int out_stride, int heads,
-                                 int kv_heads, int head_dim, int page_size, int window, float scale, int decode, void* stream) {
+                                 int kv_heads, int head_dim, int page_size, int window, float scale, int decode,
+                                 float* scratch, long long scratch_floats, int32_t* counters, int num_counters,
+                                 void* stream) {
   if (num_tiles <= 0) return 0;
   if (num_pages <= 0) return -2;
   if (kv_heads <= 0 || heads % kv_heads) return -2;
@@ -788,12 +901,14 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   a.scale_log2 = scale * 1.44269504088896340736f;
   if (kv_heads * a.nsub > 65535) return -2;
   hipStream_t s = (hipStream_t)stream;
-#define BW_CASE(HD) case HD: launch_attention<HD>(a, decode, s); break;
+  int rc = 0;
+#define BW_CASE(HD) case HD: rc = launch_attention<HD>(a, decode, scratch, (size_t)scratch_floats, counters, num_counters, s); break;
   switch (head_dim) {
     BW_CASE(16) BW_CASE(32) BW_CASE(48) BW_CASE(64) BW_CASE(80) BW_CASE(96) BW_CASE(112) BW_CASE(128)
     BW_CASE(160) BW_CASE(192) BW_CASE(224) BW_CASE(256)
     default: return -4;
   }
 #undef BW_CASE
+  if (rc) return rc;
   return BW_LAUNCH_CHECK();
 }

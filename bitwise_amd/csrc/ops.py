@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -28,6 +28,7 @@ _ERRORS = {
     -3: "misaligned pointer or stride",
     -4: f"head size not compiled in (supported: {HEAD_DIMS})",
     -5: "page size not supported (a power of two from 4 to 64 is needed)",
+    -6: "scratch smaller than attention_decode_scratch asks for",
 }
 
 _SIGS = {
@@ -45,7 +46,9 @@ _SIGS = {
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
-                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_longlong,
+                          c_void_p, c_int, c_void_p],
+    "bw_attention_decode_scratch": [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_attention_fold_group_tiles": [c_int],
     "bw_norm_gemm_supported": [c_int, c_int],
     "bw_norm_gemm_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -342,7 +345,8 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
 def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    out: torch.Tensor, heads: int, kv_heads: int, head_dim: int, page_size: int, window: int,
-                   scale: float, decode: bool = False) -> None:
+                   scale: float, decode: bool = False,
+                   scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> None:
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
     [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).
 
@@ -353,7 +357,11 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     the tiles of a sequence must come in runs padded to that number (empty tiles allowed).
     ``decode`` True (tiles of one token each; ``tiles`` None means "tile t is row t of sequence
     t"): a workgroup per tile whose waves take one 64-key partition each and fold through LDS
-    in partition order.  The bits are the same either way."""
+    in partition order.  The bits are the same either way.
+
+    ``scratch`` (decode only): the tensors ``attention_decode_scratch`` asks for, (float32, int32
+    zeros).  With them a launch of few tiles is split over several workgroups per tile; without
+    them it is not.  The bits are the same again."""
     _need(q, torch.bfloat16, "q")
     _need(out, torch.bfloat16, "out")
     _need(k_cache, torch.bfloat16, "k_cache")
@@ -376,11 +384,30 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
     page_elems = kv_heads * page_size * head_dim
     if k_cache.dim() != 2 or k_cache.shape[1] != page_elems or v_cache.shape != k_cache.shape:
         raise ValueError(f"attention_bf16: caches must be [pages, {page_elems}]")
+    sc_f = sc_c = None
+    if scratch is not None and decode:
+        sc_f, sc_c = scratch
+        _need(sc_f, torch.float32, "scratch")
+        _need(sc_c, torch.int32, "scratch counters")
     _check(_fn("bw_attention_bf16")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
                                     block_table.stride(0), tiles.data_ptr() if tiles is not None else 0, num_tiles,
                                     k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], out.data_ptr(),
-                                    out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode), _stream()),
+                                    out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode),
+                                    sc_f.data_ptr() if sc_f is not None else 0, sc_f.numel() if sc_f is not None else 0,
+                                    sc_c.data_ptr() if sc_c is not None else 0, sc_c.numel() if sc_c is not None else 0,
+                                    _stream()),
            "attention_bf16")
+
+
+def attention_decode_scratch(num_tiles: int, heads: int, kv_heads: int, head_dim: int, table_stride: int,
+                             page_size: int) -> Tuple[int, int]:
+    """(float32 elements, int32 counters) that a decode launch of ``num_tiles`` tiles wants as
+    ``scratch`` to split its tiles over workgroups; (0, 0): it would not split."""
+    floats, counters = ctypes.c_longlong(0), ctypes.c_int(0)
+    _check(_fn("bw_attention_decode_scratch")(num_tiles, heads, kv_heads, head_dim, table_stride, page_size,
+                                              ctypes.addressof(floats), ctypes.addressof(counters)),
+           "attention_decode_scratch")
+    return int(floats.value), int(counters.value)
 
 
 def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int) -> bool:

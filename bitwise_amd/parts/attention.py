@@ -130,5 +130,13 @@ class Attention(Mixer):
         if plan.fold_count:
             ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
         if plan.decode_count:
-            ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True)
+            # few decoded tokens: several workgroups a tile, meeting in device scratch
+            floats, counters = ops.attention_decode_scratch(plan.decode_count, self.heads, self.kv_heads, self.head_dim,
+                                                            table.stride(0), rt.page_size)
+            scratch = None
+            if floats:
+                scratch = (rt.buffer("attn_split", floats, torch.float32, rows=1),
+                           rt.buffer("attn_split_count", counters, torch.int32, rows=1))
+            ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True,
+                               scratch=scratch)
         self.o.add_into(out, residual, rows)

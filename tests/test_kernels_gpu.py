@@ -258,7 +258,10 @@ def paged_setup(gpu, bf16, heads, kvh, hd, page, pages, n_keys, seed, poison=Fal
     return k, v, kc.reshape(pages, -1).to(gpu), vc.reshape(pages, -1).to(gpu), tab
 
 
-def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=0, split=False, tiles=None):
+def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=0, split=False, tiles=None,
+                  shared=False):
+    """split: the decode kernel (a wave per partition); shared: it may also split a tile over
+    workgroups that meet in device scratch (given full of NaN: only what a launch wrote may be read)."""
     rows = len(positions)
     pos = torch.tensor(positions, dtype=torch.int32, device=gpu)
     scale = 1.0 / float(hd) ** 0.5
@@ -271,8 +274,19 @@ def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, wi
     if tiles is None:
         tiles = [(r, 1, 0, 0) for r in range(rows)]
     t = torch.tensor(tiles, dtype=torch.int32, device=gpu)
+    scratch = None
+    if shared:
+        floats, counters = ops.attention_decode_scratch(len(tiles), heads, kvh, hd, tab.stride(0), page)
+        assert floats > 0 and counters > 0, "this launch was meant to be split over workgroups"
+        scratch = (torch.full((floats,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
     ops.attention_bf16(q.to(gpu), pos, tab, t, len(tiles), kc, vc, out, heads, kvh, hd, page, window, scale,
-                       decode=split)
+                       decode=split, scratch=scratch)
+    if shared:                                   # the counters are zero again, and a second launch on them agrees
+        assert not scratch[1].any()
+        again = torch.zeros_like(out)
+        ops.attention_bf16(q.to(gpu), pos, tab, t, len(tiles), kc, vc, again, heads, kvh, hd, page, window, scale,
+                           decode=True, scratch=scratch)
+        assert torch.equal(again, out) and not scratch[1].any()
     return out
 
 
@@ -313,6 +327,8 @@ def test_attention_batched_equals_alone_and_plain(gpu, bf16, heads, kvh, hd, pag
     if bf16:                                                      # a wave per partition gives the same bits
         sp = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
         assert torch.equal(sp, batch)
+        sh = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True, shared=True)
+        assert torch.equal(sh, batch)             # and so do several workgroups a tile
 
 
 @pytest.mark.parametrize("bf16", [False, True])
@@ -361,6 +377,10 @@ def test_attention_finds_a_far_key_and_respects_the_window(gpu, bf16):
             assert hit == visible, f"key {far} from position {p}: visible={hit}"
             refw = plain_rows(q.to(dt), kk, v, [p], heads, window=100)
             assert (w.cpu().double() - refw).abs().max() <= (1.5e-2 if bf16 else 3e-6) * refw.abs().max()
+            if bf16:                              # the window's first partition is where a split tile's scratch begins
+                ws = run_attention(gpu, bf16, q.to(dt), [p], tab, kc2.view(50, -1), vc, heads, kvh, hd, page, window=100,
+                                   split=True, shared=True)
+                assert torch.equal(ws, w)
 
 
 def test_attention_refuses_what_it_cannot_do(gpu):
@@ -513,6 +533,8 @@ def test_decode_attention_beyond_one_pass_of_partials(gpu):
     split = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
     assert torch.isfinite(split.float()).all()
     assert torch.equal(split, fold)
+    shared = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True, shared=True)
+    assert torch.equal(shared, fold)
     for r, p in enumerate(positions):                              # softmax(q k^T / sqrt(hd)) v for this one row, in float64
         for h in range(heads):
             qh = q[r].double().view(heads, hd)[h]
