@@ -189,6 +189,69 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
     }
 }
 
+// ------------------------------------------------------------------------------ tile epilogue
+
+// What a wave does with its NI x 4 accumulators (16 x 16 outputs each: rows row0 + 16 i + 4 g + q,
+// columns 16 j + r of the wave's 64).  Plain epilogues: output columns col0 + 16 j + r.  SwiGLU:
+// accumulators j = 0, 1 are gate columns col0 + 16 j + r, j = 2, 3 the up columns of the same outputs.
+// Rotary q|k|v: the wave's 64 columns are head ``head``; accumulators j and j + 2 hold the rotary pairs
+// (d, d + 32) in the same lane; q heads go to the q buffer, k heads rotated and v heads as they are to
+// the row's page slot (v transposed).  ``residual_in``: the values already contain the residual.
+template <int EPI, int NI>
+__device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* __restrict__ out, int M, int N, int ldo,
+                                              int row0, int col0, int head, int r, int g, bool residual_in,
+                                              const QkvRopeArgs& rp) {
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = row0 + 16 * i + 4 * g + q;
+      if (m >= M) continue;
+      if constexpr (EPI == EPI_QKV_ROPE) {
+        const int pos = rp.positions[m];
+        if (head >= rp.heads + 2 * rp.kv_heads || pos < 0) continue;
+        const int q_dim = rp.heads * 64;
+        size_t page = 0;
+        if (head >= rp.heads) page = (size_t)rp.block_table[(size_t)rp.row_seq[m] * rp.table_stride + pos / rp.page_size];
+        const int slot = pos % rp.page_size;
+        if (head < rp.heads + rp.kv_heads) {
+          bf16_t* dst = head < rp.heads ? (bf16_t*)out + (size_t)m * q_dim + (size_t)head * 64
+                                        : rp.k_cache + ((page * rp.kv_heads + (head - rp.heads)) * rp.page_size + slot) * 64;
+          if (head < rp.heads || rp.write_cache) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int d = 16 * j + r;
+              const float c = rp.cos_table[(size_t)pos * 32 + d], s = rp.sin_table[(size_t)pos * 32 + d];
+              const float x1 = acc[i][j][q], x2 = acc[i][j + 2][q];
+              const float o1 = x1 * c - x2 * s;
+              const float o2 = x2 * c + x1 * s;
+              dst[d] = f32_to_bf16(o1);
+              dst[d + 32] = f32_to_bf16(o2);
+            }
+          }
+        } else if (rp.write_cache) {
+          bf16_t* dst = rp.v_cache + (page * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size + slot;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
+        }
+      } else if constexpr (EPI == EPI_SWIGLU_BF16) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = col0 + 16 * j + r;
+          if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j + 2][q]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = col0 + 16 * j + r;
+          if (n >= N) continue;
+          if (EPI == EPI_ADD_F32 && residual_in) ((float*)out)[(size_t)m * ldo + n] = acc[i][j][q];
+          else epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j][q]);
+        }
+      }
+    }
+}
+
 // ------------------------------------------------------------------------------ wide
 
 #define WIDE_BM 128
@@ -395,63 +458,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();
   }
 
+  if constexpr (TOT) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int m = m0 + 64 * wy + 16 * i + 4 * g + q;
-      if (m >= M) continue;
-      if constexpr (EPI == EPI_QKV_ROPE) {
-        // the wave's 64 columns are one head: tiles j and j + 2 hold the rotary pairs (d, d + 32) in
-        // the same lane; q heads go to the q buffer, k heads rotated and v heads as they are to
-        // this row's page slot (v transposed)
-        const int head = (n0 >> 6) + wx;
-        const int pos = rp.positions[m];
-        if (head >= rp.heads + 2 * rp.kv_heads || pos < 0) continue;
-        const int q_dim = rp.heads * 64;
-        size_t page = 0;
-        if (head >= rp.heads) page = (size_t)rp.block_table[(size_t)rp.row_seq[m] * rp.table_stride + pos / rp.page_size];
-        const int slot = pos % rp.page_size;
-        if (head < rp.heads + rp.kv_heads) {
-          bf16_t* dst = head < rp.heads ? (bf16_t*)out + (size_t)m * q_dim + (size_t)head * 64
-                                        : rp.k_cache + ((page * rp.kv_heads + (head - rp.heads)) * rp.page_size + slot) * 64;
-          if (head < rp.heads || rp.write_cache) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int d = 16 * j + r;
-              const float c = rp.cos_table[(size_t)pos * 32 + d], s = rp.sin_table[(size_t)pos * 32 + d];
-              const float x1 = acc[i][j][q], x2 = acc[i][j + 2][q];
-              const float o1 = x1 * c - x2 * s;
-              const float o2 = x2 * c + x1 * s;
-              dst[d] = f32_to_bf16(o1);
-              dst[d + 32] = f32_to_bf16(o2);
-            }
-          }
-        } else if (rp.write_cache) {
-          bf16_t* dst = rp.v_cache + (page * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size + slot;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
-        }
-      } else if constexpr (EPI == EPI_SWIGLU_BF16) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int n = n0 + 32 * wx + 16 * j + r;
-          if (n >= N) continue;
-          const float gv = TOT ? tot[TOT ? i : 0][TOT ? j : 0][q] : acc[i][j][q];
-          const float uv = TOT ? tot[TOT ? i : 0][TOT ? j + 2 : 0][q] : acc[i][j + 2][q];
-          epilogue_store<EPI>(out, (size_t)m * ldo + n, gv, uv);
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int n = n0 + 64 * wx + 16 * j + r;
-          if (n >= N) continue;
-          const float v = TOT ? tot[TOT ? i : 0][TOT ? j : 0][q] : acc[i][j][q];
-          if (EPI == EPI_ADD_F32 && TOT) ((float*)out)[(size_t)m * ldo + n] = v;     // the residual is in already
-          else epilogue_store<EPI>(out, (size_t)m * ldo + n, v, v);
-        }
-      }
-    }
+      for (int j = 0; j < 4; ++j) acc[i][j] = tot[TOT ? i : 0][TOT ? j : 0];
+  }
+  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (EPI == EPI_SWIGLU_BF16 ? 32 : 64) * wx, (n0 >> 6) + wx, r, g,
+                        TOT, rp);
 }
 
 // The same tiles worked by eight waves (each 64 x 32 outputs), for products whose grid is too
@@ -574,6 +588,172 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// ------------------------------------------------------------------------------ big tiles
+
+// 256 x 256 outputs a workgroup (256 x 128 of SwiGLU: 128 gate and 128 up rows of W), steps of 64
+// along K, eight waves of 128 x 64 outputs each.  A compute unit can keep only so many bytes of
+// loads in flight, so what it computes per byte it loads decides how busy its matrix cores are:
+// this tile computes twice as much per byte as the 128 x 128 one.  Tiles travel from memory straight
+// into LDS (buffer loads with LDS as their destination: no registers, no LDS write instructions).
+// One load instruction of a wave brings 8 rows of a step, 128 bytes each (whole cache lines), into
+// 1 KB of LDS, lane l's 16 bytes to 16 * l.  Which 16 bytes of its row a lane fetches is permuted:
+// slot c' of row r (r counted within its block of 16 rows) holds the row's chunk c' ^ (r >> 1), so
+// that the 16 lanes that read one chunk of 16 different rows as a matrix operand hit 16 different
+// groups of banks.  LDS is a ring of five slots of 32 KB, filled in the order A0 B0 A1 B1 A2 ... (a
+// step's tile of x, then its tile of W): while the waves work on step s, B(s+1) and A(s+2) are in
+// flight and A(s+1) has landed or is landing, so the memory pipe never runs dry at a step's edge;
+// one barrier a step.  Rows past M or N lie outside the buffer descriptors.  K a multiple of 64 and
+// one segment; for products with enough tiles to go round.
+#define BIG_BM 256
+#define BIG_SLOT (32 * 1024)
+#define BIG_SLOTS 5
+#define BIG_WAIT_ALL 0x0f70     // s_waitcnt vmcnt(0) alone
+#define BIG_WAIT_BUT_4 0x0f74   // s_waitcnt vmcnt(4): all but the wave's last four loads have landed
+
+template <int EPI>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_big_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
+  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr int COLS = GLU ? 128 : 256;
+  extern __shared__ __attribute__((aligned(16))) unsigned char big_lds[];   // [5 slots][32 KB]
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int wy = wave >> 2, wx = wave & 3;
+  int bid = blockIdx.x;
+  const int nblocks = m_tiles * n_tiles;
+  if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;      // an n tile's workgroups share an XCD
+  const int m0 = (bid % m_tiles) * BIG_BM;
+  const int n0 = (bid / m_tiles) * COLS;
+
+  // this wave's loads of a stage: rows 32*wave .. 32*wave + 31 of A's 256 and of B's 256, four loads of 8 rows each
+  const int a_rows = min(BIG_BM, M - m0), b_rows = min(COLS, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+  // SwiGLU: B rows 0-127 are gate rows n0.., 128-255 the up rows N + n0..
+  const bool up = GLU && wave >= 4;
+  const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int b_row0 = GLU ? 32 * (wave & 3) : 32 * wave;
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_a[4], voff_b[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int r16 = (8 * t + lrow) & 15;                    // the row within its block of 16
+    const int chunk = lslot ^ (r16 >> 1);
+    voff_a[t] = ((32 * wave + 8 * t + lrow) * ldx + 8 * chunk) * 2;
+    voff_b[t] = ((b_row0 + 8 * t + lrow) * K + 8 * chunk) * 2;
+  }
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  // load number n of the ring: A of step n / 2 (n even) or B of it (n odd), into slot n % 5
+  auto issue_a = [&](int step) {
+    unsigned char* dst = big_lds + ((2 * step) % BIG_SLOTS) * BIG_SLOT + (4 * wave) * 1024;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, voff_a[t], step * 128, 0, 0);
+  };
+  auto issue_b = [&](int step) {
+    unsigned char* dst = big_lds + ((2 * step + 1) % BIG_SLOTS) * BIG_SLOT + (4 * wave) * 1024;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + t * 1024), 16, voff_b[t], step * 128, 0, 0);
+  };
+
+  f32x4 acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  // the wave's operands: A row blocks 8*wy + i; B row blocks 4*wx + j, or in SwiGLU mode gate blocks
+  // 2*wx, 2*wx + 1 (j = 0, 1) and up blocks 8 + 2*wx, 8 + 2*wx + 1 (j = 2, 3).  A block of 16 rows is
+  // 2 KB; lane (g, r) wants row r, chunk 4*kk + g: slot (4*kk + g) ^ (r >> 1) of that row.
+  const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
+  int slot_off[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
+  const int a_frag = (8 * wy) * 2048, b_frag = (GLU ? 2 * wx : 4 * wx) * 2048;
+  auto b_off = [&](int j) { return GLU ? ((j & 1) + 8 * (j >> 1)) * 2048 : j * 2048; };
+
+  const int steps = K / 64;
+  issue_a(0);
+  issue_b(0);
+  if (steps > 1) issue_a(1);
+  for (int step = 0; step < steps; ++step) {
+    // A(step) and B(step) have landed (only A(step + 1), the wave's last four loads, may still be in
+    // flight), for every wave; and every wave is done with the slots of the step before, which the
+    // next loads overwrite
+    if (step + 1 < steps) __builtin_amdgcn_s_waitcnt(BIG_WAIT_BUT_4);
+    else __builtin_amdgcn_s_waitcnt(BIG_WAIT_ALL);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (step + 1 < steps) issue_b(step + 1);
+    if (step + 2 < steps) issue_a(step + 2);
+    const unsigned char* a_slot = big_lds + ((2 * step) % BIG_SLOTS) * BIG_SLOT + a_frag;
+    const unsigned char* b_slot = big_lds + ((2 * step + 1) % BIG_SLOTS) * BIG_SLOT + b_frag;
+    __builtin_amdgcn_sched_barrier(0);
+    // A step is 24 operand reads (per half of the step: 4 of B, 8 of A) and 64 matrix instructions,
+    // written in the order they are needed and then interleaved explicitly: the reads of a pair of A
+    // blocks (and, at the half's end, of the next half's B blocks) are issued while the 8 matrix
+    // instructions of the pair before run, so that no matrix instruction waits for LDS.
+    u32x4 fb[2][4], fa[2][2];
+    auto read_b = [&](int kk) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fb[kk][j] = *reinterpret_cast<const u32x4*>(b_slot + b_off(j) + slot_off[kk]);
+    };
+    auto read_a = [&](int kk, int pair) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        fa[pair & 1][t] = *reinterpret_cast<const u32x4*>(a_slot + (2 * pair + t) * 2048 + slot_off[kk]);
+    };
+    auto multiply = [&](int kk, int pair) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[2 * pair + t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[pair & 1][t]), as_bf16x8(fb[kk][j]),
+                                                                         acc[2 * pair + t][j], 0, 0, 0);
+    };
+    read_b(0);
+    read_a(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int pair = 0; pair < 4; ++pair) {
+        if (pair < 3) read_a(kk, pair + 1);
+        else if (kk == 0) {
+          read_b(1);
+          read_a(1, 0);
+        }
+        multiply(kk, pair);
+      }
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int pair = 0; pair < 3; ++pair) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      }
+      if (kk == 0) {
+#pragma unroll
+        for (int t = 0; t < 6; ++t) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+  }
+  tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
+}
+
 // ------------------------------------------------------------------------------ launch
 
 template <int EPI>
@@ -612,6 +792,22 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     }
 #undef BW_SKINNY
   } else {
+    if constexpr (EPI != EPI_ADD_F32) {
+      // enough 256-row tiles to go round the compute units (a second round at least half full)
+      constexpr int BIG_COLS = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+      const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + BIG_COLS - 1) / BIG_COLS;
+      if (S == 1 && K % 64 == 0 && M >= 2 * BIG_BM && bm * bn >= 128) {
+        static bool allowed = false;                 // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    BIG_SLOTS * BIG_SLOT);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI>), dim3(bm * bn), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w, out, M, N, K, ldx,
+                           ldo, bm, bn, rp);
+        return BW_LAUNCH_CHECK();
+      }
+    }
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);

@@ -115,6 +115,28 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             ops.gemm_bf16(x[:, k0:k0 + 2048].contiguous(), w[:, k0:k0 + 2048].contiguous(), part, M, ops.EPI_F32)
             want = want + part
         assert torch.equal(acc, want), (M, N, K)
+    # enough 256 x 256 tiles for the big-tile kernel: the bits of the same rows in slices that other kernels take
+    M, N, K = 2100, 3700, 192
+    x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+    w = torch.randn(N, K, generator=g).bfloat16().to(gpu)
+    y = torch.full((M, N), 3.0, device=gpu)
+    ops.gemm_bf16(x, w, y, M, ops.EPI_F32)
+    ref = x.double() @ w.double().T
+    assert (y.double() - ref).abs().max() <= 2e-6 * K ** 0.5 * ref.abs().max()
+    for lo, n in ((0, 300), (1800, 300), (2047, 53), (2099, 1)):
+        part = torch.zeros(n, N, device=gpu)
+        ops.gemm_bf16(x[lo:lo + n].contiguous(), w, part, n, ops.EPI_F32)
+        assert torch.equal(part, y[lo:lo + n]), (lo, n)
+    yb = torch.zeros(M, N, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_bf16(x, w, yb, M, ops.EPI_BF16)
+    assert torch.equal(yb, y.bfloat16())
+    inter = N // 2
+    hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_bf16(x, w, hb, M, ops.EPI_SWIGLU_BF16)
+    for lo, n in ((0, 300), (1900, 200), (2090, 10)):
+        part = torch.zeros(n, inter, device=gpu, dtype=torch.bfloat16)
+        ops.gemm_bf16(x[lo:lo + n].contiguous(), w, part, n, ops.EPI_SWIGLU_BF16)
+        assert torch.equal(part, hb[lo:lo + n]), (lo, n)
     M, inter, K = 19, 56, 96
     x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
@@ -486,9 +508,11 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
     epilogue; q, the key pages and the value pages must be the bits of product + rope_kvwrite.
     Rows of two requests, a padding row, positions across page edges, a ragged last tile."""
     g = torch.Generator().manual_seed(21)
-    for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32)]:
-        hd, pages = 64, 40
-        cos, sin = rope_tables(10000.0, hd, 400, gpu)
+    for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
+                                   (40, 10, 128, 2100, 32)]:       # the last: enough 256 x 256 tiles for the big-tile kernel
+        hd = 64
+        pages = 40 if M < 500 else 3 * ((M + page - 1) // page + 2) + 3
+        cos, sin = rope_tables(10000.0, hd, max(400, M), gpu)
         h = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = (torch.randn((heads + 2 * kvh) * hd, K, generator=g) * 0.05).bfloat16().to(gpu)
         pos = [(r if r < M // 2 else r - M // 2 + 3) for r in range(M)]
