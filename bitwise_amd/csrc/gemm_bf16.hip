@@ -754,6 +754,109 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
 }
 
+// ------------------------------------------------------------------------------ 17 to 64 rows
+
+// All rows (up to 64) x 64 columns a workgroup (32 of SwiGLU: 32 gate and 32 up rows of W), steps of
+// 64 along K, four waves.  With more than 16 rows a wave of the skinny kernel spends most of its
+// loads on x, again for every strip; here the rows of x come into LDS once per workgroup and serve
+// four strips.  Loads and LDS layout are those of the big-tile kernel (buffer loads into LDS, 8 rows
+// of 128 bytes an instruction, chunks permuted against bank conflicts); the ring has eight stages of
+// 16 KB, so up to seven steps of weights are in flight while one is worked on.  A wave issues four
+// loads a stage, in order, so "all but the last 24 have landed" is the wait for the stage at hand;
+// stages past K are asked for outside the descriptors (zeros, no memory traffic) to keep that count
+// fixed.  One barrier a step: behind it every wave has the stage at hand and is done with the one before.
+// Plain epilogues: wave w owns strip w, all four blocks of 16 rows.  SwiGLU: wave (s, h) owns gate and
+// up strip s for the row blocks 2h, 2h + 1.  K a multiple of 64, one segment.
+#define MID_STAGE (16 * 1024)
+#define MID_STAGES 8
+#define MID_WAIT 0x4f78         // s_waitcnt vmcnt(24): 4 * (MID_STAGES - 2)
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                            void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr int COLS = GLU ? 32 : 64;
+  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][A 8 KB | B 8 KB]
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * COLS;
+  const int b_rows = min(COLS, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
+  // SwiGLU: B rows 0-31 are gate rows n0.., 32-63 the up rows N + n0..; waves 0, 1 load the first, 2, 3 the others
+  const bool up = GLU && wave >= 2;
+  const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int b_row0 = GLU ? 16 * (wave & 1) : 16 * wave;
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_a[2], voff_b[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int r16 = 8 * t + lrow;                               // the row within its block of 16
+    const int chunk = lslot ^ (r16 >> 1);
+    voff_a[t] = ((16 * wave + r16) * ldx + 8 * chunk) * 2;
+    voff_b[t] = ((b_row0 + r16) * K + 8 * chunk) * 2;
+  }
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const int steps = K / 64;
+  auto issue = [&](int step) {
+    unsigned char* dst = mid_lds + (step % MID_STAGES) * MID_STAGE + (2 * wave) * 1024;
+    const bool real = step < steps;                              // scalar
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 8 * 1024 + t * 1024), 16, real ? voff_b[t] : 0x7ffffff0,
+                                               step * 128, 0, 0);
+    }
+  };
+  constexpr int NI = GLU ? 2 : 4, NJ = GLU ? 2 : 1;
+  f32x4 acc[NI][NJ];
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  // lane (g, r) wants row r of a block of 16 rows (2 KB), chunk 4*kk + g: slot (4*kk + g) ^ (r >> 1) of that row
+  const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
+  int slot_off[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
+  const int a_block0 = GLU ? 2 * (wave >> 1) : 0;                // first block of 16 rows this wave works on
+  const int b_off0 = 8 * 1024 + (GLU ? (wave & 1) : wave) * 2048;   // its (gate) strip; the up strip lies 4 KB further
+
+#pragma unroll
+  for (int st = 0; st < MID_STAGES - 1; ++st) issue(st);
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(MID_WAIT);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    issue(step + MID_STAGES - 1);                                 // into the stage worked on a step ago
+    const unsigned char* stage = mid_lds + (step % MID_STAGES) * MID_STAGE;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      u32x4 fa[NI], fb[NJ];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) fa[i] = *reinterpret_cast<const u32x4*>(stage + (a_block0 + i) * 2048 + slot_off[kk]);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(stage + b_off0 + j * 4096 + slot_off[kk]);
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
+    }
+    asm volatile("" ::: "memory");
+  }
+  const int n = n0 + 16 * (GLU ? (wave & 1) : wave) + r;
+  if (n >= N) return;
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = 16 * (a_block0 + i) + 4 * g + q;
+      if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
+    }
+}
+
 // ------------------------------------------------------------------------------ launch
 
 template <int EPI>
@@ -763,6 +866,22 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
   constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
   if (M <= 64) {
     if constexpr (EPI == EPI_QKV_ROPE) return -2;       // the rotary epilogue belongs to the wide kernel
+    else {
+      // more than 16 rows, one segment, enough columns: the rows of x are shared through LDS
+      constexpr int MID_COLS = (EPI == EPI_SWIGLU_BF16) ? 32 : 64;
+      const int wgs = (N + MID_COLS - 1) / MID_COLS;
+      if (M > 16 && S == 1 && K % 64 == 0 && wgs >= 64 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) &&
+          (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        static bool allowed = false;                     // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    MID_STAGES * MID_STAGE);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI>), dim3(wgs), dim3(256), MID_STAGES * MID_STAGE, s, x, w, out, M, N, K, ldx, ldo);
+        return BW_LAUNCH_CHECK();
+      }
+    }
     const int row_blocks = (M + 15) / 16, strips = (N + 15) / 16;
     // Few columns and more than 16 rows: a workgroup per block of 16 rows (the strips of W are then
     // fetched once per block of rows, from cache after the first, by four times the waves).  Many
