@@ -112,7 +112,9 @@ def build(force: bool = False, verbose: bool = True) -> Path:
     with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     tmp_lib = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
-    p = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp_lib), *objs],
+    # -z defs: a kernel template that the host pass failed to instantiate (it can do so without a
+    # word) leaves an undefined symbol; better the link fails here than the load on the GPU box
+    p = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-z,defs", "-o", str(tmp_lib), *objs],
                        capture_output=True, text=True, env=env)
     if p.returncode != 0:
         raise KernelLibraryError(f"linking the kernel library failed:\n{p.stderr[-4000:]}")

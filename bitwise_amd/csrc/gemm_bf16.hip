@@ -754,62 +754,91 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
 }
 
-// ------------------------------------------------------------------------------ 17 to 64 rows
+// ------------------------------------------------------------------------------ up to 64 rows, through LDS
 
-// All rows (up to 64) x 64 columns a workgroup (32 of SwiGLU: 32 gate and 32 up rows of W), steps of
-// 64 along K, four waves.  With more than 16 rows a wave of the skinny kernel spends most of its
-// loads on x, again for every strip; here the rows of x come into LDS once per workgroup and serve
-// four strips.  Loads and LDS layout are those of the big-tile kernel (buffer loads into LDS, 8 rows
-// of 128 bytes an instruction, chunks permuted against bank conflicts); the ring has eight stages of
-// 16 KB, so up to seven steps of weights are in flight while one is worked on.  A wave issues four
-// loads a stage, in order, so "all but the last 24 have landed" is the wait for the stage at hand;
-// stages past K are asked for outside the descriptors (zeros, no memory traffic) to keep that count
-// fixed.  One barrier a step: behind it every wave has the stage at hand and is done with the one before.
-// Plain epilogues: wave w owns strip w, all four blocks of 16 rows.  SwiGLU: wave (s, h) owns gate and
-// up strip s for the row blocks 2h, 2h + 1.  K a multiple of 64, one segment.
-#define MID_STAGE (16 * 1024)
+// All rows (NRB blocks of 16: up to 16, 32 or 64 rows) x 64 columns a workgroup (32 of SwiGLU: 32 gate
+// and 32 up rows of W), steps of 64 along K.  The rows of x come into LDS once per workgroup and serve
+// all its strips; weights and x travel as in the big-tile kernel (buffer loads with LDS as destination,
+// 8 rows of 128 bytes an instruction, whole cache lines; chunks permuted against bank conflicts), and
+// since no registers hold them the ring can be deep: eight stages, so up to seven steps of weights are
+// in flight while one is worked on.  Every wave issues the same number of loads a stage (LPW: its share
+// of the weights and of x, padded with loads from outside the descriptors, which cost no memory
+// traffic), in order, so "all but the last 6 * LPW have landed" is the wait for the stage at hand;
+// stages past K are asked for outside the descriptors too, to keep that count fixed.  One barrier a
+// step: behind it every wave has the stage at hand and is done with the one before.
+// Plain epilogues: four waves, wave w owns strip w and all blocks of rows.  SwiGLU: wave (s, h) owns
+// gate and up strip s for half h of the row blocks; with one block of rows there are two waves.
+// K a multiple of 64, one segment.
 #define MID_STAGES 8
-#define MID_WAIT 0x4f78         // s_waitcnt vmcnt(24): 4 * (MID_STAGES - 2)
 
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                            void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
-  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
-  constexpr int COLS = GLU ? 32 : 64;
-  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][A 8 KB | B 8 KB]
+template <int EPI, int NRB>
+struct MidShape {
+  static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  static constexpr int NW = (GLU && NRB == 1) ? 2 : 4;               // waves
+  static constexpr int A_LOADS = (2 * NRB + NW - 1) / NW;           // per wave and stage: 8 rows of x each
+  static constexpr int B_LOADS = 8 / NW;                            // 8 rows of W each
+  static constexpr int LPW = A_LOADS + B_LOADS;
+  static constexpr int A_BYTES = NRB * 2048, STAGE = A_BYTES + 8 * 1024;
+  static constexpr int NI = GLU ? (NRB >= 2 ? NRB / 2 : 1) : NRB;    // blocks of rows a wave works on
+  static constexpr int NJ = GLU ? 2 : 1;
+  static constexpr int PENDING = LPW * (MID_STAGES - 2);            // loads that may still be in flight at a step's start
+  static_assert(PENDING < 64, "the wait count has six bits");
+};
+
+// A wave's loads of one stage of the ring: its share of the rows of x and of W, LPW instructions.
+template <int EPI, int NRB>
+__device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
+                                          const int (&voff_a)[MidShape<EPI, NRB>::A_LOADS],
+                                          const int (&voff_b)[MidShape<EPI, NRB>::B_LOADS], int wave, int step, int steps) {
+  using S = MidShape<EPI, NRB>;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = lds + (step % MID_STAGES) * S::STAGE;
+  const bool real = step < steps;                                     // scalar
+#pragma unroll
+  for (int t = 0; t < S::A_LOADS; ++t) {
+    const int block = wave * S::A_LOADS + t;                          // 1 KB of the stage's x; a padding load's zeros go behind the ring
+    unsigned char* to = block < 2 * NRB ? dst + block * 1024 : lds + MID_STAGES * S::STAGE;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)to, 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
+  }
+#pragma unroll
+  for (int t = 0; t < S::B_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + S::A_BYTES + (wave * S::B_LOADS + t) * 1024), 16,
+                                             real ? voff_b[t] : 0x7ffffff0, step * 128, 0, 0);
+}
+
+template <int EPI, int NRB>
+__global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+  using S = MidShape<EPI, NRB>;
+  constexpr bool GLU = S::GLU;
+  constexpr int COLS = GLU ? 32 : 64, NI = S::NI, NJ = S::NJ;
+  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * COLS;
   const int b_rows = min(COLS, N - n0);
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
-  // SwiGLU: B rows 0-31 are gate rows n0.., 32-63 the up rows N + n0..; waves 0, 1 load the first, 2, 3 the others
-  const bool up = GLU && wave >= 2;
+  // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
+  const int lrow = lane >> 3, lslot = lane & 7;
+  const int b_first = wave * S::B_LOADS * 8;                         // this wave's first row of the tile's 64 of W
+  const bool up = GLU && b_first >= 32;
   const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
-  const int b_row0 = GLU ? 16 * (wave & 1) : 16 * wave;
-  const int lrow = lane >> 3, lslot = lane & 7;
-  int voff_a[2], voff_b[2];
+  int voff_a[S::A_LOADS], voff_b[S::B_LOADS];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int r16 = 8 * t + lrow;                               // the row within its block of 16
-    const int chunk = lslot ^ (r16 >> 1);
-    voff_a[t] = ((16 * wave + r16) * ldx + 8 * chunk) * 2;
-    voff_b[t] = ((b_row0 + r16) * K + 8 * chunk) * 2;
+  for (int t = 0; t < S::A_LOADS; ++t) {
+    const int row = (wave * S::A_LOADS + t) * 8 + lrow;             // of the NRB * 16 rows of x; past them: a padding load
+    const int chunk = lslot ^ ((row & 15) >> 1);
+    voff_a[t] = row < NRB * 16 ? (row * ldx + 8 * chunk) * 2 : 0x7ffffff0;
   }
-  typedef __attribute__((address_space(3))) void* lds_ptr;
-  const int steps = K / 64;
-  auto issue = [&](int step) {
-    unsigned char* dst = mid_lds + (step % MID_STAGES) * MID_STAGE + (2 * wave) * 1024;
-    const bool real = step < steps;                              // scalar
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 8 * 1024 + t * 1024), 16, real ? voff_b[t] : 0x7ffffff0,
-                                               step * 128, 0, 0);
-    }
-  };
-  constexpr int NI = GLU ? 2 : 4, NJ = GLU ? 2 : 1;
+  for (int t = 0; t < S::B_LOADS; ++t) {
+    const int row = b_first + 8 * t + lrow;
+    const int chunk = lslot ^ ((row & 15) >> 1);
+    voff_b[t] = (((GLU ? row & 31 : row)) * K + 8 * chunk) * 2;
+  }
+  const int steps = K / 64;
   f32x4 acc[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -820,17 +849,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(const bf16_t* __rest
   int slot_off[2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
-  const int a_block0 = GLU ? 2 * (wave >> 1) : 0;                // first block of 16 rows this wave works on
-  const int b_off0 = 8 * 1024 + (GLU ? (wave & 1) : wave) * 2048;   // its (gate) strip; the up strip lies 4 KB further
+  const int strip = GLU ? (wave & 1) : wave;                          // of the tile's output columns
+  const int a_block0 = GLU ? NI * (wave >> 1) : 0;                    // first block of 16 rows this wave works on
+  const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
 
 #pragma unroll
-  for (int st = 0; st < MID_STAGES - 1; ++st) issue(st);
+  for (int st = 0; st < MID_STAGES - 1; ++st) mid_issue<EPI, NRB>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
   for (int step = 0; step < steps; ++step) {
-    __builtin_amdgcn_s_waitcnt(MID_WAIT);
+    // s_waitcnt vmcnt(PENDING) alone; the instruction wants a literal
+    static_assert(S::PENDING == 18 || S::PENDING == 24 || S::PENDING == 30, "a wait for this count is not written out");
+    if constexpr (S::PENDING == 18) __builtin_amdgcn_s_waitcnt(0x4f72);
+    else if constexpr (S::PENDING == 24) __builtin_amdgcn_s_waitcnt(0x4f78);
+    else __builtin_amdgcn_s_waitcnt(0x4f7e);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    issue(step + MID_STAGES - 1);                                 // into the stage worked on a step ago
-    const unsigned char* stage = mid_lds + (step % MID_STAGES) * MID_STAGE;
+    mid_issue<EPI, NRB>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + MID_STAGES - 1, steps);   // into the stage worked on a step ago
+    const unsigned char* stage = mid_lds + (step % MID_STAGES) * S::STAGE;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       u32x4 fa[NI], fb[NJ];
@@ -846,7 +880,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(const bf16_t* __rest
     }
     asm volatile("" ::: "memory");
   }
-  const int n = n0 + 16 * (GLU ? (wave & 1) : wave) + r;
+  const int n = n0 + 16 * strip + r;
   if (n >= N) return;
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -855,6 +889,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(const bf16_t* __rest
       const int m = 16 * (a_block0 + i) + 4 * g + q;
       if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
     }
+}
+
+template <int EPI, int NRB>
+static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s) {
+  using S = MidShape<EPI, NRB>;
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  constexpr int lds_bytes = MID_STAGES * S::STAGE + 1024;
+  if (!allowed && lds_bytes > 64 * 1024) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo);
+  return BW_LAUNCH_CHECK();
 }
 
 // ------------------------------------------------------------------------------ launch
@@ -867,19 +914,14 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
   if (M <= 64) {
     if constexpr (EPI == EPI_QKV_ROPE) return -2;       // the rotary epilogue belongs to the wide kernel
     else {
-      // more than 16 rows, one segment, enough columns: the rows of x are shared through LDS
+      // one segment and enough columns: the rows of x are shared through LDS
       constexpr int MID_COLS = (EPI == EPI_SWIGLU_BF16) ? 32 : 64;
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
-      if (M > 16 && S == 1 && K % 64 == 0 && wgs >= 64 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) &&
+      if (S == 1 && K % 64 == 0 && wgs >= 64 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) &&
           (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
-        static bool allowed = false;                     // more than 64 KB of dynamic LDS has to be asked for once
-        if (!allowed) {
-          (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    MID_STAGES * MID_STAGE);
-          allowed = true;
-        }
-        hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI>), dim3(wgs), dim3(256), MID_STAGES * MID_STAGE, s, x, w, out, M, N, K, ldx, ldo);
-        return BW_LAUNCH_CHECK();
+        if (M <= 16) return launch_mid<EPI, 1>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+        if (M <= 32) return launch_mid<EPI, 2>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+        return launch_mid<EPI, 4>(x, w, out, M, N, K, ldx, ldo, wgs, s);
       }
     }
     const int row_blocks = (M + 15) / 16, strips = (N + 15) / 16;

@@ -89,7 +89,7 @@ def test_gemm_f32_grid_rows_and_accumulate(gpu):
 def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     g = torch.Generator().manual_seed(3)
     for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
-                    (40, 4100, 192), (64, 4200, 2048), (17, 4096, 64),   # 17 to 64 rows, many columns: x shared through LDS
+                    (40, 4100, 192), (64, 4200, 2048), (17, 4096, 64), (9, 4100, 128), (16, 5000, 64), (30, 4096, 320),   # many columns: x shared through LDS
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
                     (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
@@ -138,16 +138,20 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
         part = torch.zeros(n, inter, device=gpu, dtype=torch.bfloat16)
         ops.gemm_bf16(x[lo:lo + n].contiguous(), w, part, n, ops.EPI_SWIGLU_BF16)
         assert torch.equal(part, hb[lo:lo + n]), (lo, n)
-    # SwiGLU of 17 to 64 rows and many columns (x shared through LDS): the bits of the rows one by one
-    M, inter, K = 41, 2100, 128
-    x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+    # SwiGLU with many columns (x shared through LDS; one, two or four blocks of 16 rows): the plain result, and
+    # the bits of the same rows inside a prompt portion's product (another kernel)
+    inter, K = 2100, 128
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
-    hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
-    ops.gemm_bf16(x, wgu, hb, M, ops.EPI_SWIGLU_BF16)
-    one = torch.zeros(1, inter, device=gpu, dtype=torch.bfloat16)
-    for r in (0, 15, 16, 40):
-        ops.gemm_bf16(x[r:r + 1].contiguous(), wgu, one, 1, ops.EPI_SWIGLU_BF16)
-        assert torch.equal(one[0], hb[r]), r
+    xl = torch.randn(200, K, generator=g).bfloat16().to(gpu)
+    big = torch.zeros(200, inter, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_bf16(xl, wgu, big, 200, ops.EPI_SWIGLU_BF16)
+    gate, up = xl.double() @ wgu[:inter].double().T, xl.double() @ wgu[inter:].double().T
+    want = pl.swiglu(gate.cpu(), up.cpu())
+    assert (big.cpu().double() - want).abs().max() <= 2 ** -8 * want.abs().max()
+    for M in (1, 13, 16, 29, 41, 64):
+        hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
+        ops.gemm_bf16(xl[100:100 + M].contiguous(), wgu, hb, M, ops.EPI_SWIGLU_BF16)
+        assert torch.equal(hb, big[100:100 + M]), M
     M, inter, K = 19, 56, 96
     x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
