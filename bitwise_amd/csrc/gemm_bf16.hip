@@ -904,6 +904,143 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N,
   return BW_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------------------ up to 16 rows, few columns
+
+// The skinny kernel's division of work (a wave per strip of CW columns and segment of K; the waves of
+// a strip join their segment sums through LDS in segment order) with the loads of the kernel above:
+// every wave owns a ring of STREAM_STAGES stages in LDS, a stage being a step's 64 elements of its CW
+// rows of W and of the 16 rows of x, fetched by buffer loads with LDS as destination in whole cache
+// lines; LPW loads a stage, so "all but the last LPW * (stages - 2)" is the wait for the stage at
+// hand.  Nothing is shared between waves, so the loop has no barrier.  K a multiple of 64.
+template <int CW>
+struct StreamShape {
+  static constexpr int B_LOADS = CW / 8, LPW = 2 + B_LOADS;
+  static constexpr int STAGE = 2048 + B_LOADS * 1024;               // x: 16 rows of 128 bytes, then W
+  static constexpr int STAGES = CW == 8 ? 10 : 8;
+  static constexpr int RING = STAGES * STAGE;
+  static_assert(LPW * (STAGES - 2) == 24, "the wait below is written for 24 loads in flight");
+};
+
+// A wave's loads of one stage of its ring (a device function rather than a lambda in the kernel: the
+// host pass drops, without a word, kernel templates whose lambdas capture arrays of dependent size).
+template <int CW>
+__device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
+                                             const int* voff_x, const int* voff_w, int step, int steps, int k_begin) {
+  using SH = StreamShape<CW>;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = ring + (step % SH::STAGES) * SH::STAGE;
+  const bool real = step < steps;                                  // scalar; past the segment: outside the descriptors
+  const int soff = (k_begin + step * 64) * 2;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, soff, 0, 0);
+#pragma unroll
+  for (int t = 0; t < SH::B_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + 2048 + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0, soff, 0, 0);
+}
+
+template <int EPI, int CW>
+__global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                               void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                               int S) {
+  using SH = StreamShape<CW>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];   // [waves][ring], then [S][4][64] floats when S > 1
+  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int c = r % CW;
+  const int n0 = blockIdx.x * CW;
+  const bool n_ok = r < CW && n0 + c < N;
+  const int w_rows = min(CW, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)w_rows * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x =
+      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
+  // loads: lane l fetches row l / 8 of its 8, chunk (l % 8) ^ (row within 16 >> 1) of the row's 128 bytes
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_x[2], voff_w[SH::B_LOADS];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) voff_x[t] = ((8 * t + lrow) * ldx + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
+#pragma unroll
+  for (int t = 0; t < SH::B_LOADS; ++t) voff_w[t] = ((8 * t + lrow) * K + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
+  // operand reads: lane (g, r) wants row r (of W: r % CW), chunk 4*kk + g: slot (4*kk + g) ^ (row >> 1)
+  int off_x[2], off_w[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    off_x[kk] = (r >> 3) * 1024 + (r & 7) * 128 + (((4 * kk + g) ^ (r >> 1)) * 16);
+    off_w[kk] = 2048 + (c >> 3) * 1024 + (c & 7) * 128 + (((4 * kk + g) ^ (c >> 1)) * 16);
+  }
+  unsigned char* ring = stream_lds + wave * SH::RING;
+  float* red = reinterpret_cast<float*>(stream_lds + nwaves * SH::RING);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = wave; s < S; s += nwaves) {
+    const int k_begin = s * GEMM_SEG;
+    const int steps = ((K - k_begin) < GEMM_SEG ? K - k_begin : GEMM_SEG) / 64;
+    acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+    for (int step = 0; step < steps; ++step) {
+      __builtin_amdgcn_s_waitcnt(0x4f78);                          // vmcnt(24): the stage at hand has landed
+      asm volatile("" ::: "memory");
+      const unsigned char* stage = ring + (step % SH::STAGES) * SH::STAGE;
+      u32x4 fa[2], fb[2];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        fa[kk] = *reinterpret_cast<const u32x4*>(stage + off_x[kk]);
+        fb[kk] = *reinterpret_cast<const u32x4*>(stage + off_w[kk]);
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk]), acc, 0, 0, 0);
+      // the reads above are done (their values were used) before the stage is asked for again
+      asm volatile("" ::: "memory");
+      stream_issue<CW>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);                            // the padding loads too, before the ring is reused
+    if (S > 1) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) red[(s * 4 + q) * 64 + lane] = acc[q];
+    }
+  }
+  if (S > 1) {
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float y = red[q * 64 + lane];
+      if constexpr (EPI == EPI_ADD_F32) {            // the chain of additions starts at the residual
+        const int m = 4 * g + q;
+        if (n_ok && m < M) y = ((const float*)out)[(size_t)m * ldo + n0 + c] + y;
+      }
+      for (int s = 1; s < S; ++s) y += red[(s * 4 + q) * 64 + lane];
+      acc[q] = y;
+    }
+  }
+  if (!n_ok) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int m = 4 * g + q;
+    if (m >= M) continue;
+    if (EPI == EPI_ADD_F32 && S > 1) ((float*)out)[(size_t)m * ldo + n0 + c] = acc[q];   // the residual is in already
+    else epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+  }
+}
+
+template <int EPI, int CW>
+static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
+  using SH = StreamShape<CW>;
+  const int waves = S < 4 ? S : 4;
+  const size_t lds_bytes = (size_t)waves * SH::RING + (S > 1 ? (size_t)S * 4 * 64 * sizeof(float) : 0);
+  if (lds_bytes > 160 * 1024) return -2;
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<EPI, CW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_bf16_stream_kernel<EPI, CW>), dim3((N + CW - 1) / CW), dim3(64 * waves), lds_bytes, s, x, w, out, M, N,
+                     K, ldx, ldo, S);
+  return BW_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------------------ launch
 
 template <int EPI>
@@ -922,6 +1059,13 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         if (M <= 16) return launch_mid<EPI, 1>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         if (M <= 32) return launch_mid<EPI, 2>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         return launch_mid<EPI, 4>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+      }
+    }
+    if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {
+      // up to 16 rows: a wave per strip and segment, streaming through its own ring in LDS
+      if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        if ((N + 15) / 16 < 256) return launch_stream<EPI, 8>(x, w, out, M, N, K, ldx, ldo, S, s);
+        return launch_stream<EPI, 16>(x, w, out, M, N, K, ldx, ldo, S, s);
       }
     }
     const int row_blocks = (M + 15) / 16, strips = (N + 15) / 16;

@@ -90,6 +90,7 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     g = torch.Generator().manual_seed(3)
     for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
                     (40, 4100, 192), (64, 4200, 2048), (17, 4096, 64), (9, 4100, 128), (16, 5000, 64), (30, 4096, 320),   # many columns: x shared through LDS
+                    (7, 200, 4160), (16, 5000, 4096), (3, 40, 128), (12, 4104, 6144),   # up to 16 rows streaming through LDS, several segments
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
                     (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
