@@ -15,12 +15,16 @@
 //     q goes to its buffer and k, v to their page slots (v transposed).
 //
 // Shape: a workgroup is a few strips of 16 output columns, one wave each (for q|k|v with
-// rotary: the strips of one head, or one strip and its rotary partner).  Loads go out in the
-// order their results are needed, because memory results are waited for in issue order: the
-// rows to normalise and the positions first, then D steps of the wave's weights, which stay in
-// flight while the rows are normalised into LDS (rows padded by 16 bytes so that operand reads
-// hit distinct banks).  Then each wave runs its chain with A operands from LDS and B operands
-// from its ring of registers.
+// rotary: the strips of one head, or one strip and its rotary partner).  A wave's weights stream
+// through a ring of its own in LDS: buffer loads with LDS as destination, 8 rows of 128 bytes an
+// instruction (whole cache lines), the 16-byte chunks of a row permuted so that operand reads hit
+// distinct banks; no registers hold weights, so the ring is deep.  Loads complete in the order
+// they are issued and the wait for a stage counts the loads issued after it, so everything else
+// the kernel reads from memory is asked for before the ring: positions and what the rotary
+// epilogue needs first (a short wait at the kernel's start), then the rows to normalise, then the
+// ring's first stages, which are in flight while the rows are normalised into LDS (rows padded by
+// 16 bytes so that operand reads hit distinct banks).  Then each wave runs its chain with both
+// operands from LDS.  K a multiple of 64.
 #include "common.h"
 #include "api.h"
 
@@ -47,14 +51,43 @@ struct DecodeGemmArgs {
   int pairs;               // rotary: 16-wide pairs of strips a head is cut into (0: a workgroup is a whole head)
 };
 
-template <int EPI, int D>
+// s_waitcnt vmcnt(n) alone
+constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
+// ST: stages of a wave's ring
+template <int EPI, int ST>
+struct DecodeShape {
+  static constexpr int NB = (EPI == DEPI_SWIGLU_BF16) ? 2 : 1;
+  static constexpr int STAGES = ST;
+  static constexpr int STAGE = NB * 2048;                                      // 16 rows of W, 128 bytes each, NB times
+  static constexpr int LPW = 2 * NB;                                           // loads a stage
+  static_assert(LPW * (STAGES - 2) < 64, "the wait count has six bits");
+};
+
+// A wave's loads of one stage of its ring (step past the end: outside the descriptors, zeros, no traffic).
+template <int EPI, int ST>
+__device__ __forceinline__ void decode_issue(unsigned char* ring, const __amdgpu_buffer_rsrc_t* rs_w, const int* voff_w,
+                                             int step, int steps) {
+  using SH = DecodeShape<EPI, ST>;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = ring + (step % SH::STAGES) * SH::STAGE;
+  const bool real = step < steps;                 // scalar
+#pragma unroll
+  for (int b = 0; b < SH::NB; ++b)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w[b], (lds_ptr)(dst + b * 2048 + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0,
+                                               step * 128, 0, 0);
+}
+
+template <int EPI, int ST>
 __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
-  constexpr int NB = (EPI == DEPI_SWIGLU_BF16) ? 2 : 1;
-  constexpr bool FULL = D * 32 >= DEC_SEG;        // the ring holds a whole segment: nothing is refilled
+  using SH = DecodeShape<EPI, ST>;
+  constexpr int NB = SH::NB;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int K = a.K, M = a.M;
   const int lds_row = K + 8;                      // bf16 elements; +16 bytes keeps operand reads conflict-free
-  bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row]
+  bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row], then the waves' rings
   const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   // rotary: a workgroup is a head (its strips in order), or, when half a head is a multiple of
@@ -74,7 +107,6 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     }
   }
   const bool n_ok = n0 + r < a.N;
-  const int k_begin = 0, k_end = K;
   // weights through buffer descriptors that cover the strip's rows (rows past N read as zeros):
   // one per-lane offset for the whole kernel, the step's offset in a scalar register
   const int w_rows = min(16, a.N - n0);
@@ -83,11 +115,37 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   for (int b = 0; b < NB; ++b)
     rs_w[b] = __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + ((size_t)b * a.N + n0) * K), 0,
                                                 (int)((size_t)(w_rows > 0 ? w_rows : 0) * K * 2), 0x00020000);
-  const int voff_w = (r * K + 8 * g) * 2;
+  // loads: lane l fetches row l / 8 of its 8, chunk (l % 8) ^ (row within 16 >> 1) of the row's 128 bytes
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_w[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) voff_w[t] = ((8 * t + lrow) * K + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
+  const int steps = K / 64;
+  unsigned char* ring = smem + (((size_t)M * lds_row * sizeof(bf16_t) + 15) & ~(size_t)15) + (size_t)wave * SH::STAGES * SH::STAGE;
 
-  // 1. Loads go out in the order in which their results are needed, because results are waited
-  // for in issue order: first the rows to normalise (their first batch) and the positions, then
-  // the weights, which stay in flight while the rows are normalised.
+  // 1. Everything but weights is asked for before the ring (see the head of the file).  The rotary
+  // epilogue's items first: what this thread's (row, pair) items need (at most 2 items a thread).
+  int r_pos[2] = {-1, -1}, r_page[2] = {0, 0};
+  float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
+  if constexpr (EPI == DEPI_ROPE_KV) {
+    const int half = a.head_dim >> 1, lh = rope_lw >> 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * blockDim.x;
+      if (e < M * lh) {
+        const int pos = a.positions[e / lh];
+        r_pos[j] = pos;
+        if (pos >= 0) {
+          const int i = rope_base + e % lh;
+          r_cos[j] = a.cos_table[(size_t)pos * half + i];
+          r_sin[j] = a.sin_table[(size_t)pos * half + i];
+          r_page[j] = a.block_table[(size_t)a.row_seq[e / lh] * a.table_stride + pos / a.page_size];
+        }
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // then the rows to normalise (their first batch)
   constexpr int RB = 4;                            // rows a wave normalises at a time
   const int nvec = K >> 2;
   NormRows<RB> nr;
@@ -98,47 +156,11 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
   }
   if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
-  int r_pos[2] = {-1, -1}, r_seq[2] = {0, 0};
-  if constexpr (EPI == DEPI_ROPE_KV) {
-    const int lh = rope_lw >> 1;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int e = threadIdx.x + j * blockDim.x;
-      if (e < M * lh) {
-        r_pos[j] = a.positions[e / lh];
-        r_seq[j] = a.row_seq[e / lh];
-      }
-    }
-  }
   __builtin_amdgcn_sched_barrier(0);
-  u32x4 bq[D][NB];
-  auto issue = [&](int d, int k) {
-    const int ks = k < k_end ? k : k_begin;       // past the end: re-read the first step, never used
+  // then the ring's first stages, which stay in flight while the rows are normalised
 #pragma unroll
-    for (int b = 0; b < NB; ++b) bq[d][b] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[b], voff_w, ks * 2, 0);
-  };
-#pragma unroll
-  for (int d = 0; d < D; ++d) issue(d, k_begin + 32 * d);
+  for (int st = 0; st < SH::STAGES - 1; ++st) decode_issue<EPI, ST>(ring, rs_w, voff_w, st, steps);
   __builtin_amdgcn_sched_barrier(0);
-
-  // rotary epilogue: what this thread's (row, pair) items need is asked for now and used after the
-  // product (at most 2 items a thread)
-  int r_page[2] = {0, 0};
-  float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
-  if constexpr (EPI == DEPI_ROPE_KV) {
-    const int half = a.head_dim >> 1, lh = rope_lw >> 1;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int e = threadIdx.x + j * blockDim.x;
-      const int pos = r_pos[j];
-      if (e < M * lh && pos >= 0) {
-        const int i = rope_base + e % lh;
-        r_cos[j] = a.cos_table[(size_t)pos * half + i];
-        r_sin[j] = a.sin_table[(size_t)pos * half + i];
-        r_page[j] = a.block_table[(size_t)r_seq[j] * a.table_stride + pos / a.page_size];
-      }
-    }
-  }
 
   // 2. the M rows into LDS as bfloat16, normalised
   for (int m0 = wave; m0 < M;) {
@@ -156,36 +178,36 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   }
   __syncthreads();
 
-  // 3. the product: A from LDS (rows past M read row 0; their results are thrown away), B from the ring
+  // 3. the product: A from the rows in LDS (rows past M read row 0; their results are thrown away), B from
+  // the wave's ring.  (A second batch of rows to normalise, with more than RB rows a wave, was loaded after
+  // the ring's first stages; the compiler's wait for it also waited for those, so the count below holds.)
   const bf16_t* ap = xs + (size_t)(r < M ? r : 0) * lds_row + 8 * g;
+  int off_w[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) off_w[kk] = (r >> 3) * 1024 + (r & 7) * 128 + (((4 * kk + g) ^ (r >> 1)) * 16);
   f32x4 acc[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  constexpr int PA = 4;                            // A operands are read from LDS this many steps ahead
-  static_assert(D % PA == 0, "the A look-ahead must divide the ring depth");
-  u32x4 aq[PA];
-  auto fetch_a = [&](int slot, int k) { aq[slot] = *reinterpret_cast<const u32x4*>(ap + (k < k_end ? k : k_begin)); };
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(SH::LPW * (SH::STAGES - 2)));   // all but the loads of the stages after this one have landed
+    asm volatile("" ::: "memory");
+    const unsigned char* stage = ring + (step % SH::STAGES) * SH::STAGE;
+    u32x4 fa[2], fb[2][NB];
 #pragma unroll
-  for (int j = 0; j < PA; ++j) fetch_a(j, k_begin + 32 * j);
-  for (int k0 = k_begin; k0 < k_end; k0 += 32 * D) {
+    for (int kk = 0; kk < 2; ++kk) {
+      fa[kk] = *reinterpret_cast<const u32x4*>(ap + 64 * step + 32 * kk);
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int k = k0 + 32 * d;
-      const u32x4 af = aq[d % PA];
-      u32x4 bc[NB];
-#pragma unroll
-      for (int b = 0; b < NB; ++b) bc[b] = bq[d][b];
-      if constexpr (!FULL) issue(d, k + 32 * D);
-      fetch_a(d % PA, k + 32 * PA);
-      __builtin_amdgcn_sched_barrier(0);
-      if (k < k_end) {                             // scalar: a step past the segment's end is skipped
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(bc[b]), acc[b], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      for (int b = 0; b < NB; ++b) fb[kk][b] = *reinterpret_cast<const u32x4*>(stage + b * 2048 + off_w[kk]);
     }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk][b]), acc[b], 0, 0, 0);
+    asm volatile("" ::: "memory");
+    decode_issue<EPI, ST>(ring, rs_w, voff_w, step + SH::STAGES - 1, steps);   // into the stage of the step before
   }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));       // the padding loads too, before LDS is used for anything else
 
   // 4. epilogue
   if constexpr (EPI != DEPI_ROPE_KV) {
@@ -251,26 +273,27 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
 
 static const size_t kMaxLds = 160 * 1024 - 1024;
 
-template <int EPI, int D>
+template <int EPI, int ST>
 static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hipStream_t s) {
   static bool raised = false;
-  const size_t lds = (size_t)a.M * (a.K + 8) * sizeof(bf16_t);
+  using SH = DecodeShape<EPI, ST>;
+  const size_t lds = (((size_t)a.M * (a.K + 8) * sizeof(bf16_t) + 15) & ~(size_t)15) + (size_t)waves * SH::STAGES * SH::STAGE;
   if (lds > kMaxLds) return -2;
   if (!raised) {   // more than 64 KB of dynamic LDS has to be asked for once
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, D>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, ST>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds) != hipSuccess)
       return (int)hipGetLastError();
     raised = true;
   }
-  hipLaunchKernelGGL((decode_gemm_kernel<EPI, D>), dim3(blocks), dim3(64 * waves), lds, s, a);
+  hipLaunchKernelGGL((decode_gemm_kernel<EPI, ST>), dim3(blocks), dim3(64 * waves), lds, s, a);
   return BW_LAUNCH_CHECK();
 }
 
 // Can the rows (M of them, K wide) live in LDS, and do the waves of a strip fit a workgroup?
 static int check_decode_gemm(const DecodeGemmArgs& a) {
-  if (a.M <= 0 || a.M > 16 || a.N <= 0 || a.K <= 0 || (a.K % 32)) return -2;
+  if (a.M <= 0 || a.M > 16 || a.N <= 0 || a.K <= 0 || (a.K % 64)) return -2;
   if (a.K > DEC_SEG || (a.lda % 4) || a.lda < a.K) return -2;      // a row is normalised from a wave's registers
-  if ((size_t)a.M * (a.K + 8) * sizeof(bf16_t) > kMaxLds) return -2;
+  if ((size_t)a.M * (a.K + 8) * sizeof(bf16_t) + 64 * 1024 > kMaxLds) return -2;      // the rows and the waves' rings
   return 0;
 }
 
@@ -290,15 +313,15 @@ extern "C" int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, in
   if (bad) return bad;
   if (ldo < N) return -2;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
-  const int waves = 4;                                   // strips per workgroup
+  const int waves = 4;                                   // strips per workgroup (their rings: 64 KB of LDS)
   const int strips = (N + 15) / 16;
   const int blocks = (strips + waves - 1) / waves;
   hipStream_t s = (hipStream_t)stream;
   switch (epilogue) {
-    case DEPI_F32: return launch_decode_gemm<DEPI_F32, 32>(a, waves, blocks, s);
-    case DEPI_BF16: return launch_decode_gemm<DEPI_BF16, 32>(a, waves, blocks, s);
-    case DEPI_ADD_F32: return launch_decode_gemm<DEPI_ADD_F32, 32>(a, waves, blocks, s);
-    case DEPI_SWIGLU_BF16: return launch_decode_gemm<DEPI_SWIGLU_BF16, 20>(a, waves, blocks, s);
+    case DEPI_F32: return launch_decode_gemm<DEPI_F32, 8>(a, waves, blocks, s);
+    case DEPI_BF16: return launch_decode_gemm<DEPI_BF16, 8>(a, waves, blocks, s);
+    case DEPI_ADD_F32: return launch_decode_gemm<DEPI_ADD_F32, 8>(a, waves, blocks, s);
+    case DEPI_SWIGLU_BF16: return launch_decode_gemm<DEPI_SWIGLU_BF16, 4>(a, waves, blocks, s);
   }
   return -2;
 }
@@ -327,6 +350,6 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
   if ((size_t)(pairs ? 32 : head_dim) * sizeof(float) > (size_t)(K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
   const int all_heads = heads + 2 * kv_heads;
-  if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, 64>(a, 2, all_heads * pairs, (hipStream_t)stream);
-  return launch_decode_gemm<DEPI_ROPE_KV, 64>(a, head_dim / 16, all_heads, (hipStream_t)stream);
+  if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, 2, all_heads * pairs, (hipStream_t)stream);
+  return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, head_dim / 16, all_heads, (hipStream_t)stream);
 }

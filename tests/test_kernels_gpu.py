@@ -469,7 +469,7 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
     """RMSNorm fused into the product (and rotation plus cache write into the q|k|v product)
     must give the bits of the kernels run one after the other."""
     g = torch.Generator().manual_seed(14)
-    for M, K, N in [(1, 64, 48), (5, 96, 500), (8, 2048, 6144), (16, 224, 112), (13, 1024, 72)]:
+    for M, K, N in [(1, 64, 48), (5, 128, 500), (8, 2048, 6144), (16, 192, 112), (13, 1024, 72)]:
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
         nw = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().to(gpu)
         w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
@@ -487,8 +487,9 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
             ops.norm_gemm_bf16(x, nw.float(), 1e-5, w, fused_s, M, ops.EPI_SWIGLU_BF16)
             assert torch.equal(fused_s, sep_s), (M, K, N)
     assert not ops.can_fuse_norm(17, w, x) and not ops.can_fuse_norm(4, torch.zeros(8, 4096, dtype=torch.bfloat16), x)
+    assert not ops.can_fuse_norm(4, torch.zeros(8, 96, dtype=torch.bfloat16), torch.zeros(4, 96))   # steps of 64 along the rows
 
-    for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 96), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 160),
+    for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
                                      (2, 1, 128, 16, 256), (3, 3, 96, 16, 128)]:
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
