@@ -168,5 +168,8 @@ __device__ __forceinline__ void rmsnorm_row_small(const f32x4* __restrict__ xv, 
   norm_rows_finish<1>(nr, rows, w_is_bf16, nvec, dim, eps, lane, [&](int, int c, u32x2 pk) { store(c, pk); });
 }
 
+// The operand of s_waitcnt that waits for all but the last n memory loads of the wave and for nothing else.
+constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
 // The launch wrappers return hipGetLastError() as int; 0 is success.
 #define BW_LAUNCH_CHECK() ((int)hipGetLastError())

@@ -28,6 +28,10 @@
 #include "common.h"
 #include "api.h"
 
+// in gemm_bf16.hip
+int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w_is_bf16, float eps, const void* w, void* out,
+                     int ldo, int M, int N, int K, int epilogue, void* stream);
+
 enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI_ROPE_KV = 4 };
 
 #define DEC_SEG 2048
@@ -50,9 +54,6 @@ struct DecodeGemmArgs {
   int heads, kv_heads, head_dim, page_size, table_stride, write_cache;
   int pairs;               // rotary: 16-wide pairs of strips a head is cut into (0: a workgroup is a whole head)
 };
-
-// s_waitcnt vmcnt(n) alone
-constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
 
 // ST: stages of a wave's ring
 template <int EPI, int ST>
@@ -313,6 +314,9 @@ extern "C" int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, in
   if (bad) return bad;
   if (ldo < N) return -2;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
+  // many columns: the kernel whose workgroups share the normalised rows among four strips and one ring
+  const int mid = bw_norm_gemm_mid(x, ldx, norm_w, norm_w_is_bf16, eps, w, out, ldo, M, N, K, epilogue, stream);
+  if (mid != -7) return mid;
   const int waves = 4;                                   // strips per workgroup (their rings: 64 KB of LDS)
   const int strips = (N + 15) / 16;
   const int blocks = (strips + waves - 1) / waves;

@@ -763,41 +763,54 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // since no registers hold them the ring can be deep: eight stages, so up to seven steps of weights are
 // in flight while one is worked on.  Every wave issues the same number of loads a stage (LPW: its share
 // of the weights and of x, padded with loads from outside the descriptors, which cost no memory
-// traffic), in order, so "all but the last 6 * LPW have landed" is the wait for the stage at hand;
+// traffic), in order, so "all but the last (stages - 2) * LPW have landed" is the wait for the stage at hand;
 // stages past K are asked for outside the descriptors too, to keep that count fixed.  One barrier a
 // step: behind it every wave has the stage at hand and is done with the one before.
 // Plain epilogues: four waves, wave w owns strip w and all blocks of rows.  SwiGLU: wave (s, h) owns
-// gate and up strip s for half h of the row blocks; with one block of rows there are two waves.
+// gate and up strip s for half h of the row blocks (with one block of rows the waves of the second
+// half only load and normalise: their products are of rows that do not exist and go nowhere).
 // K a multiple of 64, one segment.
-#define MID_STAGES 8
 
-template <int EPI, int NRB>
+// NORM: the rows arrive as the 32-bit residual stream and are normalised (RMSNorm, the statements of
+// rmsnorm_bf16_kernel) into LDS by the workgroup itself, all of K at once (up to 16 rows, K one segment);
+// the ring then holds weights only, and its first stages are in flight while the rows are normalised.
+template <int EPI, int NRB, bool NORM>
 struct MidShape {
   static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
-  static constexpr int NW = (GLU && NRB == 1) ? 2 : 4;               // waves
-  static constexpr int A_LOADS = (2 * NRB + NW - 1) / NW;           // per wave and stage: 8 rows of x each
+  static constexpr int NW = 4;                                      // waves
+  static constexpr int A_LOADS = NORM ? 0 : (2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
   static constexpr int B_LOADS = 8 / NW;                            // 8 rows of W each
   static constexpr int LPW = A_LOADS + B_LOADS;
-  static constexpr int A_BYTES = NRB * 2048, STAGE = A_BYTES + 8 * 1024;
+  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STAGE = A_BYTES + 8 * 1024;
   static constexpr int NI = GLU ? (NRB >= 2 ? NRB / 2 : 1) : NRB;    // blocks of rows a wave works on
   static constexpr int NJ = GLU ? 2 : 1;
-  static constexpr int PENDING = LPW * (MID_STAGES - 2);            // loads that may still be in flight at a step's start
+  static constexpr int STAGES = 8;
+  static constexpr int PENDING = LPW * (STAGES - 2);            // loads that may still be in flight at a step's start
+  static constexpr int RING = STAGES * STAGE + 1024;            // and 1 KB where padding loads put their zeros
   static_assert(PENDING < 64, "the wait count has six bits");
+  static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
+};
+
+// What the NORM variant needs beside the product's operands.
+struct MidNormArgs {
+  const float* x32;      // [M, ldx32] rows of the residual stream
+  const void* norm_w;    // [K]
+  int ldx32, norm_w_is_bf16;
+  float eps;
 };
 
 // A wave's loads of one stage of the ring: its share of the rows of x and of W, LPW instructions.
-template <int EPI, int NRB>
+template <int EPI, int NRB, bool NORM>
 __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                          const int (&voff_a)[MidShape<EPI, NRB>::A_LOADS],
-                                          const int (&voff_b)[MidShape<EPI, NRB>::B_LOADS], int wave, int step, int steps) {
-  using S = MidShape<EPI, NRB>;
+                                          const int* voff_a, const int* voff_b, int wave, int step, int steps) {
+  using S = MidShape<EPI, NRB, NORM>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
-  unsigned char* dst = lds + (step % MID_STAGES) * S::STAGE;
+  unsigned char* dst = lds + (step % S::STAGES) * S::STAGE;
   const bool real = step < steps;                                     // scalar
 #pragma unroll
   for (int t = 0; t < S::A_LOADS; ++t) {
     const int block = wave * S::A_LOADS + t;                          // 1 KB of the stage's x; a padding load's zeros go behind the ring
-    unsigned char* to = block < 2 * NRB ? dst + block * 1024 : lds + MID_STAGES * S::STAGE;
+    unsigned char* to = block < 2 * NRB ? dst + block * 1024 : lds + S::STAGES * S::STAGE;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)to, 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
   }
 #pragma unroll
@@ -806,26 +819,27 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
                                              real ? voff_b[t] : 0x7ffffff0, step * 128, 0, 0);
 }
 
-template <int EPI, int NRB>
+template <int EPI, int NRB, bool NORM>
 __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
-  using S = MidShape<EPI, NRB>;
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+    MidNormArgs na) {
+  using S = MidShape<EPI, NRB, NORM>;
   constexpr bool GLU = S::GLU;
   constexpr int COLS = GLU ? 32 : 64, NI = S::NI, NJ = S::NJ;
-  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads
+  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * COLS;
   const int b_rows = min(COLS, N - n0);
-  const __amdgpu_buffer_rsrc_t rs_a =
-      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)x, 0, NORM ? 0 : (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
   // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
   const int lrow = lane >> 3, lslot = lane & 7;
   const int b_first = wave * S::B_LOADS * 8;                         // this wave's first row of the tile's 64 of W
   const bool up = GLU && b_first >= 32;
   const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
-  int voff_a[S::A_LOADS], voff_b[S::B_LOADS];
+  int voff_a[S::A_LOADS > 0 ? S::A_LOADS : 1] = {0}, voff_b[S::B_LOADS];
 #pragma unroll
   for (int t = 0; t < S::A_LOADS; ++t) {
     const int row = (wave * S::A_LOADS + t) * 8 + lrow;             // of the NRB * 16 rows of x; past them: a padding load
@@ -853,23 +867,57 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   const int a_block0 = GLU ? NI * (wave >> 1) : 0;                    // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
 
+  unsigned char* rows_lds = mid_lds + S::RING;
+  if constexpr (NORM) {
+    // the rows to normalise are asked for before the ring (loads complete in the order they are issued: the
+    // wait for the rows must not be a wait for weights), four rows a wave at a time
+    constexpr int RB = 4;
+    const int nvec = K >> 2;
+    NormRows<RB> nr;
+    const f32x4* nrows[RB];
+    for (int m0 = wave; m0 < M; m0 += RB * S::NW) {
 #pragma unroll
-  for (int st = 0; st < MID_STAGES - 1; ++st) mid_issue<EPI, NRB>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+      for (int i = 0; i < RB; ++i) {
+        const int m = m0 + i * S::NW;
+        nrows[i] = m < M ? reinterpret_cast<const f32x4*>(na.x32 + (size_t)m * na.ldx32) : nullptr;
+      }
+      norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
+      if (m0 == wave) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      unsigned char* rl = rows_lds;
+      const int nw = S::NW;
+      norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
+        // vector c = elements 4c..4c+3 of row m: step c / 16, 16-byte chunk (c % 16) / 2 of the step, its half c % 2
+        const int m = m0 + i * nw;
+        unsigned char* p = rl + (c >> 4) * 2048 + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ (m >> 1)) * 16) + (c & 1) * 8;
+        *reinterpret_cast<u32x2*>(p) = pk;
+      });
+    }
+    if (wave >= M) {                                                   // a wave without rows still feeds the ring
+#pragma unroll
+      for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+    }
+    // rows past M stay as LDS holds them: their products are never stored
+  } else {
+#pragma unroll
+    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+  }
   for (int step = 0; step < steps; ++step) {
-    // s_waitcnt vmcnt(PENDING) alone; the instruction wants a literal
-    static_assert(S::PENDING == 18 || S::PENDING == 24 || S::PENDING == 30, "a wait for this count is not written out");
-    if constexpr (S::PENDING == 18) __builtin_amdgcn_s_waitcnt(0x4f72);
-    else if constexpr (S::PENDING == 24) __builtin_amdgcn_s_waitcnt(0x4f78);
-    else __builtin_amdgcn_s_waitcnt(0x4f7e);
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    mid_issue<EPI, NRB>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + MID_STAGES - 1, steps);   // into the stage worked on a step ago
-    const unsigned char* stage = mid_lds + (step % MID_STAGES) * S::STAGE;
+    mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + S::STAGES - 1, steps);   // into the stage worked on a step ago
+    const unsigned char* stage = mid_lds + (step % S::STAGES) * S::STAGE;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       u32x4 fa[NI], fb[NJ];
 #pragma unroll
-      for (int i = 0; i < NI; ++i) fa[i] = *reinterpret_cast<const u32x4*>(stage + (a_block0 + i) * 2048 + slot_off[kk]);
+      for (int i = 0; i < NI; ++i)
+        fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + step * 2048 : stage) + (a_block0 + i) * 2048 + slot_off[kk]);
 #pragma unroll
       for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(stage + b_off0 + j * 4096 + slot_off[kk]);
 #pragma unroll
@@ -891,17 +939,37 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     }
 }
 
-template <int EPI, int NRB>
-static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s) {
-  using S = MidShape<EPI, NRB>;
+template <int EPI, int NRB, bool NORM>
+static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
+                      const MidNormArgs& na = MidNormArgs{}) {
+  using S = MidShape<EPI, NRB, NORM>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
-  constexpr int lds_bytes = MID_STAGES * S::STAGE + 1024;
-  if (!allowed && lds_bytes > 64 * 1024) {
-    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  const int lds_bytes = S::RING + (NORM ? (K / 64) * 2048 : 0);
+  if (lds_bytes > 160 * 1024) return -2;
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo);
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na);
   return BW_LAUNCH_CHECK();
+}
+
+// RMSNorm of up to 16 rows of the residual stream + product with many columns in one kernel; -7: not this shape.
+int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w_is_bf16, float eps, const void* w, void* out,
+                     int ldo, int M, int N, int K, int epilogue, void* stream) {
+  const int cols = epilogue == EPI_SWIGLU_BF16 ? 32 : 64;
+  const int wgs = (N + cols - 1) / cols;
+  if (M > 16 || K > GEMM_SEG || K % 64 || wgs < 64 || (size_t)2 * N * K * 2 >= ((size_t)1 << 31)) return -7;
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
+  const bf16_t* wp = (const bf16_t*)w;
+  hipStream_t s = (hipStream_t)stream;
+  switch (epilogue) {
+    case EPI_F32: return launch_mid<EPI_F32, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
+    case EPI_BF16: return launch_mid<EPI_BF16, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
+    case EPI_ADD_F32: return launch_mid<EPI_ADD_F32, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
+    case EPI_SWIGLU_BF16: return launch_mid<EPI_SWIGLU_BF16, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
+  }
+  return -7;
 }
 
 // ------------------------------------------------------------------------------ up to 16 rows, few columns
@@ -1056,9 +1124,9 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
       if (S == 1 && K % 64 == 0 && wgs >= 64 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) &&
           (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
-        if (M <= 16) return launch_mid<EPI, 1>(x, w, out, M, N, K, ldx, ldo, wgs, s);
-        if (M <= 32) return launch_mid<EPI, 2>(x, w, out, M, N, K, ldx, ldo, wgs, s);
-        return launch_mid<EPI, 4>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+        if (M <= 16) return launch_mid<EPI, 1, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+        if (M <= 32) return launch_mid<EPI, 2, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+        return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
       }
     }
     if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {

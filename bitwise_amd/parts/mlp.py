@@ -42,6 +42,18 @@ class SwiGLU(FeedForward):
     def weight_bytes(self) -> int:
         return self.gate_up.nbytes() + self.down.nbytes()
 
+    def forward_with_norm(self, ctx, x, norm, residual) -> bool:
+        """Decode steps of few rows: norm, the stacked product and SwiGLU are one kernel."""
+        from .norm import RMSNorm
+        rt = self.rt
+        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.gate_up.mfma and self.down.mfma
+                and ops.can_fuse_norm(ctx.rows, self.gate_up.weight, x)):
+            return False
+        act = rt.buffer("mlp_h", self.inter, torch.bfloat16)
+        ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.gate_up.weight, act, ctx.rows, ops.EPI_SWIGLU_BF16)
+        self.down.add_into(act, residual, ctx.rows)
+        return True
+
     def forward(self, ctx, h, residual) -> None:
         rt, rows = self.rt, ctx.rows
         if self.gate_up.mfma:

@@ -469,7 +469,8 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
     """RMSNorm fused into the product (and rotation plus cache write into the q|k|v product)
     must give the bits of the kernels run one after the other."""
     g = torch.Generator().manual_seed(14)
-    for M, K, N in [(1, 64, 48), (5, 128, 500), (8, 2048, 6144), (16, 192, 112), (13, 1024, 72)]:
+    for M, K, N in [(1, 64, 48), (5, 128, 500), (8, 2048, 6144), (16, 192, 112), (13, 1024, 72),
+                    (16, 192, 4100), (1, 64, 4096), (11, 2048, 4224)]:   # many columns: another kernel
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
         nw = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().to(gpu)
         w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
