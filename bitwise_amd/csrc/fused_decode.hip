@@ -32,6 +32,11 @@
 int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w_is_bf16, float eps, const void* w, void* out,
                      int ldo, int M, int N, int K, int epilogue, void* stream);
 
+int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int norm_w_is_bf16, float eps, const void* w_qkv,
+                         void* q_out, const int32_t* positions, const int32_t* row_seq, const int32_t* block_table,
+                         int table_stride, const float* cos_table, const float* sin_table, void* k_cache, void* v_cache, int M,
+                         int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream);
+
 enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI_ROPE_KV = 4 };
 
 #define DEC_SEG 2048
@@ -353,6 +358,11 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
   if (bad) return bad;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
   if ((size_t)(pairs ? 32 : head_dim) * sizeof(float) > (size_t)(K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
+  // many heads of 64: the kernel whose workgroups are a head each, four strips sharing the normalised rows and one ring
+  const int mid = bw_norm_qkv_rope_mid(x, ldx, norm_w, norm_w_is_bf16, eps, w_qkv, q_out, positions, row_seq, block_table,
+                                       table_stride, cos_table, sin_table, k_cache, v_cache, M, heads, kv_heads, head_dim, K,
+                                       page_size, write_cache, stream);
+  if (mid != -7) return mid;
   const int all_heads = heads + 2 * kv_heads;
   if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, 2, all_heads * pairs, (hipStream_t)stream);
   return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, head_dim / 16, all_heads, (hipStream_t)stream);

@@ -822,7 +822,7 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
 template <int EPI, int NRB, bool NORM>
 __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-    MidNormArgs na) {
+    MidNormArgs na, QkvRopeArgs rp) {
   using S = MidShape<EPI, NRB, NORM>;
   constexpr bool GLU = S::GLU;
   constexpr int COLS = GLU ? 32 : 64, NI = S::NI, NJ = S::NJ;
@@ -867,6 +867,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   const int a_block0 = GLU ? NI * (wave >> 1) : 0;                    // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
 
+  // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's 64 columns are head blockIdx.x):
+  // what this thread's (row, pair) items need is asked for first of all, positions and then what depends on
+  // them, so that no load of the kernel other than weights is issued after the ring's (see the waits below).
+  int r_pos[2] = {-1, -1}, r_page[2] = {0, 0};
+  float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
+  if constexpr (EPI == EPI_QKV_ROPE) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * 256;
+      if (e < M * 32) {
+        const int pos = rp.positions[e >> 5];
+        r_pos[j] = pos;
+        if (pos >= 0) {
+          r_cos[j] = rp.cos_table[(size_t)pos * 32 + (e & 31)];
+          r_sin[j] = rp.sin_table[(size_t)pos * 32 + (e & 31)];
+          r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> 5] * rp.table_stride + pos / rp.page_size];
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   unsigned char* rows_lds = mid_lds + S::RING;
   if constexpr (NORM) {
     // the rows to normalise are asked for before the ring (loads complete in the order they are issued: the
@@ -928,20 +949,61 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     }
     asm volatile("" ::: "memory");
   }
-  const int n = n0 + 16 * strip + r;
-  if (n >= N) return;
-#pragma unroll
-  for (int i = 0; i < NI; ++i)
+  if constexpr (EPI == EPI_QKV_ROPE) {
+    // The rotary pairs (i, i + 32) sit in different waves: the 32-bit products meet in LDS.  Heads come in the
+    // order q heads, k heads, v heads; q rotated to its buffer, k rotated and v as it is to the row's page slot.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                       // the padding loads have landed: LDS is free
+    __syncthreads();
+    float* os = reinterpret_cast<float*>(mid_lds);                    // [M][64]
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int m = 16 * (a_block0 + i) + 4 * g + q;
-      if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
+      const int m = 4 * g + q;
+      if (m < M) os[m * 64 + 16 * wave + r] = acc[0][0][q];
     }
+    __syncthreads();
+    const int head = blockIdx.x;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * 256;
+      const int pos = r_pos[j];
+      if (e >= M * 32 || pos < 0) continue;
+      const int m = e >> 5, i = e & 31;
+      const float x1 = os[m * 64 + i], x2 = os[m * 64 + i + 32];
+      if (head < rp.heads + rp.kv_heads) {
+        const float c = r_cos[j], sn = r_sin[j];
+        const float o1 = x1 * c - x2 * sn;
+        const float o2 = x2 * c + x1 * sn;
+        bf16_t* dst = nullptr;
+        if (head < rp.heads) dst = (bf16_t*)out + (size_t)m * rp.heads * 64 + (size_t)head * 64;
+        else if (rp.write_cache)
+          dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + pos % rp.page_size) * 64;
+        if (dst != nullptr) {
+          dst[i] = f32_to_bf16(o1);
+          dst[i + 32] = f32_to_bf16(o2);
+        }
+      } else if (rp.write_cache) {
+        bf16_t* dst = rp.v_cache + ((size_t)r_page[j] * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size +
+                      pos % rp.page_size;
+        dst[(size_t)i * rp.page_size] = f32_to_bf16(x1);
+        dst[(size_t)(i + 32) * rp.page_size] = f32_to_bf16(x2);
+      }
+    }
+  } else {
+    const int n = n0 + 16 * strip + r;
+    if (n >= N) return;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = 16 * (a_block0 + i) + 4 * g + q;
+        if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
+      }
+  }
 }
 
 template <int EPI, int NRB, bool NORM>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
-                      const MidNormArgs& na = MidNormArgs{}) {
+                      const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}) {
   using S = MidShape<EPI, NRB, NORM>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
   const int lds_bytes = S::RING + (NORM ? (K / 64) * 2048 : 0);
@@ -950,7 +1012,7 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N,
     (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na);
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp);
   return BW_LAUNCH_CHECK();
 }
 
@@ -970,6 +1032,22 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
     case EPI_SWIGLU_BF16: return launch_mid<EPI_SWIGLU_BF16, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
   }
   return -7;
+}
+
+// RMSNorm of up to 16 rows + the stacked q|k|v product + rotation + cache write in one kernel, for heads of 64
+// and at least 64 of them (a workgroup a head); -7: not this shape.
+int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int norm_w_is_bf16, float eps, const void* w_qkv,
+                         void* q_out, const int32_t* positions, const int32_t* row_seq, const int32_t* block_table,
+                         int table_stride, const float* cos_table, const float* sin_table, void* k_cache, void* v_cache, int M,
+                         int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream) {
+  const int all_heads = heads + 2 * kv_heads;
+  if (head_dim != 64 || M > 16 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)all_heads * 64 * K * 2 >= ((size_t)1 << 31))
+    return -7;
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
+  QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                 heads, kv_heads, page_size, table_stride, write_cache};
+  return launch_mid<EPI_QKV_ROPE, 1, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64, all_heads,
+                                           (hipStream_t)stream, na, rp);
 }
 
 // ------------------------------------------------------------------------------ up to 16 rows, few columns

@@ -491,7 +491,7 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
     assert not ops.can_fuse_norm(4, torch.zeros(8, 96, dtype=torch.bfloat16), torch.zeros(4, 96))   # steps of 64 along the rows
 
     for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
-                                     (2, 1, 128, 16, 256), (3, 3, 96, 16, 128)]:
+                                     (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128)]:   # the last: a workgroup a head
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
