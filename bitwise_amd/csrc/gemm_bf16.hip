@@ -870,12 +870,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's 64 columns are head blockIdx.x):
   // what this thread's (row, pair) items need is asked for first of all, positions and then what depends on
   // them, so that no load of the kernel other than weights is issued after the ring's (see the waits below).
-  int r_pos[2] = {-1, -1}, r_page[2] = {0, 0};
-  float r_cos[2] = {1.f, 1.f}, r_sin[2] = {0.f, 0.f};
+  constexpr int ITEMS = EPI == EPI_QKV_ROPE ? 2 * NRB : 1;           // (row, pair) items a thread: 16 * NRB rows x 32 pairs
+  int r_pos[ITEMS], r_page[ITEMS];
+  float r_cos[ITEMS], r_sin[ITEMS];
   if constexpr (EPI == EPI_QKV_ROPE) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
       const int e = threadIdx.x + j * 256;
+      r_pos[j] = -1;
+      r_page[j] = 0;
+      r_cos[j] = 1.f;
+      r_sin[j] = 0.f;
       if (e < M * 32) {
         const int pos = rp.positions[e >> 5];
         r_pos[j] = pos;
@@ -956,14 +961,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     __syncthreads();
     float* os = reinterpret_cast<float*>(mid_lds);                    // [M][64]
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int m = 4 * g + q;
-      if (m < M) os[m * 64 + 16 * wave + r] = acc[0][0][q];
-    }
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = 16 * i + 4 * g + q;
+        if (m < M) os[m * 64 + 16 * wave + r] = acc[i][0][q];
+      }
     __syncthreads();
     const int head = blockIdx.x;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
       const int e = threadIdx.x + j * 256;
       const int pos = r_pos[j];
       if (e >= M * 32 || pos < 0) continue;
@@ -1032,6 +1039,20 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
     case EPI_SWIGLU_BF16: return launch_mid<EPI_SWIGLU_BF16, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
   }
   return -7;
+}
+
+// The stacked q|k|v product of up to 64 normalised rows with rotation and cache write in its epilogue, for heads of
+// 64 and at least 64 of them (a workgroup a head); -7: not this shape.
+static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, void* q_out, int M, int K, const QkvRopeArgs& rp,
+                               hipStream_t s) {
+  const int all_heads = rp.heads + 2 * rp.kv_heads;
+  if (M > 64 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)all_heads * 64 * K * 2 >= ((size_t)1 << 31) ||
+      (size_t)M * ldx * 2 >= ((size_t)1 << 31))
+    return -7;
+  const int N = all_heads * 64, ldo = rp.heads * 64;
+  if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
+  if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
+  return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
 }
 
 // RMSNorm of up to 16 rows + the stacked q|k|v product + rotation + cache write in one kernel, for heads of 64
@@ -1297,8 +1318,8 @@ extern "C" int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int 
   return -2;
 }
 
-// The stacked q|k|v product of a prompt portion with rotation and cache write in its epilogue
-// (heads of 64 elements, more than 64 rows, K of one segment): q rotated to q_out [M, heads*64],
+// The stacked q|k|v product with rotation and cache write in its epilogue (heads of 64 elements, K of one
+// segment; more than 64 rows, or up to 64 with at least 64 heads and K in steps of 64): q rotated to q_out [M, heads*64],
 // k rotated and v to their page slots.  The bits of gemm_bf16 (32-bit store) + rope_kvwrite.
 extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out, const int32_t* positions,
                                      const int32_t* row_seq, const int32_t* block_table, int table_stride,
@@ -1307,10 +1328,14 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
                                      int write_cache, void* stream) {
   if (M <= 0) return 0;
   if (head_dim != 64) return -4;
-  if (M <= 64 || K <= 0 || K > GEMM_SEG || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
+  if (K <= 0 || K > GEMM_SEG || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_qkv)) & 15) return -3;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
                  heads, kv_heads, page_size, table_stride, write_cache};
+  if (M <= 64) {
+    const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
+    return mid == -7 ? -2 : mid;
+  }
   const int N = (heads + 2 * kv_heads) * 64;
   return launch_gemm_bf16<EPI_QKV_ROPE>((const bf16_t*)x, (const bf16_t*)w_qkv, q_out, M, N, K, ldx, heads * 64,
                                         (hipStream_t)stream, rp);

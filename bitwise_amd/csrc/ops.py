@@ -410,9 +410,13 @@ def attention_decode_scratch(num_tiles: int, heads: int, kv_heads: int, head_dim
     return int(floats.value), int(counters.value)
 
 
-def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int) -> bool:
-    """Whether the q|k|v product of a prompt portion can take rotation and cache write into its epilogue."""
-    return rows > 64 and head_dim == 64 and inner <= 2048 and inner % 8 == 0
+def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int, all_heads: int = 0) -> bool:
+    """Whether the q|k|v product of normalised rows can take rotation and cache write into its
+    epilogue: heads of 64 and one segment of K; more than 64 rows, or (a workgroup a head) up to
+    64 rows of at least 64 heads (q, k and v heads together) with K in steps of 64."""
+    if head_dim != 64 or inner > 2048 or inner % 8:
+        return False
+    return rows > 64 or (all_heads >= 64 and inner % 64 == 0)
 
 
 def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
@@ -432,7 +436,7 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
     _need(cos, torch.float32, "cos table")
     _need(sin, torch.float32, "sin table")
     N, K = w_qkv.shape
-    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_gemm_ok(rows, head_dim, K):
+    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_gemm_ok(rows, head_dim, K, heads + 2 * kv_heads):
         raise ValueError("gemm_qkv_rope_bf16: not a [q|k|v] weight of 64-element heads, or too few rows")
     if x.shape[1] != K or x.shape[0] < rows or q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows:
         raise ValueError("gemm_qkv_rope_bf16: buffers do not fit")

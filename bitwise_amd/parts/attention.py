@@ -93,8 +93,9 @@ class Attention(Mixer):
         rt, rows = self.rt, ctx.rows
         table = ctx.block_tables[call.group]
         window = int(self.window or 0)
-        if rt.bf16 and self.qkv.mfma and ops.qkv_rope_gemm_ok(rows, self.head_dim, self.qkv.weight.shape[1]):
-            # prompt portions: rotation and cache write ride in the product's epilogue
+        if rt.bf16 and self.qkv.mfma and ops.qkv_rope_gemm_ok(rows, self.head_dim, self.qkv.weight.shape[1],
+                                                              self.heads + 2 * self.kv_heads):
+            # rotation and cache write ride in the product's epilogue
             q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
             ops.gemm_qkv_rope_bf16(h, self.qkv.weight, q, ctx.positions, ctx.row_seq, table, self.position.cos,
                                    self.position.sin, call.k_cache, call.v_cache, rows, self.heads, self.kv_heads,

@@ -527,7 +527,8 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
     Rows of two requests, a padding row, positions across page edges, a ragged last tile."""
     g = torch.Generator().manual_seed(21)
     for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
-                                   (40, 10, 128, 2100, 32)]:       # the last: enough 256 x 256 tiles for the big-tile kernel
+                                   (40, 10, 128, 2100, 32),        # enough 256 x 256 tiles for the big-tile kernel
+                                   (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16)]:   # up to 64 rows, a workgroup a head
         hd = 64
         pages = 40 if M < 500 else 3 * ((M + page - 1) // page + 2) + 3
         cos, sin = rope_tables(10000.0, hd, max(400, M), gpu)
@@ -546,7 +547,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
             vc = torch.full((pages, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
             q = torch.zeros(M, heads * hd, dtype=torch.bfloat16, device=gpu)
             if fused:
-                assert ops.qkv_rope_gemm_ok(M, hd, K)
+                assert ops.qkv_rope_gemm_ok(M, hd, K, heads + 2 * kvh)
                 ops.gemm_qkv_rope_bf16(h, w, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh, hd, page)
             else:
                 qkv = torch.zeros(M, w.shape[0], device=gpu)
@@ -556,7 +557,8 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
         live = [r for r in range(M) if pos[r] >= 0]
         assert torch.equal(outs[0][0][live], outs[1][0][live]), (heads, kvh, K, M)
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), (heads, kvh, K, M)
-    assert not ops.qkv_rope_gemm_ok(64, 64, 256) and not ops.qkv_rope_gemm_ok(200, 128, 256)
+    assert not ops.qkv_rope_gemm_ok(64, 64, 256, 63) and not ops.qkv_rope_gemm_ok(200, 128, 256, 96)
+    assert not ops.qkv_rope_gemm_ok(64, 64, 96, 96)
 
 
 def test_decode_attention_beyond_one_pass_of_partials(gpu):
