@@ -22,6 +22,9 @@ int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, i
                 int accumulate, void* stream);
 int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, int epilogue,
                  void* stream);
+int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_floats, int* counters);
+int bw_gemm_add_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, float* scratch,
+                     long long scratch_floats, int32_t* counters, int num_counters, void* stream);
 int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out, const int32_t* positions,
                           const int32_t* row_seq, const int32_t* block_table, int table_stride, const float* cos_table,
                           const float* sin_table, void* k_cache, void* v_cache, int M, int heads, int kv_heads,

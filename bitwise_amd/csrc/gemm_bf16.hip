@@ -774,21 +774,36 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // NORM: the rows arrive as the 32-bit residual stream and are normalised (RMSNorm, the statements of
 // rmsnorm_bf16_kernel) into LDS by the workgroup itself, all of K at once (up to 16 rows, K one segment);
 // the ring then holds weights only, and its first stages are in flight while the rows are normalised.
-template <int EPI, int NRB, bool NORM>
+// NARROW (plain epilogues, at least two blocks of rows): 32 columns a workgroup, the waves arranged as for SwiGLU
+// (strip s, half h of the row blocks), for products with so few columns that 64 a workgroup would leave most
+// compute units idle.
+template <int EPI, int NRB, bool NORM, bool NARROW = false>
 struct MidShape {
   static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  static constexpr bool HALVES = GLU || NARROW;                     // waves are (strip, half of the row blocks)
   static constexpr int NW = 4;                                      // waves
+  static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
+  static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a stage (SwiGLU: 32 gate, 32 up)
   static constexpr int A_LOADS = NORM ? 0 : (2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
-  static constexpr int B_LOADS = 8 / NW;                            // 8 rows of W each
+  static constexpr int B_LOADS = B_ROWS / 8 / NW;                   // 8 rows of W each
   static constexpr int LPW = A_LOADS + B_LOADS;
-  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STAGE = A_BYTES + 8 * 1024;
-  static constexpr int NI = GLU ? (NRB >= 2 ? NRB / 2 : 1) : NRB;    // blocks of rows a wave works on
+  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STAGE = A_BYTES + B_ROWS * 128;
+  static constexpr int NI = HALVES ? (NRB >= 2 ? NRB / 2 : 1) : NRB; // blocks of rows a wave works on
   static constexpr int NJ = GLU ? 2 : 1;
   static constexpr int STAGES = 8;
-  static constexpr int PENDING = LPW * (STAGES - 2);            // loads that may still be in flight at a step's start
-  static constexpr int RING = STAGES * STAGE + 1024;            // and 1 KB where padding loads put their zeros
+  static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
+  static constexpr int RING = STAGES * STAGE + 1024;                // and 1 KB where padding loads put their zeros
   static_assert(PENDING < 64, "the wait count has six bits");
   static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
+  static_assert(!NARROW || (!GLU && EPI != EPI_QKV_ROPE && NRB >= 2), "narrow tiles are for plain epilogues and 17 rows or more");
+};
+
+// Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
+// segments' sums meet (device scratch, [tile][segment][wave][block of rows][lane] x 16 bytes) and the tiles'
+// counters (zero before and after every launch).
+struct MidSplitArgs {
+  float* scratch;
+  int* counters;
 };
 
 // What the NORM variant needs beside the product's operands.
@@ -800,10 +815,10 @@ struct MidNormArgs {
 };
 
 // A wave's loads of one stage of the ring: its share of the rows of x and of W, LPW instructions.
-template <int EPI, int NRB, bool NORM>
+template <int EPI, int NRB, bool NORM, bool NARROW>
 __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                          const int* voff_a, const int* voff_b, int wave, int step, int steps) {
-  using S = MidShape<EPI, NRB, NORM>;
+                                          const int* voff_a, const int* voff_b, int wave, int step, int steps, int k_base) {
+  using S = MidShape<EPI, NRB, NORM, NARROW>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   unsigned char* dst = lds + (step % S::STAGES) * S::STAGE;
   const bool real = step < steps;                                     // scalar
@@ -811,21 +826,21 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
   for (int t = 0; t < S::A_LOADS; ++t) {
     const int block = wave * S::A_LOADS + t;                          // 1 KB of the stage's x; a padding load's zeros go behind the ring
     unsigned char* to = block < 2 * NRB ? dst + block * 1024 : lds + S::STAGES * S::STAGE;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)to, 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)to, 16, real ? voff_a[t] : 0x7ffffff0, (k_base + step * 64) * 2, 0, 0);
   }
 #pragma unroll
   for (int t = 0; t < S::B_LOADS; ++t)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + S::A_BYTES + (wave * S::B_LOADS + t) * 1024), 16,
-                                             real ? voff_b[t] : 0x7ffffff0, step * 128, 0, 0);
+                                             real ? voff_b[t] : 0x7ffffff0, (k_base + step * 64) * 2, 0, 0);
 }
 
-template <int EPI, int NRB, bool NORM>
+template <int EPI, int NRB, bool NORM, bool NARROW>
 __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-    MidNormArgs na, QkvRopeArgs rp) {
-  using S = MidShape<EPI, NRB, NORM>;
+    MidNormArgs na, QkvRopeArgs rp, MidSplitArgs sp) {
+  using S = MidShape<EPI, NRB, NORM, NARROW>;
   constexpr bool GLU = S::GLU;
-  constexpr int COLS = GLU ? 32 : 64, NI = S::NI, NJ = S::NJ;
+  constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ;
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
@@ -852,7 +867,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     const int chunk = lslot ^ ((row & 15) >> 1);
     voff_b[t] = (((GLU ? row & 31 : row)) * K + 8 * chunk) * 2;
   }
-  const int steps = K / 64;
+  const int k_base = blockIdx.y * GEMM_SEG;                           // gridDim.y > 1: this workgroup's segment of K
+  const int steps = ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64;
   f32x4 acc[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -863,8 +879,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   int slot_off[2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
-  const int strip = GLU ? (wave & 1) : wave;                          // of the tile's output columns
-  const int a_block0 = GLU ? NI * (wave >> 1) : 0;                    // first block of 16 rows this wave works on
+  const int strip = S::HALVES ? (wave & 1) : wave;                    // of the tile's output columns
+  const int a_block0 = S::HALVES ? NI * (wave >> 1) : 0;              // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
 
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's 64 columns are head blockIdx.x):
@@ -911,7 +927,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
       if (m0 == wave) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+        for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
         __builtin_amdgcn_sched_barrier(0);
       }
       unsigned char* rl = rows_lds;
@@ -925,18 +941,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     }
     if (wave >= M) {                                                   // a wave without rows still feeds the ring
 #pragma unroll
-      for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+      for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
     }
     // rows past M stay as LDS holds them: their products are never stored
   } else {
 #pragma unroll
-    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
   }
   for (int step = 0; step < steps; ++step) {
     __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    mid_issue<EPI, NRB, NORM>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + S::STAGES - 1, steps);   // into the stage worked on a step ago
+    mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + S::STAGES - 1, steps, k_base);   // into the stage worked on a step ago
     const unsigned char* stage = mid_lds + (step % S::STAGES) * S::STAGE;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
@@ -997,6 +1013,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     }
   } else {
     const int n = n0 + 16 * strip + r;
+    if constexpr (EPI == EPI_ADD_F32 && !NORM) {
+      const int nseg = gridDim.y;
+      if (nseg > 1) {
+        // Every segment's workgroup leaves its sums in device scratch (stores of device scope: in memory, not in
+        // this die's L2, once the barrier's wait for the wave's stores is over) and counts itself in; the one that
+        // finds all others counted in adds all segments' sums to the residual in segment order, every one of them
+        // read back from the scratch (its own too).  The counter is back at zero when the kernel ends.
+        const int cell = 4 * NI * 1024;                              // bytes of a workgroup's sums: [wave][i][lane] x 16
+        const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)((unsigned char*)sp.scratch + (size_t)blockIdx.x * nseg * cell), 0, nseg * cell, 0x00020000);
+        const int mine = (wave * NI) * 1024 + lane * 16;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][0]), rs_s, mine + i * 1024, (int)blockIdx.y * cell, 16);
+        __syncthreads();                                             // also: every wave is done with the ring, whose first word is the flag now
+        int* is_last = reinterpret_cast<int*>(mid_lds);
+        if (threadIdx.x == 0) *is_last = atomicAdd(&sp.counters[blockIdx.x], 1) == nseg - 1;
+        __syncthreads();
+        if (!*is_last) return;
+        if (threadIdx.x == 0) sp.counters[blockIdx.x] = 0;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          f32x4 y;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int m = 16 * (a_block0 + i) + 4 * g + q;
+            y[q] = (m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;   // the chain starts at the residual
+          }
+          for (int sg = 0; sg < nseg; ++sg)
+            y = y + __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_s, mine + i * 1024, sg * cell, 16));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int m = 16 * (a_block0 + i) + 4 * g + q;
+            if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] = y[q];
+          }
+        }
+        return;
+      }
+    }
     if (n >= N) return;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -1008,18 +1063,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   }
 }
 
-template <int EPI, int NRB, bool NORM>
+template <int EPI, int NRB, bool NORM, bool NARROW = false>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
-                      const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}) {
-  using S = MidShape<EPI, NRB, NORM>;
+                      const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
+                      const MidSplitArgs& sp = MidSplitArgs{}) {
+  using S = MidShape<EPI, NRB, NORM, NARROW>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
   const int lds_bytes = S::RING + (NORM ? (K / 64) * 2048 : 0);
   if (lds_bytes > 160 * 1024) return -2;
   if (!allowed) {
-    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM>), dim3(wgs), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp);
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW>), dim3(wgs, segments), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
   return BW_LAUNCH_CHECK();
 }
 
@@ -1210,9 +1266,23 @@ static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int
 
 // ------------------------------------------------------------------------------ launch
 
+// How a residual add of 17 to 64 rows runs in the kernel above: 64 or 32 columns a workgroup (as many workgroups
+// as there are compute units, if the product has them), a workgroup per tile and segment of K if there are several
+// (they meet in device scratch the caller brings).  tiles 0: it does not run there.
+static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
+  const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
+  tiles = 0;
+  narrow = false;
+  if (M <= 16 || M > 64 || K % 64) return;
+  narrow = ((N + 63) / 64) * S < 256;
+  tiles = narrow ? (N + 31) / 32 : (N + 63) / 64;
+  if (tiles * S < 32) tiles = 0;
+}
+
 template <int EPI>
 static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo,
-                            hipStream_t s, const QkvRopeArgs& rp = QkvRopeArgs{}) {
+                            hipStream_t s, const QkvRopeArgs& rp = QkvRopeArgs{}, const MidSplitArgs& sp = MidSplitArgs{},
+                            size_t scratch_floats = 0, int num_counters = 0) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
   constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
   if (M <= 64) {
@@ -1221,11 +1291,29 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       // one segment and enough columns: the rows of x are shared through LDS
       constexpr int MID_COLS = (EPI == EPI_SWIGLU_BF16) ? 32 : 64;
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
-      if (S == 1 && K % 64 == 0 && wgs >= 64 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) &&
-          (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+      const bool fits = (size_t)2 * N * K * 2 < ((size_t)1 << 31) && (size_t)M * ldx * 2 < ((size_t)1 << 31);
+      if (S == 1 && K % 64 == 0 && wgs >= 64 && fits) {
         if (M <= 16) return launch_mid<EPI, 1, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         if (M <= 32) return launch_mid<EPI, 2, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
+      }
+      // a residual add of more than 16 rows and fewer columns (the other kernel for it fetches W once per block of
+      // 16 rows): narrower tiles, and several segments if the caller brought scratch for them to meet in
+      if constexpr (EPI == EPI_ADD_F32) {
+        int tiles;
+        bool narrow;
+        add_rows_shape(M, N, K, tiles, narrow);
+        if (tiles && fits && (S == 1 || (sp.scratch != nullptr && sp.counters != nullptr))) {
+          if (S > 1 && (scratch_floats < (size_t)tiles * S * 4096 || num_counters < tiles)) return -6;
+          const MidNormArgs na{};
+          const QkvRopeArgs no{};
+          if (narrow) {
+            if (M <= 32) return launch_mid<EPI, 2, false, true>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp);
+            return launch_mid<EPI, 4, false, true>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp);
+          }
+          if (M <= 32) return launch_mid<EPI, 2, false>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp);
+          return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp);
+        }
       }
     }
     if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {
@@ -1299,6 +1387,29 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
   }
   return BW_LAUNCH_CHECK();
+}
+
+// What a residual add wants beside its operands to give every segment of K workgroups of its own: floats of
+// scratch and counters (int32, zero before the first launch; every launch leaves them zero).  Both 0: it would not.
+extern "C" int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_floats, int* counters) {
+  int tiles = 0;
+  bool narrow = false;
+  const int S = K > 0 ? (K + GEMM_SEG - 1) / GEMM_SEG : 0;
+  if (M > 0 && N > 0 && S > 1) add_rows_shape(M, N, K, tiles, narrow);
+  *scratch_floats = (long long)tiles * S * 4096;
+  *counters = tiles;
+  return 0;
+}
+
+// out += x W^T with the scratch that bw_gemm_add_scratch asks for: the bits of bw_gemm_bf16's residual add.
+extern "C" int bw_gemm_add_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo,
+                                float* scratch, long long scratch_floats, int32_t* counters, int num_counters,
+                                void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K % 8) || (ldx % 8) || ldx < K || ldo < N) return -2;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return -3;
+  return launch_gemm_bf16<EPI_ADD_F32>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldx, ldo, (hipStream_t)stream,
+                                       QkvRopeArgs{}, MidSplitArgs{scratch, counters}, (size_t)scratch_floats, num_counters);
 }
 
 extern "C" int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo,

@@ -41,6 +41,9 @@ _SIGS = {
                         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_f32": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_add_scratch": [c_int, c_int, c_int, c_void_p, c_void_p],
+    "bw_gemm_add_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p,
+                         c_int, c_void_p],
     "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -216,9 +219,20 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, acc
                               x.stride(0), out.stride(0), int(accumulate), _stream()), "gemm_f32")
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, epilogue: int) -> None:
+def gemm_add_scratch(rows: int, N: int, K: int) -> Tuple[int, int]:
+    """(float32 elements, int32 counters) that a residual add of this shape wants as ``scratch``
+    to give every 2048-segment of K workgroups of its own; (0, 0): it would not."""
+    floats, counters = ctypes.c_longlong(0), ctypes.c_int(0)
+    _check(_fn("bw_gemm_add_scratch")(rows, N, K, ctypes.addressof(floats), ctypes.addressof(counters)), "gemm_add_scratch")
+    return int(floats.value), int(counters.value)
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, epilogue: int,
+              scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> None:
     """out[:rows] = epilogue(x[:rows] @ w.T) on the matrix cores; see gemm_bf16.hip for the
-    arithmetic.  EPI_SWIGLU_BF16 takes the stacked weight [2N, K] (gate rows, then up rows)."""
+    arithmetic.  EPI_SWIGLU_BF16 takes the stacked weight [2N, K] (gate rows, then up rows).
+    ``scratch`` (EPI_ADD_F32 only): the tensors ``gemm_add_scratch`` asks for (float32, int32
+    zeros); the bits do not depend on it."""
     _need(x, torch.bfloat16, "x")
     _need(w, torch.bfloat16, "weight")
     if w.dim() != 2:
@@ -234,6 +248,13 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
         raise ValueError(f"gemm_bf16: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
     if K % 8:
         raise ValueError(f"gemm_bf16: inner size {K} must be a multiple of 8 (16-byte operand loads)")
+    if scratch is not None and epilogue == EPI_ADD_F32:
+        sc_f, sc_c = scratch
+        _need(sc_f, torch.float32, "scratch")
+        _need(sc_c, torch.int32, "scratch counters")
+        _check(_fn("bw_gemm_add_bf16")(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, N, K, x.stride(0), out.stride(0),
+                                       sc_f.data_ptr(), sc_f.numel(), sc_c.data_ptr(), sc_c.numel(), _stream()), "gemm_bf16")
+        return
     _check(_fn("bw_gemm_bf16")(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, N, K, x.stride(0), out.stride(0),
                                epilogue, _stream()), "gemm_bf16")
 

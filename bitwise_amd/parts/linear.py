@@ -47,6 +47,13 @@ class Linear:
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, rows: int) -> None:
         """residual[:rows] += x[:rows] @ W.T, the sum in 32-bit (src/model.cpp:300, :305)."""
         if self.mfma:
-            ops.gemm_bf16(x, self.weight, residual, rows, ops.EPI_ADD_F32)
+            # a long inner size and 17 to 64 rows: every 2048-segment of it gets workgroups of its own,
+            # which meet in device scratch
+            scratch = None
+            floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features) if 16 < rows <= 64 else (0, 0)
+            if floats:
+                scratch = (self.rt.buffer("gemm_add_split", floats, torch.float32, rows=1),
+                           self.rt.buffer("gemm_add_split_count", counters, torch.int32, rows=1))
+            ops.gemm_bf16(x, self.weight, residual, rows, ops.EPI_ADD_F32, scratch=scratch)
         else:
             ops.gemm_f32(self._x32(x, rows), self.weight, residual, rows, accumulate=True)

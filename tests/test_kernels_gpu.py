@@ -91,6 +91,7 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     for M, N, K in [(1, 16, 32), (5, 100, 64), (16, 64, 96), (17, 500, 96), (50, 300, 608), (130, 96, 224), (33, 72, 40),
                     (40, 4100, 192), (64, 4200, 2048), (17, 4096, 64), (9, 4100, 128), (16, 5000, 64), (30, 4096, 320),   # many columns: x shared through LDS
                     (7, 200, 4160), (16, 5000, 4096), (3, 40, 128), (12, 4104, 6144),   # up to 16 rows streaming through LDS, several segments
+                    (50, 1030, 128), (20, 2048, 256),   # 17 to 64 rows, one segment, few columns: narrow tiles for the residual add
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
                     (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
@@ -139,6 +140,21 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
         part = torch.zeros(n, inter, device=gpu, dtype=torch.bfloat16)
         ops.gemm_bf16(x[lo:lo + n].contiguous(), w, part, n, ops.EPI_SWIGLU_BF16)
         assert torch.equal(part, hb[lo:lo + n]), (lo, n)
+    # a residual add of 17 to 64 rows over several segments of K with scratch: a workgroup per tile and segment; the
+    # bits of the add without scratch, twice in a row on the same scratch (full of NaN at first), counters zero after
+    for M, N, K in [(64, 2048, 8192), (23, 800, 2048 * 2 + 320), (40, 1100, 4096)]:
+        x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
+        res = torch.randn(M, N, generator=g).to(gpu)
+        want = res.clone()
+        ops.gemm_bf16(x, w, want, M, ops.EPI_ADD_F32)
+        floats, counters = ops.gemm_add_scratch(M, N, K)
+        assert floats > 0 and counters > 0 and ops.gemm_add_scratch(8, N, K) == (0, 0)
+        scratch = (torch.full((floats,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
+        for _ in range(2):
+            got = res.clone()
+            ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
+            assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
     # SwiGLU with many columns (x shared through LDS; one, two or four blocks of 16 rows): the plain result, and
     # the bits of the same rows inside a prompt portion's product (another kernel)
     inter, K = 2100, 128
