@@ -36,6 +36,7 @@ struct QkvRopeArgs {
   bf16_t* k_cache;
   bf16_t* v_cache;
   int heads, kv_heads, page_size, table_stride, write_cache;
+  int page_shift;              // page_size is a power of two: positions are split by shift and mask, not by division
 };
 
 #define GEMM_SEG 2048
@@ -201,19 +202,40 @@ template <int EPI, int NI>
 __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* __restrict__ out, int M, int N, int ldo,
                                               int row0, int col0, int head, int r, int g, bool residual_in,
                                               const QkvRopeArgs& rp) {
+  // Rotary: what the rows need from memory (position, then the page it selects) is asked for at once for all of
+  // them, from addresses that are always valid, so that the waits for it are two and not two a row.
+  constexpr int NR = EPI == EPI_QKV_ROPE ? NI : 1;
+  int pos_all[NR][4], page_all[NR][4];
+  if constexpr (EPI == EPI_QKV_ROPE) {
 #pragma unroll
-  for (int i = 0; i < NI; ++i)
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = row0 + 16 * i + 4 * g + q;
+        pos_all[i][q] = rp.positions[m < M ? m : M - 1];
+      }
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = row0 + 16 * i + 4 * g + q;
+        const int seq = rp.row_seq[m < M ? m : M - 1];
+        const int pidx = (pos_all[i][q] > 0 ? pos_all[i][q] : 0) >> rp.page_shift;
+        page_all[i][q] = head >= rp.heads ? rp.block_table[(size_t)seq * rp.table_stride + pidx] : 0;
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = row0 + 16 * i + 4 * g + q;
       if (m >= M) continue;
       if constexpr (EPI == EPI_QKV_ROPE) {
-        const int pos = rp.positions[m];
+        const int pos = pos_all[i][q];
         if (head >= rp.heads + 2 * rp.kv_heads || pos < 0) continue;
         const int q_dim = rp.heads * 64;
-        size_t page = 0;
-        if (head >= rp.heads) page = (size_t)rp.block_table[(size_t)rp.row_seq[m] * rp.table_stride + pos / rp.page_size];
-        const int slot = pos % rp.page_size;
+        const size_t page = (size_t)page_all[i][q];
+        const int slot = pos & (rp.page_size - 1);
         if (head < rp.heads + rp.kv_heads) {
           bf16_t* dst = head < rp.heads ? (bf16_t*)out + (size_t)m * q_dim + (size_t)head * 64
                                         : rp.k_cache + ((page * rp.kv_heads + (head - rp.heads)) * rp.page_size + slot) * 64;
@@ -230,9 +252,24 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* _
             }
           }
         } else if (rp.write_cache) {
-          bf16_t* dst = rp.v_cache + (page * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size + slot;
+          // values lie transposed in their page ([d][slot]).  The lane's four rows are most often four consecutive
+          // slots of one page starting at a multiple of four: then the first row stores all four at once.
+          bool quad = row0 + 16 * i + 4 * g + 3 < M && (pos_all[i][0] & 3) == 0;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
+          for (int t = 1; t < 4; ++t) quad = quad && pos_all[i][t] == pos_all[i][0] + t && page_all[i][t] == page_all[i][0];
+          bf16_t* dst = rp.v_cache + (page * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size + slot;
+          if (quad) {
+            if (q == 0) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const u32x2 four = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
+                *reinterpret_cast<u32x2*>(dst + (size_t)(16 * j + r) * rp.page_size) = four;
+              }
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
+          }
         }
       } else if constexpr (EPI == EPI_SWIGLU_BF16) {
 #pragma unroll
@@ -250,6 +287,7 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* _
         }
       }
     }
+  }
 }
 
 // ------------------------------------------------------------------------------ wide
@@ -903,7 +941,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         if (pos >= 0) {
           r_cos[j] = rp.cos_table[(size_t)pos * 32 + (e & 31)];
           r_sin[j] = rp.sin_table[(size_t)pos * 32 + (e & 31)];
-          r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> 5] * rp.table_stride + pos / rp.page_size];
+          r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> 5] * rp.table_stride + (pos >> rp.page_shift)];
         }
       }
     }
@@ -999,14 +1037,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         bf16_t* dst = nullptr;
         if (head < rp.heads) dst = (bf16_t*)out + (size_t)m * rp.heads * 64 + (size_t)head * 64;
         else if (rp.write_cache)
-          dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + pos % rp.page_size) * 64;
+          dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + (pos & (rp.page_size - 1))) * 64;
         if (dst != nullptr) {
           dst[i] = f32_to_bf16(o1);
           dst[i + 32] = f32_to_bf16(o2);
         }
       } else if (rp.write_cache) {
         bf16_t* dst = rp.v_cache + ((size_t)r_page[j] * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size +
-                      pos % rp.page_size;
+                      (pos & (rp.page_size - 1));
         dst[(size_t)i * rp.page_size] = f32_to_bf16(x1);
         dst[(size_t)(i + 32) * rp.page_size] = f32_to_bf16(x2);
       }
@@ -1121,8 +1159,9 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
   if (head_dim != 64 || M > 16 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)all_heads * 64 * K * 2 >= ((size_t)1 << 31))
     return -7;
   MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
+  if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
-                 heads, kv_heads, page_size, table_stride, write_cache};
+                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size)};
   return launch_mid<EPI_QKV_ROPE, 1, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64, all_heads,
                                            (hipStream_t)stream, na, rp);
 }
@@ -1441,8 +1480,9 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
   if (head_dim != 64) return -4;
   if (K <= 0 || K > GEMM_SEG || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_qkv)) & 15) return -3;
+  if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
-                 heads, kv_heads, page_size, table_stride, write_cache};
+                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size)};
   if (M <= 64) {
     const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
     return mid == -7 ? -2 : mid;

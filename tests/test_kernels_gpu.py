@@ -552,6 +552,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
         w = (torch.randn((heads + 2 * kvh) * hd, K, generator=g) * 0.05).bfloat16().to(gpu)
         pos = [(r if r < M // 2 else r - M // 2 + 3) for r in range(M)]
         pos[7] = -1
+        pos[2] = -1                                                # padding rows, one the second of a pair of rows and one the first
         positions = torch.tensor(pos, dtype=torch.int32, device=gpu)
         row_seq = torch.tensor([0 if r < M // 2 else 1 for r in range(M)], dtype=torch.int32, device=gpu)
         per = (M + page - 1) // page + 2
