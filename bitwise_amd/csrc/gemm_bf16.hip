@@ -9,17 +9,32 @@
 // is added into a residual the chain starts there: y = ((res + p0) + p1) + ...  An output's bits
 // therefore depend only on its own row of x and row of W (and its own residual).
 //
-// Two kernels run this arithmetic.  The skinny one (up to 64 rows: decode) gives every
-// 16-column strip of W and every segment a wave of its own, which streams its 16 x 2048
-// weights once through a ring of operand registers kept full of loads in flight; the waves
-// of a strip join their segment results through LDS in segment order.  The wide one (prompt
-// portions) stages 128x64 tiles of x and W through LDS (double buffered, rows padded to 144
-// bytes so that 16-byte operand reads hit distinct banks) and gives each of four waves a
-// 64x64 block of outputs.
+// Several kernels run this arithmetic; which one is a matter of the shape alone (rows, columns, K), never of the
+// values, and they agree bit for bit (the tests compare them).  What bounds them all is how many bytes of loads
+// a compute unit keeps in flight and fetches through its L1, so each shape gets the kernel that fetches least:
+//   * up to 64 rows (decode steps, short prompt portions):
+//       - many columns: the "mid" kernel, a workgroup per 64 columns (32 of SwiGLU, or 32 where there are few
+//         columns and more than 16 rows), the rows of x shared by its four strips; optionally RMSNorm of up to 16
+//         rows fused in front (the rows normalised into LDS by the workgroup) and rotation + cache write behind;
+//         a residual add of 17 to 64 rows over several segments gives every segment workgroups of its own, which
+//         meet in device scratch and are added in segment order by the last to arrive;
+//       - up to 16 rows and few columns, or several segments: the "stream" kernel, a wave per strip and segment;
+//       - both stream weights and x through rings in LDS filled by buffer loads with LDS as their destination,
+//         8 rows of 128 bytes an instruction (whole cache lines; half lines cost nearly as much as whole ones),
+//         no registers in between, so the rings are deep; the 16-byte chunks of a row are permuted so that operand
+//         reads hit distinct banks; a wave waits for "all but the loads of the stages after this one", which
+//         works because loads complete in the order they are issued and nothing else is loaded meanwhile;
+//       - anything else (K no multiple of 64, SwiGLU with few columns): the "skinny" kernel, a wave per strip
+//         and segment streaming through a ring of registers;
+//   * more rows (prompt portions): 128 x 128 x 64 tiles staged through LDS by four or eight waves ("wide"), and
+//     for products with at least 128 tiles of 256 x 256 the "big" kernel, which computes twice as much per byte
+//     it fetches (buffer loads into a ring of five 32 KB slots in LDS, operand reads pipelined under the matrix
+//     instructions).
 //
 // Epilogues: store 32-bit, store bfloat16, add into a 32-bit residual (each output owned
-// by one lane: no atomics), or SwiGLU of two products (gate rows n, up rows N+n of a
-// stacked weight) stored as bfloat16: h = g * (1/(1+exp(-g))) * u in 32-bit.
+// by one lane: no atomics), SwiGLU of two products (gate rows n, up rows N+n of a
+// stacked weight) stored as bfloat16: h = g * (1/(1+exp(-g))) * u in 32-bit, or (heads of 64) rotary
+// encoding of the stacked q|k|v product and the write of k and v to their page slots.
 #include "common.h"
 #include "api.h"
 
