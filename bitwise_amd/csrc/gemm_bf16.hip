@@ -26,10 +26,12 @@
 //         works because loads complete in the order they are issued and nothing else is loaded meanwhile;
 //       - anything else (K no multiple of 64, SwiGLU with few columns): the "skinny" kernel, a wave per strip
 //         and segment streaming through a ring of registers;
-//   * more rows (prompt portions): 128 x 128 x 64 tiles staged through LDS by four or eight waves ("wide"), and
-//     for products with at least 128 tiles of 256 x 256 the "big" kernel, which computes twice as much per byte
-//     it fetches (buffer loads into a ring of five 32 KB slots in LDS, operand reads pipelined under the matrix
-//     instructions).
+//   * more rows (prompt portions): 128 x 128 x 64 tiles, eight waves, fed through a four-stage LDS ring by the
+//     same kind of loads ("tile128"), and for products with at least 128 tiles of 256 x 256 the "big" kernel,
+//     which computes twice as much per byte it fetches (a ring of five 32 KB slots, operand reads pipelined
+//     under the matrix instructions); the "wide" kernel (128 x 128 tiles staged through registers by four waves)
+//     takes what those do not: K no multiple of 64, several segments with another epilogue than the residual
+//     add, and the rotary epilogue below 512 rows.
 //
 // Epilogues: store 32-bit, store bfloat16, add into a 32-bit residual (each output owned
 // by one lane: no atomics), SwiGLU of two products (gate rows n, up rows N+n of a
@@ -521,126 +523,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         TOT, rp);
 }
 
-// The same tiles worked by eight waves (each 64 x 32 outputs), for products whose grid is too
-// small to give every compute unit two workgroups of four: two waves per SIMD inside one
-// workgroup, so that one wave's LDS traffic hides behind the other's matrix instructions.
-// K in whole double steps; epilogues store / bf16 / residual add (several segments: added into
-// the output segment by segment, the chain starting at the residual).
-template <int EPI>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_wide8_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles) {
-  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][WIDE_BM * WIDE_LDS_ROW];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][WIDE_BN * WIDE_LDS_ROW];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int r = lane & 15, g = lane >> 4;
-  const int wy = wave >> 2, wx = wave & 3;
-  int bid = blockIdx.x;
-  const int nblocks = m_tiles * n_tiles;
-  if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;
-  const int m0 = (bid % m_tiles) * WIDE_BM;
-  const int n0 = (bid / m_tiles) * WIDE_BN;
-  const int lr = tid >> 3, lc = tid & 7;             // rows lr, lr + 64; 16-byte chunk lc
-  const int a_rows = min(WIDE_BM, M - m0), b_rows = min(WIDE_BN, N - n0);
-  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rs_b =
-      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
-  const int voff_a = (lr * ldx + lc * 8) * 2, voff_b = (lr * K + lc * 8) * 2;
-
-  f32x4 acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  u32x4 ra[2][2], rb[2][2];
-  auto fetch = [&](int set, int k0) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      ra[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, voff_a, (64 * j * ldx + k0) * 2, 0);
-      rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_b, voff_b, (64 * j * K + k0) * 2, 0);
-    }
-  };
-  auto stash = [&](int set, int buf) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      *reinterpret_cast<u32x4*>(&lds_a[buf][(lr + 64 * j) * WIDE_LDS_ROW + lc * 8]) = ra[set][j];
-      *reinterpret_cast<u32x4*>(&lds_b[buf][(lr + 64 * j) * WIDE_LDS_ROW + lc * 8]) = rb[set][j];
-    }
-  };
-  auto fast_step = [&](int k0, int set_fetch, int buf) {
-    fetch(set_fetch, k0 + 2 * WIDE_BK);               // past K: outside the descriptors, zeros, never used
-    u32x4 fa[2][4], fb[2][2];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        fa[kk][i] = *reinterpret_cast<const u32x4*>(&lds_a[buf][(64 * wy + 16 * i + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        fb[kk][j] = *reinterpret_cast<const u32x4*>(&lds_b[buf][(32 * wx + 16 * j + r) * WIDE_LDS_ROW + kk * 32 + g * 8]);
-    }
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
-    stash(set_fetch ^ 1, buf ^ 1);
-    // 8 operand reads; 4 x [2 matrix instructions, 1 operand read, 1 global load]; 4 x [2 matrix instructions, 1 LDS write]
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    }
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    }
-    __syncthreads();
-  };
-  fetch(0, 0);
-  fetch(1, WIDE_BK);
-  stash(0, 0);
-  __syncthreads();
-  for (int k0 = 0; k0 < K; k0 += 2 * WIDE_BK) {
-    fast_step(k0, 0, 0);
-    fast_step(k0 + WIDE_BK, 1, 1);
-    if constexpr (EPI == EPI_ADD_F32) {
-      const int kn = k0 + 2 * WIDE_BK;
-      if (kn % GEMM_SEG == 0 && kn < K) {            // a segment ends before the last: add it into the output now
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 32 * wx + 16 * j + r;
-              if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] += acc[i][j][q];
-            }
-            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-          }
-      }
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int m = m0 + 64 * wy + 16 * i + 4 * g + q;
-      if (m >= M) continue;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int n = n0 + 32 * wx + 16 * j + r;
-        if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j][q]);
-      }
-    }
-}
-
 // ------------------------------------------------------------------------------ big tiles
 
 // 256 x 256 outputs a workgroup (256 x 128 of SwiGLU: 128 gate and 128 up rows of W), steps of 64
@@ -805,6 +687,148 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     asm volatile("" ::: "memory");
   }
   tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
+}
+
+// ------------------------------------------------------------------------------ 128 x 128 tiles through an LDS ring
+
+// 128 x 128 outputs a workgroup (128 x 64 of SwiGLU: 64 gate and 64 up rows of W), steps of 64 along K, eight waves
+// of 64 x 32 outputs each, for prompt portions whose product has too few tiles of 256 x 256 to go round.  Tiles
+// travel as in the big-tile kernel (buffer loads with LDS as destination, 8 rows of 128 bytes an instruction, chunks
+// permuted against bank conflicts); a stage is a step's tiles of x and W (32 KB), the ring has four, a wave issues
+// four loads a stage, and "all but the last 8 have landed" is the wait for the stage at hand; one barrier a step.
+// A residual add over several segments of K adds each finished segment into the output (the chain of additions
+// starts at the residual, segments in order).  K a multiple of 64; SwiGLU, store: one segment.
+#define T128_STAGE (32 * 1024)
+#define T128_STAGES 4
+
+__device__ __forceinline__ void t128_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
+                                           const int* voff_a, const int* voff_b, int wave, int step, int steps) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = lds + (step % T128_STAGES) * T128_STAGE + (2 * wave) * 1024;
+  const bool real = step < steps;                                     // scalar; past K: outside the descriptors
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 16 * 1024 + t * 1024), 16, real ? voff_b[t] : 0x7ffffff0,
+                                             step * 128, 0, 0);
+  }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile128_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
+    int ldo, int m_tiles, int n_tiles) {
+  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr int COLS = GLU ? 64 : 128;
+  extern __shared__ __attribute__((aligned(16))) unsigned char t128_lds[];   // [4 stages][x 16 KB | W 16 KB]
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int wy = wave >> 2, wx = wave & 3;
+  int bid = blockIdx.x;
+  const int nblocks = m_tiles * n_tiles;
+  if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;      // an n tile's workgroups share an XCD
+  const int m0 = (bid % m_tiles) * 128;
+  const int n0 = (bid / m_tiles) * COLS;
+  // this wave's loads of a stage: rows 16*wave .. 16*wave + 15 of x's 128 and of W's 128 (SwiGLU: W rows 0-63 of
+  // the tile are gate rows n0.., 64-127 the up rows N + n0..)
+  const int a_rows = min(128, M - m0), b_rows = min(COLS, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+  const bool up = GLU && wave >= 4;
+  const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int b_row0 = GLU ? 16 * (wave & 3) : 16 * wave;
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_a[2], voff_b[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int r16 = 8 * t + lrow;
+    const int chunk = lslot ^ (r16 >> 1);
+    voff_a[t] = ((16 * wave + r16) * ldx + 8 * chunk) * 2;
+    voff_b[t] = ((b_row0 + r16) * K + 8 * chunk) * 2;
+  }
+  f32x4 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  // operands: x row blocks 4*wy + i; W row blocks 2*wx + j, or in SwiGLU mode gate block wx (j = 0) and up block 4 + wx
+  const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
+  int slot_off[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
+  const int a_frag = (4 * wy) * 2048;
+  const int b_frag = 16 * 1024 + (GLU ? wx : 2 * wx) * 2048;
+  constexpr int b_step = GLU ? 4 * 2048 : 2048;                        // from the wave's first W block to its second
+  const int steps = K / 64;
+#pragma unroll
+  for (int st = 0; st < T128_STAGES - 1; ++st) t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(4 * (T128_STAGES - 2)));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, step + T128_STAGES - 1, steps);   // into the stage worked on a step ago
+    const unsigned char* stage = t128_lds + (step % T128_STAGES) * T128_STAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    // 12 operand reads and 16 matrix instructions a step, the second half's reads under the first half's products
+    u32x4 fa[2][4], fb[2][2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[kk][j] = *reinterpret_cast<const u32x4*>(stage + b_frag + j * b_step + slot_off[kk]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) fa[kk][i] = *reinterpret_cast<const u32x4*>(stage + a_frag + i * 2048 + slot_off[kk]);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int t = 0; t < 6; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 10, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    if constexpr (EPI == EPI_ADD_F32) {
+      const int kn = (step + 1) * 64;
+      if (kn % GEMM_SEG == 0 && kn < K) {              // a segment ends before the last: add it into the output now
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 32 * wx + 16 * j + r;
+              if (m < M && n < N) ((float*)out)[(size_t)m * ldo + n] += acc[i][j][q];
+            }
+            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = m0 + 64 * wy + 16 * i + 4 * g + q;
+      if (m >= M) continue;
+      if constexpr (GLU) {
+        const int n = n0 + 16 * wx + r;
+        if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][1][q]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = n0 + 32 * wx + 16 * j + r;
+          if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j][q]);
+        }
+      }
+    }
 }
 
 // ------------------------------------------------------------------------------ up to 64 rows, through LDS
@@ -1425,11 +1449,17 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
-    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_ADD_F32) {
-      // too few tiles for two workgroups of four waves per compute unit: eight waves a tile
-      // (and every residual add over several segments: it joins them in the output itself)
-      if (K % (2 * WIDE_BK) == 0 && ((S == 1 && m_tiles * n_tiles <= 256) || (S > 1 && EPI == EPI_ADD_F32))) {
-        hipLaunchKernelGGL((gemm_bf16_wide8_kernel<EPI>), grid, dim3(512), 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles);
+    if constexpr (EPI != EPI_QKV_ROPE) {
+      // K in whole steps of 64 (and one segment, or a residual add): the tiles go straight into an LDS ring
+      if (K % 64 == 0 && (S == 1 || EPI == EPI_ADD_F32)) {
+        static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_tile128_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    T128_STAGES * T128_STAGE);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI>), grid, dim3(512), T128_STAGES * T128_STAGE, s, x, w, out, M, N, K, ldx,
+                           ldo, m_tiles, n_tiles);
         return BW_LAUNCH_CHECK();
       }
     }
