@@ -149,6 +149,9 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
         }
       }
     }
+    // these loads stay here, before the ring's: the waits in the loop count the loads issued after a stage's own,
+    // and must find nothing but the ring's among them
+    asm volatile("" ::: "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
   // then the rows to normalise (their first batch)

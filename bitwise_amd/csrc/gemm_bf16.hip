@@ -984,6 +984,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         }
       }
     }
+    // these loads stay here, before the ring's: the waits in the loop count the loads issued after a stage's own,
+    // and must find nothing but the ring's among them
+    asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
   }
   unsigned char* rows_lds = mid_lds + S::RING;
