@@ -1164,7 +1164,7 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
                      int ldo, int M, int N, int K, int epilogue, void* stream) {
   const int cols = epilogue == EPI_SWIGLU_BF16 ? 32 : 64;
   const int wgs = (N + cols - 1) / cols;
-  if (M > 16 || K > GEMM_SEG || K % 64 || wgs < 64 || (size_t)2 * N * K * 2 >= ((size_t)1 << 31)) return -7;
+  if (M > 16 || K > GEMM_SEG || K % 64 || wgs < 64) return -7;
   MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
   const bf16_t* wp = (const bf16_t*)w;
   hipStream_t s = (hipStream_t)stream;
@@ -1182,8 +1182,7 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
 static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, void* q_out, int M, int K, const QkvRopeArgs& rp,
                                hipStream_t s) {
   const int all_heads = rp.heads + 2 * rp.kv_heads;
-  if (M > 64 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)all_heads * 64 * K * 2 >= ((size_t)1 << 31) ||
-      (size_t)M * ldx * 2 >= ((size_t)1 << 31))
+  if (M > 64 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31))
     return -7;
   const int N = all_heads * 64, ldo = rp.heads * 64;
   if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
@@ -1198,7 +1197,7 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
                          int table_stride, const float* cos_table, const float* sin_table, void* k_cache, void* v_cache, int M,
                          int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream) {
   const int all_heads = heads + 2 * kv_heads;
-  if (head_dim != 64 || M > 16 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)all_heads * 64 * K * 2 >= ((size_t)1 << 31))
+  if (head_dim != 64 || M > 16 || K > GEMM_SEG || K % 64 || all_heads < 64)
     return -7;
   MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
@@ -1372,7 +1371,8 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       // one segment and enough columns: the rows of x are shared through LDS
       constexpr int MID_COLS = (EPI == EPI_SWIGLU_BF16) ? 32 : 64;
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
-      const bool fits = (size_t)2 * N * K * 2 < ((size_t)1 << 31) && (size_t)M * ldx * 2 < ((size_t)1 << 31);
+      // (the descriptors of W cover a tile's rows each, so only the rows of x have to fit 31 bits of offset)
+      const bool fits = (size_t)M * ldx * 2 < ((size_t)1 << 31);
       if (S == 1 && K % 64 == 0 && wgs >= 64 && fits) {
         if (M <= 16) return launch_mid<EPI, 1, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         if (M <= 32) return launch_mid<EPI, 2, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
@@ -1399,7 +1399,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     }
     if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {
       // up to 16 rows: a wave per strip and segment, streaming through its own ring in LDS
-      if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)2 * N * K * 2 < ((size_t)1 << 31) && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+      if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
         if ((N + 15) / 16 < 256) return launch_stream<EPI, 8>(x, w, out, M, N, K, ldx, ldo, S, s);
         return launch_stream<EPI, 16>(x, w, out, M, N, K, ldx, ldo, S, s);
       }
@@ -1416,7 +1416,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     dim3 grid(half ? (N + 7) / 8 : strips, split_rows ? row_blocks : 1), block(64 * waves);
     const size_t lds = S > 1 ? (size_t)S * NB * wm * 4 * 64 * sizeof(float) : 0;
     if (lds > 64 * 1024) return -2;
-    if ((size_t)2 * N * K * 2 >= ((size_t)1 << 31) || (size_t)M * ldx * 2 >= ((size_t)1 << 31)) return -2;
+    if ((size_t)M * ldx * 2 >= ((size_t)1 << 31) || (size_t)16 * K * 2 >= ((size_t)1 << 31)) return -2;   // offsets within x, within a strip of W
 #define BW_SKINNY(WMV, DV, CWV)                                                                                    \
   if (K % 32)                                                                                                      \
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, true, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S); \

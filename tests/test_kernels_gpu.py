@@ -182,6 +182,25 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
                       torch.zeros(4, 12, device=gpu, dtype=torch.bfloat16), torch.zeros(2, 4, device=gpu), 2, ops.EPI_F32)
 
 
+def test_gemm_bf16_weight_beyond_two_gib(gpu):
+    """A weight of more than 2^31 bytes (a large vocabulary's head): every kernel addresses W through descriptors
+    of a tile's rows, so only the tile has to fit 32-bit offsets.  The first and last columns equal the product
+    with those rows of W alone, for a decode step, a short portion and a long one."""
+    N, K = 270000, 4096                                            # 2.2 GB
+    g = torch.Generator(device=gpu).manual_seed(3)
+    w = (torch.randn(N, K, device=gpu, generator=g) * 0.05).bfloat16()
+    for M in (3, 40, 300):
+        x = torch.randn(M, K, device=gpu, generator=g).bfloat16()
+        y = torch.zeros(M, N, device=gpu)
+        ops.gemm_bf16(x, w, y, M, ops.EPI_F32)
+        for lo in (0, N - 200):
+            part = torch.zeros(M, 200, device=gpu)
+            ops.gemm_bf16(x, w[lo:lo + 200].contiguous(), part, M, ops.EPI_F32)
+            assert torch.equal(part, y[:, lo:lo + 200]), (M, lo)
+        ref = x[:, :].double() @ w[N - 200:].double().T
+        assert (y[:, N - 200:].double() - ref).abs().max() <= 2e-6 * K ** 0.5 * ref.abs().max()
+
+
 # ----------------------------------------------------------------------------- row kernels
 
 def test_rmsnorm(gpu):
