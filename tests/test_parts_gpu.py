@@ -244,6 +244,107 @@ def test_toy_mixer_with_state_and_a_schedule_that_repeats_and_shares(gpu, mode):
     assert np.abs(lg - ref["b"]).max() <= (2e-2 if mode == "bfloat16" else 2e-5) * np.abs(ref["b"]).max()
 
 
+# ----------------------------------------------------------------------------- a toy routed feed-forward, a toy position encoding
+
+@base.register_feed_forward("toy_top1")
+class TopOneExperts(base.FeedForward):
+    """Two square experts and a router: every row goes through the expert whose router logit (32-bit) is larger,
+    ties to the first.  The choice depends on the row alone, so it does not matter what else is in the batch."""
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.width = params["width"]
+
+    def tensors(self):
+        return {"router.weight": TensorSpec((2, self.width)), "experts.0.weight": TensorSpec((self.width, self.width)),
+                "experts.1.weight": TensorSpec((self.width, self.width))}
+
+    def bind(self, tensors):
+        self.router = tensors["router.weight"].to(self.rt.device).float()
+        self.experts = [tensors[f"experts.{e}.weight"].to(self.rt.device).float() for e in range(2)]
+
+    def forward(self, ctx, h, residual):
+        rows = h[:ctx.rows].float()
+        logits = rows @ self.router.T
+        second = logits[:, 1] > logits[:, 0]
+        out = torch.where(second[:, None], rows @ self.experts[1].T, rows @ self.experts[0].T)
+        residual[:ctx.rows] += out
+
+
+@base.register_position_encoding("toy_stretched_rope")
+class StretchedRotary(base.PositionEncoding):
+    """Rotary angles of position / stretch (positions interpolated): the tables a mixer's kernels read, built by
+    another rule.  params: theta, head_dim, max_positions, stretch."""
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        hd, n = int(params["head_dim"]), int(params["max_positions"])
+        inv = pl.rope_inv_freq(float(params["theta"]), hd)
+        places = (np.arange(n, dtype=np.float32) / np.float32(params["stretch"]))[:, None]
+        angle = (places * inv[None, :]).astype(np.float32).astype(np.float64)
+        self.cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(runtime.device).contiguous()
+        self.sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(runtime.device).contiguous()
+
+    @classmethod
+    def shared(cls, params, runtime):
+        return cls(params, runtime)
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_another_position_encoding(gpu, mode):
+    """A model of one layer whose feed-forward routes rows between two experts and whose attention reads the tables
+    of a position encoding defined here: registered, built, stepped in portions and compared with plain code; nothing
+    in the framework's files knows of either."""
+    width, vocab, hd, stretch = 32, 40, 16, 4.0
+    pos = PartSpec("toy_stretched_rope", {"theta": 1000.0, "head_dim": hd, "max_positions": 64, "stretch": stretch})
+    attn = PartSpec("attention", {"width": width, "heads": 2, "kv_heads": 2, "head_dim": hd, "window": None, "position": pos},
+                    "l.attn.")
+    layer = LayerSpec("prenorm", attn, PartSpec("toy_top1", {"width": width}, "l.moe."),
+                      PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm1."),
+                      PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm2."))
+    spec = ModelSpec("ToyRouted", vocab, width, PartSpec("embedding", {"vocab": vocab, "width": width}, "embed."), [layer],
+                     [LayerCall(0, 0)], PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "norm."),
+                     PartSpec("lm_head", {"vocab": vocab, "width": width, "tied": True}, "head."), 64)
+    rt = Runtime(mode, gpu, max_rows=32, page_size=8)
+    model = AssembledModel(spec, rt)
+    w = dict(random_tensors(model.tensor_specs(), 17, 0.3))
+    model.bind_tensors({k: v.to(gpu) for k, v in w.items()})
+    storage = CacheStorage(model, num_pages=8, num_slots=2)
+    manager = CacheManager([GroupSpec(None)], 8, 8, 2, prefix_caching=False)
+    runner = ModelRunner(model, storage, max_model_len=64, use_graphs=False)
+    toks = [int(t) for t in torch.randint(0, vocab, (21,), generator=torch.Generator().manual_seed(5))]
+    rnd = rnd_for(mode)
+
+    # plain: whole sequence, the toy parts written out again
+    n = len(toks)
+    x = pl.embed(toks, w["embed.weight"])
+    hn = rnd(pl.rmsnorm(x, w["l.norm1.weight"], 1e-5))
+    inv = pl.rope_inv_freq(1000.0, hd)
+    places = [p / stretch for p in range(n)]
+    q = rnd(pl.rope(pl.linear(hn, w["l.attn.q_proj.weight"]).view(n, 2, hd), places, inv))
+    k = rnd(pl.rope(pl.linear(hn, w["l.attn.k_proj.weight"]).view(n, 2, hd), places, inv))
+    v = rnd(pl.linear(hn, w["l.attn.v_proj.weight"]).view(n, 2, hd))
+    x = x + pl.linear(rnd(pl.attention(q, k, v, rnd)).reshape(n, -1), w["l.attn.o_proj.weight"])
+    hn = rnd(pl.rmsnorm(x, w["l.norm2.weight"], 1e-5))
+    logits = hn.float().double() @ w["l.moe.router.weight"].double().T
+    chosen = (logits[:, 1] > logits[:, 0]).long()
+    assert 0 < int(chosen.sum()) < n                                # both experts get rows
+    experts = [w[f"l.moe.experts.{e}.weight"].double() for e in range(2)]
+    x = x + torch.stack([hn[i].double() @ experts[int(chosen[i])].T for i in range(n)])
+    ref = pl.linear(rnd(pl.rmsnorm(x, w["norm.weight"], 1e-5)), w["embed.weight"]).numpy()
+
+    rc = manager.open()
+    got, done = [], 0
+    for cut in (8, 1, 5, 7):
+        assert manager.ensure(rc, done + cut)
+        lg = runner.step([Segment(toks[done:done + cut], done, rc.tables, rc.slot, list(range(cut)))])
+        got.append(lg.cpu().numpy())
+        done += cut
+        manager.advance(rc, toks, done)
+    out = np.concatenate(got)
+    assert np.abs(out - ref).max() <= (2e-2 if mode == "bfloat16" else 2e-5) * np.abs(ref).max()
+
+
 def test_schedule_errors(gpu):
     rt = Runtime("float32", gpu, max_rows=16, page_size=8)
     spec = toy_spec()
