@@ -61,7 +61,9 @@ class CacheManager:
             for page in table:
                 if page >= 0:
                     pool.release(page)
-            table.clear()
+        # new lists, not cleared ones: a table only ever grows at its end while it is the same object (the step
+        # function's host copy of a block table relies on that)
+        rc.tables = [[] for _ in self.pools]
         rc.hashes.clear()
         rc.computed = 0
 

@@ -53,6 +53,9 @@ class _StaticDecodeContext:
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
         self.segments: List[Segment] = []
+        # what the host copy of each block-table row was last filled from: (the request's list, its length then);
+        # a request's list only grows at its end from step to step, so mostly there is nothing or one entry to write
+        self._row_source = [[(None, 0)] * size for _ in range(num_groups)]
 
     def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
         return self._plan
@@ -75,10 +78,18 @@ class _StaticDecodeContext:
         base = 3 * size
         for g in range(len(self.block_tables)):
             t = h[base + g * size * self.max_pages:base + (g + 1) * size * self.max_pages].reshape(size, self.max_pages)
+            source = self._row_source[g]
             for i, s in enumerate(segments):
                 row = s.tables[g]
-                t[i, :len(row)] = row
-            np.maximum(t[:n], 0, out=t[:n])  # pages given back (-1) are never read
+                was, had = source[i]
+                if was is row and had <= len(row):
+                    lo = had                        # the same request as last step: only what it got since
+                else:
+                    lo = 0
+                if lo < len(row):
+                    # pages given back (-1; outside the window, never read) become 0: any valid page number
+                    t[i, lo:len(row)] = [p if p > 0 else 0 for p in row[lo:]]
+                    source[i] = (row, len(row))
         self._dev.copy_(self._host, non_blocking=True)
 
 
