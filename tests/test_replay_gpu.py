@@ -207,3 +207,57 @@ def test_trace_run_program(folders, tmp_path):
         assert got.shape[0] == len(rows)
         for g, r in zip(got, rows):
             assert np.abs(g - r).max() <= TOL[dtype] * np.abs(r).max()
+
+
+def test_real_layer_sizes_are_cut_invariant(gpu):
+    """Two layers of the SmolLM2-1.7B sizes, so that every shape-dependent route of the kernels runs at the shapes it
+    was written for (K = 2048 and 8192, 6144 / 2048 / 16384 / 49152 columns): a prompt whole; in portions of 1600, 300,
+    100, 61, 29 and 10 tokens; with its last 40 tokens decoded one by one from graphs; and decoded beside 8 and then 19
+    other requests.  The logits of the last 40 positions are the same bits every time."""
+    import bitwise_amd as bw
+    from bitwise_amd.replay import Replayer
+
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "vocab_size": 49152,
+           "hidden_size": 2048, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 32,
+           "head_dim": 64, "intermediate_size": 8192, "rope_theta": 130000.0, "rms_norm_eps": 1e-5,
+           "tie_word_embeddings": True, "max_position_embeddings": 4096, "bos_token_id": 1, "eos_token_id": 2}
+    model = bw.Model.random(cfg, seed=3, dtype="bfloat16", sigma=0.02, on_device=True)
+    g = torch.Generator().manual_seed(11)
+    toks = torch.randint(0, 49152, (2100,), generator=g).tolist()
+    others = {f"o{i}": torch.randint(0, 49152, (30,), generator=g).tolist() for i in range(19)}
+    tail = 40
+    head = len(toks) - tail
+
+    def last(rp_steps, max_tokens=4096):
+        rp = Replayer("", "bfloat16", max_tokens, block_size=16, model=model)
+        rows = []
+        for st in rp_steps:
+            lg = rp.step(st["entries"], st.get("end", []))
+            row = 0
+            for e in st["entries"]:
+                for _ in e["want"]:
+                    if e["id"] == "r":
+                        rows.append(lg[row].copy())
+                    row += 1
+        return np.stack(rows)
+
+    whole = last([{"entries": [{"id": "r", "tokens": toks, "want": list(range(head, len(toks)))}]}])
+    assert whole.shape == (tail, 49152) and np.isfinite(whole).all()
+    steps, pos = [], 0
+    for n in (1600, 300, 100, 61, 29, 10):
+        want = [i - pos for i in range(max(pos, head), pos + n)]
+        steps.append({"entries": [{"id": "r", "tokens": toks[pos:pos + n], "want": want}]})
+        pos += n
+    assert np.array_equal(last(steps), whole), "portions of 1600, 300, 100, 61, 29, 10"
+    one = [{"entries": [{"id": "r", "tokens": toks[:head + 1], "want": [head]}]}]
+    one += [{"entries": [{"id": "r", "tokens": [t], "want": [0]}]} for t in toks[head + 1:]]
+    assert np.array_equal(last(one), whole), "last tokens one by one"
+    for crowd in (8, 19):
+        names = list(others)[:crowd]
+        mixed = [{"entries": [{"id": "r", "tokens": toks[:head + 1], "want": [head]}] +
+                             [{"id": n, "tokens": others[n], "want": []} for n in names]}]
+        for j, t in enumerate(toks[head + 1:]):
+            mixed.append({"entries": [{"id": n, "tokens": [others[n][j % 30]], "want": [0]} for n in names[:crowd // 2]] +
+                                     [{"id": "r", "tokens": [t], "want": [0]}] +
+                                     [{"id": n, "tokens": [others[n][j % 30]], "want": [0]} for n in names[crowd // 2:]]})
+        assert np.array_equal(last(mixed, max_tokens=8192), whole), f"decoded beside {crowd} others"
