@@ -36,15 +36,24 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
   int best_i = 0x7fffffff;
   if ((vocab & 3) == 0 && (ld & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
     const f32x4* lv = reinterpret_cast<const f32x4*>(l);
-    for (int v = tid; v < (vocab >> 2); v += SMP_THREADS) {
-      const f32x4 x = lv[v];
+    const int nv = vocab >> 2;
+    auto scan = [&](const f32x4& x, int v) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (x[e] > best || best_i == 0x7fffffff) {  // the share's first element, or strictly greater
           best = x[e];
           best_i = 4 * v + e;
         }
+    };
+    int v = tid;
+    for (; v + 3 * SMP_THREADS < nv; v += 4 * SMP_THREADS) {   // four loads in flight, scanned in ascending order
+      const f32x4 x0 = lv[v], x1 = lv[v + SMP_THREADS], x2 = lv[v + 2 * SMP_THREADS], x3 = lv[v + 3 * SMP_THREADS];
+      scan(x0, v);
+      scan(x1, v + SMP_THREADS);
+      scan(x2, v + 2 * SMP_THREADS);
+      scan(x3, v + 3 * SMP_THREADS);
     }
+    for (; v < nv; v += SMP_THREADS) scan(lv[v], v);
   } else {
     for (int i = tid; i < vocab; i += SMP_THREADS)
       if (l[i] > best || best_i == 0x7fffffff) {
