@@ -697,7 +697,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // permuted against bank conflicts); a stage is a step's tiles of x and W (32 KB), the ring has four, a wave issues
 // four loads a stage, and "all but the last 8 have landed" is the wait for the stage at hand; one barrier a step.
 // A residual add over several segments of K adds each finished segment into the output (the chain of additions
-// starts at the residual, segments in order).  K a multiple of 64; SwiGLU, store: one segment.
+// starts at the residual, segments in order); the other epilogues join the segments' sums left to right in
+// registers.  K a multiple of 64.
 #define T128_STAGE (32 * 1024)
 #define T128_STAGES 4
 
@@ -747,11 +748,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     voff_a[t] = ((16 * wave + r16) * ldx + 8 * chunk) * 2;
     voff_b[t] = ((b_row0 + r16) * K + 8 * chunk) * 2;
   }
-  f32x4 acc[4][2];
+  f32x4 acc[4][2], tot[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 2; ++j) {
+      acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
   // operands: x row blocks 4*wy + i; W row blocks 2*wx + j, or in SwiGLU mode gate block wx (j = 0) and up block 4 + wx
   const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
   int slot_off[2];
@@ -810,7 +814,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
           }
       }
+    } else {
+      const int kn = (step + 1) * 64;
+      if (kn % GEMM_SEG == 0 && kn < K) {              // a segment ends before the last: joined left to right
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
+            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          }
+      }
     }
+  }
+  if (EPI != EPI_ADD_F32 && K > GEMM_SEG) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = tot[i][j] + acc[i][j];
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -944,13 +965,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     const int chunk = lslot ^ ((row & 15) >> 1);
     voff_b[t] = (((GLU ? row & 31 : row)) * K + 8 * chunk) * 2;
   }
-  const int k_base = blockIdx.y * GEMM_SEG;                           // gridDim.y > 1: this workgroup's segment of K
-  const int steps = ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64;
-  f32x4 acc[NI][NJ];
+  // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
+  // segment after segment, each segment's sums joined to those before it when it ends
+  const int k_base = blockIdx.y * GEMM_SEG;
+  const int steps = gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64;
+  f32x4 acc[NI][NJ], tot[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; ++j) {
+      acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
   // lane (g, r) wants row r of a block of 16 rows (2 KB), chunk 4*kk + g: slot (4*kk + g) ^ (r >> 1) of that row
   const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
   int slot_off[2];
@@ -1049,6 +1075,26 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
     }
     asm volatile("" ::: "memory");
+    if constexpr (EPI != EPI_QKV_ROPE && !NORM) {
+      const int kn = (step + 1) * 64;
+      if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {            // a segment ends before the last: left to right
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) {
+            tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
+            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          }
+      }
+    }
+  }
+  if constexpr (EPI != EPI_QKV_ROPE && !NORM) {
+    if (K > GEMM_SEG && gridDim.y == 1) {                               // the last segment joins the others
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) acc[i][j] = tot[i][j] + acc[i][j];
+    }
   }
   if constexpr (EPI == EPI_QKV_ROPE) {
     // The rotary pairs (i, i + 32) sit in different waves: the 32-bit products meet in LDS.  Heads come in the
@@ -1373,7 +1419,8 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
       // (the descriptors of W cover a tile's rows each, so only the rows of x have to fit 31 bits of offset)
       const bool fits = (size_t)M * ldx * 2 < ((size_t)1 << 31);
-      if (S == 1 && K % 64 == 0 && wgs >= 64 && fits) {
+      // (a residual add of several segments starts its chain at the residual: the kernels further down do that)
+      if ((S == 1 || EPI != EPI_ADD_F32) && K % 64 == 0 && wgs >= 64 && fits) {
         if (M <= 16) return launch_mid<EPI, 1, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         if (M <= 32) return launch_mid<EPI, 2, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
         return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, wgs, s);
@@ -1453,8 +1500,8 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
     if constexpr (EPI != EPI_QKV_ROPE) {
-      // K in whole steps of 64 (and one segment, or a residual add): the tiles go straight into an LDS ring
-      if (K % 64 == 0 && (S == 1 || EPI == EPI_ADD_F32)) {
+      // K in whole steps of 64: the tiles go straight into an LDS ring
+      if (K % 64 == 0) {
         static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
         if (!allowed) {
           (void)hipFuncSetAttribute((const void*)gemm_bf16_tile128_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -157,18 +157,18 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
     # SwiGLU with many columns (x shared through LDS; one, two or four blocks of 16 rows): the plain result, and
     # the bits of the same rows inside a prompt portion's product (another kernel)
-    inter, K = 2100, 128
-    wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
-    xl = torch.randn(200, K, generator=g).bfloat16().to(gpu)
-    big = torch.zeros(200, inter, device=gpu, dtype=torch.bfloat16)
-    ops.gemm_bf16(xl, wgu, big, 200, ops.EPI_SWIGLU_BF16)
-    gate, up = xl.double() @ wgu[:inter].double().T, xl.double() @ wgu[inter:].double().T
-    want = pl.swiglu(gate.cpu(), up.cpu())
-    assert (big.cpu().double() - want).abs().max() <= 2 ** -8 * want.abs().max()
-    for M in (1, 13, 16, 29, 41, 64):
-        hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
-        ops.gemm_bf16(xl[100:100 + M].contiguous(), wgu, hb, M, ops.EPI_SWIGLU_BF16)
-        assert torch.equal(hb, big[100:100 + M]), M
+    for inter, K in ((2100, 128), (2100, 2048 + 128)):             # the second: two segments of K
+        wgu = (torch.randn(2 * inter, K, generator=g) * (0.5 if K > 2048 else 1.0)).bfloat16().to(gpu)
+        xl = torch.randn(200, K, generator=g).bfloat16().to(gpu)
+        big = torch.zeros(200, inter, device=gpu, dtype=torch.bfloat16)
+        ops.gemm_bf16(xl, wgu, big, 200, ops.EPI_SWIGLU_BF16)
+        gate, up = xl.double() @ wgu[:inter].double().T, xl.double() @ wgu[inter:].double().T
+        want = pl.swiglu(gate.cpu(), up.cpu())
+        assert (big.cpu().double() - want).abs().max() <= 2 ** -8 * want.abs().max()
+        for M in (1, 13, 16, 29, 41, 64):
+            hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
+            ops.gemm_bf16(xl[100:100 + M].contiguous(), wgu, hb, M, ops.EPI_SWIGLU_BF16)
+            assert torch.equal(hb, big[100:100 + M]), (M, K)
     M, inter, K = 19, 56, 96
     x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
