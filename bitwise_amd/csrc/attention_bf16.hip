@@ -520,17 +520,31 @@ __device__ __forceinline__ void stage_store(const WorkgroupCtx& wc, const StageP
   }
 }
 
+// Which piece of work (0 = the group of the last tiles, the longest of a prompt; consecutive ranks = the heads of
+// one group) the workgroup with this index takes.  Workgroups go to the 8 dies of the chip in turn, and on a die
+// to its 32 compute units in turn; a prompt's groups often all fit the chip at once, and then what a compute unit
+// gets in its first and in its second turn should add up to the same everywhere: the ranks run forward over the
+// compute units in even turns and backward in odd ones, so a long piece meets a short one.
+__device__ __forceinline__ int fold_work_rank(int index, int count) {
+  if (count % 8 != 0) return index;
+  const int die = index & 7, j = index >> 3, per_die = count >> 3;
+  const int turn = j >> 5, cu = j & 31;
+  const int in_turn = min(32, per_die - 32 * turn);
+  return (32 * turn + ((turn & 1) ? in_turn - 1 - cu : cu)) * 8 + die;
+}
+
 template <int HD>
-__global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves_per_eu(FoldShape<HD>::WAVES, FoldShape<HD>::WAVES))) void attention_fold_kernel(AttnBf16Args a) {
+__global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves_per_eu(FoldShape<HD>::WAVES, FoldShape<HD>::WAVES))) void attention_fold_kernel(AttnBf16Args a, int groups, int items) {
   using S = FoldShape<HD>;
   constexpr int NT = HD / 16, KS = (HD + 31) / 32, QT = S::QT, NW = S::NW;
   extern __shared__ __align__(16) unsigned char lds[];
   __shared__ int ranges[2 * NW];
   const int wave = wave_index();
-  const int first_tile = (int)(gridDim.x - 1 - blockIdx.x) * S::GROUP;
+  const int rank = fold_work_rank((int)blockIdx.x, (int)gridDim.x);
+  const int first_tile = (groups - 1 - rank / items) * S::GROUP;
   GroupCtx gc;
   TileCtx<HD> tc[QT];
-  const bool live = group_setup<HD, QT>(a, first_tile + wave * QT, blockIdx.y, gc, tc);
+  const bool live = group_setup<HD, QT>(a, first_tile + wave * QT, rank % items, gc, tc);
   if (gc.lane == 0) {
     ranges[2 * wave] = live ? gc.kmin : 0x7fffffff;
     ranges[2 * wave + 1] = live ? gc.kmax : -1;
@@ -849,8 +863,8 @@ static int launch_attention(const AttnBf16Args& a, int decode, float* scratch, s
       (void)hipFuncSetAttribute((const void*)attention_fold_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       allowed = true;
     }
-    hipLaunchKernelGGL((attention_fold_kernel<HD>), dim3((a.num_tiles + S::GROUP - 1) / S::GROUP, items), dim3(64 * S::NW),
-                       lds_bytes, s, a);
+    const int groups = (a.num_tiles + S::GROUP - 1) / S::GROUP;
+    hipLaunchKernelGGL((attention_fold_kernel<HD>), dim3(groups * items), dim3(64 * S::NW), lds_bytes, s, a, groups, items);
   }
   return 0;
 }
