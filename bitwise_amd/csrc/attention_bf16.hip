@@ -384,9 +384,15 @@ __device__ __forceinline__ void fold(float& m, float& l, f32x4 (&o)[NT], float m
   fold_scalars(m, m_p, mn, fa, fb);
   l = fmaf(l, fa, l_p * fb);
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[dt][i] = fmaf(o[dt][i], fa, o_p[dt][i] * fb);
+  for (int dt = 0; dt < NT; ++dt) {
+    // o = fmaf(o, fa, o_p * fb), the fused multiply-add written out in its three-address form: the compiler picks
+    // the two-address one, whose result lands in the product's register, and then moves every element back to
+    // where the loop keeps the state.  (The wait state in front: fa may come straight from the exponential unit.)
+    const f32x4 t = {o_p[dt][0] * fb, o_p[dt][1] * fb, o_p[dt][2] * fb, o_p[dt][3] * fb};
+    asm("s_nop 0\n\tv_fma_f32 %0, %0, %4, %5\n\tv_fma_f32 %1, %1, %4, %6\n\tv_fma_f32 %2, %2, %4, %7\n\tv_fma_f32 %3, %3, %4, %8"
+        : "+v"(o[dt][0]), "+v"(o[dt][1]), "+v"(o[dt][2]), "+v"(o[dt][3])
+        : "v"(fa), "v"(t[0]), "v"(t[1]), "v"(t[2]), "v"(t[3]));
+  }
   m = mn;
 }
 
@@ -487,13 +493,17 @@ template <int HD>
 __device__ __forceinline__ void stage_load(const AttnBf16Args& a, const StagePlan<HD>& sp, const StagePages<HD>& pg,
                                            Staged<HD>& sg) {
   using S = FoldShape<HD>;
-  const size_t kpage = (size_t)a.kv_heads * a.page_size * HD;   // values: the same number of elements
+  // (a page's bytes fit 32 bits, so page * bytes is one 32 x 32 -> 64-bit multiply-add onto the chunk's base)
+  const unsigned page_bytes = (unsigned)(a.kv_heads * a.page_size * HD) * 2u;   // values: the same number of elements
+  const unsigned last_page = (unsigned)(a.num_pages - 1);
 #pragma unroll
   for (int j = 0; j < S::KJ; ++j)
-    sg.k[j] = *reinterpret_cast<const u32x4*>(a.k_cache + clamp_page(a, pg.k[j]) * kpage + sp.k_off[j]);
+    sg.k[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(a.k_cache + sp.k_off[j]) +
+                                              (unsigned long long)min((unsigned)pg.k[j], last_page) * page_bytes);
 #pragma unroll
   for (int j = 0; j < S::VJ; ++j)
-    sg.v[j] = *reinterpret_cast<const u32x2*>(a.v_cache + clamp_page(a, pg.v[j]) * kpage + sp.v_off[j]);
+    sg.v[j] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const unsigned char*>(a.v_cache + sp.v_off[j]) +
+                                              (unsigned long long)min((unsigned)pg.v[j], last_page) * page_bytes);
 }
 
 // Staged partition -> LDS; in a partition that is not wholly live the stale keys' values are zeroed.
@@ -914,6 +924,7 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   if (!(scale > 0.0f)) return -2;                // the maximum is taken before the scaling
   a.scale_log2 = scale * 1.44269504088896340736f;
   if (kv_heads * a.nsub > 65535) return -2;
+  if ((long long)kv_heads * page_size * head_dim * 2 >= (1ll << 31)) return -2;    // a page's bytes as a 32-bit factor
   hipStream_t s = (hipStream_t)stream;
   int rc = 0;
 #define BW_CASE(HD) case HD: rc = launch_attention<HD>(a, decode, scratch, (size_t)scratch_floats, counters, num_counters, s); break;

@@ -888,12 +888,13 @@ struct MidShape {
   static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STAGE = A_BYTES + B_ROWS * 128;
   static constexpr int NI = HALVES ? (NRB >= 2 ? NRB / 2 : 1) : NRB; // blocks of rows a wave works on
   static constexpr int NJ = GLU ? 2 : 1;
-  static constexpr int STAGES = 8;
+  static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
+  static constexpr int STAGES = ROPE_NARROW && NRB <= 2 ? 16 : 8;   // (half the weights a stage: twice the stages, where they fit)
   static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
   static constexpr int RING = STAGES * STAGE + 1024;                // and 1 KB where padding loads put their zeros
   static_assert(PENDING < 64, "the wait count has six bits");
   static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
-  static_assert(!NARROW || (!GLU && EPI != EPI_QKV_ROPE && NRB >= 2), "narrow tiles are for plain epilogues and 17 rows or more");
+  static_assert(!NARROW || (!GLU && (EPI == EPI_QKV_ROPE || NRB >= 2)), "narrow tiles: plain epilogues of 17 rows or more, or the rotary one");
 };
 
 // Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
@@ -942,8 +943,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * COLS;
-  const int b_rows = min(COLS, N - n0);
+  // rotary epilogue with narrow tiles: workgroup 2h + q has columns 16q..16q+15 and 32+16q..32+16q+15 of head h,
+  // 16 whole rotary pairs, as rows 0-15 and 16-31 of its tile of W
+  constexpr bool RN = S::ROPE_NARROW;
+  const int n0 = RN ? (blockIdx.x >> 1) * 64 : blockIdx.x * COLS;
+  const int b_rows = RN ? 64 : min(COLS, N - n0);
   const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)x, 0, NORM ? 0 : (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
   // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
@@ -963,7 +967,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   for (int t = 0; t < S::B_LOADS; ++t) {
     const int row = b_first + 8 * t + lrow;
     const int chunk = lslot ^ ((row & 15) >> 1);
-    voff_b[t] = (((GLU ? row & 31 : row)) * K + 8 * chunk) * 2;
+    const int w_row = RN ? 16 * (blockIdx.x & 1) + row + (row >= 16 ? 16 : 0) : (GLU ? row & 31 : row);
+    voff_b[t] = (w_row * K + 8 * chunk) * 2;
   }
   // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
   // segment after segment, each segment's sums joined to those before it when it ends
@@ -986,32 +991,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   const int a_block0 = S::HALVES ? NI * (wave >> 1) : 0;              // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
 
-  // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's 64 columns are head blockIdx.x):
-  // what this thread's (row, pair) items need is asked for first of all, positions and then what depends on
-  // them, so that no load of the kernel other than weights is issued after the ring's (see the waits below).
-  constexpr int ITEMS = EPI == EPI_QKV_ROPE ? 2 * NRB : 1;           // (row, pair) items a thread: 16 * NRB rows x 32 pairs
+  // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's columns are a head, or 16 pairs of
+  // one): what this thread's (row, pair) items need, cosine, sine and page, hangs on the row's position.
+  constexpr int PAIRS = RN ? 16 : 32, PSH = RN ? 4 : 5;              // rotary pairs of a row in this tile
+  constexpr int ITEMS = EPI == EPI_QKV_ROPE ? (RN ? NRB : 2 * NRB) : 1;   // (row, pair) items a thread: 16 * NRB rows x PAIRS
+  const int pair0 = RN ? 16 * (blockIdx.x & 1) : 0;                  // the tile's first pair within the head
   int r_pos[ITEMS], r_page[ITEMS];
   float r_cos[ITEMS], r_sin[ITEMS];
   if constexpr (EPI == EPI_QKV_ROPE) {
+    // the positions are asked for first of all; what depends on them (two loads in a row cost two trips to memory)
+    // is asked for once the ring is under way
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int e = threadIdx.x + j * 256;
-      r_pos[j] = -1;
-      r_page[j] = 0;
-      r_cos[j] = 1.f;
-      r_sin[j] = 0.f;
-      if (e < M * 32) {
-        const int pos = rp.positions[e >> 5];
-        r_pos[j] = pos;
-        if (pos >= 0) {
-          r_cos[j] = rp.cos_table[(size_t)pos * 32 + (e & 31)];
-          r_sin[j] = rp.sin_table[(size_t)pos * 32 + (e & 31)];
-          r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> 5] * rp.table_stride + (pos >> rp.page_shift)];
-        }
-      }
+      r_pos[j] = e < M * PAIRS ? rp.positions[e >> PSH] : -1;
     }
-    // these loads stay here, before the ring's: the waits in the loop count the loads issued after a stage's own,
-    // and must find nothing but the ring's among them
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -1053,6 +1047,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   } else {
 #pragma unroll
     for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
+  }
+  if constexpr (EPI == EPI_QKV_ROPE) {
+    // These loads are younger than the ring's first stages: the loop's waits ("all but the last PENDING loads have
+    // landed") ask for a little more than the stage at hand until these have landed too, never for less.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const int e = threadIdx.x + j * 256;
+      const int pos = r_pos[j];
+      r_page[j] = 0;
+      r_cos[j] = 1.f;
+      r_sin[j] = 0.f;
+      if (pos >= 0) {
+        r_cos[j] = rp.cos_table[(size_t)pos * 32 + pair0 + (e & (PAIRS - 1))];
+        r_sin[j] = rp.sin_table[(size_t)pos * 32 + pair0 + (e & (PAIRS - 1))];
+        r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> PSH] * rp.table_stride + (pos >> rp.page_shift)];
+      }
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   }
   for (int step = 0; step < steps; ++step) {
     __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));
@@ -1101,23 +1116,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     // order q heads, k heads, v heads; q rotated to its buffer, k rotated and v as it is to the row's page slot.
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                       // the padding loads have landed: LDS is free
     __syncthreads();
-    float* os = reinterpret_cast<float*>(mid_lds);                    // [M][64]
+    float* os = reinterpret_cast<float*>(mid_lds);                    // [M][2 * PAIRS]: a row's first halves of the pairs, then the second
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int m = 16 * i + 4 * g + q;
-        if (m < M) os[m * 64 + 16 * wave + r] = acc[i][0][q];
+        const int m = 16 * (a_block0 + i) + 4 * g + q;
+        if (m < M) os[m * 2 * PAIRS + 16 * strip + r] = acc[i][0][q];
       }
     __syncthreads();
-    const int head = blockIdx.x;
+    const int head = RN ? blockIdx.x >> 1 : blockIdx.x;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int e = threadIdx.x + j * 256;
       const int pos = r_pos[j];
-      if (e >= M * 32 || pos < 0) continue;
-      const int m = e >> 5, i = e & 31;
-      const float x1 = os[m * 64 + i], x2 = os[m * 64 + i + 32];
+      if (e >= M * PAIRS || pos < 0) continue;
+      const int m = e >> PSH, ip = e & (PAIRS - 1), i = pair0 + ip;
+      const float x1 = os[m * 2 * PAIRS + ip], x2 = os[m * 2 * PAIRS + ip + PAIRS];
       if (head < rp.heads + rp.kv_heads) {
         const float c = r_cos[j], sn = r_sin[j];
         const float o1 = x1 * c - x2 * sn;
@@ -1223,6 +1238,8 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
   return -7;
 }
 
+#define ROPE_NARROW_BELOW 256
+
 // The stacked q|k|v product of up to 64 normalised rows with rotation and cache write in its epilogue, for heads of
 // 64 and at least 64 of them (a workgroup a head); -7: not this shape.
 static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, void* q_out, int M, int K, const QkvRopeArgs& rp,
@@ -1231,6 +1248,11 @@ static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, vo
   if (M > 64 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31))
     return -7;
   const int N = all_heads * 64, ldo = rp.heads * 64;
+  if (all_heads < ROPE_NARROW_BELOW) {                 // fewer heads than compute units: half a head a workgroup
+    if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
+    if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
+    return launch_mid<EPI_QKV_ROPE, 4, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
+  }
   if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
   if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
   return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
@@ -1249,6 +1271,9 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
                  heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size)};
+  if (all_heads < ROPE_NARROW_BELOW)
+    return launch_mid<EPI_QKV_ROPE, 1, true, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64,
+                                                   2 * all_heads, (hipStream_t)stream, na, rp);
   return launch_mid<EPI_QKV_ROPE, 1, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64, all_heads,
                                            (hipStream_t)stream, na, rp);
 }

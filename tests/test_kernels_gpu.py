@@ -526,7 +526,8 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
     assert not ops.can_fuse_norm(4, torch.zeros(8, 96, dtype=torch.bfloat16), torch.zeros(4, 96))   # steps of 64 along the rows
 
     for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
-                                     (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128)]:   # the last: a workgroup a head
+                                     (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128),    # the last two: half a head a workgroup,
+                                     (200, 28, 64, 16, 64)]:                                          # a head a workgroup
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
@@ -563,7 +564,8 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
     g = torch.Generator().manual_seed(21)
     for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
                                    (40, 10, 128, 2100, 32),        # enough 256 x 256 tiles for the big-tile kernel
-                                   (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16)]:   # up to 64 rows, a workgroup a head
+                                   (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16),   # up to 64 rows, half a head a workgroup
+                                   (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32)]:   # a head a workgroup
         hd = 64
         pages = 40 if M < 500 else 3 * ((M + page - 1) // page + 2) + 3
         cos, sin = rope_tables(10000.0, hd, max(400, M), gpu)
