@@ -71,12 +71,120 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   }
 }
 
+// Up to 16 rows (decoded tokens): the same chains, one per thread.  A workgroup owns 16 columns and all rows,
+// thread (m, n) the output of row m and column 16 * blockIdx.x + n; its 256 threads together bring 256 elements
+// of k of the 16 rows of W and of the rows of x into LDS at a time (16-byte loads; the next stage's loads fly
+// while this one is worked on), widened to 32-bit there, and every thread then walks the stage in k order with
+// one 16-byte read of its row of W and one of its row of x per four multiply-adds.  Few columns a workgroup,
+// so that a product with few outputs still has loads in flight from many compute units.
+// K a multiple of 8 (of 4 for 32-bit weights), rows 16-byte aligned.
+#define F32R_NB 16
+#define F32R_KB 256
+#define F32R_STRIDE (F32R_KB + 4)   // floats from row to row in LDS: 16-byte reads of 16 rows hit 64 different banks
+
+template <typename WT>
+__global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                            float* __restrict__ y, int M, int N, int K, int ldx,
+                                                            int ldy, int accumulate) {
+  constexpr int WC = sizeof(WT) == 2 ? 8 : 4;             // elements of W in a 16-byte chunk
+  constexpr int WPR = F32R_KB / WC;                        // chunks in a stage's row of W
+  constexpr int WJ = F32R_NB * WPR / 256;                  // chunks of W a thread and stage
+  constexpr int XJ = 16 * (F32R_KB / 4) / 256;             // chunks of x a thread and stage (16 rows)
+  extern __shared__ __attribute__((aligned(16))) float rows_lds[];   // [2][W: 16 rows | x: 16 rows] of F32R_STRIDE
+  const int tid = threadIdx.x, n = tid & 15, m = tid >> 4;
+  const int n0 = blockIdx.x * F32R_NB;
+  u32x4 wreg[WJ];
+  f32x4 xreg[XJ];
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const int c = tid + 256 * j, row = c / WPR, k = k0 + (c % WPR) * WC;
+      wreg[j] = (u32x4){0u, 0u, 0u, 0u};
+      if (n0 + row < N && k < K) wreg[j] = *reinterpret_cast<const u32x4*>(w + (size_t)(n0 + row) * K + k);
+    }
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+      const int c = tid + 256 * j, row = c / (F32R_KB / 4), k = k0 + (c % (F32R_KB / 4)) * 4;
+      xreg[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (row < M && k < K) xreg[j] = *reinterpret_cast<const f32x4*>(x + (size_t)row * ldx + k);
+    }
+  };
+  auto store_stage = [&](float* buf) {
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const int c = tid + 256 * j, row = c / WPR, kk = (c % WPR) * WC;
+      float* dst = buf + row * F32R_STRIDE + kk;
+      if constexpr (sizeof(WT) == 2) {                     // bfloat16 -> 32-bit: the bits, shifted (exact)
+        *reinterpret_cast<u32x4*>(dst) = (u32x4){wreg[j][0] << 16, wreg[j][0] & 0xffff0000u, wreg[j][1] << 16, wreg[j][1] & 0xffff0000u};
+        *reinterpret_cast<u32x4*>(dst + 4) = (u32x4){wreg[j][2] << 16, wreg[j][2] & 0xffff0000u, wreg[j][3] << 16, wreg[j][3] & 0xffff0000u};
+      } else {
+        *reinterpret_cast<u32x4*>(dst) = wreg[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < XJ; ++j) {
+      const int c = tid + 256 * j, row = c / (F32R_KB / 4), kk = (c % (F32R_KB / 4)) * 4;
+      *reinterpret_cast<f32x4*>(buf + (F32R_NB + row) * F32R_STRIDE + kk) = xreg[j];
+    }
+  };
+  constexpr int BUF = 2 * 16 * F32R_STRIDE;                // floats of one buffer
+  float acc = 0.0f;
+  load_stage(0);
+  store_stage(rows_lds);
+  __syncthreads();
+  int b = 0;
+  for (int k0 = 0; k0 < K; k0 += F32R_KB) {
+    const bool more = k0 + F32R_KB < K;
+    if (more) load_stage(k0 + F32R_KB);
+    if (m < M) {
+      const float* wr = rows_lds + b * BUF + n * F32R_STRIDE;
+      const float* xr = rows_lds + b * BUF + (F32R_NB + m) * F32R_STRIDE;
+      const int kend = (K - k0) < F32R_KB ? (K - k0) : F32R_KB;
+      for (int kk = 0; kk < kend; kk += 4) {
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(wr + kk);
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(xr + kk);
+        acc = fmaf(xv[0], wv[0], acc);
+        acc = fmaf(xv[1], wv[1], acc);
+        acc = fmaf(xv[2], wv[2], acc);
+        acc = fmaf(xv[3], wv[3], acc);
+      }
+    }
+    if (more) store_stage(rows_lds + (b ^ 1) * BUF);
+    __syncthreads();
+    b ^= 1;
+  }
+  if (m < M && n0 + n < N) {
+    float* o = y + (size_t)m * ldy + n0 + n;
+    *o = accumulate ? (*o + acc) : acc;
+  }
+}
+
+template <typename WT>
+static void launch_rows(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                        hipStream_t s) {
+  constexpr int lds_bytes = 2 * 2 * 16 * F32R_STRIDE * (int)sizeof(float);
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<WT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  hipLaunchKernelGGL(gemm_f32_rows_kernel<WT>, dim3((N + F32R_NB - 1) / F32R_NB), dim3(256), lds_bytes, s, x, w, y, M, N, K,
+                     ldx, ldy, accumulate);
+}
+
 extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, int N, int K, int ldx,
                            int ldy, int accumulate, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || ldx < K || ldy < N) return -2;
   dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM), block(256);
   hipStream_t s = (hipStream_t)stream;
+  // which kernel runs depends on the shape alone, and both run the same chains
+  const int wc = w_is_bf16 ? 8 : 4;
+  if (M <= 16 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+    if (w_is_bf16) launch_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    else launch_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
   if (w_is_bf16)
     hipLaunchKernelGGL(gemm_f32_kernel<bf16_t>, grid, block, 0, s, x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate);
   else
