@@ -61,12 +61,23 @@ __device__ __forceinline__ size_t key_offset(const AttnF32Args& a, const int32_t
 
 #define ATT32_THREADS 256
 
+// Keys of a chunk of pass 2: as many as 32 KB of value rows hold, at most one a thread.
+template <int HD>
+struct Att32Shape {
+  static constexpr int T = ATT32_THREADS;
+  static constexpr int KC = (8192 / HD) < T ? (8192 / HD) : T;
+  static constexpr int SEGS = HD / 4;                              // 16-byte pieces of a key's row
+  static constexpr int VJ = (KC * SEGS + T - 1) / T;               // pieces of a chunk's value rows a thread
+  static constexpr int LDS_BYTES = 2 * KC * HD * (int)sizeof(float);
+};
+
 template <int HD>
 __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Args a) {
-  constexpr int T = ATT32_THREADS;
+  using S = Att32Shape<HD>;
+  constexpr int T = S::T, KC = S::KC, SEGS = S::SEGS, VJ = S::VJ;
+  extern __shared__ __attribute__((aligned(16))) float v_lds[];    // [2][KC][HD]: value rows of a chunk of keys
   __shared__ float q_lds[HD];
-  __shared__ float e_lds[2][T];
-  __shared__ unsigned long long off_lds[2][T];
+  __shared__ float e_lds[2][KC];
   __shared__ float red[T / 64];
   const int row = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int pos = a.positions[row];
@@ -91,40 +102,75 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
 #pragma unroll
   for (int w = 1; w < T / 64; ++w) mx = fmaxf(mx, red[w]);
 
-  // pass 2: the threads compute e_j of T keys at a time (the same deterministic function of the key as in pass
-  // 1) and park them with the keys' cache offsets; thread d < HD then walks the T keys in order for element d.
-  // The next T keys' e_j are computed before the walk, into the other buffer: one barrier per T keys.
-  auto park = [&](int j0, int buf) {
-    const int j = j0 + tid;
-    float e = 0.0f;
-    size_t off = 0;
-    if (j <= pos) {
-      off = key_offset(a, table, j, head_off, page_stride, HD);
-      e = expf(dot_canonical<HD>(q_lds, a.k_cache + off) * a.scale - mx);
+  // pass 2, KC keys at a time: the last KC threads compute e_j of a key each (the same deterministic function of
+  // the key as in pass 1) and all threads bring the keys' value rows into LDS; thread d < HD then walks the
+  // chunk in key order for element d.  The next chunk is fetched before the walk and parked after it, into the
+  // other buffers: one barrier a chunk, and the loads fly during the walk.
+  f32x4 vreg[VJ];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < VJ; ++i) {
+      const int c = tid + T * i, j = j0 + c / SEGS;
+      vreg[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (c < KC * SEGS && j <= pos)
+        vreg[i] = *reinterpret_cast<const f32x4*>(a.v_cache + key_offset(a, table, j, head_off, page_stride, HD) + 4 * (c % SEGS));
     }
-    e_lds[buf][tid] = e;
-    off_lds[buf][tid] = off;
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < VJ; ++i) {
+      const int c = tid + T * i;                           // piece c = key c / SEGS, elements 4 * (c % SEGS)..: float 4c of the buffer
+      if (c < KC * SEGS) *reinterpret_cast<f32x4*>(v_lds + buf * KC * HD + 4 * c) = vreg[i];
+    }
+  };
+  auto park = [&](int j0, int buf) {
+    const int t = tid - (T - KC);
+    if (t < 0) return;
+    const int j = j0 + t;
+    float e = 0.0f;
+    if (j <= pos)
+      e = expf(dot_canonical<HD>(q_lds, a.k_cache + key_offset(a, table, j, head_off, page_stride, HD)) * a.scale - mx);
+    e_lds[buf][t] = e;
   };
   float acc = 0.0f, sum = 0.0f;
+  fetch(lo);
   park(lo, 0);
+  stash(0);
   __syncthreads();
   int buf = 0;
-  for (int j0 = lo; j0 <= pos; j0 += T) {
-    if (j0 + T <= pos) park(j0 + T, buf ^ 1);
+  for (int j0 = lo; j0 <= pos; j0 += KC) {
+    const bool more = j0 + KC <= pos;
+    if (more) {
+      fetch(j0 + KC);
+      park(j0 + KC, buf ^ 1);
+    }
     if (tid < HD) {
-      const int cnt = (pos - j0 + 1) < T ? (pos - j0 + 1) : T;
-      const float* vd = a.v_cache + tid;
+      const int cnt = (pos - j0 + 1) < KC ? (pos - j0 + 1) : KC;
+      const float* vd = v_lds + buf * KC * HD + tid;
+      const float* ed = e_lds[buf];
 #pragma unroll 8
       for (int jj = 0; jj < cnt; ++jj) {
-        const float ej = e_lds[buf][jj];
+        const float ej = ed[jj];
         sum += ej;
-        acc = fmaf(ej, vd[off_lds[buf][jj]], acc);
+        acc = fmaf(ej, vd[jj * HD], acc);
       }
     }
+    if (more) stash(buf ^ 1);
     __syncthreads();
     buf ^= 1;
   }
   if (tid < HD) a.out[(size_t)row * a.out_stride + (size_t)h * HD + tid] = acc * (1.0f / sum);
+}
+
+template <int HD>
+static void launch_attention_f32(const AttnF32Args& a, dim3 grid, hipStream_t s) {
+  static bool allowed = false;                         // 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)attention_f32_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              Att32Shape<HD>::LDS_BYTES);
+    allowed = true;
+  }
+  hipLaunchKernelGGL(attention_f32_kernel<HD>, grid, dim3(ATT32_THREADS), Att32Shape<HD>::LDS_BYTES, s, a);
 }
 
 extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
@@ -136,9 +182,9 @@ extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* pos
   AttnF32Args a{q, positions, row_seq, block_table, k_cache, v_cache, out, rows, heads, kv_heads, head_dim,
                 page_size, table_stride, q_stride, out_stride, window, scale,
                 (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1};
-  dim3 grid(rows, heads), block(ATT32_THREADS);
+  dim3 grid(rows, heads);
   hipStream_t s = (hipStream_t)stream;
-#define BW_CASE(HD) case HD: hipLaunchKernelGGL(attention_f32_kernel<HD>, grid, block, 0, s, a); break;
+#define BW_CASE(HD) case HD: launch_attention_f32<HD>(a, grid, s); break;
   switch (head_dim) {
     BW_CASE(16) BW_CASE(32) BW_CASE(48) BW_CASE(64) BW_CASE(80) BW_CASE(96) BW_CASE(112) BW_CASE(128)
     BW_CASE(160) BW_CASE(192) BW_CASE(224) BW_CASE(256)
