@@ -68,6 +68,39 @@ __global__ void rmsnorm_f32_kernel(const float* __restrict__ x, const WT* __rest
   }
 }
 
+// The same chains and tree for rows of up to RMS32_MAX elements, a workgroup a row: its 256 threads bring the row
+// into LDS together, 16 of them run the chains from there (nothing between two steps of a chain but an LDS
+// read), and all write the result.
+#define RMS32_MAX 8192
+template <typename WT>
+__global__ __launch_bounds__(256) void rmsnorm_f32_row_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                              float* __restrict__ y, int dim, float eps) {
+  __shared__ float row_lds[RMS32_MAX];
+  __shared__ float inv_lds;
+  const float* xr = x + (size_t)blockIdx.x * dim;
+  for (int i = threadIdx.x; i < dim; i += 256) row_lds[i] = xr[i];
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < dim; i += 16) acc = fmaf(row_lds[i], row_lds[i], acc);
+    acc += __shfl_xor(acc, 8, 16);
+    acc += __shfl_xor(acc, 4, 16);
+    acc += __shfl_xor(acc, 2, 16);
+    acc += __shfl_xor(acc, 1, 16);
+    if (threadIdx.x == 0) inv_lds = 1.0f / sqrtf(acc / (float)dim + eps);
+  }
+  __syncthreads();
+  const float inv = inv_lds;
+  float* yr = y + (size_t)blockIdx.x * dim;
+  for (int i = threadIdx.x; i < dim; i += 256) {
+    float wi;
+    if constexpr (sizeof(WT) == 2) wi = bf16_to_f32(w[i]);
+    else wi = w[i];
+    yr[i] = (row_lds[i] * inv) * wi;
+  }
+}
+
 // ------------------------------------------------------------------------- RMSNorm, bfloat16 out
 
 // One wave per row.  Rows whose width is a multiple of 4 are read as 16-byte vectors: lane l
@@ -127,6 +160,13 @@ extern "C" int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16
       hipLaunchKernelGGL(rmsnorm_bf16_kernel<float>, grid, block, 0, s, x, (const float*)weight, (bf16_t*)y, rows, dim, ldy, eps);
   } else {
     if (ldy != dim) return -2;
+    if (dim <= RMS32_MAX) {
+      if (weight_is_bf16)
+        hipLaunchKernelGGL(rmsnorm_f32_row_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, x, (const bf16_t*)weight, (float*)y, dim, eps);
+      else
+        hipLaunchKernelGGL(rmsnorm_f32_row_kernel<float>, dim3(rows), dim3(256), 0, s, x, (const float*)weight, (float*)y, dim, eps);
+      return BW_LAUNCH_CHECK();
+    }
     dim3 grid((rows + 15) / 16), block(256);
     if (weight_is_bf16)
       hipLaunchKernelGGL(rmsnorm_f32_kernel<bf16_t>, grid, block, 0, s, x, (const bf16_t*)weight, (float*)y, rows, dim, eps);
