@@ -93,23 +93,24 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
   extern __shared__ __attribute__((aligned(16))) float rows_lds[];   // [2][W: 16 rows | x: 16 rows] of F32R_STRIDE
   const int tid = threadIdx.x, n = tid & 15, m = tid >> 4;
   const int n0 = blockIdx.x * F32R_NB;
-  u32x4 wreg[WJ];
-  f32x4 xreg[XJ];
-  auto load_stage = [&](int k0) {
+  // Two stages' loads are in flight while one is worked on: register sets A and B take the even and the odd stages
+  // in turn.  Every load is unconditional and inside the operands (rows past N or M and k past K are clamped: what
+  // they bring is never used), so that a wait for one set's loads need not be a wait for the other's.
+  u32x4 wa[WJ], wb[WJ];
+  f32x4 xa[XJ], xb[XJ];
+  auto load_stage = [&](int k0, u32x4 (&wreg)[WJ], f32x4 (&xreg)[XJ]) {
 #pragma unroll
     for (int j = 0; j < WJ; ++j) {
-      const int c = tid + 256 * j, row = c / WPR, k = k0 + (c % WPR) * WC;
-      wreg[j] = (u32x4){0u, 0u, 0u, 0u};
-      if (n0 + row < N && k < K) wreg[j] = *reinterpret_cast<const u32x4*>(w + (size_t)(n0 + row) * K + k);
+      const int c = tid + 256 * j, row = min(n0 + c / WPR, N - 1), k = min(k0 + (c % WPR) * WC, K - WC);
+      wreg[j] = *reinterpret_cast<const u32x4*>(w + (size_t)row * K + k);
     }
 #pragma unroll
     for (int j = 0; j < XJ; ++j) {
-      const int c = tid + 256 * j, row = c / (F32R_KB / 4), k = k0 + (c % (F32R_KB / 4)) * 4;
-      xreg[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      if (row < M && k < K) xreg[j] = *reinterpret_cast<const f32x4*>(x + (size_t)row * ldx + k);
+      const int c = tid + 256 * j, row = min(c / (F32R_KB / 4), M - 1), k = min(k0 + (c % (F32R_KB / 4)) * 4, K - 4);
+      xreg[j] = *reinterpret_cast<const f32x4*>(x + (size_t)row * ldx + k);
     }
   };
-  auto store_stage = [&](float* buf) {
+  auto store_stage = [&](float* buf, const u32x4 (&wreg)[WJ], const f32x4 (&xreg)[XJ]) {
 #pragma unroll
     for (int j = 0; j < WJ; ++j) {
       const int c = tid + 256 * j, row = c / WPR, kk = (c % WPR) * WC;
@@ -129,29 +130,72 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
   };
   constexpr int BUF = 2 * 16 * F32R_STRIDE;                // floats of one buffer
   float acc = 0.0f;
-  load_stage(0);
-  store_stage(rows_lds);
-  __syncthreads();
-  int b = 0;
-  for (int k0 = 0; k0 < K; k0 += F32R_KB) {
-    const bool more = k0 + F32R_KB < K;
-    if (more) load_stage(k0 + F32R_KB);
-    if (m < M) {
-      const float* wr = rows_lds + b * BUF + n * F32R_STRIDE;
-      const float* xr = rows_lds + b * BUF + (F32R_NB + m) * F32R_STRIDE;
-      const int kend = (K - k0) < F32R_KB ? (K - k0) : F32R_KB;
-      for (int kk = 0; kk < kend; kk += 4) {
-        const f32x4 wv = *reinterpret_cast<const f32x4*>(wr + kk);
-        const f32x4 xv = *reinterpret_cast<const f32x4*>(xr + kk);
-        acc = fmaf(xv[0], wv[0], acc);
-        acc = fmaf(xv[1], wv[1], acc);
-        acc = fmaf(xv[2], wv[2], acc);
-        acc = fmaf(xv[3], wv[3], acc);
+  auto work = [&](const float* buf, int k0) {              // the stage's steps of every chain, k ascending
+    const int kend = (K - k0) < F32R_KB ? (K - k0) : F32R_KB;
+    if (m >= M || kend <= 0) return;
+    const float* wr = buf + n * F32R_STRIDE;
+    const float* xr = buf + (F32R_NB + m) * F32R_STRIDE;
+    if (kend == F32R_KB) {
+      // a whole stage: blocks of 32 steps, the operands of the next block read from LDS while this block's steps
+      // run (the wave has little company on its SIMD: what hides its read latency is its own chain)
+      constexpr int BLK = 8, NBLK = F32R_KB / 4 / BLK;
+      f32x4 wv[2][BLK], xv[2][BLK];
+#pragma unroll
+      for (int i = 0; i < BLK; ++i) {
+        wv[0][i] = *reinterpret_cast<const f32x4*>(wr + 4 * i);
+        xv[0][i] = *reinterpret_cast<const f32x4*>(xr + 4 * i);
       }
+#pragma unroll
+      for (int blk = 0; blk < NBLK; ++blk) {
+        if (blk + 1 < NBLK) {
+#pragma unroll
+          for (int i = 0; i < BLK; ++i) {
+            wv[(blk + 1) & 1][i] = *reinterpret_cast<const f32x4*>(wr + 4 * (BLK * (blk + 1) + i));
+            xv[(blk + 1) & 1][i] = *reinterpret_cast<const f32x4*>(xr + 4 * (BLK * (blk + 1) + i));
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < BLK; ++i) {
+          acc = fmaf(xv[blk & 1][i][0], wv[blk & 1][i][0], acc);
+          acc = fmaf(xv[blk & 1][i][1], wv[blk & 1][i][1], acc);
+          acc = fmaf(xv[blk & 1][i][2], wv[blk & 1][i][2], acc);
+          acc = fmaf(xv[blk & 1][i][3], wv[blk & 1][i][3], acc);
+        }
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * BLK, 0);
+#pragma unroll
+      for (int blk = 0; blk + 1 < NBLK; ++blk) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * BLK, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4 * BLK, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x002, 4 * BLK, 0);
+      return;
     }
-    if (more) store_stage(rows_lds + (b ^ 1) * BUF);
+#pragma unroll 8
+    for (int kk = 0; kk < kend; kk += 4) {               // (unrolled: the reads of the steps ahead are under way)
+      const f32x4 wv = *reinterpret_cast<const f32x4*>(wr + kk);
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(xr + kk);
+      acc = fmaf(xv[0], wv[0], acc);
+      acc = fmaf(xv[1], wv[1], acc);
+      acc = fmaf(xv[2], wv[2], acc);
+      acc = fmaf(xv[3], wv[3], acc);
+    }
+  };
+  float* buf0 = rows_lds;
+  float* buf1 = rows_lds + BUF;
+  load_stage(0, wa, xa);
+  load_stage(F32R_KB, wb, xb);
+  store_stage(buf0, wa, xa);
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += 2 * F32R_KB) {
+    load_stage(k0 + 2 * F32R_KB, wa, xa);
+    work(buf0, k0);
+    store_stage(buf1, wb, xb);
     __syncthreads();
-    b ^= 1;
+    load_stage(k0 + 3 * F32R_KB, wb, xb);
+    work(buf1, k0 + F32R_KB);
+    store_stage(buf0, wa, xa);
+    __syncthreads();
   }
   if (m < M && n0 + n < N) {
     float* o = y + (size_t)m * ldy + n0 + n;
