@@ -33,6 +33,10 @@ int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, con
                      const int32_t* block_table, int table_stride, const float* k_cache, const float* v_cache,
                      float* out, int out_stride, int rows, int heads, int kv_heads, int head_dim, int page_size,
                      int window, float scale, void* stream);
+int bw_attention_f32_tiles(const float* q, int q_stride, const int32_t* positions, const int32_t* block_table,
+                           int table_stride, const int32_t* tiles, int num_tiles, int tiled, const float* k_cache,
+                           const float* v_cache, float* out, int out_stride, int heads, int kv_heads, int head_dim,
+                           int page_size, int window, float scale, void* stream);
 int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                       int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                       const void* v_cache, int num_pages, void* out, int out_stride, int heads, int kv_heads,

@@ -46,6 +46,8 @@ _SIGS = {
                          c_int, c_void_p],
     "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_attention_f32_tiles": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
@@ -361,6 +363,32 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
                                    block_table.data_ptr(), block_table.stride(0), k_cache.data_ptr(),
                                    v_cache.data_ptr(), out.data_ptr(), out.stride(0), rows, heads, kv_heads, head_dim,
                                    page_size, int(window), float(scale), _stream()), "attention_f32")
+
+
+def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
+                        num_tiles: int, tiled: bool, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                        heads: int, kv_heads: int, head_dim: int, page_size: int, window: int, scale: float) -> None:
+    """``attention_f32`` over tiles ([tiles, 4] int32 = first row, rows, request, 0; a tile's rows are consecutive
+    rows of one request).  ``tiled``: a workgroup per tile of up to 16 rows, keys and values shared through LDS
+    (head sizes up to 128); else a workgroup per tile's first row.  The bits are those of ``attention_f32``."""
+    _need(q, torch.float32, "q")
+    _need(out, torch.float32, "out")
+    _need(k_cache, torch.float32, "k_cache")
+    _need(v_cache, torch.float32, "v_cache")
+    _need(positions, torch.int32, "positions")
+    _need(block_table, torch.int32, "block_table")
+    _need(tiles, torch.int32, "tiles")
+    if head_dim not in HEAD_DIMS or (tiled and head_dim > 128):
+        raise ValueError(f"attention: head size {head_dim} is not supported here")
+    if tiles.numel() < 4 * num_tiles or q.shape[1] < heads * head_dim or out.shape[1] != heads * head_dim:
+        raise ValueError("attention_f32_tiles: tiles, q or out too small")
+    if heads % kv_heads:
+        raise ValueError("attention: heads must be a multiple of kv_heads")
+    _check(_fn("bw_attention_f32_tiles")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
+                                         block_table.stride(0), tiles.data_ptr(), int(num_tiles), int(bool(tiled)),
+                                         k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
+                                         kv_heads, head_dim, page_size, int(window), float(scale), _stream()),
+           "attention_f32_tiles")
 
 
 def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,

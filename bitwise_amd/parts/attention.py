@@ -115,8 +115,18 @@ class Attention(Mixer):
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              rt.page_size, call.writes_cache)
             out = rt.buffer("attn_out", self.q_dim, torch.float32)
-            ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
-                              self.heads, self.kv_heads, self.head_dim, rt.page_size, window, self.scale)
+            plan = ctx.attention_plan(16, 1)
+            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                      window, self.scale)
+            if plan.fold_count and self.head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
+                # every row by itself (also: a batch of nothing but decoded tokens, row t of request t)
+                ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
+                                  self.heads, self.kv_heads, self.head_dim, rt.page_size, window, self.scale)
+            else:
+                if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
+                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.fold_tiles, plan.fold_count, True, *common)
+                if plan.decode_count:
+                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common)
             self.o.add_into(out, residual, rows)
 
     def _attend(self, ctx, call, q, residual) -> None:

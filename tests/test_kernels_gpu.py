@@ -341,6 +341,11 @@ def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, wi
     scale = 1.0 / float(hd) ** 0.5
     if not bf16:
         out = torch.zeros(rows, heads * hd, device=gpu)
+        if tiles is not None:                      # a workgroup a tile of rows, or (tiles of one row) a tile's row
+            t = torch.tensor(tiles, dtype=torch.int32, device=gpu)
+            ops.attention_f32_tiles(q.to(gpu), pos, tab, t, len(tiles), any(n != 1 for _, n, _, _ in tiles), kc, vc, out,
+                                    heads, kvh, hd, page, window, scale)
+            return out
         ops.attention_f32(q.to(gpu), pos, torch.zeros(rows, dtype=torch.int32, device=gpu), tab, kc, vc, out, rows,
                           heads, kvh, hd, page, window, scale)
         return out
@@ -414,11 +419,20 @@ def test_attention_prompt_tiles_equal_single_rows(gpu, bf16):
     positions = list(range(120, 147))
     g = torch.Generator().manual_seed(10)
     q = torch.randn(len(positions), heads * hd, generator=g).to(torch.bfloat16 if bf16 else torch.float32)
-    tpt = 16 // (heads // kvh)
+    tpt = 16 // (heads // kvh) if bf16 else 16
     tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
     portion = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, tiles=tiles)
     single = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page)
     assert torch.equal(portion, single)
+    if not bf16:
+        # a window that ends inside the tile's keys, tiles of other sizes, and tiles of one row through the row kernel
+        for window, tpt in ((0, 1), (37, 16), (37, 7), (5, 16), (70, 3)):
+            tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+            tiled = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles)
+            alone = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window)
+            assert torch.equal(tiled, alone), (window, tpt)
+        first = run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page, tiles=[(0, 16, 0, 0), (16, 4, 0, 0)])
+        assert torch.equal(first, run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page))
     ref = plain_rows(q, k, v, positions, heads)
     assert (portion.cpu().double() - ref).abs().max() <= (1.5e-2 if bf16 else 3e-6) * ref.abs().max()
 
