@@ -71,6 +71,111 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   }
 }
 
+// Prompt portions: the same chains in tiles of 128x128 outputs, 8x8 per thread (as 2x2 blocks of 4x4, 64 rows
+// or columns apart, so that every LDS read is 16 bytes and free of bank conflicts), k staged through LDS 16 at a
+// time in two buffers (the next stage's loads fly while this one is worked on; one barrier a stage).
+// K a multiple of 16, rows 16-byte aligned.
+#define F32T_BM 128
+#define F32T_BN 128
+#define F32T_BK 16
+#define F32T_STR 132            // floats from k to k in LDS
+
+template <typename WT>
+__global__ __launch_bounds__(256) void gemm_f32_tile_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                            float* __restrict__ y, int M, int N, int K, int ldx,
+                                                            int ldy, int accumulate) {
+  __shared__ __attribute__((aligned(16))) float xs[2][F32T_BK][F32T_STR];
+  __shared__ __attribute__((aligned(16))) float ws[2][F32T_BK][F32T_STR];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * F32T_BM, n0 = blockIdx.x * F32T_BN;
+  // loads of a stage: x rows lm and lm + 64, elements 4*lq..; W row wr, elements 8*wh.. (rows past the end are
+  // clamped: what they bring is never stored)
+  const int lm = tid >> 2, lq = tid & 3, wr = tid >> 1, wh = tid & 1;
+  const float* xp0 = x + (size_t)min(m0 + lm, M - 1) * ldx + 4 * lq;
+  const float* xp1 = x + (size_t)min(m0 + lm + 64, M - 1) * ldx + 4 * lq;
+  const WT* wp = w + (size_t)min(n0 + wr, N - 1) * K + 8 * wh;
+  f32x4 xr0, xr1;
+  u32x4 wq0, wq1;                                          // bfloat16: 8 elements in wq0; 32-bit: 4 and 4
+  auto load_stage = [&](int k0) {
+    xr0 = *reinterpret_cast<const f32x4*>(xp0 + k0);
+    xr1 = *reinterpret_cast<const f32x4*>(xp1 + k0);
+    wq0 = *reinterpret_cast<const u32x4*>(wp + k0);
+    if constexpr (sizeof(WT) == 4) wq1 = *reinterpret_cast<const u32x4*>(wp + k0 + 4);
+  };
+  auto store_stage = [&](int b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xs[b][4 * lq + i][lm] = xr0[i];
+      xs[b][4 * lq + i][lm + 64] = xr1[i];
+    }
+    if constexpr (sizeof(WT) == 2) {                       // bfloat16 -> 32-bit: the bits, shifted (exact)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ws[b][8 * wh + 2 * i][wr] = __uint_as_float(wq0[i] << 16);
+        ws[b][8 * wh + 2 * i + 1][wr] = __uint_as_float(wq0[i] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ws[b][8 * wh + i][wr] = __uint_as_float(wq0[i]);
+        ws[b][8 * wh + 4 + i][wr] = __uint_as_float(wq1[i]);
+      }
+    }
+  };
+  float acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  int b = 0;
+  for (int k0 = 0; k0 < K; k0 += F32T_BK) {
+    const bool more = k0 + F32T_BK < K;
+    if (more) load_stage(k0 + F32T_BK);
+#pragma unroll
+    for (int kk = 0; kk < F32T_BK; ++kk) {
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&xs[b][kk][4 * ty]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&xs[b][kk][64 + 4 * ty]);
+      const f32x4 b0 = *reinterpret_cast<const f32x4*>(&ws[b][kk][4 * tx]);
+      const f32x4 b1 = *reinterpret_cast<const f32x4*>(&ws[b][kk][64 + 4 * tx]);
+      const float av[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      const float bv[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    if (more) store_stage(b ^ 1);
+    __syncthreads();
+    b ^= 1;
+  }
+  const bool vec = (ldy & 3) == 0 && ((uintptr_t)y & 15) == 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + (i < 4 ? 4 * ty + i : 64 + 4 * ty + i - 4);
+    if (m >= M) continue;
+#pragma unroll
+    for (int jh = 0; jh < 2; ++jh) {
+      const int n = n0 + 64 * jh + 4 * tx;
+      float* o = y + (size_t)m * ldy + n;
+      if (vec && n + 3 < N) {
+        f32x4 v = {acc[i][4 * jh], acc[i][4 * jh + 1], acc[i][4 * jh + 2], acc[i][4 * jh + 3]};
+        if (accumulate) {
+          const f32x4 old = *reinterpret_cast<const f32x4*>(o);
+          v = (f32x4){old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
+        }
+        *reinterpret_cast<f32x4*>(o) = v;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < N) o[j] = accumulate ? (o[j] + acc[i][4 * jh + j]) : acc[i][4 * jh + j];
+      }
+    }
+  }
+}
+
 // Up to 16 rows (decoded tokens): the same chains, one per thread.  A workgroup owns 16 columns and all rows,
 // thread (m, n) the output of row m and column 16 * blockIdx.x + n; its 256 threads together bring 256 elements
 // of k of the 16 rows of W and of the rows of x into LDS at a time (16-byte loads; the next stage's loads fly
@@ -227,6 +332,14 @@ extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* 
   if (M <= 16 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
     if (w_is_bf16) launch_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
     else launch_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
+  if (M > 16 && K % F32T_BK == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+    dim3 tgrid((N + F32T_BN - 1) / F32T_BN, (M + F32T_BM - 1) / F32T_BM);
+    if (w_is_bf16)
+      hipLaunchKernelGGL(gemm_f32_tile_kernel<bf16_t>, tgrid, block, 0, s, x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate);
+    else
+      hipLaunchKernelGGL(gemm_f32_tile_kernel<float>, tgrid, block, 0, s, x, (const float*)w, y, M, N, K, ldx, ldy, accumulate);
     return BW_LAUNCH_CHECK();
   }
   if (w_is_bf16)
