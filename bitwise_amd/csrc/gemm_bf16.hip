@@ -548,10 +548,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_big_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char big_lds[];   // [5 slots][32 KB]
+  // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
+  // elements (a residual add's segments, joined in order by add_segments_kernel afterwards)
+  const int k_base = (int)blockIdx.y * GEMM_SEG;
+  if (gridDim.y > 1) out = (void*)((float*)out + (size_t)blockIdx.y * seg_stride);
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int wy = wave >> 2, wx = wave & 3;
@@ -585,13 +589,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     unsigned char* dst = big_lds + ((2 * step) % BIG_SLOTS) * BIG_SLOT + (4 * wave) * 1024;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, voff_a[t], step * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, voff_a[t], k_base * 2 + step * 128, 0, 0);
   };
   auto issue_b = [&](int step) {
     unsigned char* dst = big_lds + ((2 * step + 1) % BIG_SLOTS) * BIG_SLOT + (4 * wave) * 1024;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + t * 1024), 16, voff_b[t], step * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + t * 1024), 16, voff_b[t], k_base * 2 + step * 128, 0, 0);
   };
 
   f32x4 acc[8][4];
@@ -609,7 +613,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int a_frag = (8 * wy) * 2048, b_frag = (GLU ? 2 * wx : 4 * wx) * 2048;
   auto b_off = [&](int j) { return GLU ? ((j & 1) + 8 * (j >> 1)) * 2048 : j * 2048; };
 
-  const int steps = K / 64;
+  const int steps = gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64;
   issue_a(0);
   issue_b(0);
   if (steps > 1) issue_a(1);
@@ -1420,6 +1424,29 @@ static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int
 // How a residual add of 17 to 64 rows runs in the kernel above: 64 or 32 columns a workgroup (as many workgroups
 // as there are compute units, if the product has them), a workgroup per tile and segment of K if there are several
 // (they meet in device scratch the caller brings).  tiles 0: it does not run there.
+// out = (((out + p[0]) + p[1]) + ...) + p[S-1], element by element: the segments of a residual add that
+// gemm_bf16_big_kernel left in scratch ([S][M][N]), joined in segment order.
+__global__ __launch_bounds__(256) void add_segments_kernel(float* __restrict__ out, const float* __restrict__ parts, int S,
+                                                           int M, int N, int ldo) {
+  const size_t quads = (size_t)M * (N >> 2);
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= quads) return;
+  const int m = (int)(i / (N >> 2)), n = 4 * (int)(i % (N >> 2));
+  float* o = out + (size_t)m * ldo + n;
+  f32x4 y = *reinterpret_cast<const f32x4*>(o);
+  for (int sg = 0; sg < S; ++sg) y = y + *reinterpret_cast<const f32x4*>(parts + ((size_t)sg * M + m) * N + n);
+  *reinterpret_cast<f32x4*>(o) = y;
+}
+
+// A residual add of a prompt portion over several segments of K with 256 x 256 tiles, a workgroup per tile and
+// segment: for products whose 128 x 128 tiles would be bound by what a compute unit can fetch (half as many
+// bytes a flop here), if the caller brings scratch for the segments' sums.
+static bool big_add_shape(int M, int N, int K, int ldo) {
+  const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
+  const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
+  return S > 1 && K % 64 == 0 && M >= 2 * BIG_BM && bm * bn * S >= 128 && N % 4 == 0 && ldo % 4 == 0;
+}
+
 static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
   tiles = 0;
@@ -1517,7 +1544,25 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
           allowed = true;
         }
         hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI>), dim3(bm * bn), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w, out, M, N, K, ldx,
-                           ldo, bm, bn, rp);
+                           ldo, bm, bn, rp, (size_t)0);
+        return BW_LAUNCH_CHECK();
+      }
+    }
+    if constexpr (EPI == EPI_ADD_F32) {
+      if (sp.scratch != nullptr && big_add_shape(M, N, K, ldo) && ((uintptr_t)out & 15) == 0) {
+        if (scratch_floats < (size_t)S * M * N) return -6;
+        const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
+        static bool allowed = false;                 // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<EPI_F32>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    BIG_SLOTS * BIG_SLOT);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI_F32>), dim3(bm * bn, S), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w,
+                           (void*)sp.scratch, M, N, K, ldx, N, bm, bn, rp, (size_t)M * N);
+        const size_t quads = (size_t)M * (N >> 2);
+        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+                           M, N, ldo);
         return BW_LAUNCH_CHECK();
       }
     }
@@ -1554,7 +1599,12 @@ extern "C" int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_float
   int tiles = 0;
   bool narrow = false;
   const int S = K > 0 ? (K + GEMM_SEG - 1) / GEMM_SEG : 0;
-  if (M > 0 && N > 0 && S > 1) add_rows_shape(M, N, K, tiles, narrow);
+  if (M > 64 && N > 0 && big_add_shape(M, N, K, 4)) {      // a prompt portion: the segments' sums, whole
+    *scratch_floats = (long long)S * M * N;
+    *counters = 1;                                          // (none is used)
+    return 0;
+  }
+  if (M > 0 && M <= 64 && N > 0 && S > 1) add_rows_shape(M, N, K, tiles, narrow);
   *scratch_floats = (long long)tiles * S * 4096;
   *counters = tiles;
   return 0;

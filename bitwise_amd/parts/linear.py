@@ -49,8 +49,14 @@ class Linear:
         if self.mfma:
             # a long inner size and 17 to 64 rows: every 2048-segment of it gets workgroups of its own,
             # which meet in device scratch
+            # (and a prompt portion of 512 rows or more: 256 x 256 tiles, a workgroup per tile and segment; its scratch
+            # is sized for the longest step, so that one buffer serves every portion)
             scratch = None
-            floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features) if 16 < rows <= 64 else (0, 0)
+            floats, counters = 0, 0
+            if 16 < rows <= 64:
+                floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features)
+            elif rows >= 512 and ops.gemm_add_scratch(rows, self.out_features, self.in_features)[0]:
+                floats, counters = ops.gemm_add_scratch(self.rt.max_rows, self.out_features, self.in_features)
             if floats:
                 scratch = (self.rt.buffer("gemm_add_split", floats, torch.float32, rows=1),
                            self.rt.buffer("gemm_add_split_count", counters, torch.int32, rows=1))

@@ -168,6 +168,24 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             got = res.clone()
             ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
             assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
+    # a residual add of a prompt portion over several segments with scratch: 256 x 256 tiles, a workgroup per tile
+    # and segment, the segments joined in order afterwards: the bits of the add without scratch; ragged edges, a
+    # short last segment, scratch full of NaN and larger than needed
+    for M, N, K in [(700, 3000, 3 * 2048 + 128), (2048, 2048, 8192), (513, 8192, 4096)]:
+        x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
+        res = torch.randn(M, N, generator=g).to(gpu)
+        want = res.clone()
+        ops.gemm_bf16(x, w, want, M, ops.EPI_ADD_F32)
+        floats, counters = ops.gemm_add_scratch(M, N, K)
+        assert floats == ((K + 2047) // 2048) * M * N and counters > 0
+        scratch = (torch.full((floats + 1000,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
+        got = res.clone()
+        ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
+        assert torch.equal(got, want), (M, N, K)
+        with pytest.raises(RuntimeError, match="scratch smaller"):
+            ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=(scratch[0][:floats - 8], scratch[1]))
+    assert ops.gemm_add_scratch(2048, 2048, 2048) == (0, 0) and ops.gemm_add_scratch(300, 2048, 8192) == (0, 0)
     # SwiGLU with many columns (x shared through LDS; one, two or four blocks of 16 rows): the plain result, and
     # the bits of the same rows inside a prompt portion's product (another kernel)
     for inter, K in ((2100, 128), (2100, 2048 + 128)):             # the second: two segments of K
