@@ -15,7 +15,8 @@
 //   * up to 64 rows (decode steps, short prompt portions):
 //       - many columns: the "mid" kernel, a workgroup per 64 columns (32 of SwiGLU, or 32 where there are few
 //         columns and more than 16 rows), the rows of x shared by its four strips; optionally RMSNorm of up to 16
-//         rows fused in front (the rows normalised into LDS by the workgroup) and rotation + cache write behind;
+//         rows fused in front (the rows normalised into LDS by the workgroup) and rotation + cache write behind
+//         (a head a workgroup, or with fewer than 256 heads 16 rotary pairs of one);
 //         a residual add of 17 to 64 rows over several segments gives every segment workgroups of its own, which
 //         meet in device scratch and are added in segment order by the last to arrive;
 //       - up to 16 rows and few columns, or several segments: the "stream" kernel, a wave per strip and segment;
@@ -27,11 +28,13 @@
 //       - anything else (K no multiple of 64, SwiGLU with few columns): the "skinny" kernel, a wave per strip
 //         and segment streaming through a ring of registers;
 //   * more rows (prompt portions): 128 x 128 x 64 tiles, eight waves, fed through a four-stage LDS ring by the
-//     same kind of loads ("tile128"), and for products with at least 128 tiles of 256 x 256 the "big" kernel,
+//     same kind of loads ("tile128"; several segments are joined in registers, or for the residual add added
+//     into the output as they end), and for products with at least 128 tiles of 256 x 256 the "big" kernel,
 //     which computes twice as much per byte it fetches (a ring of five 32 KB slots, operand reads pipelined
-//     under the matrix instructions); the "wide" kernel (128 x 128 tiles staged through registers by four waves)
-//     takes what those do not: K no multiple of 64, several segments with another epilogue than the residual
-//     add, and the rotary epilogue below 512 rows.
+//     under the matrix instructions; one segment, or for a residual add with scratch a workgroup per tile and
+//     segment, the segments' sums joined in order by a second kernel); the "wide" kernel (128 x 128 tiles staged
+//     through registers by four waves) takes what those do not: K no multiple of 64 and the rotary epilogue
+//     below 512 rows.
 //
 // Epilogues: store 32-bit, store bfloat16, add into a 32-bit residual (each output owned
 // by one lane: no atomics), SwiGLU of two products (gate rows n, up rows N+n of a
