@@ -725,13 +725,15 @@ __device__ __forceinline__ void t128_issue(unsigned char* lds, __amdgpu_buffer_r
 template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile128_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles) {
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr bool ROPE = EPI == EPI_QKV_ROPE;           // waves of 32 x 64 outputs: a head's 64 columns in one wave
+  constexpr int NI = ROPE ? 2 : 4, NJ = ROPE ? 4 : 2;
   constexpr int COLS = GLU ? 64 : 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char t128_lds[];   // [4 stages][x 16 KB | W 16 KB]
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
-  const int wy = wave >> 2, wx = wave & 3;
+  const int wy = ROPE ? wave >> 1 : wave >> 2, wx = ROPE ? wave & 1 : wave & 3;
   int bid = blockIdx.x;
   const int nblocks = m_tiles * n_tiles;
   if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;      // an n tile's workgroups share an XCD
@@ -755,11 +757,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     voff_a[t] = ((16 * wave + r16) * ldx + 8 * chunk) * 2;
     voff_b[t] = ((b_row0 + r16) * K + 8 * chunk) * 2;
   }
-  f32x4 acc[4][2], tot[4][2];
+  f32x4 acc[NI][NJ], tot[NI][NJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
       tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
@@ -768,8 +770,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int slot_off[2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
-  const int a_frag = (4 * wy) * 2048;
-  const int b_frag = 16 * 1024 + (GLU ? wx : 2 * wx) * 2048;
+  const int a_frag = (NI * wy) * 2048;
+  const int b_frag = 16 * 1024 + (GLU ? wx : NJ * wx) * 2048;
   constexpr int b_step = GLU ? 4 * 2048 : 2048;                        // from the wave's first W block to its second
   const int steps = K / 64;
 #pragma unroll
@@ -782,20 +784,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned char* stage = t128_lds + (step % T128_STAGES) * T128_STAGE;
     __builtin_amdgcn_sched_barrier(0);
     // 12 operand reads and 16 matrix instructions a step, the second half's reads under the first half's products
-    u32x4 fa[2][4], fb[2][2];
+    u32x4 fa[2][NI], fb[2][NJ];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[kk][j] = *reinterpret_cast<const u32x4*>(stage + b_frag + j * b_step + slot_off[kk]);
+      for (int j = 0; j < NJ; ++j) fb[kk][j] = *reinterpret_cast<const u32x4*>(stage + b_frag + j * b_step + slot_off[kk]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) fa[kk][i] = *reinterpret_cast<const u32x4*>(stage + a_frag + i * 2048 + slot_off[kk]);
+      for (int i = 0; i < NI; ++i) fa[kk][i] = *reinterpret_cast<const u32x4*>(stage + a_frag + i * 2048 + slot_off[kk]);
     }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
     __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
 #pragma unroll
@@ -825,9 +827,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const int kn = (step + 1) * 64;
       if (kn % GEMM_SEG == 0 && kn < K) {              // a segment ends before the last: joined left to right
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
+          for (int j = 0; j < NJ; ++j) {
             tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
             acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
           }
@@ -836,10 +838,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   if (EPI != EPI_ADD_F32 && K > GEMM_SEG) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = tot[i][j] + acc[i][j];
+      for (int j = 0; j < NJ; ++j) acc[i][j] = tot[i][j] + acc[i][j];
   }
+  if constexpr (ROPE) {
+    tile_epilogue<EPI, NI>(acc, out, M, N, ldo, m0 + 32 * wy, n0 + 64 * wx, (n0 >> 6) + wx, r, g, false, rp);
+  } else {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -857,6 +862,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
       }
     }
+  }
 }
 
 // ------------------------------------------------------------------------------ up to 64 rows, through LDS
@@ -1572,7 +1578,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
-    if constexpr (EPI != EPI_QKV_ROPE) {
+    {
       // K in whole steps of 64: the tiles go straight into an LDS ring
       if (K % 64 == 0) {
         static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
@@ -1582,7 +1588,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
           allowed = true;
         }
         hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI>), grid, dim3(512), T128_STAGES * T128_STAGE, s, x, w, out, M, N, K, ldx,
-                           ldo, m_tiles, n_tiles);
+                           ldo, m_tiles, n_tiles, rp);
         return BW_LAUNCH_CHECK();
       }
     }
