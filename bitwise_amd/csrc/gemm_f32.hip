@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void gemm_f32_tile_kernel(const float* __restr
   }
 }
 
-// Up to 16 rows (decoded tokens): the same chains, one per thread.  A workgroup owns 16 columns and all rows,
+// Up to 64 rows (decoded tokens): the same chains, one per thread and block of 16 rows.  A workgroup owns 16 columns and all rows,
 // thread (m, n) the output of row m and column 16 * blockIdx.x + n; its 256 threads together bring 256 elements
 // of k of the 16 rows of W and of the rows of x into LDS at a time (16-byte loads; the next stage's loads fly
 // while this one is worked on), widened to 32-bit there, and every thread then walks the stage in k order with
@@ -184,17 +184,19 @@ __global__ __launch_bounds__(256) void gemm_f32_tile_kernel(const float* __restr
 // so that a product with few outputs still has loads in flight from many compute units.
 // K a multiple of 8 (of 4 for 32-bit weights), rows 16-byte aligned.
 #define F32R_NB 16
-#define F32R_KB 256
-#define F32R_STRIDE (F32R_KB + 4)   // floats from row to row in LDS: 16-byte reads of 16 rows hit 64 different banks
 
-template <typename WT>
+// MR blocks of 16 rows (up to 64 rows): thread (m, n) then runs the chains of rows m, m + 16, ... of its column,
+// and a stage is 128 elements of k instead of 256 (the rows of x take LDS).
+template <typename WT, int MR>
 __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restrict__ x, const WT* __restrict__ w,
                                                             float* __restrict__ y, int M, int N, int K, int ldx,
                                                             int ldy, int accumulate) {
+  constexpr int F32R_KB = MR == 1 ? 256 : 128;            // elements of k a stage
+  constexpr int F32R_STRIDE = F32R_KB + 4;                 // floats from row to row in LDS: 16-byte reads of 16 rows hit 64 different banks
   constexpr int WC = sizeof(WT) == 2 ? 8 : 4;             // elements of W in a 16-byte chunk
   constexpr int WPR = F32R_KB / WC;                        // chunks in a stage's row of W
   constexpr int WJ = F32R_NB * WPR / 256;                  // chunks of W a thread and stage
-  constexpr int XJ = 16 * (F32R_KB / 4) / 256;             // chunks of x a thread and stage (16 rows)
+  constexpr int XJ = 16 * MR * (F32R_KB / 4) / 256;        // chunks of x a thread and stage (16 * MR rows)
   extern __shared__ __attribute__((aligned(16))) float rows_lds[];   // [2][W: 16 rows | x: 16 rows] of F32R_STRIDE
   const int tid = threadIdx.x, n = tid & 15, m = tid >> 4;
   const int n0 = blockIdx.x * F32R_NB;
@@ -233,13 +235,31 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
       *reinterpret_cast<f32x4*>(buf + (F32R_NB + row) * F32R_STRIDE + kk) = xreg[j];
     }
   };
-  constexpr int BUF = 2 * 16 * F32R_STRIDE;                // floats of one buffer
+  constexpr int BUF = (1 + MR) * 16 * F32R_STRIDE;         // floats of one buffer
   float acc = 0.0f;
+  float accs[MR];                                          // (MR > 1)
+#pragma unroll
+  for (int r = 0; r < MR; ++r) accs[r] = 0.0f;
   auto work = [&](const float* buf, int k0) {              // the stage's steps of every chain, k ascending
     const int kend = (K - k0) < F32R_KB ? (K - k0) : F32R_KB;
     if (m >= M || kend <= 0) return;
     const float* wr = buf + n * F32R_STRIDE;
     const float* xr = buf + (F32R_NB + m) * F32R_STRIDE;
+    if constexpr (MR > 1) {
+#pragma unroll 4
+      for (int kk = 0; kk < kend; kk += 4) {
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(wr + kk);
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+          const f32x4 xv = *reinterpret_cast<const f32x4*>(xr + 16 * r * F32R_STRIDE + kk);   // (rows past M: finite, never stored)
+          accs[r] = fmaf(xv[0], wv[0], accs[r]);
+          accs[r] = fmaf(xv[1], wv[1], accs[r]);
+          accs[r] = fmaf(xv[2], wv[2], accs[r]);
+          accs[r] = fmaf(xv[3], wv[3], accs[r]);
+        }
+      }
+      return;
+    }
     if (kend == F32R_KB) {
       // a whole stage: blocks of 32 steps, the operands of the next block read from LDS while this block's steps
       // run (the wave has little company on its SIMD: what hides its read latency is its own chain)
@@ -302,23 +322,36 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
     store_stage(buf0, wa, xa);
     __syncthreads();
   }
-  if (m < M && n0 + n < N) {
-    float* o = y + (size_t)m * ldy + n0 + n;
-    *o = accumulate ? (*o + acc) : acc;
+  if (n0 + n >= N) return;
+#pragma unroll
+  for (int r = 0; r < MR; ++r) {
+    const int mr = m + 16 * r;
+    if (mr >= M) continue;
+    float* o = y + (size_t)mr * ldy + n0 + n;
+    const float v = MR == 1 ? acc : accs[r];
+    *o = accumulate ? (*o + v) : v;
   }
+}
+
+template <typename WT, int MR>
+static void launch_rows_mr(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                           hipStream_t s) {
+  constexpr int lds_bytes = 2 * (1 + MR) * 16 * ((MR == 1 ? 256 : 128) + 4) * (int)sizeof(float);
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<WT, MR>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<WT, MR>), dim3((N + F32R_NB - 1) / F32R_NB), dim3(256), lds_bytes, s, x, w, y, M, N, K,
+                     ldx, ldy, accumulate);
 }
 
 template <typename WT>
 static void launch_rows(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
                         hipStream_t s) {
-  constexpr int lds_bytes = 2 * 2 * 16 * F32R_STRIDE * (int)sizeof(float);
-  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
-  if (!allowed) {
-    (void)hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<WT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    allowed = true;
-  }
-  hipLaunchKernelGGL(gemm_f32_rows_kernel<WT>, dim3((N + F32R_NB - 1) / F32R_NB), dim3(256), lds_bytes, s, x, w, y, M, N, K,
-                     ldx, ldy, accumulate);
+  if (M <= 16) launch_rows_mr<WT, 1>(x, w, y, M, N, K, ldx, ldy, accumulate, s);
+  else if (M <= 32) launch_rows_mr<WT, 2>(x, w, y, M, N, K, ldx, ldy, accumulate, s);
+  else launch_rows_mr<WT, 4>(x, w, y, M, N, K, ldx, ldy, accumulate, s);
 }
 
 extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, int N, int K, int ldx,
@@ -329,12 +362,12 @@ extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* 
   hipStream_t s = (hipStream_t)stream;
   // which kernel runs depends on the shape alone, and both run the same chains
   const int wc = w_is_bf16 ? 8 : 4;
-  if (M <= 16 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+  if (M <= 64 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
     if (w_is_bf16) launch_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
     else launch_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
     return BW_LAUNCH_CHECK();
   }
-  if (M > 16 && K % F32T_BK == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+  if (M > 64 && K % F32T_BK == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
     dim3 tgrid((N + F32T_BN - 1) / F32T_BN, (M + F32T_BM - 1) / F32T_BM);
     if (w_is_bf16)
       hipLaunchKernelGGL(gemm_f32_tile_kernel<bf16_t>, tgrid, block, 0, s, x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate);

@@ -85,13 +85,15 @@ def test_gemm_f32_grid_rows_and_accumulate(gpu):
     ops.gemm_f32(x, wb, batch, 9, accumulate=True)
     assert torch.equal(batch, before + before)                     # y + acc, one addition per output
     # prompt portions (128 x 128 tiles, or 64 x 64 where K is no multiple of 16): a row's bits are those of the row alone
-    for M, N, K in [(150, 200, 1024), (129, 130, 64), (300, 77, 48), (70, 140, 1000)]:
+    # (and 17 to 64 rows: the chain-per-thread kernel with two or four blocks of rows)
+    for M, N, K in [(150, 200, 1024), (129, 130, 64), (300, 77, 48), (70, 140, 1000), (40, 130, 1024), (20, 77, 264),
+                    (64, 50, 136), (33, 16, 8)]:
         x, w = torch.randn(M, K, generator=g).to(gpu), torch.randn(N, K, generator=g).to(gpu)
         for weight in (w, w.bfloat16()):
             batch, one = torch.full((M, N), 3.0, device=gpu), torch.zeros(1, N, device=gpu)
             ops.gemm_f32(x, weight, batch, M)
             assert (batch.double() - x.double() @ weight.double().T).abs().max() <= 1e-6 * K ** 0.5 * batch.abs().max()
-            for r in (0, 63, 64, M // 2, M - 1):
+            for r in sorted({0, min(63, M - 1), min(64, M - 1), M // 2, M - 1}):
                 ops.gemm_f32(x[r:r + 1].contiguous(), weight, one, 1)
                 assert torch.equal(one[0], batch[r]), (M, N, K, r)
             before = batch.clone()
