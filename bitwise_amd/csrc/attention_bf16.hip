@@ -832,6 +832,9 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
 }
 
 #define DECODE_W 8
+#define DECODE_W_MANY 4          // waves a workgroup where there are several workgroups for every compute unit
+#define DECODE_MANY 1024          // that many workgroups: a workgroup's last, partly empty round of partitions costs more
+                                  // than what a compute unit gains from eight waves' loads in flight
 
 // How a decode launch over ``num_tiles`` tiles is split: workgroups per tile (1 = no split) and
 // the partitions a tile's scratch must hold.  Depends on nothing that changes from step to step.
@@ -861,6 +864,10 @@ static int launch_attention(const AttnBf16Args& a, int decode, float* scratch, s
         return -6;
       hipLaunchKernelGGL((attention_decode_kernel<HD, W, true>), dim3(a.num_tiles, items, nsplit), dim3(64 * W), pcap * cell, s,
                          a, pcap, scratch, counters, max_parts);
+    } else if (a.num_tiles * items >= DECODE_MANY) {
+      constexpr int WM = DECODE_W_MANY;            // (the partials are folded in partition order whatever the waves: the same bits)
+      hipLaunchKernelGGL((attention_decode_kernel<HD, WM, false>), dim3(a.num_tiles, items), dim3(64 * WM), pcap * cell, s, a,
+                         pcap, nullptr, nullptr, 0);
     } else {
       hipLaunchKernelGGL((attention_decode_kernel<HD, W, false>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a,
                          pcap, nullptr, nullptr, 0);

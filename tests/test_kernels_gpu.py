@@ -443,6 +443,21 @@ def test_attention_batched_equals_alone_and_plain(gpu, bf16, heads, kvh, hd, pag
         assert torch.equal(sh, batch)             # and so do several workgroups a tile
 
 
+def test_decode_attention_with_many_workgroups(gpu):
+    """So many tokens and kv heads that there are several workgroups for every compute unit (the decode kernel then
+    runs with fewer waves a workgroup): still the bits of the fold kernel."""
+    heads, kvh, hd, page = 32, 32, 16, 16
+    k, v, kc, vc, tab = paged_setup(gpu, True, heads, kvh, hd, page, 40, 500, seed=19, poison=True)
+    positions = [(37 * i + 5) % 500 for i in range(40)]           # 40 x 32 = 1280 workgroups
+    g = torch.Generator().manual_seed(20)
+    q = torch.randn(len(positions), heads * hd, generator=g).bfloat16()
+    fold = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page)
+    split = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True)
+    assert torch.equal(split, fold)
+    few = run_attention(gpu, True, q[:3], positions[:3], tab, kc, vc, heads, kvh, hd, page, split=True)
+    assert torch.equal(few, fold[:3])                              # (and of the same kernel with eight waves)
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 def test_attention_prompt_tiles_equal_single_rows(gpu, bf16):
     """Rows of a prompt portion share a tile with consecutive positions; each must equal the
