@@ -246,6 +246,21 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* _
   }
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
+    // Rotary: the cosines and sines of the block's four rows are asked for together, from addresses that are
+    // always valid (a padding row's position counts as 0), so that their latency is paid once a block, not once a row.
+    float cs[4][2], sn[4][2];
+    if constexpr (EPI == EPI_QKV_ROPE) {
+      if (head < rp.heads + rp.kv_heads) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const size_t at = (size_t)(pos_all[i][q] > 0 ? pos_all[i][q] : 0) * 32 + 16 * j + r;
+            cs[q][j] = rp.cos_table[at];
+            sn[q][j] = rp.sin_table[at];
+          }
+      }
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = row0 + 16 * i + 4 * g + q;
@@ -263,7 +278,7 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* _
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               const int d = 16 * j + r;
-              const float c = rp.cos_table[(size_t)pos * 32 + d], s = rp.sin_table[(size_t)pos * 32 + d];
+              const float c = cs[q][j], s = sn[q][j];
               const float x1 = acc[i][j][q], x2 = acc[i][j + 2][q];
               const float o1 = x1 * c - x2 * s;
               const float o2 = x2 * c + x1 * s;
