@@ -215,6 +215,62 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
                       torch.zeros(4, 12, device=gpu, dtype=torch.bfloat16), torch.zeros(2, 4, device=gpu), 2, ops.EPI_F32)
 
 
+def test_gemm_bf16_random_shapes(gpu):
+    """Which kernel runs is a matter of the shape: shapes drawn at random (edges of the row blocks, of the strips,
+    of the segments of K) through every epilogue, against float64 and, bit for bit, against the same rows alone."""
+    import random
+    rnd = random.Random(11)
+    g = torch.Generator().manual_seed(12)
+    ms = [1, 2, 7, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 127, 128, 129, 255, 256, 300, 511, 512, 513, 700]
+    ns = [8, 16, 24, 40, 64, 72, 128, 136, 200, 256, 264, 1000, 1024, 2048, 2056, 4096, 4104]
+    ks = [8, 32, 64, 72, 128, 192, 320, 1024, 2048, 2056, 2112, 4096, 4160]
+    done = 0
+    while done < 90:
+        M, N, K, epi = rnd.choice(ms), rnd.choice(ns), rnd.choice(ks), rnd.choice(["f32", "bf16", "add", "swiglu"])
+        if M * N > 1_500_000 or N * K > 9_000_000:
+            continue
+        done += 1
+        x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+        w = (torch.randn(N, K, generator=g) * (0.3 if epi == "swiglu" else 1.0)).bfloat16().to(gpu)
+        rows = sorted({0, M - 1, M // 2, min(15, M - 1), min(16, M - 1), min(64, M - 1)})
+        what = (M, N, K, epi)
+        if epi == "swiglu":
+            out = torch.zeros(M, N // 2, device=gpu, dtype=torch.bfloat16)
+            one = torch.zeros(1, N // 2, device=gpu, dtype=torch.bfloat16)
+            ops.gemm_bf16(x, w, out, M, ops.EPI_SWIGLU_BF16)
+            for r in rows:
+                ops.gemm_bf16(x[r:r + 1].contiguous(), w, one, 1, ops.EPI_SWIGLU_BF16)
+                assert torch.equal(one[0], out[r]), (what, r)
+            gate, up = x.double() @ w[:N // 2].double().T, x.double() @ w[N // 2:].double().T
+            ref = gate * torch.sigmoid(gate) * up
+            assert (out.double() - ref).abs().max() <= 2 ** -7 * ref.abs().max() + 1e-3, what
+            continue
+        ref = x.double() @ w.double().T
+        if epi == "add":
+            res = torch.randn(M, N, generator=g).to(gpu)
+            out, one = res.clone(), torch.zeros(1, N, device=gpu)
+            ops.gemm_bf16(x, w, out, M, ops.EPI_ADD_F32)
+            floats, counters = ops.gemm_add_scratch(M, N, K)
+            if floats:
+                scratch = (torch.full((floats,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
+                again = res.clone()
+                ops.gemm_bf16(x, w, again, M, ops.EPI_ADD_F32, scratch=scratch)
+                assert torch.equal(again, out), what
+            for r in rows:
+                one.copy_(res[r:r + 1])
+                ops.gemm_bf16(x[r:r + 1].contiguous(), w, one, 1, ops.EPI_ADD_F32)
+                assert torch.equal(one[0], out[r]), (what, r)
+            assert (out.double() - res.double() - ref).abs().max() <= 3e-6 * K ** 0.5 * ref.abs().max() + 1e-4, what
+            continue
+        dt, e = (torch.float32, ops.EPI_F32) if epi == "f32" else (torch.bfloat16, ops.EPI_BF16)
+        out, one = torch.zeros(M, N, device=gpu, dtype=dt), torch.zeros(1, N, device=gpu, dtype=dt)
+        ops.gemm_bf16(x, w, out, M, e)
+        for r in rows:
+            ops.gemm_bf16(x[r:r + 1].contiguous(), w, one, 1, e)
+            assert torch.equal(one[0], out[r]), (what, r)
+        assert (out.double() - ref).abs().max() <= (3e-6 * K ** 0.5 if epi == "f32" else 2 ** -8) * ref.abs().max() + 1e-4, what
+
+
 def test_gemm_bf16_weight_beyond_two_gib(gpu):
     """A weight of more than 2^31 bytes (a large vocabulary's head): every kernel addresses W through descriptors
     of a tile's rows, so only the tile has to fit 32-bit offsets.  The first and last columns equal the product
@@ -441,6 +497,48 @@ def test_attention_batched_equals_alone_and_plain(gpu, bf16, heads, kvh, hd, pag
         assert torch.equal(sp, batch)
         sh = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, split=True, shared=True)
         assert torch.equal(sh, batch)             # and so do several workgroups a tile
+
+
+def test_attention_random_shapes(gpu):
+    """Head sizes, groups, page sizes, windows and key counts drawn at random: a prompt portion's tiles, single rows,
+    the decode kernel and its split over workgroups agree bit for bit (bfloat16), tiles of rows and single rows
+    agree in 32-bit, and all are the plain result."""
+    import random
+    rnd = random.Random(21)
+    for case in range(36):
+        bf16 = rnd.random() < 0.6
+        hd = rnd.choice([16, 32, 48, 64, 80, 96, 128, 160, 256] if bf16 else [16, 32, 64, 96, 128, 160])
+        kvh = rnd.choice([1, 2, 3, 5])
+        group = rnd.choice([1, 2, 3, 4, 7] if bf16 else [1, 2, 4])
+        heads = kvh * group
+        page = rnd.choice([4, 8, 16, 32, 64] if bf16 else [4, 8, 16, 32])
+        nkeys = rnd.choice([5, 40, 64, 65, 130, 300])
+        pages = (nkeys + page - 1) // page + rnd.choice([1, 2, 3])
+        while pages % 7 == 0:
+            pages += 1
+        window = rnd.choice([0, 0, 3, 50, 200])
+        what = (case, bf16, heads, kvh, hd, page, nkeys, window)
+        k, v, kc, vc, tab = paged_setup(gpu, bf16, heads, kvh, hd, page, pages, nkeys, seed=100 + case, poison=True)
+        g = torch.Generator().manual_seed(200 + case)
+        positions = list(range(rnd.randrange(0, nkeys), nkeys))[:40]
+        q = torch.randn(len(positions), heads * hd, generator=g).to(torch.bfloat16 if bf16 else torch.float32)
+        single = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window)
+        if bf16:
+            tpt = max(1, 16 // min(group, 16))
+            tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+            while len(tiles) % ops.fold_group_tiles(hd):
+                tiles.append((0, 0, 0, 0))
+            assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles), single), what
+            assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, split=True), single), what
+            if ops.attention_decode_scratch(len(positions), heads, kvh, hd, tab.stride(0), page)[0]:
+                assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, split=True,
+                                                 shared=True), single), what
+        elif hd <= 128:
+            tpt = rnd.choice([1, 3, 16])
+            tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+            assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles), single), what
+        ref = plain_rows(q, k, v, positions, heads, window=window or None)
+        assert (single.cpu().double() - ref).abs().max() <= (2e-2 if bf16 else 5e-6) * ref.abs().max().clamp(min=0.05), what
 
 
 def test_decode_attention_with_many_workgroups(gpu):
