@@ -57,6 +57,7 @@ struct QkvRopeArgs {
   bf16_t* v_cache;
   int heads, kv_heads, page_size, table_stride, write_cache;
   int page_shift;              // page_size is a power of two: positions are split by shift and mask, not by division
+  int head_dim = 64;           // (the kernels for up to 64 rows take multiples of 64; the tiled ones 64)
 };
 
 #define GEMM_SEG 2048
@@ -971,11 +972,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
-  // rotary epilogue with narrow tiles: workgroup 2h + q has columns 16q..16q+15 and 32+16q..32+16q+15 of head h,
-  // 16 whole rotary pairs, as rows 0-15 and 16-31 of its tile of W
+  // rotary epilogue: a workgroup has PAIRS whole rotary pairs (i, i + head size / 2) of one head, 32 or (narrow
+  // tiles) 16: the pairs' first columns as the first half of its tile's rows of W, their second columns as the second
+  constexpr bool ROPE = EPI == EPI_QKV_ROPE;
   constexpr bool RN = S::ROPE_NARROW;
-  const int n0 = RN ? (blockIdx.x >> 1) * 64 : blockIdx.x * COLS;
-  const int b_rows = RN ? 64 : min(COLS, N - n0);
+  constexpr int PAIRS = RN ? 16 : 32, PSH = RN ? 4 : 5;              // rotary pairs of a row in this tile
+  const int hd = ROPE ? rp.head_dim : 64, half = hd >> 1;
+  const int tiles_per_head = half / PAIRS;
+  const int head = ROPE ? (int)blockIdx.x / tiles_per_head : 0;
+  const int pair0 = ROPE ? PAIRS * ((int)blockIdx.x % tiles_per_head) : 0;   // the tile's first pair within the head
+  const int n0 = ROPE ? head * hd : blockIdx.x * COLS;
+  const int b_rows = ROPE ? hd : min(COLS, N - n0);
   const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)x, 0, NORM ? 0 : (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
   // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
@@ -995,7 +1002,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   for (int t = 0; t < S::B_LOADS; ++t) {
     const int row = b_first + 8 * t + lrow;
     const int chunk = lslot ^ ((row & 15) >> 1);
-    const int w_row = RN ? 16 * (blockIdx.x & 1) + row + (row >= 16 ? 16 : 0) : (GLU ? row & 31 : row);
+    const int w_row = ROPE ? (row < PAIRS ? pair0 + row : half + pair0 + row - PAIRS) : (GLU ? row & 31 : row);
     voff_b[t] = (w_row * K + 8 * chunk) * 2;
   }
   // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
@@ -1021,9 +1028,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
 
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's columns are a head, or 16 pairs of
   // one): what this thread's (row, pair) items need, cosine, sine and page, hangs on the row's position.
-  constexpr int PAIRS = RN ? 16 : 32, PSH = RN ? 4 : 5;              // rotary pairs of a row in this tile
   constexpr int ITEMS = EPI == EPI_QKV_ROPE ? (RN ? NRB : 2 * NRB) : 1;   // (row, pair) items a thread: 16 * NRB rows x PAIRS
-  const int pair0 = RN ? 16 * (blockIdx.x & 1) : 0;                  // the tile's first pair within the head
   int r_pos[ITEMS], r_page[ITEMS];
   float r_cos[ITEMS], r_sin[ITEMS];
   if constexpr (EPI == EPI_QKV_ROPE) {
@@ -1089,8 +1094,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
       r_cos[j] = 1.f;
       r_sin[j] = 0.f;
       if (pos >= 0) {
-        r_cos[j] = rp.cos_table[(size_t)pos * 32 + pair0 + (e & (PAIRS - 1))];
-        r_sin[j] = rp.sin_table[(size_t)pos * 32 + pair0 + (e & (PAIRS - 1))];
+        r_cos[j] = rp.cos_table[(size_t)pos * half + pair0 + (e & (PAIRS - 1))];
+        r_sin[j] = rp.sin_table[(size_t)pos * half + pair0 + (e & (PAIRS - 1))];
         r_page[j] = rp.block_table[(size_t)rp.row_seq[e >> PSH] * rp.table_stride + (pos >> rp.page_shift)];
       }
     }
@@ -1118,7 +1123,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
     }
     asm volatile("" ::: "memory");
-    if constexpr (EPI != EPI_QKV_ROPE && !NORM) {
+    if constexpr (!NORM) {
       const int kn = (step + 1) * 64;
       if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {            // a segment ends before the last: left to right
 #pragma unroll
@@ -1131,7 +1136,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
       }
     }
   }
-  if constexpr (EPI != EPI_QKV_ROPE && !NORM) {
+  if constexpr (!NORM) {
     if (K > GEMM_SEG && gridDim.y == 1) {                               // the last segment joins the others
 #pragma unroll
       for (int i = 0; i < NI; ++i)
@@ -1153,7 +1158,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         if (m < M) os[m * 2 * PAIRS + 16 * strip + r] = acc[i][0][q];
       }
     __syncthreads();
-    const int head = RN ? blockIdx.x >> 1 : blockIdx.x;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int e = threadIdx.x + j * 256;
@@ -1166,18 +1170,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         const float o1 = x1 * c - x2 * sn;
         const float o2 = x2 * c + x1 * sn;
         bf16_t* dst = nullptr;
-        if (head < rp.heads) dst = (bf16_t*)out + (size_t)m * rp.heads * 64 + (size_t)head * 64;
+        if (head < rp.heads) dst = (bf16_t*)out + (size_t)m * rp.heads * hd + (size_t)head * hd;
         else if (rp.write_cache)
-          dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + (pos & (rp.page_size - 1))) * 64;
+          dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + (pos & (rp.page_size - 1))) * hd;
         if (dst != nullptr) {
           dst[i] = f32_to_bf16(o1);
-          dst[i + 32] = f32_to_bf16(o2);
+          dst[i + half] = f32_to_bf16(o2);
         }
       } else if (rp.write_cache) {
-        bf16_t* dst = rp.v_cache + ((size_t)r_page[j] * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * 64 * rp.page_size +
+        bf16_t* dst = rp.v_cache + ((size_t)r_page[j] * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * hd * rp.page_size +
                       (pos & (rp.page_size - 1));
         dst[(size_t)i * rp.page_size] = f32_to_bf16(x1);
-        dst[(size_t)(i + 32) * rp.page_size] = f32_to_bf16(x2);
+        dst[(size_t)(i + half) * rp.page_size] = f32_to_bf16(x2);
       }
     }
   } else {
@@ -1272,18 +1276,19 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
 // 64 and at least 64 of them (a workgroup a head); -7: not this shape.
 static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, void* q_out, int M, int K, const QkvRopeArgs& rp,
                                hipStream_t s) {
-  const int all_heads = rp.heads + 2 * rp.kv_heads;
-  if (M > 64 || K > GEMM_SEG || K % 64 || all_heads < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31))
+  const int all_heads = rp.heads + 2 * rp.kv_heads, hd = rp.head_dim;
+  const int wide_tiles = all_heads * (hd / 64);         // workgroups with 32 pairs each
+  if (M > 64 || K % 64 || hd % 64 || wide_tiles < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31))
     return -7;
-  const int N = all_heads * 64, ldo = rp.heads * 64;
-  if (all_heads < ROPE_NARROW_BELOW) {                 // fewer heads than compute units: half a head a workgroup
-    if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
-    if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
-    return launch_mid<EPI_QKV_ROPE, 4, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * all_heads, s, MidNormArgs{}, rp);
+  const int N = all_heads * hd, ldo = rp.heads * hd;
+  if (wide_tiles < ROPE_NARROW_BELOW) {                // fewer workgroups than compute units: 16 pairs a workgroup
+    if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp);
+    if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp);
+    return launch_mid<EPI_QKV_ROPE, 4, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp);
   }
-  if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
-  if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
-  return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, all_heads, s, MidNormArgs{}, rp);
+  if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, wide_tiles, s, MidNormArgs{}, rp);
+  if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, wide_tiles, s, MidNormArgs{}, rp);
+  return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, wide_tiles, s, MidNormArgs{}, rp);
 }
 
 // RMSNorm of up to 16 rows + the stacked q|k|v product + rotation + cache write in one kernel, for heads of 64
@@ -1293,17 +1298,18 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
                          int table_stride, const float* cos_table, const float* sin_table, void* k_cache, void* v_cache, int M,
                          int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream) {
   const int all_heads = heads + 2 * kv_heads;
-  if (head_dim != 64 || M > 16 || K > GEMM_SEG || K % 64 || all_heads < 64)
+  const int wide_tiles = all_heads * (head_dim / 64);
+  if (head_dim % 64 || M > 16 || K > GEMM_SEG || K % 64 || wide_tiles < 64)
     return -7;
   MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
-                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size)};
-  if (all_heads < ROPE_NARROW_BELOW)
-    return launch_mid<EPI_QKV_ROPE, 1, true, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64,
-                                                   2 * all_heads, (hipStream_t)stream, na, rp);
-  return launch_mid<EPI_QKV_ROPE, 1, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * 64, K, 0, heads * 64, all_heads,
-                                           (hipStream_t)stream, na, rp);
+                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size), head_dim};
+  if (wide_tiles < ROPE_NARROW_BELOW)
+    return launch_mid<EPI_QKV_ROPE, 1, true, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * head_dim, K, 0,
+                                                   heads * head_dim, 2 * wide_tiles, (hipStream_t)stream, na, rp);
+  return launch_mid<EPI_QKV_ROPE, 1, true>(nullptr, (const bf16_t*)w_qkv, q_out, M, all_heads * head_dim, K, 0, heads * head_dim,
+                                           wide_tiles, (hipStream_t)stream, na, rp);
 }
 
 // ------------------------------------------------------------------------------ up to 16 rows, few columns
@@ -1671,12 +1677,12 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
                                      int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                                      int write_cache, void* stream) {
   if (M <= 0) return 0;
-  if (head_dim != 64) return -4;
-  if (K <= 0 || K > GEMM_SEG || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
+  if (head_dim != 64 && (M > 64 || head_dim % 64)) return -4;     // the tiled kernels' epilogue: heads of 64
+  if (K <= 0 || (K > GEMM_SEG && M > 64) || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_qkv)) & 15) return -3;
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
-                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size)};
+                 heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size), head_dim};
   if (M <= 64) {
     const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
     return mid == -7 ? -2 : mid;

@@ -461,19 +461,20 @@ def attention_decode_scratch(num_tiles: int, heads: int, kv_heads: int, head_dim
 
 def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int, all_heads: int = 0) -> bool:
     """Whether the q|k|v product of normalised rows can take rotation and cache write into its
-    epilogue: heads of 64 and one segment of K; more than 64 rows, or (a workgroup a head) up to
-    64 rows of at least 64 heads (q, k and v heads together) with K in steps of 64."""
-    if head_dim != 64 or inner > 2048 or inner % 8:
-        return False
-    return rows > 64 or (all_heads >= 64 and inner % 64 == 0)
+    epilogue.  More than 64 rows: heads of 64 and one segment of K.  Up to 64 rows (a workgroup per 32 or 16
+    rotary pairs of a head): head sizes in multiples of 64, K in steps of 64, and enough heads (q, k and v
+    heads together) for 64 workgroups."""
+    if rows > 64:
+        return head_dim == 64 and inner <= 2048 and inner % 8 == 0
+    return head_dim % 64 == 0 and inner % 64 == 0 and all_heads * (head_dim // 64) >= 64
 
 
 def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
                        row_seq: torch.Tensor, block_table: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                        k_cache: torch.Tensor, v_cache: torch.Tensor, rows: int, heads: int, kv_heads: int,
                        head_dim: int, page_size: int, write_cache: bool = True) -> None:
-    """The stacked q|k|v product of more than 64 rows with rotation and cache write in its epilogue
-    (heads of 64); the bits of gemm_bf16 into a 32-bit buffer followed by rope_kvwrite."""
+    """The stacked q|k|v product with rotation and cache write in its epilogue (the shapes of
+    ``qkv_rope_gemm_ok``); the bits of gemm_bf16 into a 32-bit buffer followed by rope_kvwrite."""
     _need(x, torch.bfloat16, "x")
     _need(w_qkv, torch.bfloat16, "qkv weight")
     _need(q_out, torch.bfloat16, "q_out")
@@ -486,7 +487,7 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
     _need(sin, torch.float32, "sin table")
     N, K = w_qkv.shape
     if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_gemm_ok(rows, head_dim, K, heads + 2 * kv_heads):
-        raise ValueError("gemm_qkv_rope_bf16: not a [q|k|v] weight of 64-element heads, or too few rows")
+        raise ValueError("gemm_qkv_rope_bf16: not a [q|k|v] weight, or a shape the rotary epilogue does not take")
     if x.shape[1] != K or x.shape[0] < rows or q_out.shape[1] != heads * head_dim or q_out.shape[0] < rows:
         raise ValueError("gemm_qkv_rope_bf16: buffers do not fit")
     if positions.numel() < rows or row_seq.numel() < rows or cos.shape[1] != head_dim // 2 or sin.shape != cos.shape:

@@ -688,7 +688,8 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
 
     for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
                                      (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128),    # the last two: half a head a workgroup,
-                                     (200, 28, 64, 16, 64)]:                                          # a head a workgroup
+                                     (200, 28, 64, 16, 64),                                           # a head a workgroup
+                                     (24, 4, 128, 16, 128), (12, 2, 256, 8, 64), (100, 14, 128, 16, 64)]:     # larger heads: 16 or 32 pairs a workgroup
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
@@ -723,12 +724,15 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
     epilogue; q, the key pages and the value pages must be the bits of product + rope_kvwrite.
     Rows of two requests, a padding row, positions across page edges, a ragged last tile."""
     g = torch.Generator().manual_seed(21)
-    for heads, kvh, K, M, page in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
+    for case in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
                                    (5, 2, 96, 150, 16), (2, 2, 40, 190, 8),   # K no multiple of 64: tiles through registers
                                    (40, 10, 128, 2100, 32),        # enough 256 x 256 tiles for the big-tile kernel
                                    (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16),   # up to 64 rows, half a head a workgroup
-                                   (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32)]:   # a head a workgroup
-        hd = 64
+                                   (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32),   # a head a workgroup
+                                   (40, 12, 4160, 16, 16),                                 # several segments of K
+                                   (32, 8, 4096, 8, 16, 128), (24, 4, 128, 40, 8, 128), (100, 14, 64, 12, 16, 128),
+                                   (16, 8, 2112, 20, 16, 256)]:                            # larger heads, up to 64 rows
+        heads, kvh, K, M, page, hd = (tuple(case) + (64,))[:6]
         pages = 40 if M < 500 else 3 * ((M + page - 1) // page + 2) + 3
         cos, sin = rope_tables(10000.0, hd, max(400, M), gpu)
         h = torch.randn(M, K, generator=g).bfloat16().to(gpu)
@@ -758,7 +762,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
         assert torch.equal(outs[0][0][live], outs[1][0][live]), (heads, kvh, K, M)
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), (heads, kvh, K, M)
     assert not ops.qkv_rope_gemm_ok(64, 64, 256, 63) and not ops.qkv_rope_gemm_ok(200, 128, 256, 96)
-    assert not ops.qkv_rope_gemm_ok(64, 64, 96, 96)
+    assert not ops.qkv_rope_gemm_ok(64, 64, 96, 96) and not ops.qkv_rope_gemm_ok(8, 96, 128, 200) and not ops.qkv_rope_gemm_ok(200, 64, 4096, 96)
 
 
 def test_decode_attention_beyond_one_pass_of_partials(gpu):
