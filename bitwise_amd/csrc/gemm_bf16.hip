@@ -709,7 +709,100 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
   }
-  tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
+  if constexpr (EPI == EPI_QKV_ROPE) {
+    // What the rows of the tile need from memory is fetched once for the workgroup, into the ring (free now), not
+    // by every lane for each of its rows: position and page of each of the 256 rows (a thread a row), then the
+    // rows' cosines and sines (16-byte loads; a row of 32 + 32 floats, 36 apart against bank conflicts).
+    constexpr int CS = 36;
+    __builtin_amdgcn_s_waitcnt(BIG_WAIT_ALL);
+    __syncthreads();                                                // every wave is done with the ring
+    int* pos_lds = reinterpret_cast<int*>(big_lds);                 // [256]
+    int* page_lds = pos_lds + BIG_BM;                               // [256]
+    float* cos_lds = reinterpret_cast<float*>(page_lds + BIG_BM);   // [256][CS]
+    float* sin_lds = cos_lds + BIG_BM * CS;                         // [256][CS]
+    const int first_head = n0 >> 6;
+    const bool any_cache = first_head + 4 > rp.heads;               // some of the tile's four heads are k or v heads
+    const bool any_rotary = first_head < rp.heads + rp.kv_heads;
+    if (threadIdx.x < BIG_BM) {
+      const int m = m0 + (int)threadIdx.x;
+      const int mm = m < M ? m : M - 1;
+      const int pos = rp.positions[mm];
+      int page = 0;
+      if (any_cache) page = rp.block_table[(size_t)rp.row_seq[mm] * rp.table_stride + ((pos > 0 ? pos : 0) >> rp.page_shift)];
+      pos_lds[threadIdx.x] = m < M ? pos : -1;
+      page_lds[threadIdx.x] = page;
+    }
+    __syncthreads();
+    if (any_rotary) {
+      const int row = threadIdx.x >> 1, part = threadIdx.x & 1;     // 16 cosines and 16 sines of a row a thread
+      const int pos = pos_lds[row];
+      const size_t at = (size_t)(pos > 0 ? pos : 0) * 32 + 16 * part;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        *reinterpret_cast<f32x4*>(cos_lds + row * CS + 16 * part + 4 * t) = *reinterpret_cast<const f32x4*>(rp.cos_table + at + 4 * t);
+        *reinterpret_cast<f32x4*>(sin_lds + row * CS + 16 * part + 4 * t) = *reinterpret_cast<const f32x4*>(rp.sin_table + at + 4 * t);
+      }
+    }
+    __syncthreads();
+    const int head = first_head + wx;
+    if (head >= rp.heads + 2 * rp.kv_heads) return;
+    const int q_dim = rp.heads * 64;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int lrow0 = 128 * wy + 16 * i + 4 * g;                  // the lane's four rows of the block, within the tile
+      int pos4[4], page4[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        pos4[q] = pos_lds[lrow0 + q];
+        page4[q] = page_lds[lrow0 + q];
+      }
+      if (head < rp.heads + rp.kv_heads) {
+        if (head >= rp.heads && !rp.write_cache) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int pos = pos4[q];
+          if (pos < 0) continue;
+          const int m = m0 + lrow0 + q;
+          bf16_t* dst = head < rp.heads
+                            ? (bf16_t*)out + (size_t)m * q_dim + (size_t)head * 64
+                            : rp.k_cache + (((size_t)page4[q] * rp.kv_heads + (head - rp.heads)) * rp.page_size + (pos & (rp.page_size - 1))) * 64;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int d = 16 * j + r;
+            const float c = cos_lds[(lrow0 + q) * CS + d], sn = sin_lds[(lrow0 + q) * CS + d];
+            const float x1 = acc[i][j][q], x2 = acc[i][j + 2][q];
+            dst[d] = f32_to_bf16(x1 * c - x2 * sn);
+            dst[d + 32] = f32_to_bf16(x2 * c + x1 * sn);
+          }
+        }
+      } else if (rp.write_cache) {
+        // values lie transposed in their page ([d][slot]).  The lane's four rows are most often four consecutive
+        // slots of one page starting at a multiple of four: then all four are stored at once.
+        bool quad = pos4[0] >= 0 && (pos4[0] & 3) == 0;
+#pragma unroll
+        for (int t = 1; t < 4; ++t) quad = quad && pos4[t] == pos4[0] + t && page4[t] == page4[0];
+        const int vh = head - rp.heads - rp.kv_heads;
+        if (quad) {
+          bf16_t* dst = rp.v_cache + ((size_t)page4[0] * rp.kv_heads + vh) * 64 * rp.page_size + (pos4[0] & (rp.page_size - 1));
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x2 four = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
+            *reinterpret_cast<u32x2*>(dst + (size_t)(16 * j + r) * rp.page_size) = four;
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (pos4[q] < 0) continue;
+            bf16_t* dst = rp.v_cache + ((size_t)page4[q] * rp.kv_heads + vh) * 64 * rp.page_size + (pos4[q] & (rp.page_size - 1));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
+          }
+        }
+      }
+    }
+  } else {
+    tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
+  }
 }
 
 // ------------------------------------------------------------------------------ 128 x 128 tiles through an LDS ring
