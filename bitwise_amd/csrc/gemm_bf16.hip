@@ -33,20 +33,20 @@
 //     which computes twice as much per byte it fetches (a ring of five 32 KB slots, operand reads pipelined
 //     under the matrix instructions; one segment, or for a residual add with scratch a workgroup per tile and
 //     segment, the segments' sums joined in order by a second kernel); the "wide" kernel (128 x 128 tiles staged
-//     through registers by four waves) takes what those do not: K no multiple of 64 and the rotary epilogue
-//     below 512 rows.
+//     through registers by four waves) takes what those do not: K no multiple of 64.
 //
 // Epilogues: store 32-bit, store bfloat16, add into a 32-bit residual (each output owned
 // by one lane: no atomics), SwiGLU of two products (gate rows n, up rows N+n of a
-// stacked weight) stored as bfloat16: h = g * (1/(1+exp(-g))) * u in 32-bit, or (heads of 64) rotary
-// encoding of the stacked q|k|v product and the write of k and v to their page slots.
+// stacked weight) stored as bfloat16: h = g * (1/(1+exp(-g))) * u in 32-bit, or rotary encoding of the
+// stacked q|k|v product and the write of k and v to their page slots (heads of 64; up to 64 rows: head sizes
+// in multiples of 64).
 #include "common.h"
 #include "api.h"
 
 enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3, EPI_QKV_ROPE = 4 };
 
-// What the rotary epilogue of the stacked q|k|v product needs (wide kernel, heads of 64): the
-// statements of rope_kvwrite_bf16_kernel on the 32-bit products while they are still in registers.
+// What the rotary epilogue of the stacked q|k|v product needs: the statements of
+// rope_kvwrite_bf16_kernel on the 32-bit products while they are still in registers.
 struct QkvRopeArgs {
   const int32_t* positions;    // [rows]; negative = padding row
   const int32_t* row_seq;      // [rows] -> row of the block table
