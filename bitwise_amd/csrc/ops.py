@@ -274,10 +274,13 @@ def norm_gemm_supported(rows: int, inner: int) -> bool:
     return _decode_ok[key]
 
 
-def qkv_rope_head_dim_ok(head_dim: int) -> bool:
+def qkv_rope_head_dim_ok(head_dim: int, inner: int) -> bool:
     """Head sizes the fused norm + q|k|v + rotation kernel takes: multiples of 32 (a workgroup
-    is a pair of 16-column strips half a head apart) and 16 or 48 (a workgroup is a head)."""
-    return head_dim % 16 == 0 and head_dim >= 16 and (head_dim % 32 == 0 or head_dim <= 64)
+    is a pair of 16-column strips half a head apart) and 16 or 48 (a workgroup is a head); its epilogue
+    reuses the LDS that held the rows, so a workgroup's 32-bit products must fit a row of ``inner`` elements."""
+    if head_dim % 16 or head_dim < 16 or not (head_dim % 32 == 0 or head_dim <= 64):
+        return False
+    return (32 if head_dim % 32 == 0 else head_dim) * 4 <= (inner + 8) * 2
 
 
 def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor) -> bool:
@@ -323,7 +326,7 @@ def norm_qkv_rope_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w
     _need(cos, torch.float32, "cos table")
     _need(sin, torch.float32, "sin table")
     N, K = w_qkv.shape
-    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_head_dim_ok(head_dim):
+    if N != (heads + 2 * kv_heads) * head_dim or not qkv_rope_head_dim_ok(head_dim, K):
         raise ValueError("norm_qkv_rope_bf16: weight is not [q|k|v] heads of a supported size")
     if not can_fuse_norm(rows, w_qkv, x) or norm_weight.numel() != K:
         raise ValueError("norm_qkv_rope_bf16: this step cannot be fused")

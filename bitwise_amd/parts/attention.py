@@ -78,7 +78,8 @@ class Attention(Mixer):
         """Decode steps of few rows: norm, q|k|v product, rotation and cache write are one kernel."""
         from .norm import RMSNorm
         rt = self.rt
-        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma and ops.qkv_rope_head_dim_ok(self.head_dim)
+        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma
+                and ops.qkv_rope_head_dim_ok(self.head_dim, self.qkv.weight.shape[1])
                 and ops.can_fuse_norm(ctx.rows, self.qkv.weight, x)):
             return False
         q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)

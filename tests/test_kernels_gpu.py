@@ -685,6 +685,7 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
             assert torch.equal(fused_s, sep_s), (M, K, N)
     assert not ops.can_fuse_norm(17, w, x) and not ops.can_fuse_norm(4, torch.zeros(8, 4096, dtype=torch.bfloat16), x)
     assert not ops.can_fuse_norm(4, torch.zeros(8, 96, dtype=torch.bfloat16), torch.zeros(4, 96))   # steps of 64 along the rows
+    assert not ops.qkv_rope_head_dim_ok(48, 64) and ops.qkv_rope_head_dim_ok(48, 192) and ops.qkv_rope_head_dim_ok(256, 64)   # the epilogue's LDS
 
     for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
                                      (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128),    # the last two: half a head a workgroup,

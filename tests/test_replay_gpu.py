@@ -209,6 +209,37 @@ def test_trace_run_program(folders, tmp_path):
             assert np.abs(g - r).max() <= TOL[dtype] * np.abs(r).max()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_awkward_sizes(gpu, tmp_path, dtype):
+    """Configurations whose sizes fall between the kernels' favourite ones (head sizes 48, 80 and 256, 14 heads on 2,
+    a width of 64 with heads of 48, a feed-forward of 8, a vocabulary of 17; one segment of K and a bit): every
+    fusion that does not take them must step aside, and the logits are the plain ones whatever the cutting."""
+    import bitwise_amd as bw
+    from bitwise_amd.model import write_random_model
+
+    base = dict(tiny.TINY_A, max_position_embeddings=512)
+    configs = [
+        dict(base, hidden_size=136, num_attention_heads=6, num_key_value_heads=3, head_dim=80, intermediate_size=344,
+             vocab_size=1001, num_hidden_layers=3, tie_word_embeddings=False),
+        dict(base, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=256, intermediate_size=520,
+             vocab_size=4099, num_hidden_layers=2),
+        dict(base, hidden_size=64, num_attention_heads=14, num_key_value_heads=2, head_dim=48, intermediate_size=8,
+             vocab_size=17, num_hidden_layers=1),
+        dict(base, hidden_size=2048 + 64, num_attention_heads=33, num_key_value_heads=33, head_dim=64,
+             intermediate_size=2056, vocab_size=1000, num_hidden_layers=1, tie_word_embeddings=False),
+    ]
+    for i, cfg in enumerate(configs):
+        folder = tmp_path / f"awkward{i}"
+        write_random_model(folder, cfg, 10 + i, 0.05, "bfloat16")
+        model = bw.Model.load(folder, dtype)
+        g = torch.Generator().manual_seed(30 + i)
+        toks = torch.randint(0, cfg["vocab_size"], (75,), generator=g).tolist()
+        whole = model.logits(toks)
+        want = pl.forward(cfg, tiny.read_weights(folder), toks, pl.round_bf16 if dtype == "bfloat16" else pl.identity).numpy()
+        assert np.abs(whole - want).max() <= TOL[dtype] * np.abs(want).max(), (i, dtype)
+        assert np.array_equal(model.logits(toks, chunk=5), whole) and np.array_equal(model.logits(toks, chunk=1), whole), (i, dtype)
+
+
 def test_real_layer_sizes_are_cut_invariant(gpu):
     """Two layers of the SmolLM2-1.7B sizes, so that every shape-dependent route of the kernels runs at the shapes it
     was written for (K = 2048 and 8192, 6144 / 2048 / 16384 / 49152 columns): a prompt whole; in portions of 1600, 300,
