@@ -1055,6 +1055,36 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
                                              real ? voff_b[t] : 0x7ffffff0, (k_base + step * 64) * 2, 0, 0);
 }
 
+// The NORM variant's rows: wave ``wave`` normalises rows wave, wave + 4, ... (RB of them at most) into LDS, the
+// ring's first stages asked for between the rows' loads and the arithmetic.
+template <int RB, int EPI, int NRB, bool NARROW>
+__device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int K, int wave, int lane, unsigned char* rows_lds,
+                                              unsigned char* mid_lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
+                                              const int* voff_a, const int* voff_b, int steps, int k_base) {
+  using S = MidShape<EPI, NRB, true, NARROW>;
+  const int nvec = K >> 2;
+  NormRows<RB> nr;
+  const f32x4* nrows[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int m = wave + i * S::NW;
+    nrows[i] = m < M ? reinterpret_cast<const f32x4*>(na.x32 + (size_t)m * na.ldx32) : nullptr;
+  }
+  norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
+  __builtin_amdgcn_sched_barrier(0);
+  unsigned char* rl = rows_lds;
+  const int nw = S::NW;
+  norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
+    // vector c = elements 4c..4c+3 of row m: step c / 16, 16-byte chunk (c % 16) / 2 of the step, its half c % 2
+    const int m = wave + i * nw;
+    unsigned char* p = rl + (c >> 4) * 2048 + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ (m >> 1)) * 16) + (c & 1) * 8;
+    *reinterpret_cast<u32x2*>(p) = pk;
+  });
+}
+
 template <int EPI, int NRB, bool NORM, bool NARROW>
 __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
@@ -1138,32 +1168,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   unsigned char* rows_lds = mid_lds + S::RING;
   if constexpr (NORM) {
     // the rows to normalise are asked for before the ring (loads complete in the order they are issued: the
-    // wait for the rows must not be a wait for weights), four rows a wave at a time
-    constexpr int RB = 4;
-    const int nvec = K >> 2;
-    NormRows<RB> nr;
-    const f32x4* nrows[RB];
-    for (int m0 = wave; m0 < M; m0 += RB * S::NW) {
-#pragma unroll
-      for (int i = 0; i < RB; ++i) {
-        const int m = m0 + i * S::NW;
-        nrows[i] = m < M ? reinterpret_cast<const f32x4*>(na.x32 + (size_t)m * na.ldx32) : nullptr;
-      }
-      norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
-      if (m0 == wave) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      unsigned char* rl = rows_lds;
-      const int nw = S::NW;
-      norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
-        // vector c = elements 4c..4c+3 of row m: step c / 16, 16-byte chunk (c % 16) / 2 of the step, its half c % 2
-        const int m = m0 + i * nw;
-        unsigned char* p = rl + (c >> 4) * 2048 + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ (m >> 1)) * 16) + (c & 1) * 8;
-        *reinterpret_cast<u32x2*>(p) = pk;
-      });
+    // wait for the rows must not be a wait for weights); wave w takes rows w, w + 4, ...: as many at a time as
+    // there are (a slot without a row would fetch a row for nothing)
+    if (wave < M) {
+      if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
+      else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
+      else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
+      else mid_norm_rows<4, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
     }
     if (wave >= M) {                                                   // a wave without rows still feeds the ring
 #pragma unroll
