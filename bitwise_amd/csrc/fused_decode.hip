@@ -86,6 +86,43 @@ __device__ __forceinline__ void decode_issue(unsigned char* ring, const __amdgpu
                                                step * 128, 0, 0);
 }
 
+// The rows of the residual stream, normalised into LDS as bfloat16: wave ``wave`` has rows wave, wave + nwaves,
+// ..., RB of them at a time.  The ring's first stages are asked for after the first batch's loads and before its
+// arithmetic, so that they stay in flight meanwhile.  (A second batch, with more than RB rows a wave, is loaded
+// after the ring's first stages; the compiler's wait for it also waits for those, so the caller's wait counts hold.)
+template <int RB, int EPI, int ST>
+__device__ __forceinline__ void decode_norm_rows(const DecodeGemmArgs& a, int wave, int nwaves, int lane, bf16_t* xs, int lds_row,
+                                                 unsigned char* ring, const __amdgpu_buffer_rsrc_t* rs_w, const int* voff_w,
+                                                 int steps) {
+  using SH = DecodeShape<EPI, ST>;
+  const int M = a.M, K = a.K, nvec = K >> 2;
+  NormRows<RB> nr;
+  const f32x4* nrows[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int m = wave + i * nwaves;               // rows are dealt to the waves round robin
+    nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
+  }
+  if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int st = 0; st < SH::STAGES - 1; ++st) decode_issue<EPI, ST>(ring, rs_w, voff_w, st, steps);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int m0 = wave; m0 < M;) {
+    norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
+      *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
+    });
+    m0 += RB * nwaves;
+    if (m0 >= M) break;
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      const int m = m0 + i * nwaves;
+      nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
+    }
+    norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
+  }
+}
+
 template <int EPI, int ST>
 __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   using SH = DecodeShape<EPI, ST>;
@@ -154,42 +191,17 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
     asm volatile("" ::: "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
-  // then the rows to normalise (their first batch)
-  constexpr int RB = 4;                            // rows a wave normalises at a time
-  const int nvec = K >> 2;
-  NormRows<RB> nr;
-  const f32x4* nrows[RB];
-#pragma unroll
-  for (int i = 0; i < RB; ++i) {
-    const int m = wave + i * nwaves;               // rows are dealt to the waves round robin
-    nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
-  }
-  if (wave < M) norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
-  __builtin_amdgcn_sched_barrier(0);
-  // then the ring's first stages, which stay in flight while the rows are normalised
-#pragma unroll
-  for (int st = 0; st < SH::STAGES - 1; ++st) decode_issue<EPI, ST>(ring, rs_w, voff_w, st, steps);
-  __builtin_amdgcn_sched_barrier(0);
-
-  // 2. the M rows into LDS as bfloat16, normalised
-  for (int m0 = wave; m0 < M;) {
-    norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
-      *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
-    });
-    m0 += RB * nwaves;
-    if (m0 >= M) break;
-#pragma unroll
-    for (int i = 0; i < RB; ++i) {
-      const int m = m0 + i * nwaves;
-      nrows[i] = m < M ? reinterpret_cast<const f32x4*>(a.a + (size_t)m * a.lda) : nullptr;
-    }
-    norm_rows_load<RB>(nr, nrows, a.norm_w, a.norm_w_is_bf16, nvec, lane);
-  }
+  // then the rows to normalise, the ring's first stages asked for between their loads and the arithmetic; a wave
+  // fetches as many rows at a time as it has (four at most)
+  const int rows_a_wave = (M + nwaves - 1) / nwaves;
+  if (rows_a_wave <= 1) decode_norm_rows<1, EPI, ST>(a, wave, nwaves, lane, xs, lds_row, ring, rs_w, voff_w, steps);
+  else if (rows_a_wave == 2) decode_norm_rows<2, EPI, ST>(a, wave, nwaves, lane, xs, lds_row, ring, rs_w, voff_w, steps);
+  else if (rows_a_wave == 3) decode_norm_rows<3, EPI, ST>(a, wave, nwaves, lane, xs, lds_row, ring, rs_w, voff_w, steps);
+  else decode_norm_rows<4, EPI, ST>(a, wave, nwaves, lane, xs, lds_row, ring, rs_w, voff_w, steps);
   __syncthreads();
 
   // 3. the product: A from the rows in LDS (rows past M read row 0; their results are thrown away), B from
-  // the wave's ring.  (A second batch of rows to normalise, with more than RB rows a wave, was loaded after
-  // the ring's first stages; the compiler's wait for it also waited for those, so the count below holds.)
+  // the wave's ring.
   const bf16_t* ap = xs + (size_t)(r < M ? r : 0) * lds_row + 8 * g;
   int off_w[2];
 #pragma unroll
