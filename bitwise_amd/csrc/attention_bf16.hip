@@ -411,13 +411,21 @@ struct FoldShape {
   static constexpr int GROUP = NW * QT;
   static constexpr int NBUF = HD <= 128 ? 2 : 1;
   static constexpr int WAVES = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);   // waves per SIMD the register budget is set for
-  static constexpr int KSTR = HD * 2 + 16;          // bytes from key to key in LDS (16 of padding against bank conflicts)
-  static constexpr int VSTR = ATT_PART * 2 + 16;    // bytes from d to d
+  // LDS layout, measured on the part: 16-byte operand reads of 16 rows by 4 chunks run at full rate when the rows lie
+  // an odd multiple of 32 bytes apart (at twice the time 16 bytes off that, four times at a multiple of 128); 8-byte
+  // reads want rows an odd multiple of 8 bytes apart, or 128-byte rows whose 8-byte slots are permuted (fold_v_slot)
+  static constexpr int KSTR = HD * 2 + (HD % 32 == 0 ? 32 : 0);   // bytes from key to key
+  static constexpr int VSTR = ATT_PART * 2;                       // bytes from d to d: no padding, slots permuted
   static constexpr int KBYTES = ATT_PART * KSTR;
   static constexpr int BYTES = KBYTES + HD * VSTR;  // one partition
   static constexpr int KJ = (ATT_PART * (HD / 8) + 64 * NW - 1) / (64 * NW);   // 16-byte key chunks per thread
   static constexpr int VJ = (HD * (ATT_PART / 4) + 64 * NW - 1) / (64 * NW);   // 8-byte value chunks per thread
 };
+
+// Where the 8-byte slot ``slot`` (keys 4 * slot .. 4 * slot + 3) of the values' row d lies in the row: the two low
+// bit pairs of d, swapped, are xor-ed onto the slot number.  The 16 rows of an operand read then hit 16 different
+// slots, and so do the 4 consecutive rows by 4 consecutive slots that 16 lanes store from pages of 16.
+__device__ __forceinline__ int fold_v_slot(int slot, int d) { return (slot ^ (((d & 3) << 2) | ((d >> 2) & 3))) & 15; }
 
 template <int HD>
 struct Staged {
@@ -526,7 +534,7 @@ __device__ __forceinline__ void stage_store(const WorkgroupCtx& wc, const StageP
       v2 = (u32x2){v2[0] & m0, v2[1] & m1};
     }
     if (sp.v_key[j] < ATT_PART)
-      *reinterpret_cast<u32x2*>(buf + S::KBYTES + sp.v_d[j] * S::VSTR + sp.v_key[j] * 2) = v2;
+      *reinterpret_cast<u32x2*>(buf + S::KBYTES + sp.v_d[j] * S::VSTR + 8 * fold_v_slot(sp.v_key[j] >> 2, sp.v_d[j])) = v2;
   }
 }
 
@@ -633,8 +641,10 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
         for (int t = 0; t < QT; ++t) o_p[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-          const unsigned char* vrow = vb + (16 * dt + gc.r) * S::VSTR + (32 * w + 4 * gc.g) * 2;
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow), hi = *reinterpret_cast<const u32x2*>(vrow + 32);
+          // keys 32w + 4g .. + 3 and 32w + 16 + 4g .. + 3 of row d = 16 dt + r: slots 8w + g and 8w + 4 + g
+          const unsigned char* vrow = vb + (16 * dt + gc.r) * S::VSTR;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow + 8 * fold_v_slot(8 * w + gc.g, gc.r));
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(vrow + 8 * fold_v_slot(8 * w + 4 + gc.g, gc.r));
           const u32x4 vfrag = {lo[0], lo[1], hi[0], hi[1]};
 #pragma unroll
           for (int t = 0; t < QT; ++t)
