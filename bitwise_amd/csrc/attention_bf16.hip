@@ -413,19 +413,24 @@ struct FoldShape {
   static constexpr int WAVES = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);   // waves per SIMD the register budget is set for
   // LDS layout, measured on the part: 16-byte operand reads of 16 rows by 4 chunks run at full rate when the rows lie
   // an odd multiple of 32 bytes apart (at twice the time 16 bytes off that, four times at a multiple of 128); 8-byte
-  // reads want rows an odd multiple of 8 bytes apart, or 128-byte rows whose 8-byte slots are permuted (fold_v_slot)
+  // reads want rows an odd multiple of 8 bytes apart; 128-byte rows read at full rate when their 16-byte chunks are
+  // permuted by the row (fold_v_chunk)
   static constexpr int KSTR = HD * 2 + (HD % 32 == 0 ? 32 : 0);   // bytes from key to key
-  static constexpr int VSTR = ATT_PART * 2;                       // bytes from d to d: no padding, slots permuted
+  static constexpr int VSTR = ATT_PART * 2;                       // bytes from d to d: no padding, chunks permuted
   static constexpr int KBYTES = ATT_PART * KSTR;
   static constexpr int BYTES = KBYTES + HD * VSTR;  // one partition
   static constexpr int KJ = (ATT_PART * (HD / 8) + 64 * NW - 1) / (64 * NW);   // 16-byte key chunks per thread
   static constexpr int VJ = (HD * (ATT_PART / 4) + 64 * NW - 1) / (64 * NW);   // 8-byte value chunks per thread
 };
 
-// Where the 8-byte slot ``slot`` (keys 4 * slot .. 4 * slot + 3) of the values' row d lies in the row: the two low
-// bit pairs of d, swapped, are xor-ed onto the slot number.  The 16 rows of an operand read then hit 16 different
-// slots, and so do the 4 consecutive rows by 4 consecutive slots that 16 lanes store from pages of 16.
-__device__ __forceinline__ int fold_v_slot(int slot, int d) { return (slot ^ (((d & 3) << 2) | ((d >> 2) & 3))) & 15; }
+// Where the 8-byte slot ``slot`` (keys 4 * slot .. 4 * slot + 3) of the values' row d lies in the row's 128 bytes.
+// The second product's operand of lane (g, r) for keys 32w .. 32w + 31 is keys 32w + 4g .. + 3 and 32w + 16 + 4g .. + 3
+// of row d = 16 dt + r: those two slots lie side by side as 16-byte chunk 4w + g, so that one read brings the operand,
+// and the chunk's place in the row is permuted by the row as the keys' chunks are in the product kernels.
+__device__ __forceinline__ int fold_v_chunk(int chunk, int d) { return 16 * (chunk ^ ((d >> 1) & 7)); }
+__device__ __forceinline__ int fold_v_offset(int slot, int d) {
+  return fold_v_chunk(((slot >> 3) << 2) | (slot & 3), d) + 8 * ((slot >> 2) & 1);
+}
 
 template <int HD>
 struct Staged {
@@ -534,7 +539,7 @@ __device__ __forceinline__ void stage_store(const WorkgroupCtx& wc, const StageP
       v2 = (u32x2){v2[0] & m0, v2[1] & m1};
     }
     if (sp.v_key[j] < ATT_PART)
-      *reinterpret_cast<u32x2*>(buf + S::KBYTES + sp.v_d[j] * S::VSTR + 8 * fold_v_slot(sp.v_key[j] >> 2, sp.v_d[j])) = v2;
+      *reinterpret_cast<u32x2*>(buf + S::KBYTES + sp.v_d[j] * S::VSTR + fold_v_offset(sp.v_key[j] >> 2, sp.v_d[j])) = v2;
   }
 }
 
@@ -641,11 +646,7 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
         for (int t = 0; t < QT; ++t) o_p[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-          // keys 32w + 4g .. + 3 and 32w + 16 + 4g .. + 3 of row d = 16 dt + r: slots 8w + g and 8w + 4 + g
-          const unsigned char* vrow = vb + (16 * dt + gc.r) * S::VSTR;
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow + 8 * fold_v_slot(8 * w + gc.g, gc.r));
-          const u32x2 hi = *reinterpret_cast<const u32x2*>(vrow + 8 * fold_v_slot(8 * w + 4 + gc.g, gc.r));
-          const u32x4 vfrag = {lo[0], lo[1], hi[0], hi[1]};
+          const u32x4 vfrag = *reinterpret_cast<const u32x4*>(vb + (16 * dt + gc.r) * S::VSTR + fold_v_chunk(4 * w + gc.g, gc.r));
 #pragma unroll
           for (int t = 0; t < QT; ++t)
             o_p[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vfrag), as_bf16x8(pf[t][w]), o_p[t][dt], 0, 0, 0);
