@@ -501,18 +501,29 @@ __device__ __forceinline__ void stage_pages(const AttnBf16Args& a, const Workgro
   }
 }
 
-// Unconditional loads from addresses that are always inside the cache; see the operand loaders above.
+// Unconditional loads from addresses that are always inside the cache; see the operand loaders above.  Keys and
+// values separately: all waves of a workgroup ask for their chunks at the same point of the loop, and a compute
+// unit's one path to memory takes a few hundred clocks to accept a whole partition's requests, so the loop asks for
+// the next partition piece by piece, between the phases of its arithmetic.
 template <int HD>
-__device__ __forceinline__ void stage_load(const AttnBf16Args& a, const StagePlan<HD>& sp, const StagePages<HD>& pg,
-                                           Staged<HD>& sg) {
+__device__ __forceinline__ void stage_load_keys(const AttnBf16Args& a, const StagePlan<HD>& sp, const StagePages<HD>& pg,
+                                                Staged<HD>& sg) {
   using S = FoldShape<HD>;
   // (a page's bytes fit 32 bits, so page * bytes is one 32 x 32 -> 64-bit multiply-add onto the chunk's base)
-  const unsigned page_bytes = (unsigned)(a.kv_heads * a.page_size * HD) * 2u;   // values: the same number of elements
+  const unsigned page_bytes = (unsigned)(a.kv_heads * a.page_size * HD) * 2u;
   const unsigned last_page = (unsigned)(a.num_pages - 1);
 #pragma unroll
   for (int j = 0; j < S::KJ; ++j)
     sg.k[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(a.k_cache + sp.k_off[j]) +
                                               (unsigned long long)min((unsigned)pg.k[j], last_page) * page_bytes);
+}
+
+template <int HD>
+__device__ __forceinline__ void stage_load_values(const AttnBf16Args& a, const StagePlan<HD>& sp, const StagePages<HD>& pg,
+                                                  Staged<HD>& sg) {
+  using S = FoldShape<HD>;
+  const unsigned page_bytes = (unsigned)(a.kv_heads * a.page_size * HD) * 2u;   // values: the same number of elements
+  const unsigned last_page = (unsigned)(a.num_pages - 1);
 #pragma unroll
   for (int j = 0; j < S::VJ; ++j)
     sg.v[j] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const unsigned char*>(a.v_cache + sp.v_off[j]) +
@@ -602,7 +613,8 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
   StagePages<HD> pg;
   stage_pages<HD>(a, wc, sp, first, pg);
   Staged<HD> sg;
-  stage_load<HD>(a, sp, pg, sg);
+  stage_load_keys<HD>(a, sp, pg, sg);
+  stage_load_values<HD>(a, sp, pg, sg);
   stage_pages<HD>(a, wc, sp, first + 1, pg);
   int b = 0;
   for (int part = first; part <= last; ++part) {
@@ -610,13 +622,15 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
     if constexpr (S::NBUF == 1) __syncthreads();   // everyone is done with the partition before
     stage_store<HD>(wc, sp, part, sg, buf);
     __syncthreads();
-    if (part < last) {
-      stage_load<HD>(a, sp, pg, sg);
-      stage_pages<HD>(a, wc, sp, part + 2, pg);
-    }
-    if (part >= my_first && part <= my_last) {
+    // The next partition is asked for in three pieces, each in front of a phase of this one's arithmetic (the
+    // addresses are inside the cache for any partition number, so nothing here is conditional).
+    const bool mine = part >= my_first && part <= my_last;    // the same for the whole wave
+    f32x4 st[QT][4];
+    float m_p[QT], l_p[QT];
+    u32x4 pf[QT][2];
+    stage_load_keys<HD>(a, sp, pg, sg);
+    if (mine) {
       // scores of all the wave's tiles; a key operand is read once and used for each of them
-      f32x4 st[QT][4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
 #pragma unroll
@@ -631,13 +645,17 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
             st[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kfrag), as_bf16x8(tc[t].qf[ks]), st[t][u], 0, 0, 0);
         }
       }
-      float m_p[QT], l_p[QT];
-      u32x4 pf[QT][2];
+    }
+    stage_load_values<HD>(a, sp, pg, sg);
+    if (mine) {
 #pragma unroll
       for (int t = 0; t < QT; ++t) {
         softmax_partition<HD>(a, gc, tc[t], part * ATT_PART, st[t], m_p[t], pf[t]);
         l_p[t] = probability_sum(pf[t]);
       }
+    }
+    stage_pages<HD>(a, wc, sp, part + 2, pg);
+    if (mine) {
       f32x4 o_p[QT][NT];
       const unsigned char* vb = buf + S::KBYTES;
 #pragma unroll
