@@ -755,7 +755,7 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
   constexpr int EPT = (16 * HD + THREADS - 1) / THREADS;   // output elements per thread at most (16 live columns)
   constexpr int CELL = HD + 2;                              // m, l, then hd values
   constexpr bool PREFETCH = HD <= 64 && !SPLIT;
-  extern __shared__ float parts[];                          // [pcap][hpt][CELL]
+  extern __shared__ __attribute__((aligned(16))) float parts[];   // [pcap][hpt][CELL]
   __shared__ int is_last;
   GroupCtx gc;
   TileCtx<HD> tc[1];
@@ -785,7 +785,16 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
         float m_p, l_p;
         f32x4 o_p[NT];
         partition_partial<HD>(a, gc, tc[0], part, pg, kf, vf, m_p, l_p, o_p);
-        store_partial<HD, true>(a, gc, mine + (size_t)(part - first) * a.hpt * CELL, m_p, l_p, o_p);
+        // The partial goes to the scratch through the wave's own cell of LDS, so that whole runs of bytes are
+        // written, 8 a lane: device-scope stores write through, and the words of the accumulator layout (a few
+        // lanes, 4 bytes each, 16 bytes apart) would each be a write of part of a line.  (A wave's LDS
+        // instructions are carried out in order: the reads below see the stores above.)
+        float* park = parts + (size_t)wave * a.hpt * CELL;
+        store_partial<HD, false>(a, gc, park, m_p, l_p, o_p);
+        const unsigned long long* from = reinterpret_cast<const unsigned long long*>(park);
+        unsigned long long* to = reinterpret_cast<unsigned long long*>(mine + (size_t)(part - first) * a.hpt * CELL);
+        for (int i = gc.lane; i < a.hpt * CELL / 2; i += 64)
+          __hip_atomic_store(to + i, from[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
     // The barrier waits for every thread's stores (device-scope ones: they are in memory then, no
@@ -800,8 +809,24 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
     for (int pass0 = first; pass0 <= last; pass0 += pcap) {
       const int count = (last - pass0) < pcap ? last - pass0 + 1 : pcap;
       const float* src = mine + (size_t)(pass0 - first) * a.hpt * CELL;
-      for (int i = threadIdx.x; i < count * a.hpt * CELL; i += THREADS)
-        parts[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // eight loads of 8 bytes in flight a thread (a loop of one load and its store waits a memory round trip for
+      // each: 40 us for the 66 KB of a group of four heads of 128 over 32 partitions)
+      const int total = count * a.hpt * CELL / 2;
+      const unsigned long long* src64 = reinterpret_cast<const unsigned long long*>(src);
+      unsigned long long* parts64 = reinterpret_cast<unsigned long long*>(parts);
+      for (int base = 0; base < total; base += 8 * THREADS) {
+        unsigned long long v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = base + j * THREADS + (int)threadIdx.x;
+          v[j] = __hip_atomic_load(src64 + (i < total ? i : 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = base + j * THREADS + (int)threadIdx.x;
+          if (i < total) parts64[i] = v[j];
+        }
+      }
       __syncthreads();
       decode_fold_pass<HD, W>(a, parts, count, m, l, o);
       __syncthreads();
@@ -946,6 +971,7 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   if (kv_heads <= 0 || heads % kv_heads) return -2;
   if (page_size < 4 || (page_size & (page_size - 1)) || page_size > ATT_PART) return -5;  // 4-key loads stay inside a page
   if ((q_stride % 8) || (out_stride % 4)) return -3;
+  if (reinterpret_cast<uintptr_t>(scratch) & 7) return -3;      // partials travel in 8-byte words
   const int group = heads / kv_heads;
   AttnBf16Args a;
   a.q = (const bf16_t*)q; a.positions = positions; a.block_table = block_table; a.tiles = tiles;
