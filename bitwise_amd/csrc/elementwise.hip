@@ -128,12 +128,27 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16_kernel(const float* __restri
     }
     acc = row_sumsq_vec(xv, nvec, lane);
     const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
-    for (int c = lane; c < nvec; c += 64) {
-      const f32x4 v = xv[c];
-      const f32x4 wv = load_norm_w4(w, sizeof(WT) == 2, c);
-      u32x2 pk = {pack_bf16x2((v[0] * inv) * wv[0], (v[1] * inv) * wv[1]),
-                  pack_bf16x2((v[2] * inv) * wv[2], (v[3] * inv) * wv[3])};
-      *reinterpret_cast<u32x2*>(yr + 4 * c) = pk;
+    // eight vectors of the row and of the weight asked for before the first is used (a loop of one load and its
+    // store waits a memory round trip for every vector: 9 us for rows of 4096)
+    constexpr int UN = 8;
+    for (int c0 = 0; c0 < nvec; c0 += 64 * UN) {
+      f32x4 v[UN];
+      u32x4 wr[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j) {
+        const int c = c0 + 64 * j + lane < nvec ? c0 + 64 * j + lane : nvec - 1;
+        v[j] = xv[c];
+        wr[j] = load_norm_w_raw(w, sizeof(WT) == 2, c);
+      }
+#pragma unroll
+      for (int j = 0; j < UN; ++j) {
+        const int c = c0 + 64 * j + lane;
+        if (c >= nvec) continue;
+        const f32x4 wv = norm_w_floats(wr[j], sizeof(WT) == 2);
+        u32x2 pk = {pack_bf16x2((v[j][0] * inv) * wv[0], (v[j][1] * inv) * wv[1]),
+                    pack_bf16x2((v[j][2] * inv) * wv[2], (v[j][3] * inv) * wv[3])};
+        *reinterpret_cast<u32x2*>(yr + 4 * c) = pk;
+      }
     }
     return;
   }
