@@ -51,6 +51,7 @@ class _StaticDecodeContext:
         self.sampled = torch.zeros(size, dtype=torch.int32, device=device)
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
+        self.wants_every_row = True                      # row i is wanted place i: the model need not gather
         self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
         self.segments: List[Segment] = []
         # what the host copy of each block-table row was last filled from: (the request's list, its length then);

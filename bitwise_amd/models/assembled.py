@@ -134,8 +134,11 @@ class AssembledModel:
         count = ctx.num_wanted
         if count == 0:
             return None
-        last = self.rt.buffer("wanted_rows", self.spec.width, torch.float32, rows=self.rt.max_logit_rows)
-        ops.gather_rows(x, ctx.want_rows, last, count)
+        if getattr(ctx, "wants_every_row", False):
+            last = x                                     # rows 0 .. count-1 are the wanted ones already
+        else:
+            last = self.rt.buffer("wanted_rows", self.spec.width, torch.float32, rows=self.rt.max_logit_rows)
+            ops.gather_rows(x, ctx.want_rows, last, count)
         logits = self.lm_head.forward_with_norm(ctx, last, self.final_norm, count)
         if logits is None:
             normed = self.final_norm.forward(ctx, last, out_name="final_normed", rows=count)
