@@ -1,7 +1,8 @@
 // C entry points of the kernel library.  Every function launches on the given stream and
 // returns 0, a HIP error code (> 0), or a negative code for arguments it refuses:
 //   -2 sizes or strides out of range, -3 misaligned pointer or stride,
-//   -4 head size not compiled in, -5 page size not supported.
+//   -4 head size not compiled in, -5 page size not supported, -6 scratch smaller than asked for,
+//   -7 sizes beyond what the library's own static scratch holds.
 // All pointers are device pointers.  Nothing here allocates.
 #pragma once
 #include <stdint.h>
@@ -25,6 +26,17 @@ int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, i
 int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_floats, int* counters);
 int bw_gemm_add_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, float* scratch,
                      long long scratch_floats, int32_t* counters, int num_counters, void* stream);
+// No counterpart in the reference.  For callers that cannot allocate device memory and cannot bring a
+// workspace either (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+// bw_gemm_add_bf16 with its scratch (the segments' sums, the tiles' counters) in a static array of the
+// library's device image, 8 MB + 4 KB on every GPU the library runs on, held until the process ends.
+// Shapes whose scratch would exceed that (bw_gemm_add_bf16_static_max gives the limits, bw_gemm_add_scratch
+// what a shape needs) are refused with -7.  It calls no hipMalloc, no hipFree and no allocating library
+// routine.  All calls on one GPU share that GPU's array: calls that overlap on one GPU race; calls on one
+// stream, one after the other, do not.  The bits are those of bw_gemm_add_bf16.
+int bw_gemm_add_bf16_static(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo,
+                            void* stream);
+int bw_gemm_add_bf16_static_max(long long* scratch_floats, int* counters);
 int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out, const int32_t* positions,
                           const int32_t* row_seq, const int32_t* block_table, int table_stride, const float* cos_table,
                           const float* sin_table, void* k_cache, void* v_cache, int M, int heads, int kv_heads,

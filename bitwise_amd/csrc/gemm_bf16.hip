@@ -40,6 +40,8 @@
 // stacked weight) stored as bfloat16: h = g * (1/(1+exp(-g))) * u in 32-bit, or rotary encoding of the
 // stacked q|k|v product and the write of k and v to their page slots (heads of 64; up to 64 rows: head sizes
 // in multiples of 64).
+#include <mutex>
+
 #include "common.h"
 #include "api.h"
 
@@ -1794,4 +1796,73 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
   const int N = (heads + 2 * kv_heads) * 64;
   return launch_gemm_bf16<EPI_QKV_ROPE>((const bf16_t*)x, (const bf16_t*)w_qkv, q_out, M, N, K, ldx, heads * 64,
                                         (hipStream_t)stream, rp);
+}
+
+// ------------------------------------------------------------------------------ a residual add that allocates nothing
+
+// out += x W^T like bw_gemm_add_bf16, for callers that can neither allocate device memory nor bring a
+// workspace (code under graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+// segments' sums and the tiles' counters live in one array in the library's own device image.  Every GPU
+// that loads the library holds a copy of the array at an address of its own until the process ends; the
+// name of the array is no device address in host code, so the address is asked for once per device and
+// kept.  Calls on one GPU share the array: calls that overlap there (two streams, two threads) race.
+#define BW_STATIC_SCRATCH_FLOATS (2 * 1024 * 1024)          // 8 MB of sums
+#define BW_STATIC_SCRATCH_COUNTERS 1024                      // 4 KB of counters behind them
+#define BW_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[BW_STATIC_SCRATCH_FLOATS + BW_STATIC_SCRATCH_COUNTERS];
+
+__global__ __launch_bounds__(256) void zero_words_kernel(int32_t* __restrict__ p, int n) {
+  const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+  if (i < n) p[i] = 0;
+}
+
+static float* static_scratch_of_device[BW_STATIC_MAX_DEVICES];
+static std::mutex static_scratch_mutex;
+
+// The current device's copy of the array (asked for at the first call on that device).
+static int static_scratch_address(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= BW_STATIC_MAX_DEVICES) return -2;
+  std::lock_guard<std::mutex> hold(static_scratch_mutex);
+  if (static_scratch_of_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return -2;
+    static_scratch_of_device[dev] = (float*)p;
+  }
+  *out = static_scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" int bw_gemm_add_bf16_static_max(long long* scratch_floats, int* counters) {
+  *scratch_floats = BW_STATIC_SCRATCH_FLOATS;
+  *counters = BW_STATIC_SCRATCH_COUNTERS;
+  return 0;
+}
+
+extern "C" int bw_gemm_add_bf16_static(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo,
+                                       void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K % 8) || (ldx % 8) || ldx < K || ldo < N) return -2;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return -3;
+  long long need_floats = 0;
+  int need_counters = 0;
+  bw_gemm_add_scratch(M, N, K, &need_floats, &need_counters);
+  if (need_floats > BW_STATIC_SCRATCH_FLOATS || need_counters > BW_STATIC_SCRATCH_COUNTERS) return -7;
+  if (need_floats == 0)      // this shape's kernel joins its segments in registers: nothing to share
+    return launch_gemm_bf16<EPI_ADD_F32>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldx, ldo, (hipStream_t)stream);
+  float* base = nullptr;
+  const int rc = static_scratch_address(&base);
+  if (rc != 0) return rc;
+  int32_t* count = reinterpret_cast<int32_t*>(base + BW_STATIC_SCRATCH_FLOATS);
+  // The counters must be zero when the kernel starts.  Every launch leaves them so, but the array outlives a
+  // launch that was aborted half way; a small kernel clears them (a memset node in a captured graph is no
+  // safe thing on this hardware's runtime).  The sums need no clearing: every cell is written before it is read.
+  hipLaunchKernelGGL(zero_words_kernel, dim3((need_counters + 255) / 256), dim3(256), 0, (hipStream_t)stream, count,
+                     need_counters);
+  return launch_gemm_bf16<EPI_ADD_F32>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldx, ldo, (hipStream_t)stream,
+                                       QkvRopeArgs{}, MidSplitArgs{base, count}, (size_t)need_floats, need_counters);
 }

@@ -29,6 +29,7 @@ _ERRORS = {
     -4: f"head size not compiled in (supported: {HEAD_DIMS})",
     -5: "page size not supported (a power of two from 4 to 64 is needed)",
     -6: "scratch smaller than attention_decode_scratch asks for",
+    -7: "sizes beyond what the library's static scratch holds",
 }
 
 _SIGS = {
@@ -44,6 +45,8 @@ _SIGS = {
     "bw_gemm_add_scratch": [c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_gemm_add_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p,
                          c_int, c_void_p],
+    "bw_gemm_add_bf16_static": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_add_bf16_static_max": [c_void_p, c_void_p],
     "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32_tiles": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
