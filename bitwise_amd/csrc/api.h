@@ -13,6 +13,8 @@ int bw_embed(const int32_t* tokens, const void* table, int table_is_bf16, float*
 int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16, int rows,
                int dim, int ldy, float eps, void* stream);
 int bw_add(float* x, const float* y, long long n, void* stream);
+int bw_convert(const void* src, int src_is_bf16, void* dst, int dst_is_bf16, int rows, int cols, int lds, int ldd,
+               void* stream);
 int bw_swiglu_f32(const float* gate_up, float* h, int rows, int inter, void* stream);
 int bw_gather_rows_f32(const float* x, const int32_t* idx, float* out, int count, int width, int ldx, void* stream);
 int bw_rope_kvwrite(float* qkv, void* q_out, const int32_t* positions, const int32_t* row_seq,

@@ -797,9 +797,13 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
           __hip_atomic_store(to + i, from[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    // The barrier waits for every thread's stores (device-scope ones: they are in memory then, no
-    // cache has to be written back) before the workgroup counts itself in, and orders the last
-    // workgroup's loads (device scope again) behind its count.
+    // Every wave waits until its own device-scope stores are acknowledged (they write through: once the
+    // wave's count of outstanding memory operations is zero they are in memory, no cache has to be written
+    // back), then the barrier: when thread 0 counts the workgroup in, all of its partials are visible to the
+    // device.  The count's atomic returns a value, so thread 0 has it before the second barrier, and the last
+    // workgroup issues its loads (device scope again: they do not read a stale line of this die's L2) only
+    // after that barrier.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
     __syncthreads();
     if (threadIdx.x == 0) is_last = atomicAdd(&counters[item], 1) == (int)gridDim.z - 1;
     __syncthreads();

@@ -188,7 +188,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
   auto park = [&](int j0, int buf) {                       // ``krow`` holds key j0 + et; afterwards key j0 + KC + et
     if (et < 0) return;
     const int j = j0 + et;
-    const float e = expf(dot_canonical<HD>(q_lds, krow) * a.scale - mx);
+    const float e = bw_expf(dot_canonical<HD>(q_lds, krow) * a.scale - mx);
     load_row<HD>(krow, a.k_cache + offset_of(j + KC));
     e_lds[buf][et] = j <= pos ? e : 0.0f;
   };
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
     for (int u = 0; u < CH / 16; ++u) {
       const int key = c0 + kl + 16 * u;
       float e = 0.0f;
-      if (key >= lo_q && key <= pos_q) e = expf(dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR) * a.scale - mx);
+      if (key >= lo_q && key <= pos_q) e = bw_expf(dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR) * a.scale - mx);
       e_lds[qi * CH + kl + 16 * u] = e;
     }
     __syncthreads();

@@ -40,6 +40,31 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   return c.b;
 }
 
+// exp(x) of the 32-bit path: one fixed sequence of IEEE operations (a rounding to the nearest integer,
+// fused multiply-adds, multiplications by powers of two) and no library call, so that a scalar program
+// on any IEEE machine gives the same bits.  x = k ln2 + r with k = rint(x * log2e), |r| <= 0.35 (ln2 in
+// two parts, the high one with trailing zero bits); e^r by the Taylor polynomial of degree 7 in Horner
+// form (its remainder is below a tenth of an ulp); the result scaled by 2^k in two exact steps.
+// Arguments below -87 give 0 (the result would be under the smallest normal number), arguments above 89
+// give +inf, NaN stays NaN; exp(0) is exactly 1.
+__device__ __forceinline__ float bw_expf(float x) {
+  if (!(x >= -87.0f)) return (x != x) ? x : 0.0f;
+  if (x > 89.0f) return __builtin_inff();
+  const float kf = __builtin_rintf(x * 0x1.715476p+0f);
+  float r = fmaf(kf, -0x1.62e4p-1f, x);
+  r = fmaf(kf, -0x1.7f7d1cp-20f, r);
+  float p = 0x1.a01a02p-13f;
+  p = fmaf(p, r, 0x1.6c16c2p-10f);
+  p = fmaf(p, r, 0x1.111112p-7f);
+  p = fmaf(p, r, 0x1.555556p-5f);
+  p = fmaf(p, r, 0x1.555556p-3f);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.0f);
+  p = fmaf(p, r, 1.0f);
+  const int k = (int)kf, k1 = k >> 1, k2 = k - k1;          // both within [-64, 64]
+  return (p * __uint_as_float((uint32_t)(k1 + 127) << 23)) * __uint_as_float((uint32_t)(k2 + 127) << 23);
+}
+
 // exp(x) through the hardware exp2; one fixed instruction sequence wherever it is used.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 

@@ -204,6 +204,37 @@ extern "C" int bw_add(float* x, const float* y, long long n, void* stream) {
   return BW_LAUNCH_CHECK();
 }
 
+// dst[r, c] = src[r, c] between 32-bit and bfloat16 rows (widening is exact; narrowing rounds to nearest even
+// with the hardware conversion).  For the routes on which a weight's dtype is not the mode's.
+template <typename S, typename D>
+__global__ void convert_kernel(const S* __restrict__ src, D* __restrict__ dst, int rows, int cols, int lds, int ldd) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)rows * cols) return;
+  const int r = (int)(i / cols), c = (int)(i % cols);
+  const S v = src[(size_t)r * lds + c];
+  if constexpr (sizeof(S) == 4 && sizeof(D) == 2) dst[(size_t)r * ldd + c] = f32_to_bf16(v);
+  else if constexpr (sizeof(S) == 2 && sizeof(D) == 4) dst[(size_t)r * ldd + c] = bf16_to_f32(v);
+  else dst[(size_t)r * ldd + c] = v;
+}
+
+extern "C" int bw_convert(const void* src, int src_is_bf16, void* dst, int dst_is_bf16, int rows, int cols, int lds,
+                          int ldd, void* stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (lds < cols || ldd < cols) return -2;
+  const size_t n = (size_t)rows * cols;
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  if (src_is_bf16 && dst_is_bf16)
+    hipLaunchKernelGGL((convert_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)src, (bf16_t*)dst, rows, cols, lds, ldd);
+  else if (src_is_bf16)
+    hipLaunchKernelGGL((convert_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)src, (float*)dst, rows, cols, lds, ldd);
+  else if (dst_is_bf16)
+    hipLaunchKernelGGL((convert_kernel<float, bf16_t>), grid, block, 0, s, (const float*)src, (bf16_t*)dst, rows, cols, lds, ldd);
+  else
+    hipLaunchKernelGGL((convert_kernel<float, float>), grid, block, 0, s, (const float*)src, (float*)dst, rows, cols, lds, ldd);
+  return BW_LAUNCH_CHECK();
+}
+
 // h = g * (1/(1+exp(-g))) * u over rows laid out [gate | up] (src/kernels.cpp:291-298).
 __global__ void swiglu_f32_kernel(const float* __restrict__ gate_up, float* __restrict__ h, int rows, int inter) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -211,7 +242,7 @@ __global__ void swiglu_f32_kernel(const float* __restrict__ gate_up, float* __re
   const int r = (int)(i / inter), c = (int)(i % inter);
   const float g = gate_up[(size_t)r * 2 * inter + c];
   const float u = gate_up[(size_t)r * 2 * inter + inter + c];
-  h[i] = g * (1.0f / (1.0f + expf(-g))) * u;
+  h[i] = g * (1.0f / (1.0f + bw_expf(-g))) * u;
 }
 
 extern "C" int bw_swiglu_f32(const float* gate_up, float* h, int rows, int inter, void* stream) {

@@ -1295,10 +1295,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     if constexpr (EPI == EPI_ADD_F32 && !NORM) {
       const int nseg = gridDim.y;
       if (nseg > 1) {
-        // Every segment's workgroup leaves its sums in device scratch (stores of device scope: in memory, not in
-        // this die's L2, once the barrier's wait for the wave's stores is over) and counts itself in; the one that
-        // finds all others counted in adds all segments' sums to the residual in segment order, every one of them
-        // read back from the scratch (its own too).  The counter is back at zero when the kernel ends.
+        // Every segment's workgroup leaves its sums in device scratch (stores of device scope: they write through,
+        // and each wave waits below until its own are acknowledged, so they are in memory, not in this die's L2,
+        // before the barrier) and counts itself in; the one that finds all others counted in adds all segments'
+        // sums to the residual in segment order, every one of them read back from the scratch (its own too) with
+        // device-scope loads issued after the barrier behind the count.  The counter is back at zero when the
+        // kernel ends.
         const int cell = 4 * NI * 1024;                              // bytes of a workgroup's sums: [wave][i][lane] x 16
         const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(
             (void*)((unsigned char*)sp.scratch + (size_t)blockIdx.x * nseg * cell), 0, nseg * cell, 0x00020000);
@@ -1306,6 +1308,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
 #pragma unroll
         for (int i = 0; i < NI; ++i)
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][0]), rs_s, mine + i * 1024, (int)blockIdx.y * cell, 16);
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                   // this wave's stores have been acknowledged
         __syncthreads();                                             // also: every wave is done with the ring, whose first word is the flag now
         int* is_last = reinterpret_cast<int*>(mid_lds);
         if (threadIdx.x == 0) *is_last = atomicAdd(&sp.counters[blockIdx.x], 1) == nseg - 1;

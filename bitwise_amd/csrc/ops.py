@@ -36,6 +36,7 @@ _SIGS = {
     "bw_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_add": [c_void_p, c_void_p, c_longlong, c_void_p],
+    "bw_convert": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_swiglu_f32": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "bw_gather_rows_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_rope_kvwrite": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -153,6 +154,18 @@ def add_(x: torch.Tensor, y: torch.Tensor, rows: int) -> None:
     if x.shape[1:] != y.shape[1:] or x.shape[0] < rows or y.shape[0] < rows:
         raise ValueError("add_: shapes differ")
     _check(_fn("bw_add")(x.data_ptr(), y.data_ptr(), rows * x.stride(0), _stream()), "add")
+
+
+def convert(src: torch.Tensor, dst: torch.Tensor, rows: int) -> None:
+    """dst[:rows] = src[:rows] between float32 and bfloat16 (narrowing rounds to nearest even)."""
+    if not (src.is_cuda and dst.is_cuda) or src.dim() != 2 or dst.dim() != 2:
+        raise ValueError("convert: two GPU matrices are needed")
+    if src.shape[1] != dst.shape[1] or src.shape[0] < rows or dst.shape[0] < rows:
+        raise ValueError(f"convert: {tuple(src.shape)} does not fit {tuple(dst.shape)} for {rows} rows")
+    if src.stride(1) != 1 or dst.stride(1) != 1:
+        raise ValueError("convert: rows must be contiguous")
+    _check(_fn("bw_convert")(src.data_ptr(), _is_bf16(src, "src"), dst.data_ptr(), _is_bf16(dst, "dst"), rows, src.shape[1],
+                             src.stride(0), dst.stride(0), _stream()), "convert")
 
 
 def swiglu_f32(gate_up: torch.Tensor, out: torch.Tensor, rows: int) -> None:

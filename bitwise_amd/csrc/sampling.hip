@@ -1,7 +1,7 @@
 // Token choice and logits fingerprints on the device, one workgroup per logits row.
 //
 // Greedy: the first maximum wins (the reference scans with a strict '>', src/engine.cpp:40-45).
-// Temperature: w[i] = expf((l[i] - max) / T) in 32-bit, sums in double, the token is the first
+// Temperature: w[i] = bw_expf((l[i] - max) / T) in 32-bit, sums in double, the token is the first
 // i whose running sum exceeds u * total, else the last i with positive weight
 // (src/engine.cpp:50-73).  The reference adds the weights one after the other; here each of
 // the 256 threads adds its own contiguous stretch of the vocabulary in order and the
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
   double part = 0.0;
   int lastpos = -1;
   for (int i = begin; i < end; ++i) {
-    const float w = expf((l[i] - mx) / T);
+    const float w = bw_expf((l[i] - mx) / T);
     if (w > 0.0f) {
       part += (double)w;
       lastpos = i;
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(const float* __rest
   double cum = s_sum[tid];
   if (cum <= target) {
     for (int i = begin; i < end; ++i) {
-      const float w = expf((l[i] - mx) / T);
+      const float w = bw_expf((l[i] - mx) / T);
       if (w <= 0.0f) continue;
       cum += (double)w;
       if (cum > target) {

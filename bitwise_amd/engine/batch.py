@@ -1,17 +1,16 @@
 """One step's batch as the parts see it: flat rows of several requests (portions of prompts
 beside single decoded tokens), with positions, the request each row belongs to, block tables
 per cache group, state slots and the rows whose logits are wanted (the reference's BatchRow
-list, src/model.h:78-85, turned into device arrays)."""
+list, src/model.h:78-85, turned into device arrays), together with what belongs to the engine
+that runs the step: its workspace and its layer calls bound to its caches."""
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
-
-from ..parts.attention import DECODE_MIN_CONTEXT
 
 
 @dataclass
@@ -24,20 +23,23 @@ class Segment:
     want: Sequence[int] = ()           # offsets into ``tokens`` whose logits are wanted
 
 
-@dataclass
-class AttentionPlan:
-    fold_tiles: Optional[torch.Tensor]
-    fold_count: int
-    decode_tiles: Optional[torch.Tensor]      # None with a positive count: tile t is row t of request t
-    decode_count: int
-
-
 class StepContext:
-    """Device arrays of one step.  Rows of a request are contiguous and in position order."""
+    """Device arrays of one step.  Rows of a request are contiguous and in position order.
 
-    def __init__(self, segments: Sequence[Segment], num_groups: int, device: torch.device):
+    ``ws``: the workspace of the engine that runs the step (scratch buffers, page size, limits).
+    ``calls``: the model's layer calls bound to that engine's caches and state.  ``num_pages``:
+    the size of the engine's page pools; a block table that names a page outside is refused
+    here, on the host, since the cache writes do not clamp.  A part may keep what it derives
+    from the step's shape (tile lists and the like) with ``memo`` for its other layers.
+    """
+
+    def __init__(self, segments: Sequence[Segment], num_groups: int, ws, calls: Sequence[Any] = (),
+                 num_pages: Optional[int] = None):
         self.segments = list(segments)
-        self.device = device
+        self.ws = ws
+        self.calls = list(calls)
+        self.device = device = ws.device
+        self.page_size = ws.page_size
         nseq = len(self.segments)
         rows = sum(len(s.tokens) for s in self.segments)
         self.rows, self.nseq = rows, nseq
@@ -62,6 +64,8 @@ class StepContext:
             t = np.zeros((nseq, widths[g]), np.int32)
             for i, s in enumerate(self.segments):
                 row = np.asarray(s.tables[g], np.int32)
+                if num_pages is not None and row.size and int(row.max()) >= num_pages:
+                    raise ValueError(f"a block table names page {int(row.max())}, the pool has {num_pages}")
                 t[i, :len(row)] = np.maximum(row, 0)      # pages given back (-1) are never read
             tables.append(t)
         slots = np.asarray([s.slot for s in self.segments], np.int32)
@@ -72,29 +76,10 @@ class StepContext:
         self.tokens, self.positions, self.row_seq, self.want_rows, self.slots = view[:5]
         self.block_tables = [view[5 + g].view(nseq, widths[g]) for g in range(num_groups)]
         self.host_positions = positions
-        self._plans: Dict[tuple, AttentionPlan] = {}
+        self._memo: Dict[Any, Any] = {}
 
-    def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
-        """Tiles of up to ``tokens_per_tile`` consecutive rows of one request; every request's
-        run of tiles is padded with empty tiles to a multiple of ``group_tiles`` (the tiles one
-        wave owns must belong to one request).  Single decoded tokens with a long context go
-        to the decode kernel (a wave per 64-key partition)."""
-        plan = self._plans.get((tokens_per_tile, group_tiles))
-        if plan is not None:
-            return plan
-        fold, split = [], []
-        for i, s in enumerate(self.segments):
-            n, r0 = len(s.tokens), self.seq_start[i]
-            if n == 1 and s.pos0 + 1 >= DECODE_MIN_CONTEXT:
-                split.append((r0, 1, i, 0))
-                continue
-            for off in range(0, n, tokens_per_tile):
-                fold.append((r0 + off, min(tokens_per_tile, n - off), i, 0))
-            while len(fold) % group_tiles:
-                fold.append((r0, 0, i, 0))
-        both = np.asarray(fold + split, np.int32).reshape(-1, 4)
-        dev = torch.from_numpy(both).to(self.device)
-        plan = AttentionPlan(dev[:len(fold)].contiguous() if fold else None, len(fold),
-                             dev[len(fold):].contiguous() if split else None, len(split))
-        self._plans[(tokens_per_tile, group_tiles)] = plan
-        return plan
+    def memo(self, key: Any, make: Callable[[], Any]) -> Any:
+        """``make()`` once per step and key."""
+        if key not in self._memo:
+            self._memo[key] = make()
+        return self._memo[key]

@@ -68,13 +68,15 @@ class GpuExecutor:
         rt = asm.rt
         if rt.mode != config.dtype:
             raise ValueError(f"the model was loaded as {rt.mode}, the engine is configured for {config.dtype}")
-        rt.configure(max_rows=config.max_batched_tokens, page_size=config.block_size,
-                     max_logit_rows=min(config.max_num_seqs, config.max_batched_tokens))
-        self.storage = CacheStorage(asm, config.num_blocks, config.max_num_seqs)
+        # caches, state, scratch buffers and captured graphs are this executor's own: the model holds
+        # weights only, so other engines may run it at the same time
+        self.storage = CacheStorage(asm, config.num_blocks, config.max_num_seqs, config.block_size)
         max_len = config.max_model_len or asm.spec.max_positions
         self.max_model_len = min(max_len, asm.spec.max_positions)
-        self.runner = ModelRunner(asm, self.storage, self.max_model_len, use_graphs=config.use_graphs)
-        self.sampler = Sampler(rt.device, rt.max_logit_rows)
+        max_logit_rows = min(config.max_num_seqs, config.max_batched_tokens)
+        self.runner = ModelRunner(asm, self.storage, self.max_model_len, max_rows=config.max_batched_tokens,
+                                  max_logit_rows=max_logit_rows, use_graphs=config.use_graphs)
+        self.sampler = Sampler(rt.device, max_logit_rows)
         self.group_specs = [GroupSpec(g.window) for g in asm.group_specs]
         self.has_state = bool(asm.state_specs)
         self.vocab_size = asm.spec.vocab_size

@@ -17,7 +17,8 @@ import torch
 
 from ..csrc import ops
 from ..models.assembled import AssembledModel
-from .batch import AttentionPlan, Segment, StepContext
+from ..runtime import Workspace
+from .batch import Segment, StepContext
 from .storage import CacheStorage
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -27,18 +28,28 @@ class _StaticDecodeContext:
     """Fixed device arrays for a decode batch of up to ``size`` requests, one row each: the
     step's index arrays and, for sampling inside the graph, each row's temperature and
     uniform.  All of them are views of one device buffer that a step refreshes with a single
-    copy from pinned host memory."""
+    copy from pinned host memory.  Rows beyond the step's requests are padding: token -1,
+    position -1, slot -1; every kernel skips a row with a negative position, and a mixer
+    with per-request state must skip a row with a negative position or slot."""
 
-    def __init__(self, size: int, num_groups: int, max_pages: int, device: torch.device):
+    one_row_per_request = True                           # row t is the one token of request t
+    wants_every_row = True                               # row i is wanted place i: the model need not gather
+
+    def __init__(self, size: int, num_groups: int, max_pages: int, ws: Workspace, calls, num_pages: int):
         self.rows = self.nseq = self.num_wanted = size
-        self.device = device
+        self.ws, self.calls = ws, list(calls)
+        self.device = device = ws.device
+        self.page_size = ws.page_size
         self.max_pages = max_pages
+        self.num_pages = num_pages
         off_temp = 3 * size + num_groups * size * max_pages
         off_uni = off_temp + size + ((off_temp + size) & 1)        # 64-bit values start at an even word
         words = off_uni + 2 * size
         self._host = torch.zeros(words, dtype=torch.int32, pin_memory=True)
         self._host_np = self._host.numpy()
         self._dev = torch.zeros(words, dtype=torch.int32, device=device)
+        self._copied = torch.cuda.Event()                # the last copy out of the pinned buffer
+        self._copy_pending = False
         self.tokens = self._dev[0:size]
         self.positions = self._dev[size:2 * size]
         self.slots = self._dev[2 * size:3 * size]
@@ -51,18 +62,23 @@ class _StaticDecodeContext:
         self.sampled = torch.zeros(size, dtype=torch.int32, device=device)
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
-        self.wants_every_row = True                      # row i is wanted place i: the model need not gather
-        self._plan = AttentionPlan(None, 0, None, size)      # implicit tiles: tile t = row t of request t
         self.segments: List[Segment] = []
+        self.seq_start = list(range(size))
+        self._memo: Dict = {}
         # what the host copy of each block-table row was last filled from: (the request's list, its length then);
         # a request's list only grows at its end from step to step, so mostly there is nothing or one entry to write
         self._row_source = [[(None, 0)] * size for _ in range(num_groups)]
 
-    def attention_plan(self, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
-        return self._plan
+    def memo(self, key, make):
+        if key not in self._memo:
+            self._memo[key] = make()
+        return self._memo[key]
 
     def fill(self, segments: Sequence[Segment], sampling=None) -> None:
         """``sampling``: (temperatures, uniforms) of the rows, or None (greedy everywhere)."""
+        if self._copy_pending:
+            self._copied.synchronize()      # the pinned buffer is rewritten below: the last copy must have read it
+            self._copy_pending = False
         size, n = self.rows, len(segments)
         self._host_temps[:] = 0.0
         self._host_unis[:] = 0.0
@@ -71,9 +87,7 @@ class _StaticDecodeContext:
             self._host_unis[:n] = sampling[1]
         self.segments = list(segments)
         h = self._host_np
-        h[0:size] = -1                      # padding rows: token -1, position -1
-        h[size:2 * size] = -1
-        h[2 * size:3 * size] = 0
+        h[0:3 * size] = -1                  # padding rows: token -1, position -1, slot -1
         for i, s in enumerate(segments):
             h[i], h[size + i], h[2 * size + i] = s.tokens[0], s.pos0, s.slot
         base = 3 * size
@@ -88,20 +102,30 @@ class _StaticDecodeContext:
                 else:
                     lo = 0
                 if lo < len(row):
+                    fresh = row[lo:]
+                    if max(fresh) >= self.num_pages:
+                        raise ValueError(f"a block table names page {max(fresh)}, the pool has {self.num_pages}")
                     # pages given back (-1; outside the window, never read) become 0: any valid page number
-                    t[i, lo:len(row)] = [p if p > 0 else 0 for p in row[lo:]]
+                    t[i, lo:len(row)] = [p if p > 0 else 0 for p in fresh]
                     source[i] = (row, len(row))
         self._dev.copy_(self._host, non_blocking=True)
+        self._copied.record()
+        self._copy_pending = True
 
 
 class ModelRunner:
-    def __init__(self, model: AssembledModel, storage: CacheStorage, max_model_len: int, use_graphs: bool = True):
+    """The step function of one engine over one model: it owns the workspace (scratch buffers
+    sized for ``max_rows`` tokens a step and ``max_logit_rows`` wanted places) and runs on the
+    storage's caches.  It keeps nothing in the model, so several runners may share one."""
+
+    def __init__(self, model: AssembledModel, storage: CacheStorage, max_model_len: int, max_rows: int = 256,
+                 max_logit_rows: Optional[int] = None, use_graphs: bool = True):
         self.model, self.storage = model, storage
         self.rt = model.rt
-        self.max_model_len = int(max_model_len)
+        self.ws = Workspace(model.rt.device, max_rows, storage.page_size, max_logit_rows)
+        self.max_model_len = min(int(max_model_len), model.spec.max_positions)
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs: Dict[int, tuple] = {}
-        self._graph_generation = -1
         self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
 
     # ------------------------------------------------------------------ the step function
@@ -117,37 +141,36 @@ class ModelRunner:
             return None
         rows = sum(len(s.tokens) for s in segments)
         wanted = sum(len(s.want) for s in segments)
-        if rows > self.rt.max_rows:
-            raise ValueError(f"a step of {rows} tokens exceeds the engine's {self.rt.max_rows}")
-        if wanted > self.rt.max_logit_rows:
-            raise ValueError(f"logits wanted at {wanted} places, the engine allows {self.rt.max_logit_rows}")
+        if rows > self.ws.max_rows:
+            raise ValueError(f"a step of {rows} tokens exceeds the engine's {self.ws.max_rows}")
+        if wanted > self.ws.max_logit_rows:
+            raise ValueError(f"logits wanted at {wanted} places, the engine allows {self.ws.max_logit_rows}")
         for s in segments:
             if not len(s.tokens):
                 raise ValueError("a request without tokens in a step")
             if s.pos0 + len(s.tokens) > self.max_model_len:
                 raise ValueError(f"position {s.pos0 + len(s.tokens) - 1} is beyond the model length {self.max_model_len}")
-            need = (s.pos0 + len(s.tokens) + self.rt.page_size - 1) // self.rt.page_size
+            need = (s.pos0 + len(s.tokens) + self.ws.page_size - 1) // self.ws.page_size
             for t in s.tables:
                 if len(t) < need:
                     raise ValueError("a request's block table does not cover its positions")
         decode_only = all(len(s.tokens) == 1 and tuple(s.want) == (0,) for s in segments)
         if self.use_graphs and decode_only and len(segments) <= GRAPH_BUCKETS[-1]:
             return self._step_graph(segments, sampling)
-        ctx = StepContext(segments, len(self.model.group_specs), self.rt.device)
-        return self.model.forward(ctx)
+        return self.model.forward(self._context(segments))
+
+    def _context(self, segments: Sequence[Segment]) -> StepContext:
+        return StepContext(segments, len(self.model.group_specs), self.ws, self.storage.bindings, self.storage.num_pages)
 
     # ------------------------------------------------------------------ graph replay
     def _step_graph(self, segments: Sequence[Segment], sampling=None) -> torch.Tensor:
         n = len(segments)
         bucket = next(b for b in GRAPH_BUCKETS if b >= n)
-        if bucket > self.rt.max_rows or bucket > self.rt.max_logit_rows:
-            ctx = StepContext(segments, len(self.model.group_specs), self.rt.device)
-            return self.model.forward(ctx)
-        if self._graph_generation != self.rt.scratch_generation:
-            self._graphs.clear()                      # a scratch tensor moved: old captures are stale
+        if bucket > self.ws.max_rows or bucket > self.ws.max_logit_rows:
+            return self.model.forward(self._context(segments))
         entry = self._graphs.get(bucket)
         if entry is None:
-            entry = self._capture(bucket, segments)
+            entry = self._capture(bucket)
         ctx, graph, logits = entry
         ctx.fill(segments, sampling)
         graph.replay()
@@ -155,20 +178,21 @@ class ModelRunner:
             self.last_sampled = ctx.sampled[:n]
         return logits[:n]
 
-    def _capture(self, bucket: int, segments: Sequence[Segment]):
-        rt = self.rt
-        max_pages = (self.max_model_len + rt.page_size - 1) // rt.page_size
-        ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, rt.device)
-        ctx.fill(segments)
-        # One eager run first: it creates every scratch buffer the capture will use and it is
-        # the step's real work (writing the same cache slots twice with the same values is harmless).
+    def _capture(self, bucket: int):
+        ws = self.ws
+        max_pages = (self.max_model_len + ws.page_size - 1) // ws.page_size
+        ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, ws, self.storage.bindings,
+                                   self.storage.num_pages)
+        # One eager run first, on rows that are all padding: it creates every scratch buffer the capture
+        # will use and touches neither cache nor state (a real step run here and then replayed from the
+        # fresh graph would advance a stateful mixer twice).
+        ctx.fill([])
         self.model.forward(ctx)
-        torch.cuda.synchronize(rt.device)
+        torch.cuda.synchronize(ws.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
             ops.sample(logits, bucket, ctx.temps, ctx.unis, ctx.sampled)
-        self._graph_generation = rt.scratch_generation
         entry = (ctx, graph, logits)
         self._graphs[bucket] = entry
         return entry

@@ -98,21 +98,26 @@ class Model:
         return self.assembled.weight_bytes()
 
     # ------------------------------------------------------------------ numerics entry
-    def logits(self, tokens: Sequence[int], chunk: Optional[int] = None) -> np.ndarray:
+    def logits(self, tokens: Sequence[int], chunk: Optional[int] = None, block_size: int = 16) -> np.ndarray:
         """Logits [n, vocab] at every position of one sequence, run as a prompt through a
-        fresh cache (python/bindings.cpp:35-52); ``chunk`` cuts the prompt into steps."""
+        fresh cache of its own (python/bindings.cpp:35-52); ``chunk`` cuts the prompt into
+        steps.  It shares nothing with engines that run the same model."""
         from .engine.runner import ModelRunner
         from .engine.batch import Segment
         from .engine.storage import CacheStorage
 
-        rt = self.assembled.rt
+        asm = self.assembled
         n = len(tokens)
-        step = min(chunk or rt.max_rows, rt.max_rows, rt.max_logit_rows)
-        pages = (n + rt.page_size - 1) // rt.page_size
-        storage = CacheStorage(self.assembled, pages, 1)
-        runner = ModelRunner(self.assembled, storage, max_model_len=max(n, 1), use_graphs=False)
-        tables = [list(range(pages)) for _ in self.assembled.group_specs]
-        out = np.empty((n, self.assembled.spec.vocab_size), np.float32)
+        if n > asm.spec.max_positions:
+            raise ValueError(f"{n} tokens exceed the model's {asm.spec.max_positions} positions")
+        if n == 0:
+            return np.empty((0, asm.spec.vocab_size), np.float32)
+        step = max(1, min(chunk or 256, 256, n))
+        pages = (n + block_size - 1) // block_size
+        storage = CacheStorage(asm, pages, 1, block_size)
+        runner = ModelRunner(asm, storage, max_model_len=n, max_rows=step, use_graphs=False)
+        tables = [list(range(pages)) for _ in asm.group_specs]
+        out = np.empty((n, asm.spec.vocab_size), np.float32)
         for start in range(0, n, step):
             part = list(tokens[start:start + step])
             lg = runner.step([Segment(part, start, tables, 0, list(range(len(part))))])

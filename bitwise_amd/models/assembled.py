@@ -11,14 +11,15 @@ import torch
 from ..csrc import ops
 from ..parts import base
 from ..parts.base import CacheSpec, LayerCall, ModelSpec, StateSpec, TensorSpec, lookup
-from ..parts.embedding import Embedding, LMHead
 from ..runtime import Runtime
 
 
 @dataclass
 class CallBinding:
-    """One schedule entry made concrete: which layer runs, which cache tensors and state
-    tensor it works on, and which cache group's block table covers them."""
+    """One schedule entry made concrete: which layer runs, which cache group's block table covers
+    its cache, and the cache tensors and state tensor it works on.  The model's own list
+    (``AssembledModel.calls``) is the plan and carries no tensors; every cache storage makes
+    bound copies of it (``CacheStorage.bindings``), so that engines on one model share nothing."""
     index: int
     layer: int
     cache: int
@@ -33,19 +34,24 @@ class CallBinding:
 class AssembledModel:
     def __init__(self, spec: ModelSpec, runtime: Runtime):
         self.spec, self.rt = spec, runtime
-        self.embedding = Embedding(spec.embedding.params, runtime)
+        self.embedding = lookup(base.EMBEDDINGS, "embedding", spec.embedding.kind)(spec.embedding.params, runtime)
         self.layers: List[base.Block] = []
         for ls in spec.layers:
-            mixer = lookup(base.MIXERS, "mixer", ls.mixer.kind)(ls.mixer.params, runtime)
-            ff = lookup(base.FEED_FORWARDS, "feed-forward", ls.feed_forward.kind)(ls.feed_forward.params, runtime)
-            n1 = lookup(base.NORMS, "norm", ls.mixer_norm.kind)(ls.mixer_norm.params, runtime)
-            n2 = lookup(base.NORMS, "norm", ls.ffn_norm.kind)(ls.ffn_norm.params, runtime)
-            self.layers.append(lookup(base.BLOCKS, "block", ls.block)(mixer, ff, n1, n2, runtime))
+            block_cls = lookup(base.BLOCKS, "block", ls.block)
+            if "mixer" not in block_cls.roles:
+                raise ValueError(f"block '{ls.block}' has no role 'mixer'")
+            parts = {}
+            for role, ps in ls.parts.items():
+                kind = block_cls.roles.get(role)
+                if kind is None:
+                    raise ValueError(f"block '{ls.block}' has no role '{role}'; its roles: {sorted(block_cls.roles)}")
+                parts[role] = lookup(base.KINDS[kind], kind.replace("_", "-"), ps.kind)(ps.params, runtime)
+            self.layers.append(block_cls(parts, runtime))
         self.final_norm = lookup(base.NORMS, "norm", spec.final_norm.kind)(spec.final_norm.params, runtime)
-        self.lm_head = LMHead(spec.lm_head.params, runtime)
+        self.lm_head = lookup(base.HEADS, "head", spec.lm_head.kind)(spec.lm_head.params, runtime)
         self._plan_caches(spec.schedule)
-        self.graph_safe = all(getattr(b.mixer, "graph_safe", False) and getattr(b.feed_forward, "graph_safe", False)
-                              for b in self.layers)
+        every = [self.embedding, self.final_norm, self.lm_head] + [p for b in self.layers for p in (b, *b.parts.values())]
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
 
     # ------------------------------------------------------------------ caches and state
     def _plan_caches(self, schedule: List[LayerCall]) -> None:
@@ -88,10 +94,8 @@ class AssembledModel:
         s = self.spec
         yield s.embedding.prefix, self.embedding
         for ls, block in zip(s.layers, self.layers):
-            yield ls.mixer_norm.prefix, block.mixer_norm
-            yield ls.ffn_norm.prefix, block.ffn_norm
-            yield ls.mixer.prefix, block.mixer
-            yield ls.feed_forward.prefix, block.feed_forward
+            for role, part in block.parts.items():
+                yield ls.parts[role].prefix, part
         yield s.final_norm.prefix, self.final_norm
         yield s.lm_head.prefix, self.lm_head
 
@@ -110,7 +114,7 @@ class AssembledModel:
         for prefix, part in self._parts_with_prefix():
             mine = {name: tensors[prefix + name] for name in part.tensors()}
             if part is self.lm_head:
-                part.bind(mine, self.embedding)
+                part.bind(mine, embedding=self.embedding)
             else:
                 part.bind(mine)
 
@@ -119,17 +123,20 @@ class AssembledModel:
         norm and the head (a tied head is the embedding table, read whole as the head)."""
         total = self.final_norm.weight_bytes() + self.lm_head.weight_bytes()
         for call in self.calls:
-            b = self.layers[call.layer]
-            total += (b.mixer.weight_bytes() + b.feed_forward.weight_bytes() + b.mixer_norm.weight_bytes()
-                      + b.ffn_norm.weight_bytes())
+            total += sum(p.weight_bytes() for p in self.layers[call.layer].parts.values())
         return total
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the step's rows through every scheduled layer call; logits [wanted, vocab]
-        (32-bit) for the wanted rows in row order, or None if nothing is wanted."""
+        (32-bit) for the wanted rows in row order, or None if nothing is wanted.  Everything
+        that belongs to one engine comes with ``ctx``: its workspace (``ctx.ws``) and the layer
+        calls bound to its caches and state (``ctx.calls``)."""
+        if len(ctx.calls) != len(self.calls):
+            raise ValueError("the step context carries no bindings for this model's layer calls")
+        ws = ctx.ws
         x = self.embedding.forward(ctx)
-        for call in self.calls:
+        for call in ctx.calls:
             self.layers[call.layer].forward(ctx, call, x)
         count = ctx.num_wanted
         if count == 0:
@@ -137,10 +144,7 @@ class AssembledModel:
         if getattr(ctx, "wants_every_row", False):
             last = x                                     # rows 0 .. count-1 are the wanted ones already
         else:
-            last = self.rt.buffer("wanted_rows", self.spec.width, torch.float32, rows=self.rt.max_logit_rows)
+            last = ws.buffer("wanted_rows", self.spec.width, torch.float32, rows=ws.max_logit_rows)
             ops.gather_rows(x, ctx.want_rows, last, count)
-        logits = self.lm_head.forward_with_norm(ctx, last, self.final_norm, count)
-        if logits is None:
-            normed = self.final_norm.forward(ctx, last, out_name="final_normed", rows=count)
-            logits = self.lm_head.forward(ctx, normed, count)
+        logits = self.lm_head.forward(ctx, last, self.final_norm, count)
         return logits[:count]

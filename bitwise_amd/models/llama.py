@@ -15,8 +15,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
     layers = []
     for i in range(cfg.num_hidden_layers):
         pre = f"model.layers.{i}."
-        layers.append(LayerSpec(
-            block="prenorm",
+        layers.append(LayerSpec.prenorm(
             mixer=PartSpec("attention", {"width": cfg.hidden_size, "heads": cfg.num_attention_heads,
                                          "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                                          "window": None, "position": position}, pre + "self_attn."),

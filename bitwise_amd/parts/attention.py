@@ -9,8 +9,10 @@ cache it reads, which block table belongs to it and where its rows sit arrive wi
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 from typing import Dict, Optional
 
+import numpy as np
 import torch
 
 from ..csrc import ops
@@ -22,12 +24,48 @@ from .linear import Linear
 DECODE_MIN_CONTEXT = 128
 
 
+@dataclass
+class AttentionPlan:
+    """Which rows of a step the attention kernels treat together: tiles (first row, rows, request, 0)."""
+    fold_tiles: Optional[torch.Tensor]
+    fold_count: int
+    decode_tiles: Optional[torch.Tensor]      # None with a positive count: tile t is row t of request t
+    decode_count: int
+
+
+def plan_tiles(ctx, tokens_per_tile: int, group_tiles: int = 1) -> AttentionPlan:
+    """Cut a step's segments into tiles of up to ``tokens_per_tile`` consecutive rows of one request; every
+    request's run of tiles is padded with empty tiles to a multiple of ``group_tiles`` (the tiles one wave owns
+    must belong to one request).  Single decoded tokens with a long context go to the decode kernel (a wave per
+    64-key partition).  A step of nothing but one row per request (``ctx.one_row_per_request``, the shape of a
+    captured decode step) needs no tile list: tile t is row t of request t.  The plan is made once per step
+    and kept in the context for the other layers."""
+    if getattr(ctx, "one_row_per_request", False):
+        return AttentionPlan(None, 0, None, ctx.rows)
+
+    def make() -> AttentionPlan:
+        fold, split = [], []
+        for i, s in enumerate(ctx.segments):
+            n, r0 = len(s.tokens), ctx.seq_start[i]
+            if n == 1 and s.pos0 + 1 >= DECODE_MIN_CONTEXT:
+                split.append((r0, 1, i, 0))
+                continue
+            for off in range(0, n, tokens_per_tile):
+                fold.append((r0 + off, min(tokens_per_tile, n - off), i, 0))
+            while len(fold) % group_tiles:
+                fold.append((r0, 0, i, 0))
+        both = np.asarray(fold + split, np.int32).reshape(-1, 4)
+        dev = torch.from_numpy(both).to(ctx.device)
+        return AttentionPlan(dev[:len(fold)].contiguous() if fold else None, len(fold),
+                             dev[len(fold):].contiguous() if split else None, len(split))
+
+    return ctx.memo(("attention_tiles", tokens_per_tile, group_tiles), make)
+
+
 @register_mixer("attention")
 class Attention(Mixer):
     """params: width, heads, kv_heads, head_dim, window (None = all keys), position (PartSpec
     of the position encoding).  tensors: q_proj/k_proj/v_proj/o_proj .weight."""
-
-    graph_safe = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
@@ -43,6 +81,7 @@ class Attention(Mixer):
         self.scale = 1.0 / math.sqrt(float(self.head_dim))     # 1.0f / sqrtf(float(hd)), src/kernels.cpp:347
         pos = p["position"]
         self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+        self.graph_safe = bool(getattr(self.position, "graph_safe", False))    # the tables must be device tensors
         self.qkv: Optional[Linear] = None
         self.o: Optional[Linear] = None
         group = self.heads // self.kv_heads
@@ -77,78 +116,78 @@ class Attention(Mixer):
     def forward_with_norm(self, ctx, call, x, norm, residual) -> bool:
         """Decode steps of few rows: norm, q|k|v product, rotation and cache write are one kernel."""
         from .norm import RMSNorm
-        rt = self.rt
+        rt, ws = self.rt, ctx.ws
         if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma
                 and ops.qkv_rope_head_dim_ok(self.head_dim, self.qkv.weight.shape[1])
                 and ops.can_fuse_norm(ctx.rows, self.qkv.weight, x)):
             return False
-        q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
+        q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
         ops.norm_qkv_rope_bf16(x, norm.weight, norm.eps, self.qkv.weight, q, ctx.positions, ctx.row_seq,
                                ctx.block_tables[call.group], self.position.cos, self.position.sin, call.k_cache,
-                               call.v_cache, ctx.rows, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                               call.v_cache, ctx.rows, self.heads, self.kv_heads, self.head_dim, ws.page_size,
                                call.writes_cache)
         self._attend(ctx, call, q, residual)
         return True
 
     def forward(self, ctx, call, h, residual) -> None:
-        rt, rows = self.rt, ctx.rows
+        rt, ws, rows = self.rt, ctx.ws, ctx.rows
         table = ctx.block_tables[call.group]
         window = int(self.window or 0)
         if rt.bf16 and self.qkv.mfma and ops.qkv_rope_gemm_ok(rows, self.head_dim, self.qkv.weight.shape[1],
                                                               self.heads + 2 * self.kv_heads):
             # rotation and cache write ride in the product's epilogue
-            q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
+            q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
             ops.gemm_qkv_rope_bf16(h, self.qkv.weight, q, ctx.positions, ctx.row_seq, table, self.position.cos,
                                    self.position.sin, call.k_cache, call.v_cache, rows, self.heads, self.kv_heads,
-                                   self.head_dim, rt.page_size, call.writes_cache)
+                                   self.head_dim, ws.page_size, call.writes_cache)
             self._attend(ctx, call, q, residual)
             return
-        qkv = rt.buffer("qkv", self.q_dim + 2 * self.kv_dim, torch.float32)
-        self.qkv.store(h, qkv, rows)
+        qkv = ws.buffer("qkv", self.q_dim + 2 * self.kv_dim, torch.float32)
+        self.qkv.store(ws, h, qkv, rows)
         if rt.bf16:
-            q = rt.buffer("q_rot", self.q_dim, torch.bfloat16)
+            q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
             ops.rope_kvwrite(qkv, q, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
-                             rt.page_size, call.writes_cache)
+                             ws.page_size, call.writes_cache)
             self._attend(ctx, call, q, residual)
         else:
             ops.rope_kvwrite(qkv, None, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
-                             rt.page_size, call.writes_cache)
-            out = rt.buffer("attn_out", self.q_dim, torch.float32)
-            plan = ctx.attention_plan(16, 1)
-            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+                             ws.page_size, call.writes_cache)
+            out = ws.buffer("attn_out", self.q_dim, torch.float32)
+            plan = plan_tiles(ctx, 16, 1)
+            common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, ws.page_size,
                       window, self.scale)
             if plan.fold_count and self.head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
                 # every row by itself (also: a batch of nothing but decoded tokens, row t of request t)
                 ops.attention_f32(qkv, ctx.positions, ctx.row_seq, table, call.k_cache, call.v_cache, out, rows,
-                                  self.heads, self.kv_heads, self.head_dim, rt.page_size, window, self.scale)
+                                  self.heads, self.kv_heads, self.head_dim, ws.page_size, window, self.scale)
             else:
                 if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
                     ops.attention_f32_tiles(qkv, ctx.positions, table, plan.fold_tiles, plan.fold_count, True, *common)
                 if plan.decode_count:
                     ops.attention_f32_tiles(qkv, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common)
-            self.o.add_into(out, residual, rows)
+            self.o.add_into(ws, out, residual, rows)
 
     def _attend(self, ctx, call, q, residual) -> None:
         """bfloat16 attention over the cache for rotated queries ``q``, then the output projection."""
-        rt, rows = self.rt, ctx.rows
+        ws, rows = ctx.ws, ctx.rows
         table = ctx.block_tables[call.group]
         window = int(self.window or 0)
-        out = rt.buffer("attn_out", self.q_dim, torch.bfloat16)
-        plan = ctx.attention_plan(self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
-        common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, rt.page_size,
+        out = ws.buffer("attn_out", self.q_dim, torch.bfloat16)
+        plan = plan_tiles(ctx, self.tokens_per_tile, ops.fold_group_tiles(self.head_dim))
+        common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, ws.page_size,
                   window, self.scale)
         if plan.fold_count:
             ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
         if plan.decode_count:
             # few decoded tokens: several workgroups a tile, meeting in device scratch
             floats, counters = ops.attention_decode_scratch(plan.decode_count, self.heads, self.kv_heads, self.head_dim,
-                                                            table.stride(0), rt.page_size)
+                                                            table.stride(0), ws.page_size)
             scratch = None
             if floats:
-                scratch = (rt.buffer("attn_split", floats, torch.float32, rows=1),
-                           rt.buffer("attn_split_count", counters, torch.int32, rows=1))
+                scratch = (ws.buffer("attn_split", floats, torch.float32, rows=1),
+                           ws.buffer("attn_split_count", counters, torch.int32, rows=1))
             ops.attention_bf16(q, ctx.positions, table, plan.decode_tiles, plan.decode_count, *common, decode=True,
                                scratch=scratch)
-        self.o.add_into(out, residual, rows)
+        self.o.add_into(ws, out, residual, rows)

@@ -36,11 +36,22 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
-    block: str                     # arrangement of the parts, e.g. "prenorm"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    """One layer: the arrangement (a registered block) and the parts it arranges, by role.
+
+    Which roles a block has, and which kind of part fills each, is the block's own business
+    (``Block.roles``); every block has a role "mixer", the part that may own a cache or state.
+    """
+    block: str                                         # arrangement of the parts, e.g. "prenorm"
+    parts: Dict[str, PartSpec] = field(default_factory=dict)   # role -> part
+
+    @classmethod
+    def prenorm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ffn_norm: PartSpec) -> "LayerSpec":
+        return cls("prenorm", {"mixer_norm": mixer_norm, "ffn_norm": ffn_norm, "mixer": mixer,
+                               "feed_forward": feed_forward})
+
+    @property
+    def mixer(self) -> PartSpec:
+        return self.parts["mixer"]
 
 
 @dataclass(frozen=True)
@@ -92,7 +103,10 @@ class StateSpec:
 # --------------------------------------------------------------------------- interfaces
 
 class Part:
-    """Base of every part.  ``runtime`` carries device, precision mode and kernels."""
+    """Base of every part.  ``runtime`` carries the device and the precision mode; what belongs
+    to one engine (scratch buffers, page size, caches) arrives with every step's context."""
+
+    graph_safe = False             # True if forward() launches only capturable device work
 
     def __init__(self, params: Dict[str, Any], runtime: "Any"):
         self.params = dict(params)
@@ -110,6 +124,23 @@ class Part:
         return 0
 
 
+class Embedding(Part):
+    def forward(self, ctx):
+        """Token ids ``ctx.tokens`` -> the 32-bit residual stream [max_rows, width] (a buffer of
+        the context's workspace; rows of negative tokens are zero)."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def bind(self, tensors: Dict[str, Any], embedding: Optional[Embedding] = None) -> None:
+        """As Part.bind; ``embedding`` is the model's embedding part (a tied head reads its table)."""
+
+    def forward(self, ctx, x, norm, count: int):
+        """x: ``count`` wanted rows of the 32-bit residual stream; runs ``norm`` and the
+        projection; returns 32-bit logits [>= count, vocab]."""
+        raise NotImplementedError
+
+
 class Norm(Part):
     def forward(self, ctx, x):
         """x: [rows, width] 32-bit residual stream -> normed rows in the activation dtype."""
@@ -121,8 +152,6 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    graph_safe = False             # True if forward() launches only capturable device work
-
     def cache_spec(self) -> Optional[CacheSpec]:
         return None
 
@@ -145,8 +174,6 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    graph_safe = False
-
     def forward_with_norm(self, ctx, x, norm, residual) -> bool:
         """As Mixer.forward_with_norm."""
         return False
@@ -157,11 +184,23 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """The arrangement of mixer, feed-forward and norms around the residual stream."""
+    """The arrangement of a layer's parts around the residual stream.
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm, runtime):
+    ``roles`` names the parts an arrangement has and the kind of each ("mixer", "feed_forward",
+    "norm"), in the order their tensors are listed; the built parts become attributes of those
+    names.  Every arrangement has a role "mixer"."""
+
+    roles: Dict[str, str] = {}
+
+    def __init__(self, parts: Dict[str, Part], runtime):
         super().__init__({}, runtime)
-        self.mixer, self.feed_forward, self.mixer_norm, self.ffn_norm = mixer, feed_forward, mixer_norm, ffn_norm
+        missing = [r for r in self.roles if r not in parts]
+        extra = [r for r in parts if r not in self.roles]
+        if missing or extra:
+            raise ValueError(f"block {type(self).__name__}: missing parts {missing}, unknown parts {extra}")
+        self.parts = {role: parts[role] for role in self.roles}
+        for role, part in self.parts.items():
+            setattr(self, role, part)
 
     def forward(self, ctx, call, x) -> None:
         raise NotImplementedError
@@ -174,6 +213,10 @@ FEED_FORWARDS: Dict[str, Type[FeedForward]] = {}
 NORMS: Dict[str, Type[Norm]] = {}
 POSITION_ENCODINGS: Dict[str, Type[PositionEncoding]] = {}
 BLOCKS: Dict[str, Type[Block]] = {}
+EMBEDDINGS: Dict[str, Type[Embedding]] = {}
+HEADS: Dict[str, Type[Head]] = {}
+# the registry of every kind of part a block's role may name
+KINDS: Dict[str, Dict[str, type]] = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
 
 
 def _register(table: Dict[str, type], what: str) -> Callable[[str], Callable[[type], type]]:
@@ -192,6 +235,8 @@ register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
 register_norm = _register(NORMS, "norm")
 register_position_encoding = _register(POSITION_ENCODINGS, "position encoding")
 register_block = _register(BLOCKS, "block")
+register_embedding = _register(EMBEDDINGS, "embedding")
+register_head = _register(HEADS, "head")
 
 
 def lookup(table: Dict[str, type], what: str, name: str) -> type:

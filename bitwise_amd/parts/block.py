@@ -9,6 +9,9 @@ from .base import Block, register_block
 class PreNormBlock(Block):
     """x += mixer(norm1(x)); x += feed_forward(norm2(x)) (src/model.cpp:281-305)."""
 
+    roles = {"mixer_norm": "norm", "ffn_norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    graph_safe = True
+
     def forward(self, ctx, call, x) -> None:
         if not self.mixer.forward_with_norm(ctx, call, x, self.mixer_norm, x):
             h = self.mixer_norm.forward(ctx, x)

@@ -7,12 +7,15 @@ from typing import Dict, Optional
 import torch
 
 from ..csrc import ops
-from .base import Part, TensorSpec
+from .base import Embedding, Head, TensorSpec, register_embedding, register_head
 from .linear import Linear
 
 
-class Embedding(Part):
+@register_embedding("embedding")
+class TokenEmbedding(Embedding):
     """params: vocab, width.  tensor: weight [vocab, width], gathered as 32-bit rows."""
+
+    graph_safe = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
@@ -29,14 +32,17 @@ class Embedding(Part):
         return 0      # a step reads one row per token, not the table
 
     def forward(self, ctx) -> torch.Tensor:
-        x = self.rt.buffer("residual", self.width, torch.float32)
+        x = ctx.ws.buffer("residual", self.width, torch.float32)
         ops.embed(ctx.tokens[:ctx.rows], self.weight, x)
         return x
 
 
-class LMHead(Part):
+@register_head("lm_head")
+class LMHead(Head):
     """params: vocab, width, tied.  tensor: weight [vocab, width] unless tied to the embedding
     (src/model.cpp:170-171).  Only the wanted rows are normed and projected."""
+
+    graph_safe = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
@@ -46,27 +52,27 @@ class LMHead(Part):
     def tensors(self) -> Dict[str, TensorSpec]:
         return {} if self.tied else {"weight": TensorSpec((self.vocab, self.width), "linear")}
 
-    def bind(self, tensors, embedding: Optional[Embedding] = None) -> None:
+    def bind(self, tensors, embedding=None) -> None:
         if self.tied:
-            self.linear = Linear(embedding.weight, self.rt)     # the same device tensor, not a copy
+            table = getattr(embedding, "weight", None)
+            if table is None or tuple(table.shape) != (self.vocab, self.width):
+                raise ValueError("a tied head needs an embedding part with a table [vocab, width]")
+            self.linear = Linear(table, self.rt)     # the same device tensor, not a copy
         else:
             self.linear = Linear(tensors["weight"], self.rt)
 
     def weight_bytes(self) -> int:
         return self.linear.nbytes()
 
-    def forward_with_norm(self, ctx, x: torch.Tensor, norm, count: int):
-        """Few wanted rows: the final norm and the head product are one kernel.  Returns the
-        logits buffer, or None if this step cannot be fused."""
+    def forward(self, ctx, x: torch.Tensor, norm, count: int) -> torch.Tensor:
+        """Final norm and projection of ``count`` rows; few rows: both are one kernel (the same bits)."""
         from .norm import RMSNorm
-        if not (self.rt.bf16 and isinstance(norm, RMSNorm) and self.linear.mfma
+        ws = ctx.ws
+        logits = ws.buffer("logits", self.vocab, torch.float32, rows=ws.max_logit_rows)
+        if (self.rt.bf16 and isinstance(norm, RMSNorm) and self.linear.mfma
                 and ops.can_fuse_norm(count, self.linear.weight, x)):
-            return None
-        logits = self.rt.buffer("logits", self.vocab, torch.float32, rows=self.rt.max_logit_rows)
-        ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.linear.weight, logits, count, ops.EPI_F32)
-        return logits
-
-    def forward(self, ctx, normed: torch.Tensor, count: int) -> torch.Tensor:
-        logits = self.rt.buffer("logits", self.vocab, torch.float32, rows=self.rt.max_logit_rows)
-        self.linear.store(normed, logits, count)
+            ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.linear.weight, logits, count, ops.EPI_F32)
+            return logits
+        normed = norm.forward(ctx, x, out_name="final_normed", rows=count)
+        self.linear.store(ws, normed, logits, count)
         return logits

@@ -26,25 +26,26 @@ class Linear:
     def nbytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
-    def _x32(self, x: torch.Tensor, rows: int) -> torch.Tensor:
+    def _x32(self, ws, x: torch.Tensor, rows: int) -> torch.Tensor:
         if x.dtype == torch.float32:
             return x
-        buf = self.rt.buffer("linear_x32", x.shape[1], torch.float32)
-        buf[:rows].copy_(x[:rows])
+        buf = ws.buffer("linear_x32", x.shape[1], torch.float32)
+        ops.convert(x, buf, rows)
         return buf
 
-    def store(self, x: torch.Tensor, out: torch.Tensor, rows: int) -> None:
-        """out[:rows] = x[:rows] @ W.T (out float32, or bfloat16 on the matrix-core path)."""
+    def store(self, ws, x: torch.Tensor, out: torch.Tensor, rows: int) -> None:
+        """out[:rows] = x[:rows] @ W.T (out float32, or bfloat16 on the matrix-core path).  ``ws`` is the
+        step's workspace (temporaries for a weight whose dtype is not the mode's)."""
         if self.mfma:
             ops.gemm_bf16(x, self.weight, out, rows, ops.EPI_BF16 if out.dtype == torch.bfloat16 else ops.EPI_F32)
         elif out.dtype == torch.float32:
-            ops.gemm_f32(self._x32(x, rows), self.weight, out, rows)
+            ops.gemm_f32(self._x32(ws, x, rows), self.weight, out, rows)
         else:
-            tmp = self.rt.buffer("linear_y32", self.out_features, torch.float32)
-            ops.gemm_f32(self._x32(x, rows), self.weight, tmp, rows)
-            out[:rows].copy_(tmp[:rows])
+            tmp = ws.buffer("linear_y32", self.out_features, torch.float32)
+            ops.gemm_f32(self._x32(ws, x, rows), self.weight, tmp, rows)
+            ops.convert(tmp, out, rows)
 
-    def add_into(self, x: torch.Tensor, residual: torch.Tensor, rows: int) -> None:
+    def add_into(self, ws, x: torch.Tensor, residual: torch.Tensor, rows: int) -> None:
         """residual[:rows] += x[:rows] @ W.T, the sum in 32-bit (src/model.cpp:300, :305)."""
         if self.mfma:
             # a long inner size and 17 to 64 rows: every 2048-segment of it gets workgroups of its own,
@@ -56,10 +57,10 @@ class Linear:
             if 16 < rows <= 64:
                 floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features)
             elif rows >= 512 and ops.gemm_add_scratch(rows, self.out_features, self.in_features)[0]:
-                floats, counters = ops.gemm_add_scratch(self.rt.max_rows, self.out_features, self.in_features)
+                floats, counters = ops.gemm_add_scratch(ws.max_rows, self.out_features, self.in_features)
             if floats:
-                scratch = (self.rt.buffer("gemm_add_split", floats, torch.float32, rows=1),
-                           self.rt.buffer("gemm_add_split_count", counters, torch.int32, rows=1))
+                scratch = (ws.buffer("gemm_add_split", floats, torch.float32, rows=1),
+                           ws.buffer("gemm_add_split_count", counters, torch.int32, rows=1))
             ops.gemm_bf16(x, self.weight, residual, rows, ops.EPI_ADD_F32, scratch=scratch)
         else:
-            ops.gemm_f32(self._x32(x, rows), self.weight, residual, rows, accumulate=True)
+            ops.gemm_f32(self._x32(ws, x, rows), self.weight, residual, rows, accumulate=True)

@@ -45,28 +45,28 @@ class SwiGLU(FeedForward):
     def forward_with_norm(self, ctx, x, norm, residual) -> bool:
         """Decode steps of few rows: norm, the stacked product and SwiGLU are one kernel."""
         from .norm import RMSNorm
-        rt = self.rt
+        rt, ws = self.rt, ctx.ws
         if not (rt.bf16 and isinstance(norm, RMSNorm) and self.gate_up.mfma and self.down.mfma
                 and ops.can_fuse_norm(ctx.rows, self.gate_up.weight, x)):
             return False
-        act = rt.buffer("mlp_h", self.inter, torch.bfloat16)
+        act = ws.buffer("mlp_h", self.inter, torch.bfloat16)
         ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.gate_up.weight, act, ctx.rows, ops.EPI_SWIGLU_BF16)
-        self.down.add_into(act, residual, ctx.rows)
+        self.down.add_into(ws, act, residual, ctx.rows)
         return True
 
     def forward(self, ctx, h, residual) -> None:
-        rt, rows = self.rt, ctx.rows
+        rt, ws, rows = self.rt, ctx.ws, ctx.rows
         if self.gate_up.mfma:
-            act = rt.buffer("mlp_h", self.inter, torch.bfloat16)
+            act = ws.buffer("mlp_h", self.inter, torch.bfloat16)
             ops.gemm_bf16(h, self.gate_up.weight, act, rows, ops.EPI_SWIGLU_BF16)   # SwiGLU in the epilogue
         else:
-            gu = rt.buffer("gate_up", 2 * self.inter, torch.float32)
-            self.gate_up.store(h, gu, rows)
-            act32 = rt.buffer("mlp_h32", self.inter, torch.float32)
+            gu = ws.buffer("gate_up", 2 * self.inter, torch.float32)
+            self.gate_up.store(ws, h, gu, rows)
+            act32 = ws.buffer("mlp_h32", self.inter, torch.float32)
             ops.swiglu_f32(gu, act32, rows)
             if rt.bf16 and self.down.mfma:
-                act = rt.buffer("mlp_h", self.inter, torch.bfloat16)
-                act[:rows].copy_(act32[:rows])
+                act = ws.buffer("mlp_h", self.inter, torch.bfloat16)
+                ops.convert(act32, act, rows)
             else:
                 act = act32
-        self.down.add_into(act, residual, rows)
+        self.down.add_into(ws, act, residual, rows)

@@ -15,6 +15,8 @@ class RMSNorm(Norm):
     """params: width, eps.  tensor: weight [width].  The sum of squares, the root and both
     products are 32-bit; the output has the mode's activation dtype."""
 
+    graph_safe = True
+
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         self.width = int(params["width"])
@@ -32,6 +34,6 @@ class RMSNorm(Norm):
 
     def forward(self, ctx, x: torch.Tensor, out_name: str = "normed", rows: int | None = None) -> torch.Tensor:
         rows = ctx.rows if rows is None else rows
-        out = self.rt.buffer(out_name, self.width, self.rt.act_dtype)
+        out = ctx.ws.buffer(out_name, self.width, self.rt.act_dtype)
         ops.rmsnorm(x, self.weight, out, rows, self.eps)
         return out

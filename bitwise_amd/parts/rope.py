@@ -18,6 +18,8 @@ from .base import PositionEncoding, register_position_encoding
 class RotaryTable(PositionEncoding):
     """params: theta, head_dim, max_positions.  No checkpoint tensors."""
 
+    graph_safe = True
+
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         self.theta = float(params["theta"])

@@ -23,13 +23,13 @@ class Replayer:
         self.model = model if model is not None else Model.load(model_dir, dtype)
         asm = self.model.assembled
         rows = max(64, min(int(max_tokens), MAX_STEP_ROWS))
-        asm.rt.configure(max_rows=rows, page_size=block_size, max_logit_rows=rows)
         pages = (int(max_tokens) + block_size - 1) // block_size
         self.manager = CacheManager([GroupSpec(g.window) for g in asm.group_specs], pages, block_size, max_live,
                                     prefix_caching=False, has_state=bool(asm.state_specs))
-        self.storage = CacheStorage(asm, pages, max_live)
+        self.storage = CacheStorage(asm, pages, max_live, block_size)
         max_len = min(asm.spec.max_positions, max(int(max_tokens), 1))
-        self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, use_graphs=use_graphs)
+        self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, max_rows=rows, max_logit_rows=rows,
+                                  use_graphs=use_graphs)
         self.live: Dict[str, RequestCache] = {}
 
     def step(self, entries: Sequence[dict], end: Sequence[str] = ()) -> Optional[np.ndarray]:
@@ -66,7 +66,7 @@ class Replayer:
         return out
 
     def _run(self, segments: List[Segment]) -> Optional[np.ndarray]:
-        limit = self.runner.rt.max_rows
+        limit = self.runner.ws.max_rows
         if sum(len(s.tokens) for s in segments) <= limit:
             lg = self.runner.step(segments)
             return None if lg is None else lg.cpu().numpy()

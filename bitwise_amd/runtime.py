@@ -1,8 +1,10 @@
-"""What every part shares on the device: precision mode, scratch buffers, position tables."""
+"""What parts see of the device: the model-wide ``Runtime`` (device, precision mode, objects
+that parts share) and the per-engine ``Workspace`` (step size limits, page size and the scratch
+buffers of one step function)."""
 
 from __future__ import annotations
 
-from typing import Any, Callable, Dict, Tuple
+from typing import Any, Callable, Dict
 
 import torch
 
@@ -10,16 +12,15 @@ MODES = ("bfloat16", "float32")
 
 
 class Runtime:
-    """Device, precision mode and persistent scratch memory of one model instance.
+    """Device and precision mode of one model instance, and objects its parts share.
 
     mode "bfloat16": the kernels and precisions of serving (bfloat16 operands on the matrix
     cores, 32-bit accumulation, 32-bit residual stream, bfloat16 cache).  mode "float32":
-    everything in true 32-bit with plain fused multiply-adds.  Scratch buffers are made once
-    for ``max_rows`` rows and never move, so captured HIP graphs stay valid.
+    everything in true 32-bit with plain fused multiply-adds.  Nothing here belongs to a
+    particular engine: any number of step functions may run one model.
     """
 
-    def __init__(self, mode: str = "bfloat16", device: str | torch.device | None = "cuda:0", max_rows: int = 256,
-                 page_size: int = 16, max_logit_rows: int | None = None):
+    def __init__(self, mode: str = "bfloat16", device: str | torch.device | None = "cuda:0"):
         if mode not in MODES:
             raise ValueError(f"dtype must be one of {MODES}, got {mode!r}")
         self.mode = mode
@@ -28,22 +29,34 @@ class Runtime:
         if self.device is not None and self.device.type != "cuda":
             raise RuntimeError("bitwise_amd runs on the GPU only; there is no CPU path")
         self.act_dtype = torch.bfloat16 if mode == "bfloat16" else torch.float32
-        self._buffers: Dict[Any, torch.Tensor] = {}
         self._shared: Dict[Any, Any] = {}
-        self.scratch_generation = 0      # bumped when the buffers are dropped (captured graphs go stale)
-        self.configure(max_rows, page_size, max_logit_rows)
-
-    def configure(self, max_rows: int, page_size: int, max_logit_rows: int | None = None) -> None:
-        """Set the step size limits; existing scratch buffers are dropped."""
-        self.max_rows = int(max_rows)
-        self.page_size = int(page_size)
-        self.max_logit_rows = int(max_logit_rows if max_logit_rows is not None else max_rows)
-        self._buffers.clear()
-        self.scratch_generation += 1
 
     @property
     def bf16(self) -> bool:
         return self.mode == "bfloat16"
+
+    def shared(self, key: Any, make: Callable[[], Any]) -> Any:
+        """Objects several parts share (one rotary table per distinct parameter set)."""
+        if key not in self._shared:
+            self._shared[key] = make()
+        return self._shared[key]
+
+
+class Workspace:
+    """Scratch memory and size limits of one step function (one engine, one replayer, one
+    ``Model.logits`` call).  Buffers are made once per name for ``max_rows`` rows and never
+    move, so HIP graphs captured over them stay valid; two workspaces share nothing."""
+
+    def __init__(self, device: torch.device, max_rows: int, page_size: int, max_logit_rows: int | None = None):
+        self.device = torch.device(device)
+        self.max_rows = int(max_rows)
+        self.page_size = int(page_size)
+        self.max_logit_rows = int(max_logit_rows if max_logit_rows is not None else max_rows)
+        if self.max_rows < 1 or self.max_logit_rows < 1:
+            raise ValueError("a workspace needs room for at least one row")
+        if self.page_size < 1 or self.page_size & (self.page_size - 1):
+            raise ValueError(f"page size must be a power of two, got {self.page_size}")
+        self._buffers: Dict[Any, torch.Tensor] = {}
 
     def buffer(self, name: str, cols: int, dtype: torch.dtype, rows: int | None = None) -> torch.Tensor:
         """A persistent zero-initialised [rows or max_rows, cols] scratch tensor by name."""
@@ -54,8 +67,5 @@ class Runtime:
             self._buffers[key] = buf
         return buf
 
-    def shared(self, key: Any, make: Callable[[], Any]) -> Any:
-        """Objects several parts share (one rotary table per distinct parameter set)."""
-        if key not in self._shared:
-            self._shared[key] = make()
-        return self._shared[key]
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._buffers.values())

@@ -15,7 +15,7 @@ from bitwise_amd.engine.storage import CacheStorage
 from bitwise_amd.models.assembled import AssembledModel, CallBinding
 from bitwise_amd.parts import base
 from bitwise_amd.parts.base import LayerCall, LayerSpec, ModelSpec, PartSpec, StateSpec, TensorSpec
-from bitwise_amd.runtime import Runtime
+from bitwise_amd.runtime import Runtime, Workspace
 from bitwise_amd.weights.loader import random_tensors
 
 pytestmark = pytest.mark.gpu
@@ -27,21 +27,21 @@ def rnd_for(mode):
     return pl.round_bf16 if mode == "bfloat16" else pl.identity
 
 
-def one_request_ctx(rt, n, groups=1, pages=None):
-    pages = pages if pages is not None else list(range((n + rt.page_size - 1) // rt.page_size))
-    return StepContext([Segment([0] * n, 0, [pages] * groups, 0, [])], groups, rt.device)
+def one_request_ctx(ws, n, groups=1, pages=None):
+    pages = pages if pages is not None else list(range((n + ws.page_size - 1) // ws.page_size))
+    return StepContext([Segment([0] * n, 0, [pages] * groups, 0, [])], groups, ws)
 
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 def test_norm_part(gpu, mode):
-    rt = Runtime(mode, gpu, max_rows=32, page_size=8)
+    rt, ws = Runtime(mode, gpu), Workspace(gpu, max_rows=32, page_size=8)
     part = base.NORMS["rmsnorm"]({"width": 72, "eps": 1e-3}, rt)
     assert part.tensors() == {"weight": TensorSpec((72,), "norm")}
     w = 1 + 0.1 * torch.randn(72)
     part.bind({"weight": w.bfloat16()})
     x = torch.zeros(32, 72, device=gpu)
     x[:5] = torch.randn(5, 72, device=gpu) * 2
-    out = part.forward(one_request_ctx(rt, 5), x)
+    out = part.forward(one_request_ctx(ws, 5), x)
     assert out.dtype == rt.act_dtype
     ref = pl.rmsnorm(x[:5].double().cpu(), w.bfloat16(), 1e-3)
     assert (out[:5].cpu().double() - ref).abs().max() <= (2 ** -8 if mode == "bfloat16" else 4e-7) * ref.abs().max()
@@ -49,7 +49,7 @@ def test_norm_part(gpu, mode):
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 def test_feed_forward_part(gpu, mode):
-    rt = Runtime(mode, gpu, max_rows=64, page_size=8)
+    rt, ws = Runtime(mode, gpu), Workspace(gpu, max_rows=64, page_size=8)
     part = base.FEED_FORWARDS["swiglu"]({"width": 40, "inter": 88}, rt)
     specs = part.tensors()
     assert specs["down_proj.weight"].shape == (40, 88) and specs["gate_proj.weight"].shape == (88, 40)
@@ -60,7 +60,7 @@ def test_feed_forward_part(gpu, mode):
     h[:n] = torch.randn(n, 40, device=gpu).to(rt.act_dtype)
     res = torch.randn(64, 40, device=gpu)
     before = res.clone()
-    part.forward(one_request_ctx(rt, n), h, res)
+    part.forward(one_request_ctx(ws, n), h, res)
     hd = h[:n].cpu().double()
     act = rnd_for(mode)(pl.swiglu(pl.linear(hd, w["gate_proj.weight"]), pl.linear(hd, w["up_proj.weight"])))
     ref = before[:n].cpu().double() + pl.linear(act, w["down_proj.weight"])
@@ -74,7 +74,7 @@ def test_attention_part(gpu, mode, heads, kvh, hd, window):
     """The mixer alone: projections, rotation, cache write through a permuted block table,
     attention (with a window as an option) and the output projection added to the residual."""
     width, page = 56, 8
-    rt = Runtime(mode, gpu, max_rows=64, page_size=page)
+    rt, ws = Runtime(mode, gpu), Workspace(gpu, max_rows=64, page_size=page)
     pos_spec = PartSpec("rope", {"theta": 5000.0, "head_dim": hd, "max_positions": 64})
     part = base.MIXERS["attention"]({"width": width, "heads": heads, "kv_heads": kvh, "head_dim": hd, "window": window,
                                      "position": pos_spec}, rt)
@@ -90,13 +90,13 @@ def test_attention_part(gpu, mode, heads, kvh, hd, window):
     # the first 30 positions as one portion, then 7 single tokens: the cache carries over
     h = torch.zeros(64, width, device=gpu, dtype=rt.act_dtype)
     h[:30] = h_all[:30].to(gpu)
-    ctx = StepContext([Segment([0] * 30, 0, [pages], 0, [])], 1, gpu)
+    ctx = StepContext([Segment([0] * 30, 0, [pages], 0, [])], 1, ws)
     part.forward(ctx, call, h, res)
     got = [res[:30].cpu().clone()]
     for p in range(30, n):
         h[0] = h_all[p].to(gpu)
         res.zero_()
-        part.forward(StepContext([Segment([0], p, [pages], 0, [])], 1, gpu), call, h, res)
+        part.forward(StepContext([Segment([0], p, [pages], 0, [])], 1, ws), call, h, res)
         got.append(res[:1].cpu().clone())
     got = torch.cat(got).double()
     x = h_all.double()
@@ -145,9 +145,9 @@ class RunningMean(base.Mixer):
 def toy_spec(width=32, vocab=50):
     def layer(i, mixer):
         pre = f"layers.{i}."
-        return LayerSpec("prenorm", mixer, PartSpec("swiglu", {"width": width, "inter": 48}, pre + "mlp."),
-                         PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm1."),
-                         PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm2."))
+        return LayerSpec.prenorm(mixer, PartSpec("swiglu", {"width": width, "inter": 48}, pre + "mlp."),
+                                 PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm1."),
+                                 PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, pre + "norm2."))
     rope = PartSpec("rope", {"theta": 10000.0, "head_dim": 16, "max_positions": 128})
     attn = PartSpec("attention", {"width": width, "heads": 2, "kv_heads": 1, "head_dim": 16, "window": None,
                                   "position": rope}, "layers.1.attn.")
@@ -195,7 +195,7 @@ def plain_toy(w, toks, rnd):
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 def test_toy_mixer_with_state_and_a_schedule_that_repeats_and_shares(gpu, mode):
-    rt = Runtime(mode, gpu, max_rows=64, page_size=8)
+    rt = Runtime(mode, gpu)
     model = AssembledModel(toy_spec(), rt)
     assert len(model.state_specs) == 2 and len(model.group_specs) == 1 and model.group_caches == [[1]]
     assert not model.graph_safe                                   # the toy part works on the host: no graph capture
@@ -203,10 +203,10 @@ def test_toy_mixer_with_state_and_a_schedule_that_repeats_and_shares(gpu, mode):
     assert "layers.0.toy.gain" in specs and "head.weight" not in specs
     w = dict(random_tensors(specs, 9, 0.2))
     model.bind_tensors({k: v.to(gpu) for k, v in w.items()})
-    storage = CacheStorage(model, num_pages=12, num_slots=3)
+    storage = CacheStorage(model, num_pages=12, num_slots=3, page_size=8)
     manager = CacheManager([GroupSpec(None)], 12, 8, 3, prefix_caching=True, has_state=True)
     assert not manager.prefix_caching                             # state outside the pages: no prefix reuse
-    runner = ModelRunner(model, storage, max_model_len=128, use_graphs=True)
+    runner = ModelRunner(model, storage, max_model_len=128, max_rows=64, use_graphs=True)
     a = [int(t) for t in torch.randint(0, 50, (23,), generator=torch.Generator().manual_seed(1))]
     b = [int(t) for t in torch.randint(0, 50, (11,), generator=torch.Generator().manual_seed(2))]
     rnd = rnd_for(mode)
@@ -299,19 +299,19 @@ def test_toy_routed_feed_forward_and_another_position_encoding(gpu, mode):
     pos = PartSpec("toy_stretched_rope", {"theta": 1000.0, "head_dim": hd, "max_positions": 64, "stretch": stretch})
     attn = PartSpec("attention", {"width": width, "heads": 2, "kv_heads": 2, "head_dim": hd, "window": None, "position": pos},
                     "l.attn.")
-    layer = LayerSpec("prenorm", attn, PartSpec("toy_top1", {"width": width}, "l.moe."),
-                      PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm1."),
-                      PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm2."))
+    layer = LayerSpec.prenorm(attn, PartSpec("toy_top1", {"width": width}, "l.moe."),
+                              PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm1."),
+                              PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "l.norm2."))
     spec = ModelSpec("ToyRouted", vocab, width, PartSpec("embedding", {"vocab": vocab, "width": width}, "embed."), [layer],
                      [LayerCall(0, 0)], PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "norm."),
                      PartSpec("lm_head", {"vocab": vocab, "width": width, "tied": True}, "head."), 64)
-    rt = Runtime(mode, gpu, max_rows=32, page_size=8)
+    rt = Runtime(mode, gpu)
     model = AssembledModel(spec, rt)
     w = dict(random_tensors(model.tensor_specs(), 17, 0.3))
     model.bind_tensors({k: v.to(gpu) for k, v in w.items()})
-    storage = CacheStorage(model, num_pages=8, num_slots=2)
+    storage = CacheStorage(model, num_pages=8, num_slots=2, page_size=8)
     manager = CacheManager([GroupSpec(None)], 8, 8, 2, prefix_caching=False)
-    runner = ModelRunner(model, storage, max_model_len=64, use_graphs=False)
+    runner = ModelRunner(model, storage, max_model_len=64, max_rows=32, use_graphs=False)
     toks = [int(t) for t in torch.randint(0, vocab, (21,), generator=torch.Generator().manual_seed(5))]
     rnd = rnd_for(mode)
 
@@ -346,7 +346,7 @@ def test_toy_routed_feed_forward_and_another_position_encoding(gpu, mode):
 
 
 def test_schedule_errors(gpu):
-    rt = Runtime("float32", gpu, max_rows=16, page_size=8)
+    rt = Runtime("float32", gpu)
     spec = toy_spec()
     spec.schedule = [LayerCall(1, 5, writes_cache=False)]
     with pytest.raises(ValueError, match="before any call wrote it"):
@@ -357,6 +357,6 @@ def test_schedule_errors(gpu):
     spec.schedule = [LayerCall(7, 0)]
     with pytest.raises(ValueError, match="names layer 7"):
         AssembledModel(spec, rt)
-    spec.layers[0].mixer.kind = "no_such_mixer"
+    spec.layers[0].parts["mixer"].kind = "no_such_mixer"
     with pytest.raises(KeyError, match="unknown mixer 'no_such_mixer'"):
         AssembledModel(spec, rt)
