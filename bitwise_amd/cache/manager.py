@@ -42,6 +42,9 @@ class CacheManager:
                                and self.groups[0].window is None)
         self.pools = [PagePool(num_pages, page_size, self.prefix_caching) for _ in self.groups]
         self.slots = StateSlots(num_slots)
+        # called with (group, page) whenever a page becomes free (tests fill such pages with NaN, so that a
+        # page that is handed out again must be written before it is read)
+        self.on_free = None
 
     # ------------------------------------------------------------------ requests
     def open(self) -> Optional[RequestCache]:
@@ -57,10 +60,10 @@ class CacheManager:
         rc.slot = -1
 
     def release_pages(self, rc: RequestCache) -> None:
-        for pool, table in zip(self.pools, rc.tables):
+        for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
             for page in table:
-                if page >= 0:
-                    pool.release(page)
+                if page >= 0 and pool.release(page) and self.on_free is not None:
+                    self.on_free(g, page)
         # new lists, not cleared ones: a table only ever grows at its end while it is the same object (the step
         # function's host copy of a block table relies on that)
         rc.tables = [[] for _ in self.pools]
@@ -113,6 +116,17 @@ class CacheManager:
                 table.append(page)
         return True
 
+    def can_ever_hold(self, tokens: int, step_tokens: int) -> bool:
+        """Whether a request of ``tokens`` tokens fits an empty engine (src/engine.cpp:130-133): every group's
+        pool must hold what the request holds there at once, all its pages in a group that keeps all keys, and
+        in a windowed group the window and one step's tokens (and the page either end may straddle)."""
+        ps = self.page_size
+        for g in self.groups:
+            held = tokens if g.window is None else min(tokens, g.window + step_tokens + 2 * ps)
+            if (held + ps - 1) // ps > self.num_pages:
+                return False
+        return True
+
     def pages_missing(self, rc: RequestCache, tokens: int) -> int:
         """Most pages any pool would have to hand out for ``ensure(rc, tokens)``."""
         need = (tokens + self.page_size - 1) // self.page_size
@@ -136,7 +150,8 @@ class CacheManager:
             lo = min(self.first_needed_page(g, computed), len(table))
             for i in range(lo):
                 if table[i] >= 0:
-                    pool.release(table[i])
+                    if pool.release(table[i]) and self.on_free is not None:
+                        self.on_free(g, table[i])
                     table[i] = -1
 
     # ------------------------------------------------------------------ accounting

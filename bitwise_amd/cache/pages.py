@@ -69,16 +69,19 @@ class PagePool:
         self._ref[page] = 1
         return page
 
-    def release(self, page: int) -> None:
+    def release(self, page: int) -> bool:
+        """Drop one reference.  True if the page is free now: nobody holds it and it is not kept
+        as a cached page either, so what it holds is dead."""
         if self._ref[page] <= 0:
             raise RuntimeError(f"release of unreferenced page {page}")
         self._ref[page] -= 1
         if self._ref[page] > 0:
-            return
+            return False
         if self._hash_of[page] is not None:
             self._evictable[page] = None          # newest at the tail
-        else:
-            self._free.append(page)
+            return False
+        self._free.append(page)
+        return True
 
     def lookup(self, hash_: int, tokens: Sequence[int]) -> Optional[int]:
         """A cached full page with this hash AND these tokens; takes a reference on a hit."""

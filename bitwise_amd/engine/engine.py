@@ -136,7 +136,7 @@ class Engine:
         if any(t < 0 or t >= self.exec.vocab_size for t in prompt):
             raise ValueError("token id out of range")
         worst = len(prompt) + params.max_new_tokens + 1
-        if worst > self.cfg.num_blocks * self.cfg.block_size:
+        if not self.manager.can_ever_hold(worst, self.cfg.max_batched_tokens):
             raise ValueError("request can never fit in the KV cache")
         if len(prompt) + params.max_new_tokens > self.exec.max_model_len:
             raise ValueError(f"prompt and new tokens exceed the model length {self.exec.max_model_len}")
@@ -166,7 +166,8 @@ class Engine:
 
     @property
     def free_blocks(self) -> int:
-        return self.manager.free_pages(0)
+        """Free pages of the first cache group (the reference's one pool); all pages if the model keeps no paged cache."""
+        return self.manager.free_pages(0) if self.manager.pools else self.cfg.num_blocks
 
     def result(self, id: int) -> RequestResult:
         return self._results[id]

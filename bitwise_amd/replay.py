@@ -19,7 +19,9 @@ MAX_STEP_ROWS = 4096
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, use_graphs: bool = True,
-                 max_live: int = 64, model: Optional[Model] = None):
+                 max_live: int = 64, model: Optional[Model] = None, poison_freed_pages: bool = False):
+        """``poison_freed_pages``: every page that comes back is filled with NaN at once (a fault finder: what a
+        later owner of the page reads before writing it shows up in its logits)."""
         self.model = model if model is not None else Model.load(model_dir, dtype)
         asm = self.model.assembled
         rows = max(64, min(int(max_tokens), MAX_STEP_ROWS))
@@ -30,6 +32,8 @@ class Replayer:
         max_len = min(asm.spec.max_positions, max(int(max_tokens), 1))
         self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, max_rows=rows, max_logit_rows=rows,
                                   use_graphs=use_graphs)
+        if poison_freed_pages:
+            self.manager.on_free = lambda group, page: self.storage.poison_pages(group, [page])
         self.live: Dict[str, RequestCache] = {}
 
     def step(self, entries: Sequence[dict], end: Sequence[str] = ()) -> Optional[np.ndarray]:

@@ -129,16 +129,17 @@ def mlp_block(x, w, pre, c, rnd):
 
 
 def forward(config: Mapping[str, object], w: Mapping[str, torch.Tensor], tokens: Sequence[int],
-            rnd: Callable = identity, first_position: int = 0) -> torch.Tensor:
+            rnd: Callable = identity, first_position: int = 0, windows: Optional[Sequence[Optional[int]]] = None) -> torch.Tensor:
     """Logits [T, vocab] (float64) at every position of one whole sequence
     (src/model.cpp:267-322 with every row wanted, as python/bindings.cpp:35-52 does).
-    ``first_position`` shifts all positions (only distances matter to rotary attention)."""
+    ``first_position`` shifts all positions (only distances matter to rotary attention).
+    ``windows``: per layer, how many keys a query sees (None: all; the reference has no window)."""
     c = read_config(config)
     positions = [first_position + i for i in range(len(tokens))]
     x = embed(tokens, w["model.embed_tokens.weight"])
     for layer in range(c["layers"]):
         pre = f"model.layers.{layer}."
-        x = x + attention_block(x, w, pre, c, positions, rnd)
+        x = x + attention_block(x, w, pre, c, positions, rnd, None if windows is None else windows[layer])
         x = x + mlp_block(x, w, pre, c, rnd)
     x = rnd(rmsnorm(x, w["model.norm.weight"], c["eps"]))
     head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]

@@ -160,3 +160,59 @@ def test_constants_and_sampling():
     assert set(cold) <= {1, 2}                                           # low temperature: only the maxima
     h1 = pl.hash_floats(1469598103934665603, np.array([1.0, 2.0, 3.0], np.float32))
     assert h1 != pl.hash_floats(1469598103934665603, np.array([1.0, 2.0, 3.0000002], np.float32))
+
+
+# ----------------------------------------------------------------------------- the scalar 32-bit decoder
+
+def test_scalar_decoder_agrees_with_the_float64_one():
+    """Two transcriptions of the same formulas, in different languages and precisions: what one gets wrong
+    (a pairing, an order, a transposed weight) the other must get wrong the same way to pass."""
+    import plain_scalar as ps
+    from bitwise_amd.model import describe
+    from bitwise_amd.weights.loader import random_tensors
+
+    for cfg, seed, sigma in ((TINY_A, 0, 0.05), (TINY_B, 1, 0.08)):
+        w = dict(random_tensors(describe(cfg), seed, sigma))
+        toks = [(i * 31 + 5) % cfg["vocab_size"] for i in range(45)]
+        a = ps.forward(cfg, w, toks)
+        b = pl.forward(cfg, w, toks).numpy()
+        assert np.abs(a - b).max() <= 2e-5 * np.abs(b).max()
+        shifted = ps.forward(cfg, w, toks, first_position=9)
+        assert np.abs(shifted - a).max() <= 3e-5 * np.abs(b).max()          # only distances count
+        assert not np.array_equal(shifted, a)
+        windowed = ps.forward(cfg, w, toks, window=11)
+        assert np.array_equal(windowed[:11], a[:11]) and not np.array_equal(windowed[11:], a[11:])
+
+
+def test_scalar_primitives():
+    import plain_scalar as ps
+
+    assert ps.expf([0.0])[0] == np.float32(1.0)                            # one key: its value, exactly
+    edge = ps.expf([-87.5, -1e30, 89.5, float("inf"), float("-inf")])
+    assert list(edge[:2]) == [0.0, 0.0] and np.isinf(edge[2]) and np.isinf(edge[3]) and edge[4] == 0.0
+    assert np.isnan(ps.expf([float("nan")])[0])
+    x = np.linspace(-80, 80, 20001, dtype=np.float32)
+    ref = np.exp(x.astype(np.float64))
+    assert (np.abs(ps.expf(x).astype(np.float64) - ref) <= 2.0 * np.spacing(ref.astype(np.float32))).all()
+    # the 16 chains and the tree, written out (tests/test_main.cpp:126-131), in exact arithmetic
+    from fractions import Fraction
+    rng = np.random.default_rng(3)
+    for n in (1, 5, 16, 31, 64, 100, 128):
+        a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        lane = [np.float32(0)] * 16
+        for i in range(n):
+            exact = Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(lane[i % 16]))
+            c = np.float32(float(exact))                                  # float(Fraction) rounds correctly to double;
+            lane[i % 16] = c                                              # a double rounds to float32 once more: close
+        s8 = [np.float32(lane[i] + lane[i + 8]) for i in range(8)]
+        s4 = [np.float32(s8[i] + s8[i + 4]) for i in range(4)]
+        want = np.float32(np.float32(s4[0] + s4[2]) + np.float32(s4[1] + s4[3]))
+        got = ps.dot_canonical(a, b)
+        assert abs(float(got) - float(want)) <= 4 * np.spacing(np.float32(abs(float(want)) + 1e-30))
+    w = np.arange(12, dtype=np.float32).reshape(3, 4)
+    onehot = np.zeros((1, 4), np.float32)
+    onehot[0, 2] = 1
+    assert np.array_equal(ps.linear(onehot, w)[0], w[:, 2])
+    assert ps.swiglu([0.0], [5.0])[0] == 0.0 and ps.swiglu([30.0], [2.0])[0] == np.float32(60.0)
+    y = ps.rmsnorm(np.full((1, 8), 3.0, np.float32), np.ones(8, np.float32), 0.5)
+    assert np.allclose(y, 3.0 / math.sqrt(9.5), rtol=1e-6)

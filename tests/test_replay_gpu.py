@@ -15,6 +15,7 @@ import pytest
 import torch
 
 import plain_llama as pl
+import plain_scalar as ps
 import tiny
 
 pytestmark = pytest.mark.gpu
@@ -38,19 +39,24 @@ def plain_logits(folder, toks, dtype):
 
 
 def replay(folder, dtype, name, steps, max_tokens, **kw):
-    """Run steps through a Replayer; returns {request: [len, vocab] logits} (every position wanted)."""
+    """Run steps through a Replayer; returns {request: [len, vocab] logits} (every position wanted), the
+    replayer, and {request: the pages it ever held in group 0}."""
     from bitwise_amd.replay import Replayer
 
     rp = Replayer(str(folder), dtype, max_tokens, block_size=tiny.CONFIGS[name][3], **kw)
-    out = {}
+    out, held = {}, {}
     for st in steps:
-        lg = rp.step(st["entries"], st.get("end", []))
+        lg = rp.step(st["entries"])
         row = 0
         for e in st["entries"]:
             for _ in e["want"]:
                 out.setdefault(e["id"], []).append(lg[row])
                 row += 1
-    assert rp.manager.all_free() or any(True for _ in rp.live)
+        for rid, rc in rp.live.items():
+            held.setdefault(rid, set()).update(p for p in rc.tables[0] if p >= 0)
+        rp.step([], st.get("end", []))          # the requests that end here give back what they hold
+        rp.manager.check()
+    rp.pages_held = held
     return {k: np.stack(v) for k, v in out.items()}, rp
 
 
@@ -77,7 +83,7 @@ def folders(tmp_path_factory, gpu):
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_cuttings_equal_plain_and_each_other(folders, name, dtype):
     cfg = tiny.read_config(folders[name])
-    lengths = [100, 67, 41, 33]
+    lengths = [100, 67, 41, 33, 20]
     reqs = requests_for(cfg, 11, lengths)
     page = tiny.CONFIGS[name][3]
     refs = {rid: plain_logits(folders[name], toks, dtype) for rid, toks in reqs.items()}
@@ -90,10 +96,16 @@ def test_cuttings_equal_plain_and_each_other(folders, name, dtype):
         scale = np.abs(refs[rid]).max()
         err = np.abs(got[rid] - refs[rid]).max()
         assert err <= TOL[dtype] * scale, f"{rid} whole: err {err:.3e} vs scale {scale:.3f}"
+        if dtype == "float32":          # and the bits of the plain scalar 32-bit decoder
+            want = ps.forward(cfg, tiny.read_weights(folders[name]), toks)
+            same = (got[rid].view(np.uint32) == want.view(np.uint32)).all(axis=1)
+            assert same.all(), f"{rid}: first position that is not the scalar decoder's bits: {int(np.argmin(same))}"
 
     # 2. most of it in one step, the last 32 tokens one by one
     for rid, toks in reqs.items():
         n = len(toks)
+        if n <= 32:
+            continue
         steps = [{"entries": [all_wanted(rid, toks[:n - 32])]}]
         steps += [{"entries": [{"id": rid, "tokens": [toks[i]], "want": [0]}]} for i in range(n - 32, n)]
         for use_graphs in (True, False):
@@ -101,24 +113,26 @@ def test_cuttings_equal_plain_and_each_other(folders, name, dtype):
             assert np.array_equal(got[rid], whole[rid]), f"{rid}: decoding differs from the whole prompt (graphs={use_graphs})"
 
     # 3. portions of changing size, down to two tokens and one
-    sizes = {100: [3, 17, 1, 19, 2, 30, 2, 26], 67: [2, 2, 31, 1, 1, 30], 41: [40, 1], 33: [16, 16, 1]}
+    sizes = {100: [3, 17, 1, 19, 2, 30, 2, 26], 67: [2, 2, 31, 1, 1, 30], 41: [40, 1], 33: [16, 16, 1], 20: [2, 16, 2]}
     for rid, toks in reqs.items():
         steps = [{"entries": [all_wanted(rid, part)]} for part in cut(toks, sizes[len(toks)])]
         got, _ = replay(folders[name], dtype, name, steps, 128)
         assert np.array_equal(got[rid], whole[rid]), f"{rid}: portions differ from the whole prompt"
 
-    # 4. mixed: up to four live requests, portions of some beside decoded tokens of others, and
-    # so few pages that finished requests' pages are used again
+    # 4. mixed: up to four live requests, portions of some beside decoded tokens of others, in a pool smaller
+    # than what the five requests need together (20 pages of 16, 36 of 8): pages that come back are filled
+    # with NaN at once and must serve a later request
     ids = list(reqs)
-    progress = {rid: 0 for rid in ids}
-    plan = {ids[0]: [30, 1, 1, 1, 20, 1, 1, 45], ids[1]: [2, 5, 1, 1, 1, 57], ids[2]: [41], ids[3]: [1, 1, 31]}
-    order = [[ids[0]], [ids[0], ids[1]], [ids[0], ids[1], ids[2]], [ids[1], ids[0]], [ids[0], ids[1]],
-             [ids[0], ids[1]], [ids[1], ids[0]], [ids[0]]]
-    steps, ended = [], set()
+    plan = {ids[0]: [30, 1, 1, 1, 20, 1, 1, 45], ids[1]: [2, 5, 1, 1, 1, 57], ids[2]: [41], ids[3]: [1, 1, 31],
+            ids[4]: [20]}
+    order = [[0], [0, 1], [0, 4, 1, 2], [1, 0, 3], [3, 0, 1], [0, 1, 3], [1, 0], [0]]
+    steps = []
     cursor = {rid: 0 for rid in ids}
+    progress = {rid: 0 for rid in ids}
     for group in order:
         entries, end = [], []
-        for rid in group:
+        for i in group:
+            rid = ids[i]
             part = plan[rid][cursor[rid]]
             cursor[rid] += 1
             toks = reqs[rid][progress[rid]:progress[rid] + part]
@@ -126,17 +140,16 @@ def test_cuttings_equal_plain_and_each_other(folders, name, dtype):
             entries.append(all_wanted(rid, toks))
             if progress[rid] == len(reqs[rid]):
                 end.append(rid)
-                ended.add(rid)
         steps.append({"entries": entries, "end": end})
-    # the fourth request arrives after the third has gone, into its pages
-    for part in plan[ids[3]]:
-        toks = reqs[ids[3]][progress[ids[3]]:progress[ids[3]] + part]
-        progress[ids[3]] += part
-        steps.append({"entries": [all_wanted(ids[3], toks)], "end": [ids[3]] if progress[ids[3]] == 33 else []})
     assert all(progress[r] == len(reqs[r]) for r in ids)
-    max_tokens = 128 + 128 + 64            # a, b and one of c/d, each rounded up to 64: pages must come back
-    got, rp = replay(folders[name], dtype, name, steps, max_tokens)
-    assert rp.manager.all_free()
+    assert max(len(st["entries"]) for st in steps) == 4
+    max_tokens = 144                       # 9 pages of 16, 18 of 8: the most that is ever held at once
+    demand = sum((len(t) + page - 1) // page for t in reqs.values())
+    assert demand > max_tokens // page, "the pool must be smaller than the requests' pages together"
+    got, rp = replay(folders[name], dtype, name, steps, max_tokens, poison_freed_pages=True)
+    assert rp.manager.all_free() and not rp.live
+    late, early = rp.pages_held[ids[3]], rp.pages_held[ids[2]] | rp.pages_held[ids[4]]
+    assert late & early, "the request that came late must have been given pages that an earlier one gave back"
     for rid in ids:
         assert np.array_equal(got[rid], whole[rid]), f"{rid}: the mixed batch differs from the whole prompt"
 
