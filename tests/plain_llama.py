@@ -174,20 +174,21 @@ def argmax_row(logits: np.ndarray) -> int:
     return best
 
 
-def sample_row(logits: np.ndarray, temperature: float, u: float) -> int:
+def sample_row(logits: np.ndarray, temperature: float, u: float, expf=np.exp) -> int:
     """w[i] = expf((l[i]-max)/T) in 32-bit, total and running sum in double, first i with
-    cum > u*total, else the last index with positive weight (src/engine.cpp:50-80)."""
+    cum > u*total, else the last index with positive weight (src/engine.cpp:50-80).  ``expf``: the
+    32-bit exponential (the library's, or the engine's own definition)."""
     l32 = np.asarray(logits, dtype=np.float32)
-    w = np.exp((l32 - l32.max()) / np.float32(temperature)).astype(np.float32)
+    w = np.asarray(expf((l32 - l32.max()) / np.float32(temperature)), dtype=np.float32)
     total = 0.0
-    for x in w:
-        total += float(x)
+    for x in w.tolist():
+        total += x
     target = u * total
     cum, last = 0.0, 0
-    for i, x in enumerate(w):
+    for i, x in enumerate(w.tolist()):
         if x <= 0.0:
             continue
-        cum += float(x)
+        cum += x
         last = i
         if cum > target:
             return last

@@ -659,6 +659,27 @@ def test_sampling_and_fingerprint(gpu):
         assert h_out.cpu().numpy().view(np.uint64).tolist() == want
 
 
+def test_sampling_at_real_vocabularies(gpu):
+    """49,152 and 128,256 logits a row: the device sums its weights in 256 stretches that it joins in order, the
+    plain code in one sequential chain of doubles; both use the engine's own 32-bit exponential, so they must
+    pick the same token wherever the uniform does not fall within rounding of a boundary."""
+    import plain_scalar as ps
+
+    g = torch.Generator().manual_seed(17)
+    for V in (49152, 128256):
+        rows = 12
+        logits = (torch.randn(rows, V, generator=g) * 2.5).to(gpu)
+        logits[0, V - 3] = 30.0                                        # nearly all weight on a late token
+        temps = [0.7, 0.7, 1.0, 1.3, 0.2, 2.0, 0.9, 0.9, 0.0, 1.0, 0.5, 1.1]
+        us = [0.5, 0.001, 0.999, 0.25, 0.75, 0.6180339887, 0.0, 1.0 - 2 ** -53, 0.4, 0.31415926, 0.9, 0.05]
+        out = torch.zeros(rows, dtype=torch.int32, device=gpu)
+        ops.sample(logits, rows, torch.tensor(temps, device=gpu), torch.tensor(us, dtype=torch.float64, device=gpu), out)
+        host = logits.cpu().numpy()
+        for r, got in enumerate(out.cpu().tolist()):
+            want = pl.argmax_row(host[r]) if temps[r] <= 0 else pl.sample_row(host[r], temps[r], us[r], ps.expf)
+            assert got == want, f"V={V} row {r}"
+
+
 # ----------------------------------------------------------------------------- decode fusions
 
 def test_fused_norm_products_equal_the_separate_kernels(gpu):

@@ -253,27 +253,38 @@ def test_awkward_sizes(gpu, tmp_path, dtype):
         assert np.array_equal(model.logits(toks, chunk=5), whole) and np.array_equal(model.logits(toks, chunk=1), whole), (i, dtype)
 
 
-def test_real_layer_sizes_are_cut_invariant(gpu):
-    """Two layers of the SmolLM2-1.7B sizes, so that every shape-dependent route of the kernels runs at the shapes it
-    was written for (K = 2048 and 8192, 6144 / 2048 / 16384 / 49152 columns): a prompt whole; in portions of 1600, 300,
-    100, 61, 29 and 10 tokens; with its last 40 tokens decoded one by one from graphs; and decoded beside 8 and then 19
-    other requests.  The logits of the last 40 positions are the same bits every time."""
+REAL_SHAPES = {
+    # SmolLM2-1.7B's layer sizes
+    "smollm2": dict(vocab_size=49152, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, head_dim=64,
+                    intermediate_size=8192, rope_theta=130000.0, tie_word_embeddings=True),
+    # Llama-3-8B's: heads of 128, four query heads a key head, a feed-forward of seven 2048-segments, an untied head
+    "llama3_8b": dict(vocab_size=128256, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=14336, rope_theta=500000.0, tie_word_embeddings=False),
+}
+
+
+@pytest.mark.parametrize("shape,dtype", [("smollm2", "bfloat16"), ("smollm2", "float32"), ("llama3_8b", "bfloat16")])
+def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
+    """Two layers of real sizes, so that every shape-dependent route of the kernels runs at the shapes it was
+    written for (K = 2048, 4096, 8192 and 14336; up to 128,256 columns), in bfloat16 and in 32-bit: a prompt whole;
+    in portions of 1600, 300, 100, 61, 29 and 10 tokens; with its last 40 tokens decoded one by one from graphs;
+    and decoded beside 8 and then 19 other requests.  The logits of the last 40 positions are the same bits every time."""
     import bitwise_amd as bw
     from bitwise_amd.replay import Replayer
 
-    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "vocab_size": 49152,
-           "hidden_size": 2048, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 32,
-           "head_dim": 64, "intermediate_size": 8192, "rope_theta": 130000.0, "rms_norm_eps": 1e-5,
-           "tie_word_embeddings": True, "max_position_embeddings": 4096, "bos_token_id": 1, "eos_token_id": 2}
-    model = bw.Model.random(cfg, seed=3, dtype="bfloat16", sigma=0.02, on_device=True)
+    cfg = dict({"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "num_hidden_layers": 2,
+                "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "bos_token_id": 1, "eos_token_id": 2},
+               **REAL_SHAPES[shape])
+    vocab = cfg["vocab_size"]
+    model = bw.Model.random(cfg, seed=3, dtype=dtype, sigma=0.02, on_device=True)
     g = torch.Generator().manual_seed(11)
-    toks = torch.randint(0, 49152, (2100,), generator=g).tolist()
-    others = {f"o{i}": torch.randint(0, 49152, (30,), generator=g).tolist() for i in range(19)}
+    toks = torch.randint(0, vocab, (2100,), generator=g).tolist()
+    others = {f"o{i}": torch.randint(0, vocab, (30,), generator=g).tolist() for i in range(19)}
     tail = 40
     head = len(toks) - tail
 
     def last(rp_steps, max_tokens=4096):
-        rp = Replayer("", "bfloat16", max_tokens, block_size=16, model=model)
+        rp = Replayer("", dtype, max_tokens, block_size=16, model=model)
         rows = []
         for st in rp_steps:
             lg = rp.step(st["entries"], st.get("end", []))
@@ -286,7 +297,7 @@ def test_real_layer_sizes_are_cut_invariant(gpu):
         return np.stack(rows)
 
     whole = last([{"entries": [{"id": "r", "tokens": toks, "want": list(range(head, len(toks)))}]}])
-    assert whole.shape == (tail, 49152) and np.isfinite(whole).all()
+    assert whole.shape == (tail, vocab) and np.isfinite(whole).all()
     steps, pos = [], 0
     for n in (1600, 300, 100, 61, 29, 10):
         want = [i - pos for i in range(max(pos, head), pos + n)]
