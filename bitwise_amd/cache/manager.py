@@ -47,11 +47,15 @@ class CacheManager:
         self.on_free = None
 
     # ------------------------------------------------------------------ requests
-    def open(self) -> Optional[RequestCache]:
-        slot = self.slots.allocate()
+    def open(self, seed: int = 0, stream: int = 0) -> Optional[RequestCache]:
+        """Take a state slot; it records the request's position (0 now) and the key of its random draws."""
+        slot = self.slots.allocate(seed, stream)
         if slot is None:
             return None
         return RequestCache(slot=slot, tables=[[] for _ in self.groups])
+
+    def record(self, rc: RequestCache):
+        return self.slots.records[rc.slot]
 
     def close(self, rc: RequestCache) -> None:
         """Give back every page and the slot."""
@@ -90,6 +94,7 @@ class CacheManager:
             rc.hashes.append(h)
             parent = h
         rc.computed = len(rc.tables[0]) * ps
+        self.slots.records[rc.slot].position = rc.computed
         return rc.computed
 
     # ------------------------------------------------------------------ growth
@@ -136,6 +141,7 @@ class CacheManager:
         """After a step: ``computed`` tokens are in the cache.  Register newly full pages
         (src/engine.cpp:196-205) and give back pages a window has passed."""
         rc.computed = computed
+        self.slots.records[rc.slot].position = computed
         ps = self.page_size
         if self.prefix_caching:
             pool, table = self.pools[0], rc.tables[0]

@@ -6,6 +6,7 @@ src/block_manager.cpp:21-88, with the page size a run-time value instead of 16).
 from __future__ import annotations
 
 from collections import OrderedDict
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 _M64 = (1 << 64) - 1
@@ -127,6 +128,15 @@ class PagePool:
                 raise AssertionError("hash index out of step")
 
 
+@dataclass
+class SlotRecord:
+    """What a request's slot holds on the host beside the device state of its mixers: how many of its tokens
+    are in the cache (the position of its next token) and the key of its random draws."""
+    position: int = 0
+    seed: int = 0
+    stream: int = 0
+
+
 class StateSlots:
     """Slots 0..n-1 for per-request state of fixed size; lowest free slot first."""
 
@@ -134,15 +144,17 @@ class StateSlots:
         self._free = list(range(num_slots - 1, -1, -1))
         self._used = set()
         self.num_slots = num_slots
+        self.records: List[SlotRecord] = [SlotRecord() for _ in range(num_slots)]
 
     def available(self) -> int:
         return len(self._free)
 
-    def allocate(self) -> Optional[int]:
+    def allocate(self, seed: int = 0, stream: int = 0) -> Optional[int]:
         if not self._free:
             return None
         s = self._free.pop()
         self._used.add(s)
+        self.records[s] = SlotRecord(0, seed, stream)
         return s
 
     def release(self, slot: int) -> None:

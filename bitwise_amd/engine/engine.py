@@ -217,8 +217,11 @@ class Engine:
             else:
                 self._stats.prefill_tokens += w.n
         t0 = self.now()
-        draw = ([w.seq.params.temperature for w in sampled], [w.seq.params.seed for w in sampled],
-                [len(w.seq.tokens) for w in sampled])
+        # a draw is keyed by what the request's slot records: its seed, and its position once this step's
+        # tokens are in the cache (the number of tokens it holds before the new one, src/engine.cpp:473)
+        records = [self.manager.record(w.seq.cache) for w in sampled]
+        draw = ([w.seq.params.temperature for w in sampled], [r.seed for r in records],
+                [r.position + w.n for r, w in zip(records, sampled)])
         if sampled and getattr(self.exec, "fused_sampling", False):
             logits = self.exec.run(segments, draw)
         else:

@@ -144,7 +144,7 @@ class Scheduler:
                 break
             s = self.waiting[0]
             if s.cache is None:
-                s.cache = self.manager.open()
+                s.cache = self.manager.open(seed=s.params.seed)
                 if s.cache is None:
                     break                     # no state slot free (cannot happen while slots == max_num_seqs)
                 if self.on_open is not None:

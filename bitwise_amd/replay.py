@@ -7,6 +7,7 @@ from __future__ import annotations
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
+import torch
 
 from .cache.manager import CacheManager, GroupSpec, RequestCache
 from .engine.batch import Segment
@@ -19,7 +20,8 @@ MAX_STEP_ROWS = 4096
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, use_graphs: bool = True,
-                 max_live: int = 64, model: Optional[Model] = None, poison_freed_pages: bool = False):
+                 max_live: int = 64, model: Optional[Model] = None, poison_freed_pages: bool = False,
+                 fingerprint_logits: bool = False):
         """``poison_freed_pages``: every page that comes back is filled with NaN at once (a fault finder: what a
         later owner of the page reads before writing it shows up in its logits)."""
         self.model = model if model is not None else Model.load(model_dir, dtype)
@@ -35,6 +37,10 @@ class Replayer:
         if poison_freed_pages:
             self.manager.on_free = lambda group, page: self.storage.poison_pages(group, [page])
         self.live: Dict[str, RequestCache] = {}
+        # per request, the chained hash of every logits row that was asked for (src/engine.cpp:18-29, :246)
+        self.fingerprint_logits = fingerprint_logits
+        self.fingerprints: Dict[str, int] = {}
+        self._sampler = None
 
     def step(self, entries: Sequence[dict], end: Sequence[str] = ()) -> Optional[np.ndarray]:
         """Run one step; returns the wanted logits [wanted, vocab] or None."""
@@ -60,7 +66,8 @@ class Replayer:
             touched.append(rc)
         out = None
         if segments:
-            out = self._run(segments)
+            owners = [str(e["id"]) for e in entries if e.get("tokens") for _ in e.get("want", [])]
+            out = self._run(segments, owners)
             for rc, seg in zip(touched, segments):
                 self.manager.advance(rc, (), rc.computed + len(seg.tokens))
         for rid in end:
@@ -69,20 +76,47 @@ class Replayer:
                 self.manager.close(rc)
         return out
 
-    def _run(self, segments: List[Segment]) -> Optional[np.ndarray]:
+    def _chain_fingerprints(self, logits: torch.Tensor, owners: Sequence[str]) -> None:
+        """Chain each owner's fingerprint over its rows of ``logits`` in order: the k-th rows of all requests
+        are hashed by one launch."""
+        from .sampling.rng import FINGERPRINT_BASIS
+        from .sampling.sampler import Sampler
+        if self._sampler is None:
+            self._sampler = Sampler(logits.device, self.runner.ws.max_logit_rows)
+        waves: List[List[int]] = []
+        seen: Dict[str, int] = {}
+        for row, rid in enumerate(owners):
+            k = seen.get(rid, 0)
+            seen[rid] = k + 1
+            if k == len(waves):
+                waves.append([])
+            waves[k].append(row)
+        for rows in waves:
+            idx = torch.as_tensor(rows, dtype=torch.long, device=logits.device)
+            prev = [self.fingerprints.get(owners[r], FINGERPRINT_BASIS) for r in rows]
+            for r, h in zip(rows, self._sampler.fingerprints(logits.index_select(0, idx).contiguous(), prev)):
+                self.fingerprints[owners[r]] = h
+
+    def _run(self, segments: List[Segment], owners: Sequence[str] = ()) -> Optional[np.ndarray]:
         limit = self.runner.ws.max_rows
         if sum(len(s.tokens) for s in segments) <= limit:
             lg = self.runner.step(segments)
+            if lg is not None and self.fingerprint_logits:
+                self._chain_fingerprints(lg, owners)
             return None if lg is None else lg.cpu().numpy()
         # A step larger than the scratch buffers runs as several launches of the step
         # function; the logits do not depend on the cut.
         outs, batch, rows = [], [], 0
+        done = [0]
 
         def flush():
             nonlocal batch, rows
             if batch:
                 lg = self.runner.step(batch)
                 if lg is not None:
+                    if self.fingerprint_logits:
+                        self._chain_fingerprints(lg, owners[done[0]:done[0] + lg.shape[0]])
+                    done[0] += lg.shape[0]
                     outs.append(lg.cpu().numpy())
             batch, rows = [], 0
 

@@ -48,21 +48,30 @@ def read_file(path: str | Path) -> Dict[str, torch.Tensor]:
     header, base = read_header(path)
     data = np.memmap(path, dtype=np.uint8, mode="r")
     out: Dict[str, torch.Tensor] = {}
+    spans = []
     for name, info in header.items():
         tag = info["dtype"]
         if tag not in _NP_OF:
             raise SafetensorsError(f"{path}: unsupported dtype {tag} for {name}")
-        start, end = info["data_offsets"]
+        start, end = (int(v) for v in info["data_offsets"])
         shape = tuple(int(s) for s in info["shape"])
+        if any(s < 0 for s in shape) or not 0 <= start <= end:
+            raise SafetensorsError(f"{path}: tensor {name} has a negative size or offsets that run backwards")
         count = int(np.prod(shape, dtype=np.int64)) if shape else 1
         item = np.dtype(_NP_OF[tag]).itemsize
         if end - start != count * item or base + end > data.size:
             raise SafetensorsError(f"{path}: truncated tensor {name}")
+        if end > start:
+            spans.append((start, end, name))
         arr = np.frombuffer(data, dtype=_NP_OF[tag], count=count, offset=base + start).reshape(shape)
         t = torch.from_numpy(arr)
         if tag == "BF16":
             t = t.view(torch.int16).view(torch.bfloat16)
         out[name] = t
+    spans.sort()
+    for (_, e0, n0), (s1, _, n1) in zip(spans, spans[1:]):
+        if s1 < e0:
+            raise SafetensorsError(f"{path}: tensors {n0} and {n1} overlap")
     return out
 
 

@@ -152,3 +152,39 @@ def test_prefix_reuse_rules():
     mgr.close(d)
     off = CacheManager([GroupSpec(None)], 8, 8, 2, prefix_caching=True, has_state=True)
     assert not off.prefix_caching                                   # state outside the pages cannot be reused
+
+
+def test_two_storages_on_one_model_share_nothing():
+    """Caches, state and page size belong to a storage, not to the model: a second storage (another engine, a
+    replayer, Model.logits) leaves the first one's tensors and the model's plan alone."""
+    from tiny import TINY_A
+    from bitwise_amd.config.llama import LlamaConfig
+    from bitwise_amd.engine.storage import CacheStorage
+    from bitwise_amd.models.assembled import AssembledModel
+    from bitwise_amd.models.llama import llama_spec
+    from bitwise_amd.runtime import Runtime
+
+    asm = AssembledModel(llama_spec(LlamaConfig.from_dict(TINY_A)), Runtime("float32", None))   # described only: host tensors
+    first = CacheStorage(asm, num_pages=4, num_slots=2, page_size=16)
+    mine = [(c.k_cache, c.v_cache) for c in first.bindings]
+    second = CacheStorage(asm, num_pages=9, num_slots=3, page_size=8)
+    assert all(c.k_cache is None and c.v_cache is None and c.state is None for c in asm.calls)
+    for c, (k, v) in zip(first.bindings, mine):
+        assert c.k_cache is k and c.v_cache is v and k.shape[0] == 4
+    assert [c.k_cache.shape for c in second.bindings] == [(9, 2 * 8 * 16)] * 2
+    assert first.bindings[0].k_cache.data_ptr() != second.bindings[0].k_cache.data_ptr()
+    assert first.page_size == 16 and second.page_size == 8
+
+
+def test_slot_records_position_and_seed():
+    from bitwise_amd.cache.manager import CacheManager, GroupSpec
+
+    m = CacheManager([GroupSpec(None)], 8, 4, 2, prefix_caching=False)
+    rc = m.open(seed=77)
+    assert (m.record(rc).position, m.record(rc).seed, m.record(rc).stream) == (0, 77, 0)
+    assert m.ensure(rc, 9)
+    m.advance(rc, list(range(9)), 9)
+    assert m.record(rc).position == 9
+    m.close(rc)
+    again = m.open(seed=5)
+    assert (m.record(again).position, m.record(again).seed) == (0, 5)

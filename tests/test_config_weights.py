@@ -120,5 +120,19 @@ def test_broken_files(tmp_path):
     (tmp_path / "model.safetensors").write_bytes(raw[:-100])
     with pytest.raises(safetensors_io.SafetensorsError, match="truncated tensor"):
         loader.load_folder(tmp_path, specs)
+    # offsets that run backwards, or two tensors on the same bytes
+    import json
+    import struct
+
+    def write(header):
+        text = json.dumps(header).encode()
+        (tmp_path / "model.safetensors").write_bytes(struct.pack("<Q", len(text)) + text + bytes(64))
+
+    write({"a": {"dtype": "F32", "shape": [4], "data_offsets": [16, 0]}})
+    with pytest.raises(safetensors_io.SafetensorsError, match="run backwards"):
+        safetensors_io.read_file(tmp_path / "model.safetensors")
+    write({"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}, "b": {"dtype": "F32", "shape": [4], "data_offsets": [8, 24]}})
+    with pytest.raises(safetensors_io.SafetensorsError, match="overlap"):
+        safetensors_io.read_file(tmp_path / "model.safetensors")
     with pytest.raises(ConfigError, match="cannot open"):
         registry.read_config(tmp_path / "nowhere")

@@ -139,7 +139,10 @@ def test_residual_and_norm_placement():
 
 def test_constants_and_sampling():
     assert pl.mix64(0x9E3779B97F4A7C15) == 0xE220A8397B1DCDAF          # first output of splitmix64 seeded with 0
-    assert pl.block_hash(0, []) == pl.block_hash(0, [])                  # pure
+    # the chain: another parent, another token or another order gives another hash
+    hashes = {pl.block_hash(0, [1, 2, 3]), pl.block_hash(1, [1, 2, 3]), pl.block_hash(0, [1, 3, 2]), pl.block_hash(0, [1, 2]),
+              pl.block_hash(pl.block_hash(0, [1, 2, 3]), [1, 2, 3])}
+    assert len(hashes) == 5
     # the reference's basis is the FNV-1a offset 14695981039346656037 without its last digit
     # (src/block_manager.cpp:10, src/engine.h:68); its text is followed, not the FNV standard
     assert 1469598103934665603 == 0xCBF29CE484222325 // 10 and 1099511628211 == 0x100000001B3

@@ -215,11 +215,17 @@ def test_trace_run_program(folders, tmp_path):
     V = cfg["vocab_size"]
     ra, rb, rc = (plain_logits(folders[name], t, dtype) for t in (a, b, c))
     want = {0: [ra[0], ra[29]], 1: [rb[19]], 2: [rc[63]], 3: [ra[32], rc[69]], 4: [ra[49]]}
+    chained = {"a": 1469598103934665603, "b": 1469598103934665603, "c": 1469598103934665603}
+    owners = {0: ["a", "a"], 1: ["b"], 2: ["c"], 3: ["a", "c"], 4: ["a"]}
     for step, rows in want.items():
         got = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, V)
         assert got.shape[0] == len(rows)
-        for g, r in zip(got, rows):
+        for g, r, rid in zip(got, rows, owners[step]):
             assert np.abs(g - r).max() <= TOL[dtype] * np.abs(r).max()
+            chained[rid] = pl.hash_floats(chained[rid], g)
+    # every request's fingerprint: the hash chained over the rows it asked for, as the files hold them
+    prints = json.loads((out / "fingerprints.json").read_text())
+    assert {k: int(v, 16) for k, v in prints.items()} == chained
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
