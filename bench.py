@@ -7,7 +7,8 @@ random weights and uniform random token ids.
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
 decoded tokens per second.  One JSON line is printed; it also carries the 2,048-token prefill,
-the decode step's HBM roofline and decode at batch 1 and 64.
+the decode step's HBM roofline, decode at batch 1 and 64 with their rooflines, the same model's true
+32-bit path (decode and prefill) and decode and prefill at Llama-3-8B's sizes.
 """
 
 from __future__ import annotations
@@ -72,6 +73,63 @@ def time_decode(engine, torch, steps: int, warmup: int):
     return time.perf_counter() - t0
 
 
+LLAMA3_8B = {
+    # Llama-3-8B's sizes (BASELINE.json configs[3]): 32 layers, width 4096, 32 heads on 8 kv heads of 128,
+    # feed-forward 14336, vocabulary 128256, rotary base 500000 without scaling, eps 1e-5, untied head.
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu",
+    "vocab_size": 128256, "hidden_size": 4096, "num_hidden_layers": 32, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336, "rope_theta": 500000.0,
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192,
+    "bos_token_id": 1, "eos_token_id": 2,
+}
+
+
+def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float) -> dict:
+    """One 2,048-token prompt in one step (model, head for the last row, sampling); the best of three."""
+    engine = make_engine(bw, model, 1, 8, dtype)
+    g = torch.Generator().manual_seed(99)
+    times = []
+    for _ in range(4):
+        prompt = torch.randint(0, cfg["vocab_size"], (PREFILL_TOKENS,), generator=g).tolist()
+        engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+        assert engine.idle()
+    ms = min(times[1:])
+    flops = prefill_flops(cfg, PREFILL_TOKENS)
+    return {"value": round(PREFILL_TOKENS / ms * 1e3, 1), "tokens": PREFILL_TOKENS, "ms": round(ms, 3),
+            "frac": round(flops / (ms * 1e-3) / peak_flops, 4)}
+
+
+def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int) -> dict:
+    """``steps`` decode steps of ``batch`` requests that each hold a 2,048-token context: tokens a second, and
+    the bytes a step has to read (every weight once, the cache of the live requests) over its time."""
+    torch.cuda.empty_cache()
+    # Requests admitted early decode while the later ones are still being prefilled (one prompt a
+    # step): every request gets enough new tokens to outlast the prefills, the warm-up and the
+    # timed steps, so that each timed step has all ``batch`` rows.
+    new_tokens = steps + warmup + batch + 8
+    eng = make_engine(bw, model, batch, new_tokens, dtype)
+    fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch)
+    assert len(eng.sched.running) == batch
+    secs = time_decode(eng, torch, steps, warmup)
+    assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
+    kv_token = eng.exec.storage.bytes_per_token()
+    del eng
+    ms = secs / steps * 1e3
+    # keys a decoded token reads, on average: the prompt, what the request decoded while later
+    # prompts were prefilled, the warm-up, and half the timed steps
+    avg_ctx = CONTEXT + (batch - 1) / 2 + warmup + (steps + 1) / 2
+    step_bytes = model.weight_bytes + batch * avg_ctx * kv_token
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+    return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(achieved / PEAK_HBM_GBS, 4)}}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,7 +138,8 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (named in config)")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode points")
+    ap.add_argument("--no-points", action="store_true",
+                    help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (use --gpus 1)")
@@ -97,60 +156,45 @@ def main() -> int:
     t_start = time.perf_counter()
     model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
     vocab = cfg["vocab_size"]
-    total = args.steps + args.warmup
+    side_steps = max(16, args.steps // 2)
 
-    # ---- prefill of one 2,048-token prompt (one step: model, head for the last row, sampling)
-    engine = make_engine(bw, model, 1, 8, dtype)
-    g = torch.Generator().manual_seed(99)
-    prefill_ms = []
-    for rep in range(3):
-        prompt = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
-        engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        engine.step()
-        torch.cuda.synchronize()
-        prefill_ms.append((time.perf_counter() - t0) * 1e3)
-        assert engine.idle()
-    pf_ms = min(prefill_ms[1:])
-    flops = prefill_flops(cfg, PREFILL_TOKENS)
-    prefill = {"value": round(PREFILL_TOKENS / pf_ms * 1e3, 1), "tokens": PREFILL_TOKENS, "ms": round(pf_ms, 3),
-               "frac": round(flops / (pf_ms * 1e-3) / PEAK_FLOPS[args.dtype], 4)}
-    del engine
-
-    def decode_point(batch: int, steps: int, warmup: int):
-        torch.cuda.empty_cache()
-        # Requests admitted early decode while the later ones are still being prefilled (one prompt a
-        # step): every request gets enough new tokens to outlast the prefills, the warm-up and the
-        # timed steps, so that each timed step has all ``batch`` rows.
-        new_tokens = steps + warmup + batch + 8
-        eng = make_engine(bw, model, batch, new_tokens, dtype)
-        fill(eng, bw, torch, batch, vocab, new_tokens, seed=batch)
-        assert len(eng.sched.running) == batch
-        secs = time_decode(eng, torch, steps, warmup)
-        assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
-        kv_token = eng.exec.storage.bytes_per_token()
-        del eng
-        return secs, kv_token
-
-    secs, kv_token = decode_point(args.batch, args.steps, args.warmup)
-    ms_step = secs / args.steps * 1e3
-    value = args.batch * args.steps / secs
-    # keys a decoded token reads, on average: the prompt, what the request decoded while later
-    # prompts were prefilled, the warm-up, and half the timed steps
-    avg_ctx = CONTEXT + (args.batch - 1) / 2 + args.warmup + (args.steps + 1) / 2
-    step_bytes = model.weight_bytes + args.batch * avg_ctx * kv_token
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
-    points = {}
+    prefill = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype])
+    head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup)
+    points, point_rooflines = {}, {}
+    extra = {}
     if not args.no_points:
         for b in (1, 64):
-            s, _ = decode_point(b, max(16, args.steps // 2), 4)
-            points[f"decode_b{b}"] = round(b * max(16, args.steps // 2) / s, 1)
+            m = measure_decode(bw, torch, model, cfg, dtype, b, side_steps, 4)
+            points[f"decode_b{b}"] = m["tok_s"]
+            point_rooflines[f"decode_b{b}"] = m["roofline"]
+        if args.dtype == "bf16":
+            # the true 32-bit path of the same model (the same bfloat16 weights, widened exactly; 32-bit caches)
+            del model
+            torch.cuda.empty_cache()
+            model32 = bw.Model.random(cfg, seed=0, dtype="float32", sigma=0.02, on_device=True)
+            m = measure_decode(bw, torch, model32, cfg, "float32", args.batch, side_steps, 4)
+            extra["fp32"] = {"decode_tok_s": m["tok_s"], "batch": args.batch, "ms_per_step": m["ms_per_step"],
+                             "roofline": m["roofline"],
+                             "prefill": measure_prefill(bw, torch, model32, cfg, "float32", PEAK_FLOPS["fp32"])}
+            del model32
+            torch.cuda.empty_cache()
+            # Llama-3-8B's sizes, all 32 layers, bfloat16: decode at batch 8 with 2,048-token contexts, one prefill
+            big = dict(LLAMA3_8B)
+            model8 = bw.Model.random(big, seed=1, dtype="bfloat16", sigma=0.02, on_device=True)
+            m = measure_decode(bw, torch, model8, big, "bfloat16", 8, side_steps, 4)
+            extra["llama3_8b"] = {"layers": big["num_hidden_layers"], "hidden": big["hidden_size"], "heads": 32, "kv_heads": 8,
+                                  "head_dim": 128, "ffn": big["intermediate_size"], "vocab": big["vocab_size"],
+                                  "decode_tok_s": m["tok_s"], "batch": 8, "ms_per_step": m["ms_per_step"],
+                                  "roofline": m["roofline"],
+                                  "prefill": measure_prefill(bw, torch, model8, big, "bfloat16", PEAK_FLOPS["bf16"])}
+            del model8
+            model = None
 
+    value = head["tok_s"]
     line = {
         "metric": "decode tok/s at batch 8, SmolLM2-1.7B shape, 2048-token contexts",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / BASELINE_TOK_S, 1), "dtype": args.dtype, "data": "synthetic",
         "config": {
             "model": "SmolLM2-1.7B shape, random weights", "layers": cfg["num_hidden_layers"],
@@ -161,11 +205,12 @@ def main() -> int:
             "baseline": "reference CPU decode, one stream, 7.26 tok/s",
         },
         "prefill": prefill,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "roofline": head["roofline"],
         "points": points,
-        "wall_s": round(time.perf_counter() - t_start, 1),
+        "point_rooflines": point_rooflines,
     }
+    line.update(extra)
+    line["wall_s"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(line))
     return 0
 
