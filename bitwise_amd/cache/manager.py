@@ -164,6 +164,10 @@ class CacheManager:
     def free_pages(self, group: int = 0) -> int:
         return self.pools[group].available()
 
+    def free_pages_least(self) -> int:
+        """Free pages of the pool that has the fewest (all pools full-sized if the model keeps no paged cache)."""
+        return min((p.available() for p in self.pools), default=self.num_pages)
+
     def all_free(self) -> bool:
         return all(p.available() == p.num_pages for p in self.pools) and self.slots.available() == self.slots.num_slots
 

@@ -30,6 +30,7 @@ class EngineConfig:
     dtype: str = "bfloat16"          # "bfloat16" (serving precision) or "float32" (true 32-bit)
     max_model_len: int = 0           # 0: the model's max_position_embeddings
     use_graphs: bool = True          # replay pure-decode steps from captured HIP graphs
+    run_ahead: bool = True           # launch the next pure-decode step before the last one's tokens are read back
 
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):

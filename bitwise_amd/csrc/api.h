@@ -8,8 +8,8 @@
 #include <stdint.h>
 
 extern "C" {
-int bw_embed(const int32_t* tokens, const void* table, int table_is_bf16, float* out, int rows, int width,
-             int vocab, void* stream);
+int bw_embed(const int32_t* tokens, const int32_t* feedback, const void* table, int table_is_bf16, float* out,
+             int rows, int width, int vocab, void* stream);
 int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16, int rows,
                int dim, int ldy, float eps, void* stream);
 int bw_add(float* x, const float* y, long long n, void* stream);

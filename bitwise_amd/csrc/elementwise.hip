@@ -9,11 +9,16 @@
 
 // ------------------------------------------------------------------------- embedding
 
+// A token of -2 stands for "the token the last step sampled for this row": it is read from ``feedback`` (the
+// sampling kernel's output), so that a decode step can be launched before the host has seen the token.
+#define BW_TOKEN_FROM_FEEDBACK (-2)
+
 template <typename TableT>
-__global__ void embed_kernel(const int32_t* __restrict__ tokens, const TableT* __restrict__ table,
-                             float* __restrict__ out, int width, int vocab) {
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ feedback,
+                             const TableT* __restrict__ table, float* __restrict__ out, int width, int vocab) {
   const int row = blockIdx.x;
-  const int tok = tokens[row];
+  int tok = tokens[row];
+  if (tok == BW_TOKEN_FROM_FEEDBACK && feedback != nullptr) tok = feedback[row];
   float* o = out + (size_t)row * width;
   if (tok < 0 || tok >= vocab) {  // padding rows of a fixed-size batch carry token -1
     for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = 0.0f;
@@ -26,14 +31,14 @@ __global__ void embed_kernel(const int32_t* __restrict__ tokens, const TableT* _
   }
 }
 
-extern "C" int bw_embed(const int32_t* tokens, const void* table, int table_is_bf16, float* out, int rows,
-                        int width, int vocab, void* stream) {
+extern "C" int bw_embed(const int32_t* tokens, const int32_t* feedback, const void* table, int table_is_bf16, float* out,
+                        int rows, int width, int vocab, void* stream) {
   if (rows <= 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (table_is_bf16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, tokens, (const bf16_t*)table, out, width, vocab);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, tokens, feedback, (const bf16_t*)table, out, width, vocab);
   else
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(rows), dim3(256), 0, s, tokens, (const float*)table, out, width, vocab);
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(rows), dim3(256), 0, s, tokens, feedback, (const float*)table, out, width, vocab);
   return BW_LAUNCH_CHECK();
 }
 

@@ -33,7 +33,7 @@ _ERRORS = {
 }
 
 _SIGS = {
-    "bw_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_embed": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_add": [c_void_p, c_void_p, c_longlong, c_void_p],
     "bw_convert": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -121,8 +121,12 @@ def _is_bf16(t: torch.Tensor, what: str) -> int:
 
 # ------------------------------------------------------------------------------ row ops
 
-def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
-    """out[r, :] = float(table[tokens[r], :]); a negative token gives a zero row."""
+TOKEN_FROM_FEEDBACK = -2     # a token id that means: take this row's token from ``feedback``
+
+
+def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, feedback: Optional[torch.Tensor] = None) -> None:
+    """out[r, :] = float(table[tokens[r], :]); a negative token gives a zero row, except TOKEN_FROM_FEEDBACK,
+    which reads the row's token from ``feedback`` (int32, a row each) if that is given."""
     _need(tokens, torch.int32, "tokens")
     _need(out, torch.float32, "out")
     rows = tokens.numel()
@@ -131,8 +135,12 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
         raise ValueError("embedding table must be a contiguous GPU tensor")
     if out.shape[0] < rows or out.shape[1] != width:
         raise ValueError(f"embed: out {tuple(out.shape)} does not fit {rows} rows of width {width}")
-    _check(_fn("bw_embed")(tokens.data_ptr(), table.data_ptr(), _is_bf16(table, "table"), out.data_ptr(), rows, width,
-                           vocab, _stream()), "embed")
+    if feedback is not None:
+        _need(feedback, torch.int32, "feedback")
+        if feedback.numel() < rows:
+            raise ValueError("embed: feedback is shorter than the rows")
+    _check(_fn("bw_embed")(tokens.data_ptr(), None if feedback is None else feedback.data_ptr(), table.data_ptr(),
+                           _is_bf16(table, "table"), out.data_ptr(), rows, width, vocab, _stream()), "embed")
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, rows: int, eps: float) -> None:

@@ -15,12 +15,53 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence as Seq
 
 import numpy as np
+import torch
 
 from ..cache.manager import CacheManager, GroupSpec
 from ..config.engine import EngineConfig, SamplingParams
+from ..csrc import ops
 from ..sampling.rng import FINGERPRINT_BASIS
 from .batch import Segment
 from .scheduler import Scheduler, Sequence, Work
+
+AHEAD_TOKEN = -2       # the token id of a row whose token the step before is still choosing (ops.TOKEN_FROM_FEEDBACK)
+
+
+class _Pending:
+    """A step that has been launched: what it will leave in pinned host memory once its event has passed."""
+
+    def __init__(self, n: int, event, tokens_host, prints_host, graph_rows: int):
+        self.n, self.event, self.tokens_host, self.prints_host, self.graph_rows = n, event, tokens_host, prints_host, graph_rows
+        self.prints_dev = None
+
+    def result(self):
+        """(tokens, fingerprints or []) of the sampled rows; waits for the device."""
+        if self.n == 0:
+            return [], []
+        self.event.synchronize()
+        tokens = self.tokens_host[:self.n].tolist()
+        prints = self.prints_host[:self.n].numpy().view(np.uint64).tolist() if self.prints_host is not None else []
+        return tokens, prints
+
+
+class _Done:
+    """The same face for an executor that computes at once (the stand-in device of the scheduler's tests)."""
+
+    def __init__(self, tokens, prints):
+        self._r = (tokens, prints)
+        self.n = len(tokens)
+
+    def result(self):
+        return self._r
+
+
+@dataclass
+class _Flight:
+    """One step between its launch and its bookkeeping."""
+    plan: List[Work]
+    sampled: List[Work]
+    pending: object
+    t0: float
 
 
 @dataclass
@@ -77,6 +118,13 @@ class GpuExecutor:
         self.runner = ModelRunner(asm, self.storage, self.max_model_len, max_rows=config.max_batched_tokens,
                                   max_logit_rows=max_logit_rows, use_graphs=config.use_graphs)
         self.sampler = Sampler(rt.device, max_logit_rows)
+        # two steps may be under way at a time (one being read back, one launched ahead): two sets of buffers
+        self._flip = 0
+        self._events = [torch.cuda.Event(), torch.cuda.Event()]
+        self._tokens_host = [torch.zeros(max_logit_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._prints_host = [torch.zeros(max_logit_rows, dtype=torch.int64, pin_memory=True) for _ in range(2)]
+        self._prints_dev = [torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device) for _ in range(2)]
+        self._prints_in = torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device)
         self.group_specs = [GroupSpec(g.window) for g in asm.group_specs]
         self.has_state = bool(asm.state_specs)
         self.vocab_size = asm.spec.vocab_size
@@ -85,25 +133,44 @@ class GpuExecutor:
     def reset_slot(self, slot: int) -> None:
         self.storage.reset_slot(slot)
 
-    fused_sampling = True      # run() takes the sampling parameters and may sample inside the step
+    # ------------------------------------------------------------------ one step, launched and read back apart
+    def launch(self, segments: Seq[Segment], draw, previous_prints, after: "Optional[_Pending]" = None) -> "_Pending":
+        """Run a batch and everything behind it on the device without waiting for any of it: the model,
+        the choice of tokens for the rows that end their request's known tokens, their logits fingerprints,
+        and the copies of tokens and fingerprints to pinned host memory.  ``draw`` = (temperatures, seeds,
+        positions) of those rows.  ``previous_prints``: their fingerprints so far (host integers), or None
+        to chain them from ``after``, the step launched just before for the same rows in the same order
+        (whose tokens this step also takes on the device)."""
+        temps, seeds, positions = draw
+        n = len(temps)
+        sampling = (np.asarray(temps, np.float32), self.sampler.uniforms(temps, seeds, positions)) if n else None
+        logits = self.runner.step(segments, sampling)
+        slot = self._flip
+        self._flip ^= 1
+        pend = _Pending(n, self._events[slot], self._tokens_host[slot], None, self.runner.last_graph_rows)
+        if n:
+            sampled = self.runner.last_sampled
+            if sampled is None:
+                sampled = self.sampler.sample_on_device(logits, temps, sampling[1])
+            pend.tokens_host[:n].copy_(sampled[:n], non_blocking=True)
+            if previous_prints is not None or after is not None:
+                h_in = self._prints_in
+                if previous_prints is not None:
+                    h_in[:n].copy_(torch.from_numpy(np.asarray(previous_prints, np.uint64).view(np.int64)))
+                else:
+                    h_in = after.prints_dev
+                pend.prints_dev = self._prints_dev[slot]
+                ops.fingerprint(logits, n, h_in, pend.prints_dev)
+                pend.prints_host = self._prints_host[slot]
+                pend.prints_host[:n].copy_(pend.prints_dev[:n], non_blocking=True)
+            pend.event.record()
+        return pend
 
-    def run(self, segments: Seq[Segment], sampling=None):
-        """``sampling`` = (temperatures, seeds, positions) of the rows that will be sampled."""
-        if sampling is not None:
-            temps, seeds, positions = sampling
-            sampling = (np.asarray(temps, np.float32), self.sampler.uniforms(temps, seeds, positions))
-        return self.runner.step(segments, sampling)
-
-    def sample(self, logits, temperatures, seeds, positions) -> List[int]:
-        done = self.runner.last_sampled
-        if done is not None and done.numel() == len(temperatures):      # the step's graph has sampled already
-            self.runner.last_sampled = None
-            return done.cpu().tolist()
-        return self.sampler.sample(logits, temperatures, seeds, positions)
-
-    def fingerprints(self, logits, previous) -> List[int]:
-        return self.sampler.fingerprints(logits, previous)
-
+    def can_run_ahead(self, pend: "_Pending", rows: int) -> bool:
+        """Whether the next decode step of the same ``rows`` requests may be launched before this one's
+        tokens are read: it was replayed from a graph that sampled them (the next replay of that graph finds
+        them on the device) and no mixer keeps state that a step thrown away would have advanced."""
+        return pend.graph_rows == rows and pend.n == rows and not self.has_state
 
 class Engine:
     def __init__(self, target, draft=None, config: Optional[EngineConfig] = None, executor=None):
@@ -123,6 +190,7 @@ class Engine:
         self._next_id = 0
         self._stats = EngineStats()
         self._start = time.perf_counter()
+        self._ahead: Optional[_Flight] = None       # a step launched before the one before it was read back
 
     # ------------------------------------------------------------------ interface
     def now(self) -> float:
@@ -154,7 +222,7 @@ class Engine:
         self._finish(seq, cancelled=True)
 
     def idle(self) -> bool:
-        return self.sched.idle()
+        return self.sched.idle() and (self._ahead is None or all(w.seq.done for w in self._ahead.plan))
 
     @property
     def num_running(self) -> int:
@@ -191,8 +259,25 @@ class Engine:
 
     # ------------------------------------------------------------------ one step
     def step(self) -> List[StepEvent]:
+        """One step's tokens.  The step is planned and launched here unless the call before launched it
+        ahead; before its tokens are waited for, the next step is launched ahead if it can only be one more
+        token for each of the same requests (src/engine.cpp:304-488 is the synchronous form of this)."""
         events: List[StepEvent] = []
         self._stats.steps += 1
+        flight, self._ahead = self._ahead, None
+        if flight is not None and all(w.seq.done for w in flight.plan):
+            flight = None                          # everyone in it has ended or was cancelled meanwhile
+        if flight is None:
+            flight = self._launch_planned()
+            if flight is None:
+                return events
+        ahead = self._launch_ahead(flight)
+        self._complete(flight, events)
+        if ahead is not None and any(not w.seq.done for w in ahead.sampled):
+            self._ahead = ahead
+        return events
+
+    def _launch_planned(self) -> Optional[_Flight]:
         plan = self.sched.plan()
         for sid in self.sched.preempted_ids:
             self._results[sid].preemptions += 1
@@ -201,8 +286,7 @@ class Engine:
         for sid, hit in self.sched.prefix_hits.items():
             self._results[sid].prefix_cached_tokens += hit
         if not plan:
-            return events
-
+            return None
         segments: List[Segment] = []
         sampled: List[Work] = []
         for w in plan:
@@ -216,30 +300,69 @@ class Engine:
                 self._stats.decode_rows += 1
             else:
                 self._stats.prefill_tokens += w.n
-        t0 = self.now()
         # a draw is keyed by what the request's slot records: its seed, and its position once this step's
         # tokens are in the cache (the number of tokens it holds before the new one, src/engine.cpp:473)
         records = [self.manager.record(w.seq.cache) for w in sampled]
         draw = ([w.seq.params.temperature for w in sampled], [r.seed for r in records],
                 [r.position + w.n for r, w in zip(records, sampled)])
-        if sampled and getattr(self.exec, "fused_sampling", False):
-            logits = self.exec.run(segments, draw)
-        else:
-            logits = self.exec.run(segments)
-        new_tokens: List[int] = []
-        prints: List[int] = []
-        if sampled:
-            new_tokens = self.exec.sample(logits, *draw)
-            if self.cfg.fingerprint_logits:
-                prints = self.exec.fingerprints(logits, [self._results[w.seq.id].logits_fingerprint for w in sampled])
-        self._stats.forward_seconds += self.now() - t0
+        prints = [self._results[w.seq.id].logits_fingerprint for w in sampled] if self.cfg.fingerprint_logits else None
+        t0 = self.now()
+        return _Flight(plan, sampled, self._exec_launch(segments, draw, prints), t0)
 
+    def _exec_launch(self, segments, draw, prints):
+        if hasattr(self.exec, "launch"):
+            return self.exec.launch(segments, draw, prints)
+        logits = self.exec.run(segments)                       # an executor that computes at once
+        tokens = self.exec.sample(logits, *draw) if draw[0] else []
+        return _Done(tokens, self.exec.fingerprints(logits, prints) if prints is not None and draw[0] else [])
+
+    def _launch_ahead(self, flight: _Flight) -> Optional[_Flight]:
+        """The step after ``flight``, launched before ``flight``'s tokens are known, if it is certain what it
+        is up to the tokens themselves: ``flight`` decodes one token for every running request, nobody
+        waits, nobody reaches its length, and every request gets its next page without taking one from
+        another.  A request that turns out to have ended with ``flight``'s token (end of sequence, a
+        cancellation) has its row of this step thrown away; the other rows do not depend on it."""
+        cfg, ex = self.cfg, self.exec
+        running = self.sched.running
+        if not (cfg.run_ahead and getattr(ex, "can_run_ahead", None) and not self.sched.waiting):
+            return None
+        if len(flight.plan) != len(running) or len(flight.sampled) != len(running):
+            return None
+        if not all(w.n == 1 and w.seq is s for w, s in zip(flight.plan, running)):
+            return None
+        if not ex.can_run_ahead(flight.pending, len(running)):
+            return None
+        for s in running:
+            if s.generated() + 2 > s.params.max_new_tokens or len(s.tokens) + 2 > ex.max_model_len:
+                return None                 # it ends with this step's token, or with the next: the plain path
+        if sum(self.manager.pages_missing(s.cache, len(s.tokens) + 1) for s in running) > self.manager.free_pages_least():
+            return None
+        for s in running:
+            if not self.manager.ensure(s.cache, len(s.tokens) + 1):
+                return None                 # (pages taken so far stay with their requests)
+        plan = [Work(s, 1, len(s.tokens)) for s in running]
+        segments = [Segment([AHEAD_TOKEN], len(s.tokens), s.cache.tables, s.cache.slot, [0]) for s in running]
+        records = [self.manager.record(s.cache) for s in running]
+        draw = ([s.params.temperature for s in running], [r.seed for r in records], [len(s.tokens) + 1 for s in running])
+        t0 = self.now()
+        pending = ex.launch(segments, draw, None, after=flight.pending if cfg.fingerprint_logits else None)
+        self._stats.decode_rows += len(running)
+        return _Flight(plan, list(plan), pending, t0)
+
+    def _complete(self, flight: _Flight, events: List[StepEvent]) -> None:
+        new_tokens, prints = flight.pending.result()
+        self._stats.forward_seconds += self.now() - flight.t0
         cursor = 0
         finished: List[Sequence] = []
-        for w in plan:
+        chosen = {id(w) for w in flight.sampled}
+        for w in flight.plan:
             s = w.seq
+            last = id(w) in chosen
+            if s.done:                                 # ended or cancelled since the launch: the row is thrown away
+                cursor += 1 if last else 0
+                continue
             self.sched.commit(w)
-            if w.start + w.n == len(s.tokens):
+            if last:
                 token = new_tokens[cursor]
                 if prints:
                     self._results[s.id].logits_fingerprint = prints[cursor]
@@ -250,7 +373,6 @@ class Engine:
             self._finish(s, cancelled=False)
             self._seqs.pop(s.id, None)
         self._stats.evictions = self.manager.evictions
-        return events
 
     # ------------------------------------------------------------------ bookkeeping
     def _append(self, s: Sequence, token: int, events: List[StepEvent]) -> bool:

@@ -60,6 +60,9 @@ class _StaticDecodeContext:
         self._host_temps = self._host_np[off_temp:off_temp + size].view(np.float32)
         self._host_unis = self._host_np[off_uni:off_uni + 2 * size].view(np.float64)
         self.sampled = torch.zeros(size, dtype=torch.int32, device=device)
+        # a row whose token id is TOKEN_FROM_FEEDBACK takes the token this graph's last replay sampled for the
+        # row: the next step of the same requests in the same order can be launched before the host has the tokens
+        self.token_feedback = self.sampled
         self.row_seq = torch.arange(size, dtype=torch.int32, device=device)
         self.want_rows = torch.arange(size, dtype=torch.int32, device=device)
         self.segments: List[Segment] = []
@@ -127,6 +130,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs: Dict[int, tuple] = {}
         self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
+        self.last_graph_rows = 0      # requests of the last step if it was replayed from a graph, else 0
 
     # ------------------------------------------------------------------ the step function
     def step(self, segments: Sequence[Segment], sampling=None) -> Optional[torch.Tensor]:
@@ -137,6 +141,7 @@ class ModelRunner:
         from a graph then also samples inside the graph (the same kernel a separate call
         would run) and leaves the tokens in ``last_sampled``; any other step leaves None there."""
         self.last_sampled = None
+        self.last_graph_rows = 0
         if not segments:
             return None
         rows = sum(len(s.tokens) for s in segments)
@@ -176,6 +181,7 @@ class ModelRunner:
         graph.replay()
         if sampling is not None:
             self.last_sampled = ctx.sampled[:n]
+        self.last_graph_rows = n
         return logits[:n]
 
     def _capture(self, bucket: int):

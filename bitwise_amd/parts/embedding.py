@@ -33,7 +33,8 @@ class TokenEmbedding(Embedding):
 
     def forward(self, ctx) -> torch.Tensor:
         x = ctx.ws.buffer("residual", self.width, torch.float32)
-        ops.embed(ctx.tokens[:ctx.rows], self.weight, x)
+        # (a step launched ahead of its tokens names them by the step before: ``ctx.token_feedback``)
+        ops.embed(ctx.tokens[:ctx.rows], self.weight, x, getattr(ctx, "token_feedback", None))
         return x
 
 

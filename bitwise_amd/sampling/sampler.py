@@ -34,12 +34,17 @@ class Sampler:
             return []
         if rows > self.max_rows or logits.shape[0] < rows:
             raise ValueError("more rows to sample than the sampler was made for")
-        temps = np.asarray(temperatures, np.float32)
-        unis = self.uniforms(temperatures, seeds, positions)
-        self._temp[:rows].copy_(torch.from_numpy(temps))
-        self._uni[:rows].copy_(torch.from_numpy(unis))
+        return self.sample_on_device(logits, temperatures, self.uniforms(temperatures, seeds, positions)).cpu().tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: np.ndarray) -> torch.Tensor:
+        """The tokens as a device tensor (a view of the sampler's buffer, valid until its next call)."""
+        rows = len(temperatures)
+        if rows > self.max_rows or logits.shape[0] < rows:
+            raise ValueError("more rows to sample than the sampler was made for")
+        self._temp[:rows].copy_(torch.from_numpy(np.asarray(temperatures, np.float32)))
+        self._uni[:rows].copy_(torch.from_numpy(np.asarray(uniforms, np.float64)))
         ops.sample(logits, rows, self._temp, self._uni, self._out)
-        return self._out[:rows].cpu().tolist()
+        return self._out[:rows]
 
     @staticmethod
     def uniforms(temperatures: Sequence[float], seeds: Sequence[int], positions: Sequence[int]) -> np.ndarray:

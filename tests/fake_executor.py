@@ -19,8 +19,39 @@ def _mix(z: int) -> int:
     return z ^ (z >> 31)
 
 
+AHEAD_TOKEN = -2
+
+
+class _LazyStep:
+    """A launched step of the stand-in device: evaluated when its result is asked for, which the engine does
+    in launch order, so reads and writes of the pages happen in the order a device stream would give them."""
+
+    def __init__(self, ex, segments, draw, prints, after):
+        self.ex, self.segments, self.draw, self.prints, self.after = ex, segments, draw, prints, after
+        self.n = len(draw[0])
+        self.decode_rows = len(segments) if all(len(s.tokens) == 1 and tuple(s.want) == (0,) for s in segments) else 0
+        self._r = None
+
+    def result(self):
+        if self._r is None:
+            segs = self.segments
+            prev = self.prints
+            if self.after is not None:
+                toks, prev_prints = self.after.result()
+                assert len(toks) == len(segs)
+                segs = [type(s)([toks[i]] if s.tokens[0] == AHEAD_TOKEN else s.tokens, s.pos0, s.tables, s.slot, s.want)
+                        for i, s in enumerate(segs)]
+                prev = prev_prints if prev_prints else None
+            assert all(t >= 0 for s in segs for t in s.tokens), "a step ahead of its tokens without the step before"
+            logits = self.ex.run(segs)
+            tokens = self.ex.sample(logits, *self.draw) if self.n else []
+            self._r = (tokens, self.ex.fingerprints(logits, prev) if prev is not None and self.n else [])
+        return self._r
+
+
 class FakeExecutor:
-    def __init__(self, page_size: int, vocab_size: int = 97, eos_token_id: int = 3, max_model_len: int = 1 << 20):
+    def __init__(self, page_size: int, vocab_size: int = 97, eos_token_id: int = 3, max_model_len: int = 1 << 20,
+                 run_ahead: bool = False):
         self.group_specs = [GroupSpec()]
         self.has_state = False
         self.vocab_size = vocab_size
@@ -31,9 +62,18 @@ class FakeExecutor:
         self.steps = 0
         self.rows_run = 0
         self.reset_slots: List[int] = []
+        self.steps_ahead = 0
+        if run_ahead:        # the device's two-part face: launch now, read back later; a step may be launched ahead
+            self.launch = self._launch
+            self.can_run_ahead = lambda pend, rows: pend.decode_rows == rows and pend.n == rows
 
     def reset_slot(self, slot: int) -> None:
         self.reset_slots.append(slot)
+
+    def _launch(self, segments, draw, prints, after=None):
+        if after is not None:
+            self.steps_ahead += 1
+        return _LazyStep(self, segments, draw, prints, after)
 
     def run(self, segments):
         self.steps += 1

@@ -11,8 +11,8 @@ from bitwise_amd.engine.engine import Engine
 from fake_executor import FakeExecutor
 
 
-def run_all(cfg, prompts, params, arrivals=None, cancels=None, guard=20000):
-    ex = FakeExecutor(cfg.block_size)
+def run_all(cfg, prompts, params, arrivals=None, cancels=None, guard=20000, run_ahead=False):
+    ex = FakeExecutor(cfg.block_size, run_ahead=run_ahead)
     eng = Engine(None, None, cfg, executor=ex)
     ids = [None] * len(prompts)
     arrivals = arrivals or [0] * len(prompts)
@@ -174,8 +174,9 @@ def test_cancel_gives_everything_back():
     assert eng.manager.slots.available() == cfg.max_num_seqs
 
 
+@pytest.mark.parametrize("run_ahead", [False, True])
 @pytest.mark.parametrize("seed", range(40))
-def test_random_traces_equal_solo(seed):
+def test_random_traces_equal_solo(seed, run_ahead):
     """The reference's simulator on the CPU (sim/simulate.cpp:120-210): random requests with
     shared and repeated prompts, staggered arrivals, cancellations, tight pools and small
     budgets; every request that was not cancelled must equal its solo run."""
@@ -202,7 +203,7 @@ def test_random_traces_equal_solo(seed):
     cfg = EngineConfig(block_size=ps, max_batched_tokens=rng.randint(4, 64), max_num_seqs=rng.randint(1, 8),
                        prefix_caching=rng.random() < 0.7)
     cfg.num_blocks = (max_need + 1 + ps - 1) // ps + rng.randint(0, 12)
-    eng, ex, results = run_all(cfg, prompts, params, arrivals, cancels)
+    eng, ex, results = run_all(cfg, prompts, params, arrivals, cancels, run_ahead=run_ahead)
     assert eng.free_blocks == cfg.num_blocks, "leaked pages"
     assert eng.manager.slots.available() == cfg.max_num_seqs
     for p, sp, r in zip(prompts, params, results):
@@ -211,6 +212,36 @@ def test_random_traces_equal_solo(seed):
         ref = solo(cfg, p, sp)
         assert r.tokens == ref.tokens
         assert r.logits_fingerprint == ref.logits_fingerprint
+
+
+def test_steps_are_launched_ahead_and_thrown_away_rows_do_no_harm():
+    """Decode steps of an unchanged set of requests are launched before the tokens of the step before are read.
+    A request that ends by its end-of-sequence token has had one more row launched: it is thrown away, its
+    stale write lands in a page that may already belong to a newcomer, and nobody's tokens change."""
+    cfg = EngineConfig(num_blocks=12, block_size=8, max_batched_tokens=32, max_num_seqs=3, prefix_caching=True)
+    prompts = [[5, 6, 7, 8, 9], [11, 12, 13], [21, 22, 23, 24, 25, 26, 27, 28, 29], [40, 41], [50, 51, 52, 53]]
+    params = [SamplingParams(max_new_tokens=40), SamplingParams(max_new_tokens=40, temperature=0.9, seed=4),
+              SamplingParams(max_new_tokens=30, ignore_eos=True), SamplingParams(max_new_tokens=25),
+              SamplingParams(max_new_tokens=12, ignore_eos=True)]
+    total_ahead = 0
+    for vocab in (5, 13, 97):               # small vocabularies: the end-of-sequence token (3) comes early and often
+        def run(run_ahead):
+            ex = FakeExecutor(cfg.block_size, vocab_size=vocab, run_ahead=run_ahead)
+            eng = Engine(None, None, cfg, executor=ex)
+            ids = [eng.add_request([t % vocab for t in p], sp) for p, sp in zip(prompts, params)]
+            for _ in range(2000):
+                if eng.idle():
+                    break
+                eng.step()
+                eng.manager.check()
+            assert eng.idle() and eng.free_blocks == cfg.num_blocks and eng.manager.slots.available() == cfg.max_num_seqs
+            return ex, [(eng.result(i).tokens, eng.result(i).logits_fingerprint) for i in ids]
+        ex_plain, plain = run(False)
+        ex_ahead, ahead = run(True)
+        assert ahead == plain
+        assert ex_plain.steps_ahead == 0
+        total_ahead += ex_ahead.steps_ahead
+    assert total_ahead > 20
 
 
 def test_random_traces_do_exercise_preemption_and_prefix_hits():
@@ -271,7 +302,7 @@ def test_injected_faults_are_caught(fault, monkeypatch):
     caught = 0
     for seed in range(30):
         try:
-            test_random_traces_equal_solo(seed)
+            test_random_traces_equal_solo(seed, seed % 2 == 1)
             prompts, params = shared_prefix_workload()
             cfg = EngineConfig(max_batched_tokens=24, num_blocks=40)
             aligned = [[(i * 7 + seed) % 97 for i in range(32)]] * 2      # a repeated prompt that fills its pages
