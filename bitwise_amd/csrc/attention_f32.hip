@@ -5,8 +5,9 @@
 //   out[d] = acc[d] * (1/sum).
 // dot_canonical is the 16-chain split with the fixed tree (src/kernels.cpp:57-64, :86-101).
 // lo is 0, or p-window+1 for a windowed cache.  A workgroup of 256 threads per (row, head): in pass 1 each
-// thread takes keys j = lo+t, lo+t+256, ...; in pass 2 the threads recompute the scores of a chunk of keys
-// (the same deterministic function, so the same bits), park e_j and the keys' value rows in LDS, and then
+// thread takes keys j = lo+t, lo+t+256, ... and leaves their scores in LDS, where they become e_j once the
+// maximum is known (contexts whose scores do not fit LDS recompute the scores of a chunk of keys in pass 2: the
+// same deterministic function, so the same bits); in pass 2 the keys' value rows come into LDS a chunk at a time and
 // thread d walks the chunk in key order for its own d.  The same code runs for a row of a prompt portion and
 // for a decoded token, so the bits cannot differ.
 #include "common.h"
@@ -107,11 +108,16 @@ __device__ __forceinline__ void walk_chunk(const float* __restrict__ ed, const f
   }
 }
 
-template <int HD>
+// KEEP: the scores of pass 1 stay in LDS (``capacity`` of them: as many keys as a row of the block table, or the
+// window, can hold), turn into e_j there once the maximum is known, and pass 2 fetches values only: the keys are
+// read once and every dot product is computed once.  The e_j are the same function of the same numbers, so the bits
+// are those of the two-pass form, which remains for contexts whose scores do not fit.
+template <int HD, bool KEEP>
 __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Args a) {
   using S = Att32Shape<HD>;
   constexpr int T = S::T, KC = S::KC, SEGS = S::SEGS, VJ = S::VJ;
-  extern __shared__ __attribute__((aligned(16))) float v_lds[];    // [2][KC][HD]: value rows of a chunk of keys
+  extern __shared__ __attribute__((aligned(16))) float v_lds[];    // [2][KC][HD]: value rows of a chunk of keys; KEEP: then the scores
+  float* scores = v_lds + 2 * KC * HD;
   __shared__ float q_lds[HD];
   __shared__ float e_lds[2][KC];
   __shared__ float red[T / 64];
@@ -151,9 +157,15 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
     load_row<HD>(ka, a.k_cache + offset_of(j));
     for (; j <= pos; j += 2 * T) {
       load_row<HD>(kb, a.k_cache + offset_of(j + T));
-      mx = fmaxf(mx, dot_canonical<HD>(q_lds, ka) * a.scale);
+      const float s0 = dot_canonical<HD>(q_lds, ka) * a.scale;
+      if constexpr (KEEP) scores[j - lo] = s0;
+      mx = fmaxf(mx, s0);
       load_row<HD>(ka, a.k_cache + offset_of(j + 2 * T));
-      if (j + T <= pos) mx = fmaxf(mx, dot_canonical<HD>(q_lds, kb) * a.scale);
+      if (j + T <= pos) {
+        const float s1 = dot_canonical<HD>(q_lds, kb) * a.scale;
+        if constexpr (KEEP) scores[j + T - lo] = s1;
+        mx = fmaxf(mx, s1);
+      }
     }
   }
   mx = wave_max(mx);
@@ -186,43 +198,94 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
   const int et = tid - (T - KC);                           // this thread's key within a chunk, if not negative
   KeyRow<HD> krow;
   auto park = [&](int j0, int buf) {                       // ``krow`` holds key j0 + et; afterwards key j0 + KC + et
-    if (et < 0) return;
+    if (KEEP || et < 0) return;
     const int j = j0 + et;
     const float e = bw_expf(dot_canonical<HD>(q_lds, krow) * a.scale - mx);
     load_row<HD>(krow, a.k_cache + offset_of(j + KC));
     e_lds[buf][et] = j <= pos ? e : 0.0f;
   };
   float acc = 0.0f, sum = 0.0f;
-  if (et >= 0) load_row<HD>(krow, a.k_cache + offset_of(lo + et));
-  fetch(lo);
-  park(lo, 0);
-  stash(0);
-  __syncthreads();
-  int buf = 0;
-  for (int j0 = lo; j0 <= pos; j0 += KC) {
-    const bool more = j0 + KC <= pos;
-    if (more) {
-      fetch(j0 + KC);
-      park(j0 + KC, buf ^ 1);
-    }
-    if (tid < HD) {
-      const int cnt = (pos - j0 + 1) < KC ? (pos - j0 + 1) : KC;
-      const float* vd = v_lds + buf * KC * HD + tid;
-      const float* ed = e_lds[buf];
-      if (cnt == KC) {
-        walk_chunk<HD>(ed, vd, sum, acc);
-      } else {
+  auto walk = [&](int j0, int buf) {                       // thread d < HD: keys j0 .. of the chunk in ``buf``, in key order
+    if (tid >= HD) return;
+    const int cnt = (pos - j0 + 1) < KC ? (pos - j0 + 1) : KC;
+    const float* vd = v_lds + buf * KC * HD + tid;
+    const float* ed = KEEP ? scores + (j0 - lo) : e_lds[buf];
+    if (cnt == KC) {
+      walk_chunk<HD>(ed, vd, sum, acc);
+    } else {
 #pragma unroll 8
-        for (int jj = 0; jj < cnt; ++jj) {
-          const float ej = ed[jj];
-          sum += ej;
-          acc = fmaf(ej, vd[jj * HD], acc);
-        }
+      for (int jj = 0; jj < cnt; ++jj) {
+        const float ej = ed[jj];
+        sum += ej;
+        acc = fmaf(ej, vd[jj * HD], acc);
       }
     }
-    if (more) stash(buf ^ 1);
+  };
+  if constexpr (KEEP) {
+    // Values only.  Three chunks of them are on their way at any time (three sets of registers in turn; a chunk in
+    // flight is what keeps a compute unit's share of the memory system busy across a trip to memory), the first
+    // three asked for before the scores turn into e_j.  Chunks past the last key fetch the last key again.
+    f32x4 r0[VJ], r1[VJ], r2[VJ];
+    auto fetch_into = [&](f32x4 (&reg)[VJ], int j0) {
+#pragma unroll
+      for (int i = 0; i < VJ; ++i) {
+        const int c = tid + T * i;
+        const int cc = c < KC * SEGS ? c : KC * SEGS - 1;
+        reg[i] = *reinterpret_cast<const f32x4*>(a.v_cache + offset_of(j0 + cc / SEGS) + 4 * (cc % SEGS));
+      }
+    };
+    auto stash_from = [&](int buf, const f32x4 (&reg)[VJ]) {
+#pragma unroll
+      for (int i = 0; i < VJ; ++i) {
+        const int c = tid + T * i;
+        if (c < KC * SEGS) *reinterpret_cast<f32x4*>(v_lds + buf * KC * HD + 4 * c) = reg[i];
+      }
+    };
+    fetch_into(r0, lo);
+    fetch_into(r1, lo + KC);
+    fetch_into(r2, lo + 2 * KC);
+    // every thread turns the scores it wrote itself into e_j; the barrier behind the first chunk's values publishes them
+    for (int j = lo + tid; j <= pos; j += T) scores[j - lo] = bw_expf(scores[j - lo] - mx);
+    stash_from(0, r0);
     __syncthreads();
-    buf ^= 1;
+    int buf = 0;
+    for (int j0 = lo; j0 <= pos; j0 += 3 * KC) {           // (pos is the same for the whole workgroup: so are the exits)
+      fetch_into(r0, j0 + 3 * KC);
+      walk(j0, buf);
+      stash_from(buf ^ 1, r1);
+      __syncthreads();
+      buf ^= 1;
+      if (j0 + KC > pos) break;
+      fetch_into(r1, j0 + 4 * KC);
+      walk(j0 + KC, buf);
+      stash_from(buf ^ 1, r2);
+      __syncthreads();
+      buf ^= 1;
+      if (j0 + 2 * KC > pos) break;
+      fetch_into(r2, j0 + 5 * KC);
+      walk(j0 + 2 * KC, buf);
+      stash_from(buf ^ 1, r0);
+      __syncthreads();
+      buf ^= 1;
+    }
+  } else {
+    if (et >= 0) load_row<HD>(krow, a.k_cache + offset_of(lo + et));
+    fetch(lo);
+    park(lo, 0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int j0 = lo; j0 <= pos; j0 += KC) {
+      const bool more = j0 + KC <= pos;
+      if (more) {
+        fetch(j0 + KC);
+        park(j0 + KC, buf ^ 1);
+      }
+      walk(j0, buf);
+      if (more) stash(buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
+    }
   }
   if (tid < HD) a.out[(size_t)row * a.out_stride + (size_t)h * HD + tid] = acc * (1.0f / sum);
 }
@@ -393,15 +456,26 @@ static void launch_attention_f32_tiles(const AttnF32Args& a, dim3 grid, hipStrea
   hipLaunchKernelGGL(attention_f32_tile_kernel<HD>, grid, dim3(ATT32_THREADS), Att32Tile<HD>::LDS_BYTES, s, a);
 }
 
+#define ATT32_KEEP_LDS (144 * 1024)     // dynamic LDS of the kernel that keeps its scores: the values' chunks and the scores
+
 template <int HD>
 static void launch_attention_f32(const AttnF32Args& a, dim3 grid, hipStream_t s) {
-  static bool allowed = false;                         // 64 KB of dynamic LDS has to be asked for once
+  static bool allowed = false;                         // 64 KB of dynamic LDS and more has to be asked for once
   if (!allowed) {
-    (void)hipFuncSetAttribute((const void*)attention_f32_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    (void)hipFuncSetAttribute((const void*)attention_f32_kernel<HD, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               Att32Shape<HD>::LDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)attention_f32_kernel<HD, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              ATT32_KEEP_LDS);
     allowed = true;
   }
-  hipLaunchKernelGGL(attention_f32_kernel<HD>, grid, dim3(ATT32_THREADS), Att32Shape<HD>::LDS_BYTES, s, a);
+  // the most keys a query of this launch can see: what a row of the block table covers, or the window
+  long long capacity = (long long)a.table_stride * a.page_size;
+  if (a.window > 0 && a.window < capacity) capacity = a.window;
+  const long long keep_bytes = Att32Shape<HD>::LDS_BYTES + ((capacity + 3) & ~3ll) * (long long)sizeof(float);
+  if (keep_bytes <= ATT32_KEEP_LDS)
+    hipLaunchKernelGGL((attention_f32_kernel<HD, true>), grid, dim3(ATT32_THREADS), (size_t)keep_bytes, s, a);
+  else
+    hipLaunchKernelGGL((attention_f32_kernel<HD, false>), grid, dim3(ATT32_THREADS), Att32Shape<HD>::LDS_BYTES, s, a);
 }
 
 static int attention_f32_dispatch(const AttnF32Args& a, int items, int tiled, hipStream_t s) {
