@@ -333,6 +333,364 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
   }
 }
 
+// ------------------------------------------------------------------------------ up to 64 rows on the matrix cores
+
+// v_mfma_f32_4x4x1_16b_f32 computes, for 16 blocks of 4 x 4 outputs at once, D[r][j] = fma(A[r], B[j], D[r][j]):
+// one step of k, a true 32-bit fused multiply-add with a single rounding (denormal numbers, infinities and all;
+// the tests hold it against std::fma bit for bit).  A chain of them over k ascending from a zero accumulator is
+// therefore the scalar chain of the definition, and it needs one element of x and one of W a lane and step where
+// the vector unit needs one of each per output: the operands' way through LDS no longer bounds the product.
+//
+// A wave owns 4 * CG columns and up to 16 rows (MR such blocks of rows for up to 64): block (rg, cg) of the
+// instruction is rows 4 rg .. 4 rg + 3 of x against columns 4 cg .. 4 cg + 3 of the wave's, RG row groups times
+// CG = 16 / RG column groups; the blocks of a row group share their A operand (the instruction broadcasts it from
+// the group's first block).  Lane (block, i) holds row 4 rg + i of x as A, column 4 cg + i of W as B, and the
+// outputs of rows 4 rg .. 4 rg + 3 at its column.  Both operands stream through a ring in LDS that is the wave's
+// own (buffer loads with LDS as destination, in whole 128-byte or 256-byte runs, the 16-byte chunks of a row
+// permuted so that operand reads hit distinct banks; bfloat16 weights are widened when they are read).  Nothing is
+// shared between waves, so the loop has no barrier; loads complete in issue order and every stage has the same
+// number of them (stages past K are asked for outside the descriptors: zeros, no traffic), so "all but the last
+// PENDING loads have landed" is the wait for the stage at hand.  K a multiple of 64.
+template <typename WT, int RG, int MR>
+struct F32MShape {
+  static constexpr int CG = 16 / RG, NCW = 4 * CG;                  // column groups, columns a wave
+  static constexpr int CBSZ = RG == 1 ? 4 : (RG == 2 ? 3 : 2);      // log2 of the blocks that share an A operand
+  static constexpr int XROWS = 4 * RG * MR;                         // rows of x a stage holds
+  static constexpr int WROW = 64 * (int)sizeof(WT);                 // bytes of a row of W a stage (64 steps of k)
+  static constexpr int X_LOADS = XROWS / 4, W_LOADS = NCW * WROW / 1024;   // 1 KB an instruction
+  static constexpr int LPW = X_LOADS + W_LOADS;
+  static constexpr int XBYTES = XROWS * 256, STAGE = XBYTES + NCW * WROW;
+  static constexpr int BY_COUNT = 63 / LPW + 2, BY_ROOM = 65536 / STAGE;
+  static constexpr int STAGES = BY_COUNT < BY_ROOM ? (BY_COUNT < 12 ? BY_COUNT : 12) : (BY_ROOM < 12 ? BY_ROOM : 12);
+  static constexpr int PENDING = LPW * (STAGES - 2);
+  static_assert(STAGES >= 3 && PENDING < 64, "the ring needs three stages and the wait count has six bits");
+  static_assert(MR == 1 || RG == 4, "more than 16 rows: blocks of 16");
+};
+
+template <typename WT, int RG, int MR>
+__device__ __forceinline__ void f32m_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
+                                           const int* voff_x, const int* voff_w, int step, int steps) {
+  using S = F32MShape<WT, RG, MR>;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = ring + (step % S::STAGES) * S::STAGE;
+  const bool real = step < steps;                                  // scalar
+#pragma unroll
+  for (int t = 0; t < S::X_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, step * 256, 0, 0);
+#pragma unroll
+  for (int t = 0; t < S::W_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + S::XBYTES + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0,
+                                             step * S::WROW, 0, 0);
+}
+
+template <typename WT, int RG, int MR>
+__global__ __launch_bounds__(64) void gemm_f32_mfma_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                           float* __restrict__ y, int M, int N, int K, int ldx, int ldy,
+                                                           int accumulate) {
+  using S = F32MShape<WT, RG, MR>;
+  constexpr bool BF = sizeof(WT) == 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char f32m_ring[];
+  const int lane = threadIdx.x, blk = lane >> 2, i = lane & 3;
+  const int rg = blk / S::CG, cg = blk % S::CG;
+  const int n0 = blockIdx.x * S::NCW;
+  const int w_rows = min(S::NCW, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)w_rows * K * sizeof(WT)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x =
+      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * sizeof(float)), 0x00020000);
+  // loads: an instruction brings 1 KB: 4 rows of x (16 chunks of 4 elements each), 8 rows of bfloat16 weights (8 chunks
+  // of 8 elements) or 4 rows of 32-bit ones; the lane that fills slot s of a row fetches chunk s ^ (row % 8).  Rows
+  // past M or N are clamped to the last: what they bring ends in outputs that are never stored.
+  int voff_x[S::X_LOADS], voff_w[S::W_LOADS];
+#pragma unroll
+  for (int t = 0; t < S::X_LOADS; ++t) {
+    const int row = 4 * t + (lane >> 4), chunk = (lane & 15) ^ (row & 7);
+    voff_x[t] = (min(row, M - 1) * ldx + 4 * chunk) * 4;
+  }
+#pragma unroll
+  for (int t = 0; t < S::W_LOADS; ++t) {
+    if constexpr (BF) {
+      const int row = 8 * t + (lane >> 3), chunk = (lane & 7) ^ (row & 7);
+      voff_w[t] = (min(row, w_rows - 1) * K + 8 * chunk) * 2;
+    } else {
+      const int row = 4 * t + (lane >> 4), chunk = (lane & 15) ^ (row & 7);
+      voff_w[t] = (min(row, w_rows - 1) * K + 4 * chunk) * 4;
+    }
+  }
+  // operand reads: this lane's row of x in every block of 16 rows, and its column's row of W
+  int x_base[MR], x_swz[MR];
+#pragma unroll
+  for (int mr = 0; mr < MR; ++mr) {
+    const int row = 16 * mr + 4 * rg + i;
+    x_base[mr] = row * 256;
+    x_swz[mr] = row & 7;
+  }
+  const int wr = 4 * cg + i;
+  const int w_base = S::XBYTES + wr * S::WROW, w_swz = wr & 7;
+  f32x4 acc[MR];
+#pragma unroll
+  for (int mr = 0; mr < MR; ++mr) acc[mr] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const int steps = K / 64;
+  // A stage is worked on in PH phases of CH chunks of 8 steps of k.  The operands of a phase are read from LDS
+  // into one of two sets of registers while the phase before runs out of the other: an LDS read takes longer than
+  // the few matrix instructions the compiler would put between it and its use.
+  constexpr int CH = MR == 4 ? 2 : 4, PH = 8 / CH;
+  constexpr int WQ = BF ? CH : 2 * CH;                              // 16-byte reads of W a phase
+  u32x4 w_a[WQ], w_b[WQ];
+  f32x4 x_a[MR][2 * CH], x_b[MR][2 * CH];
+  auto read_phase = [&](const unsigned char* stage, int ph, u32x4 (&wq)[WQ], f32x4 (&xq)[MR][2 * CH]) {
+#pragma unroll
+    for (int c = 0; c < WQ; ++c) wq[c] = *reinterpret_cast<const u32x4*>(stage + w_base + (((ph * WQ + c) ^ w_swz) * 16));
+#pragma unroll
+    for (int c = 0; c < 2 * CH; ++c)
+#pragma unroll
+      for (int mr = 0; mr < MR; ++mr)
+        xq[mr][c] = *reinterpret_cast<const f32x4*>(stage + x_base[mr] + (((ph * 2 * CH + c) ^ x_swz[mr]) * 16));
+  };
+  auto run_phase = [&](const u32x4 (&wq)[WQ], const f32x4 (&xq)[MR][2 * CH]) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      float wv[8];
+      if constexpr (BF) {                                           // bfloat16 -> 32-bit: the bits, shifted (exact)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          wv[2 * q] = __uint_as_float(wq[c][q] << 16);
+          wv[2 * q + 1] = __uint_as_float(wq[c][q] & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          wv[q] = __uint_as_float(wq[2 * c][q]);
+          wv[4 + q] = __uint_as_float(wq[2 * c + 1][q]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e)                                   // k ascending
+#pragma unroll
+        for (int mr = 0; mr < MR; ++mr)
+          acc[mr] = __builtin_amdgcn_mfma_f32_4x4x1f32(xq[mr][2 * c + (e >> 2)][e & 3], wv[e], acc[mr], S::CBSZ, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int st = 0; st < S::STAGES - 1; ++st) f32m_issue<WT, RG, MR>(f32m_ring, rs_x, rs_w, voff_x, voff_w, st, steps);
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));                // stage 0 has landed
+  asm volatile("" ::: "memory");
+  read_phase(f32m_ring, 0, w_a, x_a);
+  for (int step = 0; step < steps; ++step) {
+    const unsigned char* stage = f32m_ring + (step % S::STAGES) * S::STAGE;
+    const unsigned char* next = f32m_ring + ((step + 1) % S::STAGES) * S::STAGE;
+    // stage step - 1 has been read (its last phase was read a phase ago): it may be asked for again
+    asm volatile("" ::: "memory");
+    f32m_issue<WT, RG, MR>(f32m_ring, rs_x, rs_w, voff_x, voff_w, step + S::STAGES - 1, steps);
+#pragma unroll
+    for (int ph = 0; ph < PH; ph += 2) {
+      read_phase(stage, ph + 1, w_b, x_b);
+      __builtin_amdgcn_sched_barrier(0);
+      run_phase(w_a, x_a);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ph + 2 < PH) {
+        read_phase(stage, ph + 2, w_a, x_a);
+      } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));          // the next stage has landed (past K: zeros, unused)
+        asm volatile("" ::: "memory");
+        read_phase(next, 0, w_a, x_a);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      run_phase(w_b, x_b);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                       // the padding loads too, before the wave ends
+  const int n = n0 + 4 * cg + i;
+  if (n >= N) return;
+#pragma unroll
+  for (int mr = 0; mr < MR; ++mr)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = 16 * mr + 4 * rg + r;
+      if (m >= M) continue;
+      float* o = y + (size_t)m * ldy + n;
+      *o = accumulate ? (*o + acc[mr][r]) : acc[mr][r];
+    }
+}
+
+template <typename WT, int RG, int MR>
+static void launch_f32_mfma(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                            hipStream_t s) {
+  using S = F32MShape<WT, RG, MR>;
+  hipLaunchKernelGGL((gemm_f32_mfma_kernel<WT, RG, MR>), dim3((N + S::NCW - 1) / S::NCW), dim3(64), S::STAGES * S::STAGE, s, x, w,
+                     y, M, N, K, ldx, ldy, accumulate);
+}
+
+template <typename WT>
+static void launch_f32_mfma_rows(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                                 hipStream_t s) {
+  if (M <= 32) launch_f32_mfma<WT, 4, 2>(x, w, y, M, N, K, ldx, ldy, accumulate, s);
+  else launch_f32_mfma<WT, 4, 4>(x, w, y, M, N, K, ldx, ldy, accumulate, s);
+}
+
+// ------------------------------------------------------------------------------ prompt portions on the matrix cores
+
+// Tiles of 128 x 128 outputs, four waves of 64 x 64.  v_mfma_f32_32x32x1_2b_f32 is one step of k for two blocks of
+// 32 x 32 outputs: D[i][j] = fma(A[i], B[j], D[i][j]), the same single-rounding multiply-add as above; with the A
+// operand of the first block broadcast to the second, an instruction is 32 rows (A: lane i < 32 holds row i) against
+// 64 columns (B: lane l holds column l), and a wave issues two of them a step, for its upper and lower 32 rows: two
+// chains that are independent, so that neither waits for its own last result.  Every output is still one chain over k
+// ascending from zero.  A lane needs two elements of x and one of W a step for 4096 multiply-adds of the wave.
+// Operands come through a ring of four stages of 32 steps of k in LDS that the workgroup shares (buffer loads with
+// LDS as destination, chunks permuted against bank conflicts, one barrier a stage).  K a multiple of 32.
+#define F32P_BM 128
+#define F32P_BN 128
+#define F32P_KB 32
+#define F32P_STAGES 4
+
+template <typename WT>
+struct F32PShape {
+  static constexpr int XBYTES = F32P_BM * F32P_KB * 4;                        // 16 KB
+  static constexpr int WROW = F32P_KB * (int)sizeof(WT);                      // 64 or 128 bytes
+  static constexpr int WBYTES = F32P_BN * WROW;
+  static constexpr int STAGE = XBYTES + WBYTES;
+  static constexpr int X_LOADS = XBYTES / 1024 / 4, W_LOADS = WBYTES / 1024 / 4;   // per wave
+  static constexpr int LPW = X_LOADS + W_LOADS;
+  static constexpr int PENDING = LPW * (F32P_STAGES - 2);
+};
+
+template <typename WT>
+__device__ __forceinline__ void f32p_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
+                                           const int* voff_x, const int* voff_w, int wave, int step, int steps) {
+  using S = F32PShape<WT>;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = ring + (step % F32P_STAGES) * S::STAGE;
+  const bool real = step < steps;                                  // scalar
+#pragma unroll
+  for (int t = 0; t < S::X_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + (wave * S::X_LOADS + t) * 1024), 16,
+                                             real ? voff_x[t] : 0x7ffffff0, step * F32P_KB * 4, 0, 0);
+#pragma unroll
+  for (int t = 0; t < S::W_LOADS; ++t)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + S::XBYTES + (wave * S::W_LOADS + t) * 1024), 16,
+                                             real ? voff_w[t] : 0x7ffffff0, step * S::WROW, 0, 0);
+}
+
+typedef __attribute__((ext_vector_type(32))) float f32x32;
+
+template <typename WT>
+__global__ __launch_bounds__(256) void gemm_f32_mfma_tile_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                                float* __restrict__ y, int M, int N, int K, int ldx, int ldy,
+                                                                int accumulate) {
+  using S = F32PShape<WT>;
+  constexpr bool BF = sizeof(WT) == 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char f32p_ring[];
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int wy = wave >> 1, wx = wave & 1;
+  const int m0 = blockIdx.y * F32P_BM, n0 = blockIdx.x * F32P_BN;
+  const int x_rows = min(F32P_BM, M - m0), w_rows = min(F32P_BN, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)x_rows - 1) * ldx + K) * sizeof(float)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)w_rows * K * sizeof(WT)), 0x00020000);
+  // loads: 1 KB an instruction.  Rows of 128 bytes (x; 32-bit weights): 8 rows, lane l fills slot l % 8 of row l / 8 with
+  // chunk slot ^ (row % 8).  Rows of 64 bytes (bfloat16 weights): 16 rows, slot l % 4 of row l / 4, chunk
+  // slot ^ ((row / 2) % 4).  Rows past the operand are clamped to its last: their outputs are never stored.
+  int voff_x[S::X_LOADS], voff_w[S::W_LOADS];
+#pragma unroll
+  for (int t = 0; t < S::X_LOADS; ++t) {
+    const int row = 8 * (wave * S::X_LOADS + t) + (lane >> 3), chunk = (lane & 7) ^ (row & 7);
+    voff_x[t] = (min(row, x_rows - 1) * ldx + 4 * chunk) * 4;
+  }
+#pragma unroll
+  for (int t = 0; t < S::W_LOADS; ++t) {
+    if constexpr (BF) {
+      const int row = 16 * (wave * S::W_LOADS + t) + (lane >> 2), chunk = (lane & 3) ^ ((row >> 1) & 3);
+      voff_w[t] = (min(row, w_rows - 1) * K + 8 * chunk) * 2;
+    } else {
+      const int row = 8 * (wave * S::W_LOADS + t) + (lane >> 3), chunk = (lane & 7) ^ (row & 7);
+      voff_w[t] = (min(row, w_rows - 1) * K + 4 * chunk) * 4;
+    }
+  }
+  // operand reads: rows wy*64 + (lane % 32) and 32 further of x; column wx*64 + lane of W
+  const int xr0 = wy * 64 + (lane & 31), xr1 = xr0 + 32;
+  const int x_off0 = xr0 * 128, x_off1 = xr1 * 128, x_swz = xr0 & 7;     // (xr1 % 8 == xr0 % 8)
+  const int wc = wx * 64 + lane;
+  const int w_off = S::XBYTES + wc * S::WROW, w_swz = BF ? (wc >> 1) & 3 : wc & 7;
+  f32x32 acc0, acc1;
+#pragma unroll
+  for (int r = 0; r < 32; ++r) {
+    acc0[r] = 0.f;
+    acc1[r] = 0.f;
+  }
+  const int steps = K / F32P_KB;
+#pragma unroll
+  for (int st = 0; st < F32P_STAGES - 1; ++st) f32p_issue<WT>(f32p_ring, rs_x, rs_w, voff_x, voff_w, wave, st, steps);
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));
+    __builtin_amdgcn_s_barrier();                                    // everyone has the stage at hand and is done with the one before
+    asm volatile("" ::: "memory");
+    f32p_issue<WT>(f32p_ring, rs_x, rs_w, voff_x, voff_w, wave, step + F32P_STAGES - 1, steps);
+    const unsigned char* stage = f32p_ring + (step % F32P_STAGES) * S::STAGE;
+#pragma unroll
+    for (int c8 = 0; c8 < F32P_KB / 8; ++c8) {                        // 8 steps of k at a time
+      float wv[8];
+      if constexpr (BF) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(stage + w_off + ((c8 ^ w_swz) * 16));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {                                 // bfloat16 -> 32-bit: the bits, shifted (exact)
+          wv[2 * q] = __uint_as_float(raw[q] << 16);
+          wv[2 * q + 1] = __uint_as_float(raw[q] & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const f32x4 raw = *reinterpret_cast<const f32x4*>(stage + w_off + (((2 * c8 + h) ^ w_swz) * 16));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wv[4 * h + q] = raw[q];
+        }
+      }
+      f32x4 xa[2], xb[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        xa[h] = *reinterpret_cast<const f32x4*>(stage + x_off0 + (((2 * c8 + h) ^ x_swz) * 16));
+        xb[h] = *reinterpret_cast<const f32x4*>(stage + x_off1 + (((2 * c8 + h) ^ x_swz) * 16));
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {                                   // k ascending; the two chains alternate
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(xa[e >> 2][e & 3], wv[e], acc0, 1, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(xb[e >> 2][e & 3], wv[e], acc1, 1, 0, 0);
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                         // the padding loads too, before the waves end
+  // lane l, register r of a block: row 8 * (r / 4) + 4 * (l / 32) + r % 4 of the 32, column l % 32 (+ 32 for the
+  // second block, registers 16 to 31)
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+      const int m = m0 + wy * 64 + 32 * half + 8 * ((r & 15) >> 2) + 4 * (lane >> 5) + (r & 3);
+      const int n = n0 + wx * 64 + 32 * (r >> 4) + (lane & 31);
+      if (m < M && n < N) {
+        float* o = y + (size_t)m * ldy + n;
+        const float v = half == 0 ? acc0[r] : acc1[r];
+        *o = accumulate ? (*o + v) : v;
+      }
+    }
+}
+
+template <typename WT>
+static void launch_f32_mfma_tiles(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                                  hipStream_t s) {
+  using S = F32PShape<WT>;
+  constexpr int lds_bytes = F32P_STAGES * S::STAGE;
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_f32_mfma_tile_kernel<WT>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  hipLaunchKernelGGL(gemm_f32_mfma_tile_kernel<WT>, dim3((N + F32P_BN - 1) / F32P_BN, (M + F32P_BM - 1) / F32P_BM), dim3(256),
+                     lds_bytes, s, x, w, y, M, N, K, ldx, ldy, accumulate);
+}
+
 template <typename WT, int MR>
 static void launch_rows_mr(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
                            hipStream_t s) {
@@ -362,9 +720,26 @@ extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* 
   hipStream_t s = (hipStream_t)stream;
   // which kernel runs depends on the shape alone, and both run the same chains
   const int wc = w_is_bf16 ? 8 : 4;
+  // 17 to 64 rows, K in whole stages: the chains run on the matrix cores (offsets within x and within a wave's rows
+  // of W must fit the buffer descriptors' 31 bits).  Up to 16 rows stay on the vector unit: a matrix instruction that
+  // depends on the one before it issues some 40 clocks later, a vector one 4, and so few rows have too few chains
+  // to fill the gap.
+  if (M > 16 && M <= 64 && K % 64 == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+      (size_t)M * ldx * 4 < ((size_t)1 << 31) && (size_t)64 * K * 4 < ((size_t)1 << 31)) {
+    if (w_is_bf16) launch_f32_mfma_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    else launch_f32_mfma_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
   if (M <= 64 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
     if (w_is_bf16) launch_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
     else launch_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
+  // prompt portions, K in whole stages: tiles on the matrix cores (the same chains)
+  if (M > 64 && K % F32P_KB == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+      (size_t)F32P_BM * ldx * 4 < ((size_t)1 << 31) && (size_t)F32P_BN * K * 4 < ((size_t)1 << 31)) {
+    if (w_is_bf16) launch_f32_mfma_tiles<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    else launch_f32_mfma_tiles<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
     return BW_LAUNCH_CHECK();
   }
   if (M > 64 && K % F32T_BK == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {

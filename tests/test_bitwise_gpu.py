@@ -49,6 +49,30 @@ def test_matrix_product_at_layer_widths(gpu):
         assert np.array_equal(bits(y.cpu().numpy()), bits(ps.linear(x.numpy(), w.float().numpy()))), (M, N, K)
 
 
+def test_matrix_product_on_the_matrix_cores_is_the_same_chain(gpu):
+    """17 to 64 rows and prompt portions run their chains as 32-bit matrix instructions of one step of k each:
+    shapes around the kernels' tile edges, 32-bit and bfloat16 weights, store and residual add, against std::fma."""
+    g = torch.Generator().manual_seed(15)
+    shapes = [(17, 33, 64), (24, 16, 128), (32, 100, 192), (33, 17, 64), (64, 130, 256), (48, 64, 2048),
+              (65, 1, 32), (100, 129, 96), (128, 128, 64), (129, 300, 160), (300, 257, 2048), (200, 40, 8192)]
+    for wdt in (torch.bfloat16, torch.float32):
+        for M, N, K in shapes:
+            x = torch.randn(M, K, generator=g)
+            x[0, :5] = torch.tensor([0.0, -0.0, 1e-30, -1e-38, 3e38])        # zeros, a tiny and a huge element
+            w = (torch.randn(N, K, generator=g) * 0.2).to(wdt)
+            want = ps.linear(x.numpy(), w.float().numpy())
+            y = torch.zeros(M, N, device=gpu)
+            ops.gemm_f32(x.to(gpu), w.to(gpu), y, M)
+            same = (bits(y.cpu().numpy()) == bits(want)) | (np.isnan(want) & np.isnan(y.cpu().numpy()))
+            assert same.all(), (wdt, M, N, K, int((~same).sum()))
+            res = torch.randn(M, N, generator=g)
+            y = res.clone().to(gpu)
+            ops.gemm_f32(x.to(gpu), w.to(gpu), y, M, accumulate=True)
+            want_add = res.numpy() + want
+            same = (bits(y.cpu().numpy()) == bits(want_add)) | (np.isnan(want_add) & np.isnan(y.cpu().numpy()))
+            assert same.all(), ("add", wdt, M, N, K)
+
+
 def test_rmsnorm_bits(gpu):
     g = torch.Generator().manual_seed(6)
     for rows, dim, eps in [(1, 1, 1e-5), (3, 5, 1e-6), (4, 16, 1e-5), (2, 31, 0.5), (5, 64, 1e-5), (3, 96, 1e-6),
