@@ -8,7 +8,8 @@ A step is one decode step of the whole engine (scheduler, graph replay of the mo
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
 decoded tokens per second.  One JSON line is printed; it also carries the 2,048-token prefill,
 the decode step's HBM roofline, decode at batch 1 and 64 with their rooflines, the same model's true
-32-bit path (decode and prefill) and decode and prefill at Llama-3-8B's sizes.
+32-bit path (decode and prefill) and, at Llama-3-8B's sizes, decode, prefill and a continuous-batching workload
+of 64 requests.
 """
 
 from __future__ import annotations
@@ -130,6 +131,40 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
                          "frac": round(achieved / PEAK_HBM_GBS, 4)}}
 
 
+def measure_serving(bw, torch, model, cfg: dict, dtype: str, requests: int = 64, seed: int = 5) -> dict:
+    """The continuous-batching workload of the reference's load generator (bench/loadgen.py:170-207) with synthetic
+    tokens: ``requests`` requests at once, prompt lengths uniform in [128, 2048], generation lengths uniform in
+    [64, 512], greedy, prompts cut into portions under a budget of 2,048 tokens a step, decoded beside each other."""
+    import random
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    work = []
+    for _ in range(requests):
+        n, new = rng.randint(128, 2048), rng.randint(64, 512)
+        work.append((torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), new))
+    block = 16
+    pages = sum((len(p) + new + 2 * block) // block + 1 for p, new in work)
+    ecfg = bw.EngineConfig(num_blocks=pages, max_batched_tokens=2048, max_num_seqs=requests, prefix_caching=False,
+                           fingerprint_logits=False, block_size=block, dtype=dtype, max_model_len=4096)
+    eng = bw.Engine(model, None, ecfg)
+    for p, new in work:
+        eng.add_request(p, bw.SamplingParams(max_new_tokens=new, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while not eng.idle():
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    generated = eng.stats.generated_tokens
+    prompt_tokens = sum(len(p) for p, _ in work)
+    assert generated == sum(new for _, new in work)
+    return {"requests": requests, "prompt_tokens": prompt_tokens, "generated_tokens": generated, "steps": steps,
+            "seconds": round(secs, 3), "generated_tok_s": round(generated / secs, 1),
+            "all_tok_s": round((generated + prompt_tokens) / secs, 1), "preemptions": eng.stats.preemptions}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,7 +221,8 @@ def main() -> int:
                                   "head_dim": 128, "ffn": big["intermediate_size"], "vocab": big["vocab_size"],
                                   "decode_tok_s": m["tok_s"], "batch": 8, "ms_per_step": m["ms_per_step"],
                                   "roofline": m["roofline"],
-                                  "prefill": measure_prefill(bw, torch, model8, big, "bfloat16", PEAK_FLOPS["bf16"])}
+                                  "prefill": measure_prefill(bw, torch, model8, big, "bfloat16", PEAK_FLOPS["bf16"]),
+                                  "serving": measure_serving(bw, torch, model8, big, "bfloat16")}
             del model8
             model = None
 
