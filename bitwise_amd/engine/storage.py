@@ -25,10 +25,8 @@ class CacheStorage:
         self.keys: List[torch.Tensor] = []
         self.values: List[torch.Tensor] = []
         for spec, caches in zip(model.group_specs, model.group_caches):
-            page_elems = spec.kv_heads * self.page_size * spec.head_dim
-            shape = (len(caches), self.num_pages, page_elems)
-            self.keys.append(torch.zeros(shape, dtype=rt.act_dtype, device=rt.device))
-            self.values.append(torch.zeros(shape, dtype=rt.act_dtype, device=rt.device))
+            for pool, elems in ((self.keys, spec.key_elements(self.page_size)), (self.values, spec.value_elements(self.page_size))):
+                pool.append(torch.zeros((len(caches), self.num_pages, elems), dtype=rt.act_dtype, device=rt.device))
         self.states: Dict[int, torch.Tensor] = {}
         for idx, ss in model.state_specs.items():
             self.states[idx] = torch.zeros((self.num_slots, *ss.shape), dtype=_TORCH_DTYPE[ss.dtype], device=rt.device)
@@ -47,8 +45,8 @@ class CacheStorage:
     def bytes_per_token(self) -> int:
         """Cache bytes one token occupies over all caches (keys and values)."""
         total = 0
-        for k in self.keys:
-            total += 2 * k.shape[0] * (k.shape[2] // self.page_size) * k.element_size()
+        for t in self.keys + self.values:
+            total += t.shape[0] * (t.shape[2] // self.page_size) * t.element_size()
         return total
 
     def reset_slot(self, slot: int) -> None:

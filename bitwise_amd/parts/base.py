@@ -83,14 +83,25 @@ class ModelSpec:
 
 @dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer keeps per token: keys and values in pages.
+    """What a mixer keeps per token in pages: ``key_width`` elements in the key pool and ``value_width`` in the
+    value pool (for attention both are kv_heads * head_dim; a mixer with other needs says its own, and a width
+    of 0 leaves that pool out).  How a page's elements are laid out is the mixer's own business.
 
     ``window`` None: every earlier position stays readable.  ``window`` W: a query at
     position p reads keys p-W+1..p only, so pages wholly before that may be given back.
+    Caches with equal specs share a group: one block table, one pool of page numbers.
     """
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    key_width: Optional[int] = None        # elements per token; None: kv_heads * head_dim
+    value_width: Optional[int] = None
+
+    def key_elements(self, page_size: int) -> int:
+        return page_size * (self.kv_heads * self.head_dim if self.key_width is None else self.key_width)
+
+    def value_elements(self, page_size: int) -> int:
+        return page_size * (self.kv_heads * self.head_dim if self.value_width is None else self.value_width)
 
 
 @dataclass(frozen=True)
