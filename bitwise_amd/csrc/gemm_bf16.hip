@@ -1429,38 +1429,41 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
 // rows of W and of the 16 rows of x, fetched by buffer loads with LDS as destination in whole cache
 // lines; LPW loads a stage, so "all but the last LPW * (stages - 2)" is the wait for the stage at
 // hand.  Nothing is shared between waves, so the loop has no barrier.  K a multiple of 64.
-template <int CW>
+// XR: rows of x a stage holds, 16, or 8 where there are no more than 8 (lanes that stand for rows 8 to 15 read rows
+// 0 to 7 again; their products go nowhere): a load less a stage, so more stages of W in flight.
+template <int CW, int XR = 16>
 struct StreamShape {
-  static constexpr int B_LOADS = CW / 8, LPW = 2 + B_LOADS;
-  static constexpr int STAGE = 2048 + B_LOADS * 1024;               // x: 16 rows of 128 bytes, then W
-  static constexpr int STAGES = CW == 8 ? 10 : 8;
+  static constexpr int A_LOADS = XR / 8, B_LOADS = CW / 8, LPW = A_LOADS + B_LOADS;
+  static constexpr int A_BYTES = A_LOADS * 1024;
+  static constexpr int STAGE = A_BYTES + B_LOADS * 1024;            // x: XR rows of 128 bytes, then W
+  static constexpr int STAGES = 24 / LPW + 2;
   static constexpr int RING = STAGES * STAGE;
   static_assert(LPW * (STAGES - 2) == 24, "the wait below is written for 24 loads in flight");
 };
 
 // A wave's loads of one stage of its ring (a device function rather than a lambda in the kernel: the
 // host pass drops, without a word, kernel templates whose lambdas capture arrays of dependent size).
-template <int CW>
+template <int CW, int XR>
 __device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
                                              const int* voff_x, const int* voff_w, int step, int steps, int k_begin) {
-  using SH = StreamShape<CW>;
+  using SH = StreamShape<CW, XR>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   unsigned char* dst = ring + (step % SH::STAGES) * SH::STAGE;
   const bool real = step < steps;                                  // scalar; past the segment: outside the descriptors
   const int soff = (k_begin + step * 64) * 2;
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int t = 0; t < SH::A_LOADS; ++t)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, soff, 0, 0);
 #pragma unroll
   for (int t = 0; t < SH::B_LOADS; ++t)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + 2048 + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0, soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + SH::A_BYTES + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0, soff, 0, 0);
 }
 
-template <int EPI, int CW>
+template <int EPI, int CW, int XR = 16>
 __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
                                                                int S) {
-  using SH = StreamShape<CW>;
+  using SH = StreamShape<CW, XR>;
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];   // [waves][ring], then [S][4][64] floats when S > 1
   const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -1481,10 +1484,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
   for (int t = 0; t < SH::B_LOADS; ++t) voff_w[t] = ((8 * t + lrow) * K + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
   // operand reads: lane (g, r) wants row r (of W: r % CW), chunk 4*kk + g: slot (4*kk + g) ^ (row >> 1)
   int off_x[2], off_w[2];
+  const int rx = XR == 8 ? (r & 7) : r;                              // the row of x this lane reads
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
-    off_x[kk] = (r >> 3) * 1024 + (r & 7) * 128 + (((4 * kk + g) ^ (r >> 1)) * 16);
-    off_w[kk] = 2048 + (c >> 3) * 1024 + (c & 7) * 128 + (((4 * kk + g) ^ (c >> 1)) * 16);
+    off_x[kk] = (rx >> 3) * 1024 + (rx & 7) * 128 + (((4 * kk + g) ^ (rx >> 1)) * 16);
+    off_w[kk] = SH::A_BYTES + (c >> 3) * 1024 + (c & 7) * 128 + (((4 * kk + g) ^ (c >> 1)) * 16);
   }
   unsigned char* ring = stream_lds + wave * SH::RING;
   float* red = reinterpret_cast<float*>(stream_lds + nwaves * SH::RING);
@@ -1494,7 +1498,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
     const int steps = ((K - k_begin) < GEMM_SEG ? K - k_begin : GEMM_SEG) / 64;
     acc = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+    for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
     for (int step = 0; step < steps; ++step) {
       __builtin_amdgcn_s_waitcnt(0x4f78);                          // vmcnt(24): the stage at hand has landed
       asm volatile("" ::: "memory");
@@ -1510,7 +1514,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk]), acc, 0, 0, 0);
       // the reads above are done (their values were used) before the stage is asked for again
       asm volatile("" ::: "memory");
-      stream_issue<CW>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
+      stream_issue<CW, XR>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);                            // the padding loads too, before the ring is reused
     if (S > 1) {
@@ -1542,19 +1546,132 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
   }
 }
 
-template <int EPI, int CW>
-static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
-  using SH = StreamShape<CW>;
+template <int EPI, int CW, int XR>
+static int launch_stream_rows(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
+  using SH = StreamShape<CW, XR>;
   const int waves = S < 4 ? S : 4;
   const size_t lds_bytes = (size_t)waves * SH::RING + (S > 1 ? (size_t)S * 4 * 64 * sizeof(float) : 0);
   if (lds_bytes > 160 * 1024) return -2;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
   if (!allowed) {
-    (void)hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<EPI, CW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<EPI, CW, XR>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_stream_kernel<EPI, CW>), dim3((N + CW - 1) / CW), dim3(64 * waves), lds_bytes, s, x, w, out, M, N,
+  hipLaunchKernelGGL((gemm_bf16_stream_kernel<EPI, CW, XR>), dim3((N + CW - 1) / CW), dim3(64 * waves), lds_bytes, s, x, w, out, M, N,
                      K, ldx, ldo, S);
+  return BW_LAUNCH_CHECK();
+}
+
+template <int EPI, int CW>
+static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
+  // (how many rows a stage holds changes no bit: the chain of a row is the same statements on the same values)
+  if (M <= 8) return launch_stream_rows<EPI, CW, 8>(x, w, out, M, N, K, ldx, ldo, S, s);
+  return launch_stream_rows<EPI, CW, 16>(x, w, out, M, N, K, ldx, ldo, S, s);
+}
+
+// ------------------------------------------------------------------------------ up to 16 rows, few columns, one segment
+
+// A product so small that a ring would never fill (the output projection of a decode step: 8 MB of
+// weights for 256 compute units): a workgroup of four waves takes 8 columns, and everything it needs,
+// all of its 8 rows of W and the 16 rows of x, is asked for at once, straight into LDS, wave w asking for
+// the steps w, w + 4, ... of K; nothing waits for a ring slot, so the whole weight is in flight within
+// the kernel's first hundred nanoseconds.  Loads land in the order they were asked for: when every
+// wave's q-th step has landed, steps 4q .. 4q + 3 are there, and wave 0 runs them through the one chain
+// of the workgroup's 16 x 16 block while the later ones are still on their way.  The stage layout and
+// the chain are the stream kernel's: the same bits.  K a multiple of 64, at most BURST_STEPS steps.
+#define BURST_STEPS 32
+#define BURST_STAGE 3072                                           // x: 16 rows of 128 bytes, then 8 rows of W
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char burst_lds[];   // [BURST_STEPS][BURST_STAGE]
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int c = r & 7;
+  const int n0 = blockIdx.x * 8;
+  const bool n_ok = r < 8 && n0 + c < N;
+  const int w_rows = min(8, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0, (int)((size_t)w_rows * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x =
+      __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_x[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) voff_x[t] = ((8 * t + lrow) * ldx + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
+  const int voff_w = (lrow * K + 8 * (lslot ^ (lrow >> 1))) * 2;
+  const int steps = K / 64;
+  // eight steps a wave, whatever K: those past K are asked for outside the descriptors (no traffic, zeros), so
+  // that the counts below are the same for every wave
+#pragma unroll
+  for (int i = 0; i < BURST_STEPS / 4; ++i) {
+    const int st = wave + 4 * i;
+    const bool real = st < steps;                                  // scalar
+    unsigned char* dst = burst_lds + st * BURST_STAGE;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, st * 128, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + 2048), 16, real ? voff_w : 0x7ffffff0, st * 128, 0, 0);
+  }
+  int off_x[2], off_w[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    off_x[kk] = (r >> 3) * 1024 + (r & 7) * 128 + (((4 * kk + g) ^ (r >> 1)) * 16);
+    off_w[kk] = 2048 + c * 128 + (((4 * kk + g) ^ (c >> 1)) * 16);
+  }
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  auto run_steps = [&](int q) {                                     // steps 4q .. 4q + 3 of the chain (wave 0)
+    for (int step = 4 * q; step < 4 * q + 4 && step < steps; ++step) {
+      const unsigned char* stage = burst_lds + step * BURST_STAGE;
+      u32x4 fa[2], fb[2];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        fa[kk] = *reinterpret_cast<const u32x4*>(stage + off_x[kk]);
+        fb[kk] = *reinterpret_cast<const u32x4*>(stage + off_w[kk]);
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk]), acc, 0, 0, 0);
+    }
+  };
+  // the wave's q-th step has landed when all but its last 3 * (7 - q) loads have
+#define BURST_ROUND(Q, WAIT)                                   \
+  if (4 * (Q) < steps) {                                       \
+    __builtin_amdgcn_s_waitcnt(WAIT);                          \
+    __builtin_amdgcn_s_barrier();                              \
+    asm volatile("" ::: "memory");                             \
+    if (wave == 0) run_steps(Q);                               \
+  }
+  BURST_ROUND(0, vmcnt_only(21))
+  BURST_ROUND(1, vmcnt_only(18))
+  BURST_ROUND(2, vmcnt_only(15))
+  BURST_ROUND(3, vmcnt_only(12))
+  BURST_ROUND(4, vmcnt_only(9))
+  BURST_ROUND(5, vmcnt_only(6))
+  BURST_ROUND(6, vmcnt_only(3))
+  BURST_ROUND(7, vmcnt_only(0))
+#undef BURST_ROUND
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                        // the padding loads too, before the wave ends
+  if (wave != 0 || !n_ok) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int m = 4 * g + q;
+    if (m >= M) continue;
+    epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+  }
+}
+
+template <int EPI>
+static int launch_burst(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s) {
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_burst_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_bf16_burst_kernel<EPI>), dim3((N + 7) / 8), dim3(256), BURST_STEPS * BURST_STAGE, s, x, w, out, M, N, K,
+                     ldx, ldo);
   return BW_LAUNCH_CHECK();
 }
 
@@ -1638,6 +1755,8 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {
       // up to 16 rows: a wave per strip and segment, streaming through its own ring in LDS
       if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        // one segment and few columns: everything asked for at once
+        if ((N + 15) / 16 < 256 && K <= 64 * BURST_STEPS) return launch_burst<EPI>(x, w, out, M, N, K, ldx, ldo, s);
         if ((N + 15) / 16 < 256) return launch_stream<EPI, 8>(x, w, out, M, N, K, ldx, ldo, S, s);
         return launch_stream<EPI, 16>(x, w, out, M, N, K, ldx, ldo, S, s);
       }
