@@ -445,6 +445,336 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
   }
 }
 
+// ------------------------------------------------------------------------------ prompt portions on the matrix cores
+
+// A wave per tile of up to 32 consecutive rows of one sequence and head.  v_mfma_f32_32x32x1_2b_f32 is, for every
+// one of its 2 x 32 x 32 outputs, one fused multiply-add d = fma(a, b, d) with a single rounding: a chain of them
+// is the scalar chain, bit for bit.  So both products of the attention run there, in the reference's order:
+//   * scores, transposed (rows: 32 keys, columns: the tile's queries): chain c of dot_canonical (elements
+//     16 j + c, j ascending) is HD / 16 instructions; the instruction's two blocks run chains c and c + 8, whose
+//     sums the tree adds first (s8[c] = lane[c] + lane[c + 8]): the same registers of the two blocks.  The rest
+//     of the tree, the scale and the maximum are vector instructions on 16 scores a lane.
+//   * pass 2, keys in order: e = exp(s - max) where the query sees the key, else 0 (a key it does not see adds
+//     +0 to a sum that is never -0, and fma(0, v, acc) = acc for the finite v of a written cache slot: the bits of
+//     skipping it); sum += e along the keys, which a query's two lanes (l and l + 32 hold alternate groups of
+//     four keys) hand back and forth; acc[q][d] = fma(e[q][k], v[k][d], acc[q][d]) is one instruction a key
+//     (two for more than 64 elements), its A operand broadcast from the half of the wave that holds the key.
+// The scores are computed twice (pass 1 keeps only the maximum), as in the kernels above.
+typedef __attribute__((ext_vector_type(32))) float f32x32;
+
+template <int HD>
+struct Att32Mfma {
+  static constexpr int NJ = HD / 16;            // steps of a chain of the dot
+  static constexpr int NB = (HD + 63) / 64;     // accumulators of the second product, 64 output elements each
+};
+
+// 16 scores a lane: keys kb + 8 (r / 4) + 4 (lane / 32) + r % 4 against query lane % 32, before the scale.
+// An instruction occupies the matrix core for 64 clocks, so one chain at a time keeps it busy; two accumulators
+// alternate, the vector adds of one chain's tree running under the next chain's instructions, and the order is
+// pinned (left to itself the scheduler starts all eight chains at once: eight accumulators of 32 registers).
+// ``first`` is the chain's first key operand, kr[0][c], handed in by the caller (see the pins below).
+template <int HD>
+__device__ __forceinline__ f32x32 mfma_chain(const float (&kr)[HD / 16][8], const float (&qv)[HD / 16][8], int c, float first) {
+  f32x32 acc = {};                               // (a constant zero: the first instruction's addend)
+  acc = __builtin_amdgcn_mfma_f32_32x32x1f32(first, qv[0][c], acc, 0, 0, 0);
+#pragma unroll
+  for (int j = 1; j < HD / 16; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(kr[j][c], qv[j][c], acc, 0, 0, 0);
+  return acc;
+}
+
+// Pins 16 values and the next chain's first operand at this point of the program: statements like this one keep
+// their order, so the sums above are computed (and the accumulators they read are free) before the chain below
+// starts.  Left to itself the compiler starts all eight chains at once, eight accumulators of 32 registers, and
+// spills what else the kernel holds.
+#define BW_PIN16(v, k)                                                                                             \
+  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]),  \
+               "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]), "+v"(k))
+
+template <int HD>
+__device__ __forceinline__ void mfma_scores(const float (&kr)[HD / 16][8], const float (&qv)[HD / 16][8], float (&s)[16]) {
+  // lane[c] + lane[c + 8] of dot_canonical is block 0 + block 1 of chain c: the same registers of the two halves.
+  // Two accumulators alternate: while one chain runs on the matrix core, the vector adds fold the chain before it.
+  float x[16], t[16], k0;
+  f32x32 p = mfma_chain<HD>(kr, qv, 0, kr[0][0]);
+  f32x32 q = mfma_chain<HD>(kr, qv, 4, kr[0][4]);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = p[i] + p[16 + i];                           // s8[0]
+  k0 = kr[0][2];
+  BW_PIN16(x, k0);
+  p = mfma_chain<HD>(kr, qv, 2, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = x[i] + (q[i] + q[16 + i]);                  // s4[0] = s8[0] + s8[4]
+  k0 = kr[0][6];
+  BW_PIN16(x, k0);
+  q = mfma_chain<HD>(kr, qv, 6, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) t[i] = p[i] + p[16 + i];                           // s8[2]
+  k0 = kr[0][1];
+  BW_PIN16(t, k0);
+  p = mfma_chain<HD>(kr, qv, 1, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = x[i] + (t[i] + (q[i] + q[16 + i]));         // s4[0] + s4[2]
+  k0 = kr[0][5];
+  BW_PIN16(x, k0);
+  q = mfma_chain<HD>(kr, qv, 5, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s[i] = p[i] + p[16 + i];                           // s8[1]
+  k0 = kr[0][3];
+  BW_PIN16(s, k0);
+  p = mfma_chain<HD>(kr, qv, 3, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s[i] = s[i] + (q[i] + q[16 + i]);                  // s4[1] = s8[1] + s8[5]
+  k0 = kr[0][7];
+  BW_PIN16(s, k0);
+  q = mfma_chain<HD>(kr, qv, 7, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) t[i] = p[i] + p[16 + i];                           // s8[3]
+  k0 = 0.0f;
+  BW_PIN16(t, k0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s[i] = x[i] + (s[i] + (t[i] + (q[i] + q[16 + i])));   // (s4[0] + s4[2]) + (s4[1] + s4[3])
+  BW_PIN16(s, k0);
+}
+
+// Who takes which tile: a workgroup is eight waves of one head, and the hardware deals a workgroup's waves out to
+// the compute unit's four SIMDs in turn, so waves w and w + 4 share a matrix core.  Wave w takes tile 4 k + w from
+// the front of the list and wave w + 4 tile n - 1 - (4 k + w) from its back: the tiles of a long prompt come in
+// position order, the work of a tile grows with its position, and so every matrix core gets a short tile and a
+// long one, the same sum everywhere.  Workgroups of a head run on one die (the hardware deals workgroups out to the
+// eight dies in turn), whose L2 then holds the keys and values of its heads only.
+template <int HD>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_f32_mfma_kernel(AttnF32Args a, int num_tiles, int groups) {
+  constexpr int NJ = Att32Mfma<HD>::NJ, NB = Att32Mfma<HD>::NB;
+  const int wave = wave_index(), lane = threadIdx.x & 63, col = lane & 31, h2 = lane >> 5;
+  int h, k;
+  {
+    const int L = blockIdx.x;
+    if (a.heads % 8 == 0) {
+      const int die = L & 7, idx = L >> 3;                          // the idx-th workgroup of that die
+      h = (idx / groups) * 8 + die;
+      k = idx % groups;
+    } else {
+      h = L / groups;
+      k = L % groups;
+    }
+  }
+  const int front = 4 * k + (wave & 3), half_n = (num_tiles + 1) >> 1;
+  const int tile = wave < 4 ? front : num_tiles - 1 - front;
+  if (front >= half_n || (wave >= 4 && tile < half_n)) return;       // (the middle tile of an odd count is a front tile)
+  const int row0 = a.tiles[4 * tile], ntok = a.tiles[4 * tile + 1], seq = a.tiles[4 * tile + 2];
+  if (ntok <= 0) return;
+  const int32_t* table = a.block_table + (size_t)seq * a.table_stride;
+  const bool active = col < ntok;
+  const int my_row = row0 + (active ? col : ntok - 1);
+  const int pos_q = active ? a.positions[my_row] : -1;
+  const int lo_q = (a.window > 0 && pos_q - a.window + 1 > 0) ? pos_q - a.window + 1 : 0;
+  const int pos_first = a.positions[row0], pos_last = a.positions[row0 + ntok - 1];
+  if (pos_last < 0) return;
+  const int lo_min = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
+  const int lo_last = (a.window > 0 && pos_last - a.window + 1 > 0) ? pos_last - a.window + 1 : 0;   // the last row's first key
+  const int kvh = h / (a.heads / a.kv_heads);
+  const float* kc = a.k_cache + (size_t)kvh * a.page_size * HD;     // this head's rows of page 0
+  const float* vc = a.v_cache + (size_t)kvh * a.page_size * HD;
+  const size_t page_stride = (size_t)a.kv_heads * a.page_size * HD;
+  // where key kb + col lies: its page and its row within the page's rows of this head (keys past the tile's last are
+  // that last key again: a written slot, whose products nobody sees)
+  auto locate = [&](int kb, int& page, int& slot) {
+    int j = kb + col;
+    j = j < pos_last ? j : pos_last;
+    page = table[a.page_shift >= 0 ? j >> a.page_shift : j / a.page_size];
+    slot = a.page_shift >= 0 ? j & (a.page_size - 1) : j % a.page_size;
+  };
+  // this lane's half of its query's row: elements 16 j + 8 h2 + c
+  float qv[NJ][8];
+  {
+    const float* qh = a.q + (size_t)my_row * a.q_stride + (size_t)h * HD + 8 * h2;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const f32x4 t0 = *reinterpret_cast<const f32x4*>(qh + 16 * j), t1 = *reinterpret_cast<const f32x4*>(qh + 16 * j + 4);
+      qv[j][0] = t0[0]; qv[j][1] = t0[1]; qv[j][2] = t0[2]; qv[j][3] = t0[3];
+      qv[j][4] = t1[0]; qv[j][5] = t1[1]; qv[j][6] = t1[2]; qv[j][7] = t1[3];
+    }
+  }
+  // the same half of the row of the lane's key
+  auto load_keys_at = [&](const float* kp, float (&kr)[NJ][8]) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const f32x4 t0 = *reinterpret_cast<const f32x4*>(kp + 16 * j), t1 = *reinterpret_cast<const f32x4*>(kp + 16 * j + 4);
+      kr[j][0] = t0[0]; kr[j][1] = t0[1]; kr[j][2] = t0[2]; kr[j][3] = t0[3];
+      kr[j][4] = t1[0]; kr[j][5] = t1[1]; kr[j][6] = t1[2]; kr[j][7] = t1[3];
+    }
+  };
+  auto load_keys = [&](int page, int slot, float (&kr)[NJ][8]) {
+    load_keys_at(kc + (size_t)page * page_stride + (size_t)slot * HD + 8 * h2, kr);
+  };
+  const int key_of_reg = 4 * h2;                                    // register r: key kb + 8 (r / 4) + 4 h2 + r % 4
+  // A whole block of 32 keys that starts at a multiple of 16, in pages of 16 slots or more, is two runs of 16 rows
+  // that lie one behind the other in memory: two addresses a block, found by the scalar unit, instead of one a key
+  // (address arithmetic is instructions of this wave too, and a wave's instructions do not overlap its own matrix
+  // instructions).  Other blocks (a window's unaligned start, the tile's last block) take the general way.
+  const bool runs16 = a.page_shift >= 4;
+  auto run_start = [&](const float* cache, int j) -> const float* {  // the row of key j (a multiple of 16): scalar
+    return cache + (size_t)table[j >> a.page_shift] * page_stride + (size_t)(j & (a.page_size - 1)) * HD;
+  };
+  auto load_keys_runs = [&](int kb, float (&kr)[NJ][8]) {
+    const float* r0 = run_start(kc, kb);
+    const float* r1 = run_start(kc, kb + 16);
+    load_keys_at((col < 16 ? r0 : r1) + (col & 15) * HD + 8 * h2, kr);
+  };
+
+  // keys kb .. kb + 31 into kr; page and slot are set for the general way's value loads
+  auto fetch_keys = [&](int kb, int& page, int& slot, float (&kr)[NJ][8]) {
+    if (runs16 && (kb & 15) == 0 && kb + 31 <= pos_last) load_keys_runs(kb, kr);
+    else {
+      locate(kb, page, slot);
+      load_keys(page, slot, kr);
+    }
+  };
+
+  // pass 1: every query's maximum.  Two blocks of keys a turn of the loop, each in registers of its own, asked for a
+  // whole block ahead of its use.
+  float mx = -INFINITY;
+  {
+    float ka[NJ][8], kb2[NJ][8];
+    int page, slot;
+    fetch_keys(lo_min, page, slot, ka);
+    if (lo_min + 32 <= pos_last) fetch_keys(lo_min + 32, page, slot, kb2);
+#define ATT_PASS1(KB, KR)                                                                  \
+    {                                                                                      \
+      float s[16];                                                                         \
+      mfma_scores<HD>(KR, qv, s);                                                          \
+      if ((KB) + 64 <= pos_last) fetch_keys((KB) + 64, page, slot, KR);                    \
+      __builtin_amdgcn_sched_barrier(0);                                                   \
+      if ((KB) + 31 <= pos_first && (KB) >= lo_last) {       /* every query of the tile sees every key of the block */ \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r] * a.scale);     \
+      } else {                                                                             \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                   \
+          const int key = (KB) + 8 * (r >> 2) + key_of_reg + (r & 3);                      \
+          const float t = fmaxf(mx, s[r] * a.scale);                                       \
+          mx = (key >= lo_q && key <= pos_q) ? t : mx;                                     \
+        }                                                                                  \
+      }                                                                                    \
+    }
+    for (int kb = lo_min; kb <= pos_last; kb += 64) {
+      ATT_PASS1(kb, ka)
+      if (kb + 32 <= pos_last) ATT_PASS1(kb + 32, kb2)
+    }
+#undef ATT_PASS1
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+
+  // pass 2: the keys of the next block are asked for when this block's scores are done, its values then too (for
+  // heads of up to 64 elements, whose registers allow a second set), so both have a block's time to arrive.
+  constexpr bool VAHEAD = false;
+  f32x32 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x32{};
+  float sum = 0.0f;
+  {
+    float kr[NJ][8];
+    float va[32][NB], vb[VAHEAD ? 32 : 1][NB];
+    int page, slot;
+    page = 0;
+    slot = 0;
+    fetch_keys(lo_min, page, slot, kr);
+    // a block's 32 value rows, element 64 nb + lane of each (zero past the head's size).  Where key k lies is what
+    // lane k found for the keys' rows.  Every lane loads (clamped), and the zero is a select: nothing near a matrix
+    // instruction runs under a partial execution mask.
+#define ATT_VALUES(KB, VV)                                                                                              \
+    if (runs16 && ((KB) & 15) == 0 && (KB) + 31 <= pos_last) {                                                          \
+      const float* r0 = run_start(vc, (KB));                                                                            \
+      const float* r1 = run_start(vc, (KB) + 16);                                                                       \
+      _Pragma("unroll") for (int k = 0; k < 32; ++k) {                                                                  \
+        const float* vp = (k < 16 ? r0 : r1) + (k & 15) * HD;                                                           \
+        _Pragma("unroll") for (int nb = 0; nb < NB; ++nb) {                                                             \
+          const int d = 64 * nb + lane;                                                                                 \
+          const float t = vp[d < HD ? d : HD - 1];                                                                      \
+          VV[k][nb] = d < HD ? t : 0.0f;                                                                                \
+        }                                                                                                               \
+      }                                                                                                                 \
+    } else {                                                                                                            \
+      _Pragma("unroll") for (int k = 0; k < 32; ++k) {                                                                  \
+        const float* vp = vc + (size_t)__builtin_amdgcn_readlane(page, k) * page_stride +                               \
+                          (size_t)__builtin_amdgcn_readlane(slot, k) * HD;                                              \
+        _Pragma("unroll") for (int nb = 0; nb < NB; ++nb) {                                                             \
+          const int d = 64 * nb + lane;                                                                                 \
+          const float t = vp[d < HD ? d : HD - 1];                                                                      \
+          VV[k][nb] = d < HD ? t : 0.0f;                                                                                \
+        }                                                                                                               \
+      }                                                                                                                 \
+    }
+    // Eight keys at a time (registers 4 g2 .. 4 g2 + 3: keys 8 g2 .. + 3 in the lower half of the wave, 8 g2 + 4 .. + 7
+    // in the upper): their exponentials, sum += e in key order (the two halves hand the sum back and forth: after
+    // the swap r[0] is the lower half's value in every lane, r[1] the upper half's), and
+    // acc[q][d] = fma(e[q][k], v[k][d], acc[q][d]), k ascending; the vector work of the next eight keys runs under
+    // these matrix instructions.
+#define ATT_PASS2(KB, VCUR, VNEXT)                                                                                      \
+    {                                                                                                                   \
+      float e[16];                                                                                                      \
+      if (!VAHEAD) { ATT_VALUES(KB, VCUR) }                                                                             \
+      __builtin_amdgcn_sched_barrier(0);                                                                                \
+      mfma_scores<HD>(kr, qv, e);                                                                                       \
+      if ((KB) + 32 <= pos_last) {                                                                                      \
+        fetch_keys((KB) + 32, page, slot, kr);                                                                          \
+        if (VAHEAD) { ATT_VALUES((KB) + 32, VNEXT) }                                                                    \
+      }                                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                                \
+      /* the exponentials' arguments; a key the query does not see: an argument whose exponential is 0 */               \
+      if (!((KB) + 31 <= pos_first && (KB) >= lo_last)) {                                                               \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                                                \
+          const int key = (KB) + 8 * (r >> 2) + key_of_reg + (r & 3);                                                   \
+          e[r] = (key >= lo_q && key <= pos_q) ? e[r] * a.scale - mx : -200.0f;                                         \
+        }                                                                                                               \
+      } else {                                                                                                          \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) e[r] = e[r] * a.scale - mx;                                      \
+      }                                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                                \
+      _Pragma("unroll") for (int g2 = 0; g2 < 4; ++g2) {                                                                \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) e[4 * g2 + i] = bw_expf_select(e[4 * g2 + i]);                    \
+        float t = sum;                                                                                                  \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) t += e[4 * g2 + i];   /* meaningful in the lower half */          \
+        t = __uint_as_float(__builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false)[0]); \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) t += e[4 * g2 + i];   /* meaningful in the upper half */          \
+        sum = __uint_as_float(__builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false)[1]); \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
+          _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                             \
+            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x1f32(e[4 * g2 + i], VCUR[8 * g2 + i][nb], acc[nb], 1, 0, 0);      \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                   \
+          _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                                                             \
+            acc[nb] = __builtin_amdgcn_mfma_f32_32x32x1f32(e[4 * g2 + i], VCUR[8 * g2 + 4 + i][nb], acc[nb], 1, 1, 0);  \
+      }                                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                                \
+    }
+    if constexpr (VAHEAD) {
+      ATT_VALUES(lo_min, va)
+      for (int kb = lo_min; kb <= pos_last; kb += 64) {
+        ATT_PASS2(kb, va, vb)
+        if (kb + 32 <= pos_last) ATT_PASS2(kb + 32, vb, va)
+      }
+    } else {
+      for (int kb = lo_min; kb <= pos_last; kb += 32) ATT_PASS2(kb, va, va)
+    }
+#undef ATT_PASS2
+#undef ATT_VALUES
+  }
+  // out[q][d] = acc[q][d] * (1 / sum[q]): register r of block b is query 8 (r / 4) + 4 h2 + r % 4, element 64 nb + 32 b + col
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int q = 8 * (r >> 2) + key_of_reg + (r & 3);
+    const float inv_q = __shfl(inv, q, 64);
+    if (q >= ntok) continue;
+    float* o = a.out + (size_t)(row0 + q) * a.out_stride + (size_t)h * HD;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int d = 64 * nb + 32 * b + col;
+        if (d < HD) o[d] = acc[nb][16 * b + r] * inv_q;
+      }
+  }
+}
+
 template <int HD>
 static void launch_attention_f32_tiles(const AttnF32Args& a, dim3 grid, hipStream_t s) {
   static bool allowed = false;
@@ -481,7 +811,13 @@ static void launch_attention_f32(const AttnF32Args& a, dim3 grid, hipStream_t s)
 static int attention_f32_dispatch(const AttnF32Args& a, int items, int tiled, hipStream_t s) {
   if (a.kv_heads <= 0 || a.heads % a.kv_heads || a.heads > 65535) return -2;
   dim3 grid(items, a.heads);
-#define BW_CASE(HD) case HD: if (tiled) launch_attention_f32_tiles<HD>(a, grid, s); else launch_attention_f32<HD>(a, grid, s); break;
+#define BW_CASE(HD) case HD:                                                                                          \
+    if (tiled == 2) {                                                                                                \
+      const int groups = (((items + 1) >> 1) + 3) >> 2;                                                                  \
+      hipLaunchKernelGGL(attention_f32_mfma_kernel<HD>, dim3(groups * a.heads), dim3(512), 0, s, a, items, groups);      \
+    } else if (tiled) launch_attention_f32_tiles<HD>(a, grid, s);                                                        \
+    else launch_attention_f32<HD>(a, grid, s);                                                                           \
+    break;
 #define BW_ROWS(HD) case HD: if (tiled) return -4; launch_attention_f32<HD>(a, grid, s); break;
   switch (a.head_dim) {
     BW_CASE(16) BW_CASE(32) BW_CASE(48) BW_CASE(64) BW_CASE(80) BW_CASE(96) BW_CASE(112) BW_CASE(128)
@@ -505,8 +841,9 @@ extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* pos
 }
 
 // The same over a list of tiles ([tiles][4] = row0, tokens, sequence, 0; a tile's rows are consecutive rows of one
-// sequence in position order).  tiled = 1: a workgroup per tile of up to 16 rows (head sizes up to 128; -4
-// otherwise); tiled = 0: a workgroup per tile's first row (tiles of one row).  Both give the bits of bw_attention_f32.
+// sequence in position order).  tiled = 1: a workgroup per tile of up to 16 rows; tiled = 2: a wave per tile of up to
+// 32 rows, both products on the matrix cores (head sizes up to 128; -4 otherwise); tiled = 0: a workgroup per tile's
+// first row (tiles of one row).  All give the bits of bw_attention_f32.
 extern "C" int bw_attention_f32_tiles(const float* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                                       int table_stride, const int32_t* tiles, int num_tiles, int tiled,
                                       const float* k_cache, const float* v_cache, float* out, int out_stride, int heads,

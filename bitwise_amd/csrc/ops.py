@@ -393,11 +393,13 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
 
 
 def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
-                        num_tiles: int, tiled: bool, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                        num_tiles: int, tiled, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                         heads: int, kv_heads: int, head_dim: int, page_size: int, window: int, scale: float) -> None:
     """``attention_f32`` over tiles ([tiles, 4] int32 = first row, rows, request, 0; a tile's rows are consecutive
-    rows of one request).  ``tiled``: a workgroup per tile of up to 16 rows, keys and values shared through LDS
-    (head sizes up to 128); else a workgroup per tile's first row.  The bits are those of ``attention_f32``."""
+    rows of one request).  ``tiled`` True (1): a workgroup per tile of up to 16 rows, keys and values shared
+    through LDS; 2: a wave per tile of up to 32 rows, both products as chains of single-step matrix instructions
+    (head sizes up to 128 either way); False: a workgroup per tile's first row.  The bits are those of
+    ``attention_f32``."""
     _need(q, torch.float32, "q")
     _need(out, torch.float32, "out")
     _need(k_cache, torch.float32, "k_cache")
@@ -412,7 +414,7 @@ def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: t
     if heads % kv_heads:
         raise ValueError("attention: heads must be a multiple of kv_heads")
     _check(_fn("bw_attention_f32_tiles")(q.data_ptr(), q.stride(0), positions.data_ptr(), block_table.data_ptr(),
-                                         block_table.stride(0), tiles.data_ptr(), int(num_tiles), int(bool(tiled)),
+                                         block_table.stride(0), tiles.data_ptr(), int(num_tiles), int(tiled),
                                          k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
                                          kv_heads, head_dim, page_size, int(window), float(scale), _stream()),
            "attention_f32_tiles")

@@ -155,7 +155,10 @@ class Attention(Mixer):
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              ws.page_size, call.writes_cache)
             out = ws.buffer("attn_out", self.q_dim, torch.float32)
-            plan = plan_tiles(ctx, 16, 1)
+            # prompt portions: tiles of 32 rows, a wave a tile, both products on the matrix cores; for head sizes
+            # that fill the second product's blocks badly (80 to 112) tiles of 16 rows on the vector units
+            on_matrix_cores = self.head_dim <= 64 or self.head_dim == 128
+            plan = plan_tiles(ctx, 32 if on_matrix_cores else 16, 1)
             common = (call.k_cache, call.v_cache, out, self.heads, self.kv_heads, self.head_dim, ws.page_size,
                       window, self.scale)
             if plan.fold_count and self.head_dim > 128 or (plan.decode_count and plan.decode_tiles is None):
@@ -164,7 +167,8 @@ class Attention(Mixer):
                                   self.heads, self.kv_heads, self.head_dim, ws.page_size, window, self.scale)
             else:
                 if plan.fold_count:      # prompt portions: a tile's rows share the keys and values they load
-                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.fold_tiles, plan.fold_count, True, *common)
+                    ops.attention_f32_tiles(qkv, ctx.positions, table, plan.fold_tiles, plan.fold_count,
+                                            2 if on_matrix_cores else 1, *common)
                 if plan.decode_count:
                     ops.attention_f32_tiles(qkv, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common)
             self.o.add_into(ws, out, residual, rows)

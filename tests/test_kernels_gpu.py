@@ -422,9 +422,10 @@ def paged_setup(gpu, bf16, heads, kvh, hd, page, pages, n_keys, seed, poison=Fal
 
 
 def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=0, split=False, tiles=None,
-                  shared=False):
+                  shared=False, mfma=False):
     """split: the decode kernel (a wave per partition); shared: it may also split a tile over
-    workgroups that meet in device scratch (given full of NaN: only what a launch wrote may be read)."""
+    workgroups that meet in device scratch (given full of NaN: only what a launch wrote may be read);
+    mfma (32-bit): a wave per tile of up to 32 rows, both products on the matrix cores."""
     rows = len(positions)
     pos = torch.tensor(positions, dtype=torch.int32, device=gpu)
     scale = 1.0 / float(hd) ** 0.5
@@ -432,8 +433,8 @@ def run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, wi
         out = torch.zeros(rows, heads * hd, device=gpu)
         if tiles is not None:                      # a workgroup a tile of rows, or (tiles of one row) a tile's row
             t = torch.tensor(tiles, dtype=torch.int32, device=gpu)
-            ops.attention_f32_tiles(q.to(gpu), pos, tab, t, len(tiles), any(n != 1 for _, n, _, _ in tiles), kc, vc, out,
-                                    heads, kvh, hd, page, window, scale)
+            ops.attention_f32_tiles(q.to(gpu), pos, tab, t, len(tiles), 2 if mfma else any(n != 1 for _, n, _, _ in tiles),
+                                    kc, vc, out, heads, kvh, hd, page, window, scale)
             return out
         ops.attention_f32(q.to(gpu), pos, torch.zeros(rows, dtype=torch.int32, device=gpu), tab, kc, vc, out, rows,
                           heads, kvh, hd, page, window, scale)
@@ -537,6 +538,10 @@ def test_attention_random_shapes(gpu):
             tpt = rnd.choice([1, 3, 16])
             tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
             assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles), single), what
+            tpt = rnd.choice([1, 5, 32])                          # and on the matrix cores
+            tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+            assert torch.equal(run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles,
+                                             mfma=True), single), what
         ref = plain_rows(q, k, v, positions, heads, window=window or None)
         assert (single.cpu().double() - ref).abs().max() <= (2e-2 if bf16 else 5e-6) * ref.abs().max().clamp(min=0.05), what
 
@@ -577,6 +582,14 @@ def test_attention_prompt_tiles_equal_single_rows(gpu, bf16):
             tiled = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles)
             alone = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window)
             assert torch.equal(tiled, alone), (window, tpt)
+        # the same on the matrix cores (tiles of up to 32 rows)
+        for window, tpt in ((0, 32), (0, 1), (37, 32), (37, 7), (5, 16), (70, 3), (33, 27)):
+            tiles = [(off, min(tpt, len(positions) - off), 0, 0) for off in range(0, len(positions), tpt)]
+            tiled = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, tiles=tiles, mfma=True)
+            alone = run_attention(gpu, bf16, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window)
+            assert torch.equal(tiled, alone), ("matrix cores", window, tpt)
+        first = run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page, tiles=[(0, 20, 0, 0)], mfma=True)
+        assert torch.equal(first, run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page))
         first = run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page, tiles=[(0, 16, 0, 0), (16, 4, 0, 0)])
         assert torch.equal(first, run_attention(gpu, bf16, q[:20], list(range(20)), tab, kc, vc, heads, kvh, hd, page))
     ref = plain_rows(q, k, v, positions, heads)
