@@ -333,6 +333,139 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
   }
 }
 
+// ------------------------------------------------------------------------------ up to 16 rows: a wave a row
+
+// Decoded tokens, the same chains with the operands brought another way.  A workgroup owns 64 columns and all
+// (up to 16) rows; wave m is row m, lane l the chain of (row m, column n0 + l).  Weights and rows travel from
+// memory straight into LDS (buffer loads with LDS as destination: 8 rows of W, 128 bytes each, or 4 rows of x, 256
+// bytes each, an instruction; whole cache lines, the 16-byte chunks of a row of W permuted against bank conflicts;
+// a ring of stages, waits by counting loads).  The weights stay packed there: a lane reads its column's 16-byte
+// chunks and widens them in registers.  A row's elements are the same for the whole wave: every lane reads the same
+// address, which costs LDS one access.  Against the kernel above (every thread reads a 32-bit element of x and one
+// of W from LDS for each multiply-add) a multiply-add here needs 2 bytes of W from LDS (bfloat16 weights) instead of
+// 4 of W and 4 of x.  For products with at least as many blocks of 64 columns as there are compute units.
+// K a multiple of a stage (64 bfloat16 or 32 32-bit elements), rows 16-byte aligned.
+#define F32L_MIN_BLOCKS 256                                           // fewer blocks of 64 columns than compute units: the kernel above (16 columns a workgroup)
+#define F32L_STAGES 8
+#define F32L_W (64 * 128)                                             // 64 rows of W, 128 bytes each
+#define F32L_X (16 * 256)                                             // 16 rows of x, up to 64 elements each
+#define F32L_STAGE (F32L_W + F32L_X)
+
+// A wave's loads of one stage (a device function rather than a lambda in the kernel: the host pass drops, without a
+// word, kernel templates whose lambdas capture arrays of dependent size): LPW of W and one of x.
+template <int LPW>
+__device__ __forceinline__ void lanes_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_w, __amdgpu_buffer_rsrc_t rs_x, const int* voff,
+                                            int voff_x, int wave, int nwaves, int step, int steps, int w_step, int x_step) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = lds + (step % F32L_STAGES) * F32L_STAGE;
+  unsigned char* dump = lds + F32L_STAGES * F32L_STAGE;               // where loads that bring nothing put their zeros
+  const bool real = step < steps;                                     // scalar
+#pragma unroll
+  for (int t = 0; t < LPW; ++t) {
+    const int blk = wave + t * nwaves;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(blk < 8 ? dst + blk * 1024 : dump), 16, real ? voff[t] : 0x7ffffff0,
+                                             step * w_step, 0, 0);
+  }
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(wave < 4 ? dst + F32L_W + wave * 1024 : dump), 16,
+                                           real ? voff_x : 0x7ffffff0, step * x_step, 0, 0);
+}
+
+// LPW: loads of W a wave issues per stage (8 in all; waves past the eighth, and what does not divide, issue loads
+// outside the descriptor: no traffic, zeros into a spare KB behind the ring), so that every wave counts alike.
+template <typename WT, int LPW>
+__global__ __launch_bounds__(1024) void gemm_f32_lanes_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                              float* __restrict__ y, int M, int N, int K, int ldx, int ldy,
+                                                              int accumulate) {
+  constexpr int EPC = 16 / (int)sizeof(WT);                           // elements in a 16-byte chunk
+  constexpr int KS = 128 / (int)sizeof(WT);                           // elements of k a stage
+  extern __shared__ __attribute__((aligned(16))) unsigned char lanes_lds[];   // [stages][W: 64 rows of 128 B | x: 16 rows of 256 B], 1 KB
+  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int n0 = blockIdx.x * 64;
+  const int w_rows = min(64, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0,
+                                                                        (int)((size_t)w_rows * K * sizeof(WT)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)((((size_t)M - 1) * ldx + K) * 4), 0x00020000);
+  // loads of W: lane l of a load fetches row l / 8 of its 8 rows, chunk (l % 8) ^ (row within 16 >> 1) of the row's 128 bytes
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff[LPW];
+#pragma unroll
+  for (int t = 0; t < LPW; ++t) {
+    const int blk = wave + t * nwaves;                                // which 8 rows of the 64
+    const int row = 8 * blk + lrow;
+    voff[t] = blk < 8 ? (int)((row * K) * (int)sizeof(WT) + 16 * (lslot ^ ((row & 15) >> 1))) : 0x7ffffff0;
+  }
+  // loads of x (waves 0 to 3): lane l fetches row 4 wave + l / 16, its chunk l % 16 of the stage's KS elements (rows
+  // past M and, with 32-bit weights, chunks past the stage: outside, or never read)
+  const int xrow = 4 * wave + (lane >> 4), xchunk = lane & 15;
+  const int voff_x = (wave < 4 && xrow < M && 4 * xchunk < KS) ? (xrow * ldx + 4 * xchunk) * 4 : 0x7ffffff0;
+  const int steps = K / KS;
+#pragma unroll
+  for (int st = 0; st < F32L_STAGES - 1; ++st) lanes_issue<LPW>(lanes_lds, rs_w, rs_x, voff, voff_x, wave, nwaves, st, steps, 128, KS * 4);
+  // this lane's row of the tile: chunk j lies in slot j ^ (row within 16 >> 1)
+  const int my = (lane >> 3) * 1024 + (lane & 7) * 128, swz = (lane & 15) >> 1;
+  float acc = 0.0f;
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only((LPW + 1) * (F32L_STAGES - 2)));   // all but the loads of the stages after this one have landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    lanes_issue<LPW>(lanes_lds, rs_w, rs_x, voff, voff_x, wave, nwaves, step + F32L_STAGES - 1, steps, 128, KS * 4);   // into the stage worked on a step ago
+    const unsigned char* stage = lanes_lds + (step % F32L_STAGES) * F32L_STAGE;
+    const unsigned char* xs = stage + F32L_W + wave * 256;            // the wave's row: the same address in every lane
+    u32x4 v[8];                                                       // the stage's eight chunks of W, asked for at once
+    f32x4 xv[KS / 4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const u32x4*>(stage + my + ((j ^ swz) * 16));
+#pragma unroll
+    for (int j = 0; j < KS / 4; ++j) xv[j] = *reinterpret_cast<const f32x4*>(xs + 16 * j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (sizeof(WT) == 2) {                                // bfloat16 -> 32-bit: the bits, shifted (exact)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc = fmaf(xv[2 * j + (e >> 1)][2 * (e & 1)], __uint_as_float(v[j][e] << 16), acc);
+          acc = fmaf(xv[2 * j + (e >> 1)][2 * (e & 1) + 1], __uint_as_float(v[j][e] & 0xffff0000u), acc);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = fmaf(xv[j][e], __uint_as_float(v[j][e]), acc);
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                          // the padding loads too, before the wave ends
+  const int n = n0 + lane;
+  if (n >= N) return;
+  float* o = y + (size_t)wave * ldy + n;
+  *o = accumulate ? (*o + acc) : acc;
+}
+
+template <typename WT, int LPW>
+static void launch_lanes_lpw(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                             hipStream_t s) {
+  constexpr int lds_bytes = F32L_STAGES * F32L_STAGE + 1024;
+  static_assert((LPW + 1) * (F32L_STAGES - 2) < 64, "the wait count has six bits");
+  static bool allowed = false;                       // 64 KB of dynamic LDS and more has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_f32_lanes_kernel<WT, LPW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_f32_lanes_kernel<WT, LPW>), dim3((N + 63) / 64), dim3(64 * M), lds_bytes, s, x, w, y, M, N, K, ldx, ldy,
+                     accumulate);
+}
+
+template <typename WT>
+static void launch_lanes(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate,
+                         hipStream_t s) {
+  switch ((8 + M - 1) / M) {                         // loads a wave and stage: 8 over the waves, rounded up
+    case 8: launch_lanes_lpw<WT, 8>(x, w, y, M, N, K, ldx, ldy, accumulate, s); break;
+    case 4: launch_lanes_lpw<WT, 4>(x, w, y, M, N, K, ldx, ldy, accumulate, s); break;
+    case 3: launch_lanes_lpw<WT, 3>(x, w, y, M, N, K, ldx, ldy, accumulate, s); break;
+    case 2: launch_lanes_lpw<WT, 2>(x, w, y, M, N, K, ldx, ldy, accumulate, s); break;
+    default: launch_lanes_lpw<WT, 1>(x, w, y, M, N, K, ldx, ldy, accumulate, s); break;
+  }
+}
+
 // ------------------------------------------------------------------------------ up to 64 rows on the matrix cores
 
 // v_mfma_f32_4x4x1_16b_f32 computes, for 16 blocks of 4 x 4 outputs at once, D[r][j] = fma(A[r], B[j], D[r][j]):
@@ -728,6 +861,13 @@ extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* 
       (size_t)M * ldx * 4 < ((size_t)1 << 31) && (size_t)64 * K * 4 < ((size_t)1 << 31)) {
     if (w_is_bf16) launch_f32_mfma_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
     else launch_f32_mfma_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
+  // up to 16 rows, many columns, K in whole stages: a wave a row, weights packed in LDS
+  if (M <= 16 && (N + 63) / 64 >= F32L_MIN_BLOCKS && K % (w_is_bf16 ? 64 : 32) == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 &&
+      ((uintptr_t)w & 15) == 0 && (size_t)64 * K * 4 < ((size_t)1 << 31) && (size_t)M * ldx * 4 < ((size_t)1 << 31)) {
+    if (w_is_bf16) launch_lanes<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    else launch_lanes<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
     return BW_LAUNCH_CHECK();
   }
   if (M <= 64 && K % wc == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) {
