@@ -730,7 +730,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }                                                                                                                 \
       __builtin_amdgcn_sched_barrier(0);                                                                                \
       _Pragma("unroll") for (int g2 = 0; g2 < 4; ++g2) {                                                                \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) e[4 * g2 + i] = bw_expf_select(e[4 * g2 + i]);                    \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) e[4 * g2 + i] = bw_expf(e[4 * g2 + i]);                    \
         float t = sum;                                                                                                  \
         _Pragma("unroll") for (int i = 0; i < 4; ++i) t += e[4 * g2 + i];   /* meaningful in the lower half */          \
         t = __uint_as_float(__builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false)[0]); \

@@ -48,26 +48,7 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
 // Arguments below -87 give 0 (the result would be under the smallest normal number), arguments above 89
 // give +inf, NaN stays NaN; exp(0) is exactly 1.
 __device__ __forceinline__ float bw_expf(float x) {
-  if (!(x >= -87.0f)) return (x != x) ? x : 0.0f;
-  if (x > 89.0f) return __builtin_inff();
-  const float kf = __builtin_rintf(x * 0x1.715476p+0f);
-  float r = fmaf(kf, -0x1.62e4p-1f, x);
-  r = fmaf(kf, -0x1.7f7d1cp-20f, r);
-  float p = 0x1.a01a02p-13f;
-  p = fmaf(p, r, 0x1.6c16c2p-10f);
-  p = fmaf(p, r, 0x1.111112p-7f);
-  p = fmaf(p, r, 0x1.555556p-5f);
-  p = fmaf(p, r, 0x1.555556p-3f);
-  p = fmaf(p, r, 0.5f);
-  p = fmaf(p, r, 1.0f);
-  p = fmaf(p, r, 1.0f);
-  const int k = (int)kf, k1 = k >> 1, k2 = k - k1;          // both within [-64, 64]
-  return (p * __uint_as_float((uint32_t)(k1 + 127) << 23)) * __uint_as_float((uint32_t)(k2 + 127) << 23);
-}
-
-// The same statements without a branch (selects at the end): for kernels whose matrix instructions must not end up
-// under a partial execution mask.  The same bits for every argument.
-__device__ __forceinline__ float bw_expf_select(float x) {
+  // no branch, selects at the end: a kernel's matrix instructions must not end up under a partial execution mask
   const float xc = fminf(fmaxf(x, -87.0f), 89.0f);          // (NaN becomes -87; the selects below put it back)
   const float kf = __builtin_rintf(xc * 0x1.715476p+0f);
   float r = fmaf(kf, -0x1.62e4p-1f, xc);
@@ -80,7 +61,7 @@ __device__ __forceinline__ float bw_expf_select(float x) {
   p = fmaf(p, r, 0.5f);
   p = fmaf(p, r, 1.0f);
   p = fmaf(p, r, 1.0f);
-  const int k = (int)kf, k1 = k >> 1, k2 = k - k1;
+  const int k = (int)kf, k1 = k >> 1, k2 = k - k1;          // both within [-64, 64]
   float y = (p * __uint_as_float((uint32_t)(k1 + 127) << 23)) * __uint_as_float((uint32_t)(k2 + 127) << 23);
   y = x > 89.0f ? __builtin_inff() : y;
   y = !(x >= -87.0f) ? ((x != x) ? x : 0.0f) : y;
