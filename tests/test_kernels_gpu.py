@@ -99,6 +99,25 @@ def test_gemm_f32_grid_rows_and_accumulate(gpu):
             before = batch.clone()
             ops.gemm_f32(x, weight, batch, M, accumulate=True)
             assert torch.equal(batch, before + before)
+    # many columns and up to 16 rows (a wave a row, weights packed in LDS): the bits of the same rows inside a product of
+    # 20 rows (matrix cores) and of the chain-per-thread kernel (K + 8 is no whole stage of the first)
+    for M, N, K in [(1, 16400, 64), (8, 16384, 2048), (16, 20000, 128), (5, 16385, 192), (13, 16500, 96)]:
+        x, w = torch.randn(20, K + 8, generator=g).to(gpu), (torch.randn(N, K + 8, generator=g) * 0.1).to(gpu)
+        for weight in (w, w.bfloat16()):
+            xs, ws = x[:, :K].contiguous(), weight[:, :K].contiguous()
+            few, many = torch.full((M, N), 3.0, device=gpu), torch.zeros(20, N, device=gpu)
+            ops.gemm_f32(xs[:M].contiguous(), ws, few, M)
+            ops.gemm_f32(xs, ws, many, 20)
+            assert torch.equal(few, many[:M]), (M, N, K, weight.dtype)
+            before = few.clone()
+            ops.gemm_f32(xs[:M].contiguous(), ws, few, M, accumulate=True)
+            assert torch.equal(few, before + before)
+            # the longer rows through the other kernel: zeros in the last 8 places of x leave every chain's value
+            xz = x[:M].clone()
+            xz[:, K:] = 0.0
+            longer = torch.zeros(M, N, device=gpu)
+            ops.gemm_f32(xz, weight, longer, M)
+            assert torch.equal(longer, before), (M, N, K, weight.dtype)
 
 
 def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
