@@ -702,27 +702,159 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
 // workgroup then counts itself in, and the one that finds all others counted in folds all
 // partials, again in partition order from the first: the same statements on the same values.
 // The counter is back at zero when the kernel ends.
+// The fold of ``count`` parked partials, in partition order.  Often a single wave has all the output elements, and
+// a wave alone issues an instruction every four clocks whatever the instruction: the work is cut so that the serial
+// part is a few instructions a partition.  The factors of fold() for a partition depend only on the column's maxima
+// up to it, and a running maximum can be had without running: first a thread per (eight partitions, column) takes
+// their maximum; then a thread per (partition, column) takes the maximum of the eights before its own, of the
+// partitions of its eight before it and of the passes before, and computes the two factors with fold_scalars() from
+// the same two values fold() would see; then an output element's chain is a read, a product and a fused
+// multiply-add a partition (the sums' chains run in other threads beside them).  The same statements on the same
+// values as fold(): the same bits.  Sums and values wait in LDS between passes; the last pass divides and writes.
+//
+// The workgroup's LDS: three rows a column, padded to whole eights of partitions (a partition's two factors and its
+// sum times its factor, each row read four partitions at a time); two rows of 16 running maxima (a pass reads one
+// and writes the other) and the 16 sums; the eights' maxima; the output elements' values; then the partials
+// [pcap][hpt][m, l, hd values].
+struct FoldLds {
+  float* fa;                    // [hpt][row]: the factor of what has been folded so far
+  float* fb;                    //             the factor of the partition's partial
+  float* lb;                    //             the partial's sum times fb
+  float* mcol;
+  float* lsum;
+  float* eights;
+  float* state;
+  float* parts;
+  int row;                      // floats from column to column of the factors
+  __device__ __forceinline__ FoldLds(float* base, int pcap, int hpt, int hd) {
+    row = (pcap + 7) & ~7;
+    fa = base;
+    fb = fa + row * hpt;
+    lb = fb + row * hpt;
+    mcol = lb + row * hpt;
+    lsum = mcol + 32;
+    eights = lsum + 16;
+    state = eights + fold_lds_eights(pcap, hpt);
+    parts = state + ((hpt * hd + 1) & ~1);
+  }
+  __host__ __device__ static int fold_lds_eights(int pcap, int hpt) { return (((pcap + 7) >> 3) * hpt + 1) & ~1; }
+  static size_t bytes(int pcap, int hpt, int hd) {
+    return ((size_t)3 * ((pcap + 7) & ~7) * hpt + 48 + fold_lds_eights(pcap, hpt) + (size_t)((hpt * hd + 1) & ~1) +
+            (size_t)pcap * hpt * (hd + 2)) * sizeof(float);
+  }
+};
+
 template <int HD, int W>
-__device__ __forceinline__ void decode_fold_pass(const AttnBf16Args& a, const float* parts, int count,
-                                                 float (&m)[(16 * HD + 64 * W - 1) / (64 * W)],
-                                                 float (&l)[(16 * HD + 64 * W - 1) / (64 * W)],
-                                                 float (&o)[(16 * HD + 64 * W - 1) / (64 * W)]) {
-  constexpr int THREADS = 64 * W, EPT = (16 * HD + THREADS - 1) / THREADS, CELL = HD + 2;
-  const int elems = a.hpt * HD;
+__device__ __forceinline__ void decode_fold_pass(const AttnBf16Args& a, const GroupCtx& gc, const FoldLds& lds, int count,
+                                                 int pass, bool final_pass, int row) {
+  constexpr int THREADS = 64 * W, CELL = HD + 2;
+  const float* parts = lds.parts;
+  const float* m_before = lds.mcol + 16 * (pass & 1);
+  float* m_after = lds.mcol + 16 * ((pass & 1) ^ 1);
+  const int pairs = count * a.hpt, eights = ((count + 7) >> 3) * a.hpt;
+  for (int c = threadIdx.x; c < eights; c += THREADS) {
+    const int k0 = (c / a.hpt) * 8, col = c % a.hpt;
+    float m = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    const int e = threadIdx.x + j * THREADS;
-    if (e >= elems) continue;
-    const int col = e / HD, d = e % HD;
-    for (int wv = 0; wv < count; ++wv) {
-      const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
-      const float m_p = cell[0], l_p = cell[1], o_p = cell[2 + d];
-      float mn, fa, fb;
-      fold_scalars(m[j], m_p, mn, fa, fb);
-      l[j] = fmaf(l[j], fa, l_p * fb);
-      o[j] = fmaf(o[j], fa, o_p * fb);
-      m[j] = mn;
+    for (int u = 0; u < 8; ++u)       // (past the last partition: the last one again)
+      m = max2_raw(m, parts[((size_t)min(k0 + u, count - 1) * a.hpt + col) * CELL]);
+    lds.eights[c] = m;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += THREADS) {
+    const int wv = p / a.hpt, col = p % a.hpt, full = wv >> 3;
+    float m = pass == 0 ? -INFINITY : m_before[col];
+    // every read is asked for before the first is used, eight at a time; an index past the end reads the last
+    // again, which a maximum does not mind
+    for (int c = 0; c < full; c += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = lds.eights[min(c + u, full - 1) * a.hpt + col];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) m = max2_raw(m, v[u]);
     }
+    const float* cell = parts + ((size_t)wv * a.hpt + col) * CELL;
+    const float m_p = cell[0], l_p = cell[1];
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = parts[((size_t)min(8 * full + u, count - 1) * a.hpt + col) * CELL];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) m = max2_raw(m, 8 * full + u < wv ? v[u] : -INFINITY);
+    float mn, fa, fb;
+    fold_scalars(m, m_p, mn, fa, fb);
+    lds.fa[col * lds.row + wv] = fa;
+    lds.fb[col * lds.row + wv] = fb;
+    lds.lb[col * lds.row + wv] = l_p * fb;
+    if (wv == count - 1) m_after[col] = mn;
+  }
+  __syncthreads();
+  const int elems = a.hpt * HD, cstride = a.hpt * CELL, group = a.heads / a.kv_heads, tail = count & ~7;
+  // the sums' chains: the last threads, a column each
+  if ((int)threadIdx.x >= THREADS - a.hpt) {
+    const int col = THREADS - 1 - (int)threadIdx.x;
+    const f32x4* fa4 = reinterpret_cast<const f32x4*>(lds.fa + col * lds.row);
+    const f32x4* lb4 = reinterpret_cast<const f32x4*>(lds.lb + col * lds.row);
+    float lj = pass == 0 ? 0.0f : lds.lsum[col];
+    for (int wv = 0; wv < tail; wv += 8) {
+      const f32x4 f0 = fa4[wv >> 2], f1 = fa4[(wv >> 2) + 1], b0 = lb4[wv >> 2], b1 = lb4[(wv >> 2) + 1];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) lj = fmaf(lj, f0[u], b0[u]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) lj = fmaf(lj, f1[u], b1[u]);
+    }
+    for (int wv = tail; wv < count; ++wv) lj = fmaf(lj, lds.fa[col * lds.row + wv], lds.lb[col * lds.row + wv]);
+    lds.lsum[col] = lj;
+  }
+  for (int e = threadIdx.x; e < elems; e += THREADS) {
+    const int col = e / HD, d = e % HD;
+    const f32x4* fa4 = reinterpret_cast<const f32x4*>(lds.fa + col * lds.row);
+    const f32x4* fb4 = reinterpret_cast<const f32x4*>(lds.fb + col * lds.row);
+    const float* cell = parts + (size_t)col * CELL + 2 + d;
+    float oj = pass == 0 ? 0.0f : lds.state[e];
+    // The next eight partitions' operands are on their way while this eight's chain runs.  Past the last partition
+    // the factors' padding and the last partial again are read, and not used.
+    f32x4 fa_n[2], fb_n[2];
+    float op_n[8];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      fa_n[i] = fa4[i];
+      fb_n[i] = fb4[i];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) op_n[u] = cell[min(u, count - 1) * cstride];
+#pragma unroll 2
+    for (int wv = 0; wv < tail; wv += 8) {
+      f32x4 fa_c[2], fb_c[2];
+      float op_c[8];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa_c[i] = fa_n[i];
+        fb_c[i] = fb_n[i];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) op_c[u] = op_n[u];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa_n[i] = fa4[((wv + 8) >> 2) + i];
+        fb_n[i] = fb4[((wv + 8) >> 2) + i];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) op_n[u] = cell[min(wv + 8 + u, count - 1) * cstride];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) oj = fmaf(oj, fa_c[u >> 2][u & 3], op_c[u] * fb_c[u >> 2][u & 3]);
+    }
+#pragma unroll
+    for (int u = 0; u < 7; ++u)
+      if (tail + u < count) oj = fmaf(oj, fa_n[u >> 2][u & 3], op_n[u] * fb_n[u >> 2][u & 3]);
+    lds.state[e] = oj;
+  }
+  if (!final_pass) return;
+  __syncthreads();
+  for (int e = threadIdx.x; e < elems; e += THREADS) {
+    const int col = e / HD, d = e % HD;
+    if (gc.sub * a.hpt + col >= group) continue;       // columns of a one-token tile: column c is head sub*hpt + c of the kv head's group
+    const float inv = 1.0f / lds.lsum[col];
+    a.out[(size_t)row * a.out_stride + (size_t)(gc.kvh * group + gc.sub * a.hpt + col) * HD + d] = f32_to_bf16(lds.state[e] * inv);
   }
 }
 
@@ -748,29 +880,34 @@ __device__ __forceinline__ void store_partial(const AttnBf16Args& a, const Group
 }
 
 template <int HD, int W, bool SPLIT>
-__global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a, int pcap, float* __restrict__ scratch,
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void attention_decode_kernel(AttnBf16Args a, int pcap, float* __restrict__ scratch,
                                                                   int* __restrict__ counters, int max_parts) {
   constexpr int NT = HD / 16;
   constexpr int THREADS = 64 * W;
-  constexpr int EPT = (16 * HD + THREADS - 1) / THREADS;   // output elements per thread at most (16 live columns)
   constexpr int CELL = HD + 2;                              // m, l, then hd values
   constexpr bool PREFETCH = HD <= 64 && !SPLIT;
-  extern __shared__ __attribute__((aligned(16))) float parts[];   // [pcap][hpt][CELL]
+  extern __shared__ __attribute__((aligned(16))) float lds_base[];
+  const FoldLds lds(lds_base, pcap, a.hpt, HD);
+  float* const parts = lds.parts;                  // [pcap][hpt][CELL]
   __shared__ int is_last;
   GroupCtx gc;
   TileCtx<HD> tc[1];
+  const int wave = wave_index();
+  // Without a window and with the implicit tile list the first partition is partition 0 of sequence blockIdx.x
+  // whatever the position says: its pages are asked for beside the position, not after it (the table index is
+  // clamped into the row and the pages into the pool, so a sequence shorter than that costs a wasted load).
+  const bool early = a.window == 0 && a.tiles == nullptr;
+  PartPages pg_first;
+  if (early) {
+    gc.r = threadIdx.x & 15;
+    gc.g = (threadIdx.x & 63) >> 4;
+    gc.table = a.block_table + (size_t)blockIdx.x * a.table_stride;
+    load_pages(a, gc, (SPLIT ? (int)blockIdx.z * W : 0) + wave, pg_first);
+  }
   const bool live = group_setup<HD, 1>(a, blockIdx.x, blockIdx.y, gc, tc);   // uniform over the workgroup
   if (!SPLIT && !live) return;
-  const int wave = wave_index();
   const int first = gc.kmin / ATT_PART, last = gc.kmax / ATT_PART;
-  const int elems = a.hpt * HD;
-  float m[EPT], l[EPT], o[EPT];
-#pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    m[j] = -INFINITY;
-    l[j] = 0.0f;
-    o[j] = 0.0f;
-  }
+  const int row = a.tiles != nullptr ? a.tiles[blockIdx.x * 4] : blockIdx.x;
   if constexpr (SPLIT) {
     const int item = blockIdx.x * gridDim.y + blockIdx.y;
     float* mine = scratch + (size_t)item * max_parts * a.hpt * CELL;
@@ -779,7 +916,8 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
       KFrags<HD> kf;
       VFrags<HD> vf;
       for (int part = first + blockIdx.z * W + wave; part <= last; part += W * gridDim.z) {
-        load_pages(a, gc, part, pg);
+        if (early && part == (int)blockIdx.z * W + wave) pg = pg_first;
+        else load_pages(a, gc, part, pg);
         load_keys<HD>(a, gc, part, pg, kf);
         load_values<HD>(a, gc, pg, vf);
         float m_p, l_p;
@@ -832,7 +970,7 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
         }
       }
       __syncthreads();
-      decode_fold_pass<HD, W>(a, parts, count, m, l, o);
+      decode_fold_pass<HD, W>(a, gc, lds, count, (pass0 - first) / pcap, pass0 + pcap > last, row);
       __syncthreads();
     }
   } else {
@@ -842,7 +980,8 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
       VFrags<HD> vf, vf_next;
       PartPages pg, pg_now;
       int part = pass0 + wave;
-      load_pages(a, gc, part, pg);
+      if (early && pass0 == 0) pg = pg_first;
+      else load_pages(a, gc, part, pg);
       if constexpr (PREFETCH) {
         load_keys<HD>(a, gc, part, pg, kf);
         load_values<HD>(a, gc, pg, vf);
@@ -871,25 +1010,14 @@ __global__ __launch_bounds__(64 * W) void attention_decode_kernel(AttnBf16Args a
         }
       }
       __syncthreads();
-      decode_fold_pass<HD, W>(a, parts, pass_last - pass0 + 1, m, l, o);
+      decode_fold_pass<HD, W>(a, gc, lds, pass_last - pass0 + 1, (pass0 - first) / pcap, pass_last == last, row);
       __syncthreads();
     }
-  }
-  // columns of a one-token tile: column c is head sub*hpt + c of the kv head's group
-  const int group = a.heads / a.kv_heads;
-  const int row = a.tiles != nullptr ? a.tiles[blockIdx.x * 4] : blockIdx.x;
-#pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    const int e = threadIdx.x + j * THREADS;
-    if (e >= elems) continue;
-    const int col = e / HD, d = e % HD;
-    if (gc.sub * a.hpt + col >= group) continue;
-    const float inv = 1.0f / l[j];
-    a.out[(size_t)row * a.out_stride + (size_t)(gc.kvh * group + gc.sub * a.hpt + col) * HD + d] = f32_to_bf16(o[j] * inv);
   }
 }
 
 #define DECODE_W 8
+#define BW_LDS_BYTES (160 * 1024 - 256)   // a compute unit's LDS less the kernels' few static words
 #define DECODE_W_MANY 4          // waves a workgroup where there are several workgroups for every compute unit
 #define DECODE_MANY 1024          // that many workgroups: a workgroup's last, partly empty round of partitions costs more
                                   // than what a compute unit gains from eight waves' loads in flight
@@ -910,24 +1038,46 @@ static int launch_attention(const AttnBf16Args& a, int decode, float* scratch, s
                             int num_counters, hipStream_t s) {
   const int items = a.kv_heads * a.nsub;
   if (decode) {
-    constexpr int W = DECODE_W;
+    constexpr int W = DECODE_W, WM = DECODE_W_MANY;
     const size_t cell = (size_t)a.hpt * (HD + 2) * sizeof(float);
-    int pcap = (int)((48 * 1024) / cell);          // partitions whose partials fit 48 KB of LDS
-    pcap = pcap < W ? W : (pcap > 256 ? 256 : pcap);
+    // LDS: the partials of ``pcap`` partitions (what fits 48 KB, at least one a wave) and what the fold keeps beside them
+    auto shape = [&](int waves, int& pcap) {
+      pcap = (int)((48 * 1024) / cell);
+      pcap = pcap < waves ? waves : (pcap > 256 ? 256 : pcap);
+      return FoldLds::bytes(pcap, a.hpt, HD);
+    };
+    int pcap;
+    size_t lds_bytes = shape(W, pcap);
     int nsplit, max_parts;
     decode_split_shape(a.num_tiles, items, a.table_stride, a.page_size, nsplit, max_parts);
     if (scratch == nullptr || counters == nullptr) nsplit = 1;
+    bool few_waves = nsplit == 1 && a.num_tiles * items >= DECODE_MANY;
+    if (lds_bytes > BW_LDS_BYTES) {                // sixteen heads of 256 a workgroup: only four waves' partials fit
+      few_waves = true;
+      nsplit = 1;
+    }
+    if (few_waves) lds_bytes = shape(WM, pcap);
+    if (lds_bytes > BW_LDS_BYTES) return -8;
+    // more than 64 KB of dynamic LDS has to be asked for once per kernel
+    static bool allowed[3] = {false, false, false};
+    const int variant = nsplit > 1 ? 0 : (few_waves ? 1 : 2);
+    if (lds_bytes > 48 * 1024 && !allowed[variant]) {
+      const void* fn = variant == 0 ? (const void*)attention_decode_kernel<HD, W, true>
+                     : variant == 1 ? (const void*)attention_decode_kernel<HD, WM, false>
+                                    : (const void*)attention_decode_kernel<HD, W, false>;
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, BW_LDS_BYTES) != hipSuccess) return -8;
+      allowed[variant] = true;
+    }
     if (nsplit > 1) {
       if (scratch_floats < (size_t)a.num_tiles * items * max_parts * a.hpt * (HD + 2) || num_counters < a.num_tiles * items)
         return -6;
-      hipLaunchKernelGGL((attention_decode_kernel<HD, W, true>), dim3(a.num_tiles, items, nsplit), dim3(64 * W), pcap * cell, s,
+      hipLaunchKernelGGL((attention_decode_kernel<HD, W, true>), dim3(a.num_tiles, items, nsplit), dim3(64 * W), lds_bytes, s,
                          a, pcap, scratch, counters, max_parts);
-    } else if (a.num_tiles * items >= DECODE_MANY) {
-      constexpr int WM = DECODE_W_MANY;            // (the partials are folded in partition order whatever the waves: the same bits)
-      hipLaunchKernelGGL((attention_decode_kernel<HD, WM, false>), dim3(a.num_tiles, items), dim3(64 * WM), pcap * cell, s, a,
+    } else if (few_waves) {                        // (the partials are folded in partition order whatever the waves: the same bits)
+      hipLaunchKernelGGL((attention_decode_kernel<HD, WM, false>), dim3(a.num_tiles, items), dim3(64 * WM), lds_bytes, s, a,
                          pcap, nullptr, nullptr, 0);
     } else {
-      hipLaunchKernelGGL((attention_decode_kernel<HD, W, false>), dim3(a.num_tiles, items), dim3(64 * W), pcap * cell, s, a,
+      hipLaunchKernelGGL((attention_decode_kernel<HD, W, false>), dim3(a.num_tiles, items), dim3(64 * W), lds_bytes, s, a,
                          pcap, nullptr, nullptr, 0);
     }
   } else {

@@ -29,6 +29,7 @@ _ERRORS = {
     -4: f"head size not compiled in (supported: {HEAD_DIMS})",
     -5: "page size not supported (a power of two from 4 to 64 is needed)",
     -6: "scratch smaller than attention_decode_scratch asks for",
+    -8: "the workgroup's partials do not fit the compute unit's LDS",
     -7: "sizes beyond what the library's static scratch holds",
 }
 

@@ -580,6 +580,35 @@ def test_decode_attention_with_many_workgroups(gpu):
     assert torch.equal(few, fold[:3])                              # (and of the same kernel with eight waves)
 
 
+@pytest.mark.parametrize("heads,kvh,hd,nkeys,window", [(16, 1, 128, 700, 0), (20, 1, 256, 1500, 0), (7, 1, 64, 4000, 0),
+                                                       (7, 1, 64, 4000, 2500), (3, 3, 16, 300, 0)])
+def test_decode_attention_passes_wide_groups_and_implicit_tiles(gpu, heads, kvh, hd, nkeys, window):
+    """The decode kernel where its LDS is tight: sixteen heads a workgroup (more than 64 KB of partials; at 256 only four
+    waves' fit), contexts of more partitions than LDS holds at once (the sums wait in LDS between passes), and the
+    implicit tile list (tile t = row t of sequence t, whose first pages are asked for before the position is known):
+    the bits of the fold kernel, and the plain result."""
+    page = 16
+    pages = nkeys // page + 3
+    while pages % 7 == 0:
+        pages += 1
+    k, v, kc, vc, tab = paged_setup(gpu, True, heads, kvh, hd, page, pages, nkeys, seed=31, poison=True)
+    positions = [nkeys - 1, nkeys // 2, 70, 3, 0, nkeys - 2]
+    g = torch.Generator().manual_seed(32)
+    q = torch.randn(len(positions), heads * hd, generator=g).bfloat16()
+    fold = run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window)
+    assert torch.equal(run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, split=True), fold)
+    if ops.attention_decode_scratch(len(positions), heads, kvh, hd, tab.stride(0), page)[0]:
+        assert torch.equal(run_attention(gpu, True, q, positions, tab, kc, vc, heads, kvh, hd, page, window=window, split=True,
+                                         shared=True), fold)
+    rows = len(positions)
+    out = torch.zeros(rows, heads * hd, device=gpu, dtype=torch.bfloat16)
+    ops.attention_bf16(q.to(gpu), torch.tensor(positions, dtype=torch.int32, device=gpu), tab.repeat(rows, 1).contiguous(), None,
+                       rows, kc, vc, out, heads, kvh, hd, page, window, 1.0 / float(hd) ** 0.5, decode=True)
+    assert torch.equal(out, fold)
+    ref = plain_rows(q, k, v, positions, heads, window=window or None)
+    assert (fold.cpu().double() - ref).abs().max() <= 2e-2 * ref.abs().max()
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 def test_attention_prompt_tiles_equal_single_rows(gpu, bf16):
     """Rows of a prompt portion share a tile with consecutive positions; each must equal the
