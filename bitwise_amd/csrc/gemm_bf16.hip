@@ -999,26 +999,36 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // NARROW (plain epilogues, at least two blocks of rows): 32 columns a workgroup, the waves arranged as for SwiGLU
 // (strip s, half h of the row blocks), for products with so few columns that 64 a workgroup would leave most
 // compute units idle.
-template <int EPI, int NRB, bool NORM, bool NARROW = false>
+// EIGHT (the narrow and the SwiGLU tiles of 17 rows or more): eight waves, wave (s, b) owns strip s for block b of
+// the rows (with two blocks of rows half the waves only load), and a stage is four steps of 64 along K (two of
+// SwiGLU): what a compute unit pulls grows with its waves and with the bytes between two barriers (64 rows of the
+// output projection: 29 KB a microsecond with four waves and a stage a step, 55 with eight and four steps).  K in
+// whole stages.
+template <int EPI, int NRB, bool NORM, bool NARROW = false, bool EIGHT = false>
 struct MidShape {
   static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   static constexpr bool HALVES = GLU || NARROW;                     // waves are (strip, half of the row blocks)
-  static constexpr int NW = 4;                                      // waves
+  static constexpr int NW = EIGHT ? 8 : 4;                          // waves
+  static constexpr int SUB = EIGHT ? (GLU ? 2 : 4) : 1;             // steps of 64 along K a stage
   static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
-  static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a stage (SwiGLU: 32 gate, 32 up)
-  static constexpr int A_LOADS = NORM ? 0 : (2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
-  static constexpr int B_LOADS = B_ROWS / 8 / NW;                   // 8 rows of W each
+  static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a step (SwiGLU: 32 gate, 32 up)
+  static constexpr int A_LOADS = NORM ? 0 : (SUB * 2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
+  static constexpr int B_LOADS = SUB * B_ROWS / 8 / NW;             // 8 rows of W each
   static constexpr int LPW = A_LOADS + B_LOADS;
-  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STAGE = A_BYTES + B_ROWS * 128;
-  static constexpr int NI = HALVES ? (NRB >= 2 ? NRB / 2 : 1) : NRB; // blocks of rows a wave works on
+  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STEP_BYTES = A_BYTES + B_ROWS * 128, STAGE = SUB * STEP_BYTES;
+  static constexpr int NI = EIGHT ? 1 : (HALVES ? (NRB >= 2 ? NRB / 2 : 1) : NRB); // blocks of rows a wave works on
   static constexpr int NJ = GLU ? 2 : 1;
   static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
-  static constexpr int STAGES = ROPE_NARROW && NRB <= 2 ? 16 : 8;   // (half the weights a stage: twice the stages, where they fit)
+  static constexpr int FIT = 150 * 1024 / STAGE;
+  static constexpr int STAGES = EIGHT ? (FIT > 6 ? 6 : FIT)
+                                      : (ROPE_NARROW && NRB <= 2 ? 16 : 8);   // (half the weights a stage: twice the stages, where they fit)
   static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
   static constexpr int RING = STAGES * STAGE + 1024;                // and 1 KB where padding loads put their zeros
   static_assert(PENDING < 64, "the wait count has six bits");
+  static_assert(STAGES >= 3, "a stage at hand, one landing, one asked for");
   static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
   static_assert(!NARROW || (!GLU && (EPI == EPI_QKV_ROPE || NRB >= 2)), "narrow tiles: plain epilogues of 17 rows or more, or the rotary one");
+  static_assert(!EIGHT || (HALVES && !NORM && NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: the narrow and the SwiGLU tiles of 17 rows or more");
 };
 
 // Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
@@ -1037,24 +1047,32 @@ struct MidNormArgs {
   float eps;
 };
 
+// Where a wave's loads of a stage go and come from.  A load is 8 rows of one step of 64 along K (1 KB): of x, block
+// ``id % (2 NRB)`` of step ``id / (2 NRB)`` of the stage for the wave's id-th load; of W likewise (SwiGLU with eight
+// waves: the first four waves take the gate rows, the others the up rows, so that a wave's loads share a descriptor).
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
+struct MidLoads {
+  using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
+  int voff_a[S::A_LOADS > 0 ? S::A_LOADS : 1], voff_b[S::B_LOADS];   // byte offsets in x (0x7ffffff0: a padding load) and in the tile's rows of W
+  int dst_a[S::A_LOADS > 0 ? S::A_LOADS : 1], dst_b[S::B_LOADS];     // byte offsets in the stage
+};
+
 // A wave's loads of one stage of the ring: its share of the rows of x and of W, LPW instructions.
-template <int EPI, int NRB, bool NORM, bool NARROW>
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
 __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                          const int* voff_a, const int* voff_b, int wave, int step, int steps, int k_base) {
-  using S = MidShape<EPI, NRB, NORM, NARROW>;
+                                          const MidLoads<EPI, NRB, NORM, NARROW, EIGHT>& ld, int step, int steps, int k_base) {
+  using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   unsigned char* dst = lds + (step % S::STAGES) * S::STAGE;
   const bool real = step < steps;                                     // scalar
+  const int k_off = (k_base + step * S::SUB * 64) * 2;
 #pragma unroll
-  for (int t = 0; t < S::A_LOADS; ++t) {
-    const int block = wave * S::A_LOADS + t;                          // 1 KB of the stage's x; a padding load's zeros go behind the ring
-    unsigned char* to = block < 2 * NRB ? dst + block * 1024 : lds + S::STAGES * S::STAGE;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)to, 16, real ? voff_a[t] : 0x7ffffff0, (k_base + step * 64) * 2, 0, 0);
-  }
+  for (int t = 0; t < S::A_LOADS; ++t)                                // (a padding load's zeros go behind the ring)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(ld.dst_a[t] >= 0 ? dst + ld.dst_a[t] : lds + S::STAGES * S::STAGE), 16,
+                                             real ? ld.voff_a[t] : 0x7ffffff0, k_off, 0, 0);
 #pragma unroll
   for (int t = 0; t < S::B_LOADS; ++t)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + S::A_BYTES + (wave * S::B_LOADS + t) * 1024), 16,
-                                             real ? voff_b[t] : 0x7ffffff0, (k_base + step * 64) * 2, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + ld.dst_b[t]), 16, real ? ld.voff_b[t] : 0x7ffffff0, k_off, 0, 0);
 }
 
 // The NORM variant's rows: wave ``wave`` normalises rows wave, wave + 4, ... (RB of them at most) into LDS, the
@@ -1062,7 +1080,7 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
 template <int RB, int EPI, int NRB, bool NARROW>
 __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int K, int wave, int lane, unsigned char* rows_lds,
                                               unsigned char* mid_lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                              const int* voff_a, const int* voff_b, int steps, int k_base) {
+                                              const MidLoads<EPI, NRB, true, NARROW, false>& ld, int steps, int k_base) {
   using S = MidShape<EPI, NRB, true, NARROW>;
   const int nvec = K >> 2;
   NormRows<RB> nr;
@@ -1075,7 +1093,7 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
+  for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW, false>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
   __builtin_amdgcn_sched_barrier(0);
   unsigned char* rl = rows_lds;
   const int nw = S::NW;
@@ -1087,13 +1105,13 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   });
 }
 
-template <int EPI, int NRB, bool NORM, bool NARROW>
-__global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
+__global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW)) void gemm_bf16_mid_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
     MidNormArgs na, QkvRopeArgs rp, MidSplitArgs sp) {
-  using S = MidShape<EPI, NRB, NORM, NARROW>;
+  using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   constexpr bool GLU = S::GLU;
-  constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ;
+  constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ, THREADS = 64 * S::NW;
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
@@ -1112,28 +1130,52 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
       (void*)x, 0, NORM ? 0 : (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
   // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
   const int lrow = lane >> 3, lslot = lane & 7;
-  const int b_first = wave * S::B_LOADS * 8;                         // this wave's first row of the tile's 64 of W
-  const bool up = GLU && b_first >= 32;
+  // which 1 KB of a stage this wave's t-th load of W is: block ``blk`` (8 rows) of step ``sub`` of the stage
+  auto b_load = [&](int t, int& sub, int& blk) {
+    constexpr int PER_STEP = S::B_ROWS / 8;
+    if constexpr (EIGHT && GLU) {                                    // waves 0-3: the gate rows, 4-7: the up rows
+      const int id = (wave & 3) * S::B_LOADS + t;
+      sub = id / (PER_STEP / 2);
+      blk = id % (PER_STEP / 2) + (PER_STEP / 2) * (wave >> 2);
+    } else {
+      const int id = wave * S::B_LOADS + t;
+      sub = id / PER_STEP;
+      blk = id % PER_STEP;
+    }
+  };
+  int sub0, blk0;
+  b_load(0, sub0, blk0);
+  const bool up = GLU && blk0 >= 4;                                  // (all of a wave's loads are of one kind)
   const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
-  int voff_a[S::A_LOADS > 0 ? S::A_LOADS : 1] = {0}, voff_b[S::B_LOADS];
+  MidLoads<EPI, NRB, NORM, NARROW, EIGHT> ld;
 #pragma unroll
   for (int t = 0; t < S::A_LOADS; ++t) {
-    const int row = (wave * S::A_LOADS + t) * 8 + lrow;             // of the NRB * 16 rows of x; past them: a padding load
+    const int id = wave * S::A_LOADS + t, sub = id / (2 * NRB), block = id % (2 * NRB);
+    const int row = block * 8 + lrow;                                // of the NRB * 16 rows of x
     const int chunk = lslot ^ ((row & 15) >> 1);
-    voff_a[t] = row < NRB * 16 ? (row * ldx + 8 * chunk) * 2 : 0x7ffffff0;
+    const bool is_load = id < S::SUB * 2 * NRB;                      // past them: a padding load
+    ld.voff_a[t] = is_load ? (row * ldx + 8 * chunk + 64 * sub) * 2 : 0x7ffffff0;
+    ld.dst_a[t] = is_load ? sub * S::STEP_BYTES + block * 1024 : -1;
+  }
+  if constexpr (S::A_LOADS == 0) {
+    ld.voff_a[0] = 0;
+    ld.dst_a[0] = -1;
   }
 #pragma unroll
   for (int t = 0; t < S::B_LOADS; ++t) {
-    const int row = b_first + 8 * t + lrow;
+    int sub, blk;
+    b_load(t, sub, blk);
+    const int row = blk * 8 + lrow;                                  // of the tile's rows of W
     const int chunk = lslot ^ ((row & 15) >> 1);
     const int w_row = ROPE ? (row < PAIRS ? pair0 + row : half + pair0 + row - PAIRS) : (GLU ? row & 31 : row);
-    voff_b[t] = (w_row * K + 8 * chunk) * 2;
+    ld.voff_b[t] = (w_row * K + 8 * chunk + 64 * sub) * 2;
+    ld.dst_b[t] = sub * S::STEP_BYTES + S::A_BYTES + blk * 1024;
   }
   // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
   // segment after segment, each segment's sums joined to those before it when it ends
   const int k_base = blockIdx.y * GEMM_SEG;
-  const int steps = gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64;
+  const int steps = (gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64) / S::SUB;   // stages
   f32x4 acc[NI][NJ], tot[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -1150,10 +1192,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   const int strip = S::HALVES ? (wave & 1) : wave;                    // of the tile's output columns
   const int a_block0 = S::HALVES ? NI * (wave >> 1) : 0;              // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
+  const bool computing = !EIGHT || a_block0 < NRB;                    // (eight waves, two blocks of rows: half the waves only load)
 
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's columns are a head, or 16 pairs of
   // one): what this thread's (row, pair) items need, cosine, sine and page, hangs on the row's position.
-  constexpr int ITEMS = EPI == EPI_QKV_ROPE ? (RN ? NRB : 2 * NRB) : 1;   // (row, pair) items a thread: 16 * NRB rows x PAIRS
+  constexpr int ITEMS = EPI == EPI_QKV_ROPE ? (16 * NRB * PAIRS + THREADS - 1) / THREADS : 1;   // (row, pair) items a thread: 16 * NRB rows x PAIRS
   int r_pos[ITEMS], r_page[ITEMS];
   float r_cos[ITEMS], r_sin[ITEMS];
   if constexpr (EPI == EPI_QKV_ROPE) {
@@ -1161,7 +1204,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     // is asked for once the ring is under way
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      const int e = threadIdx.x + j * 256;
+      const int e = threadIdx.x + j * THREADS;
       r_pos[j] = e < M * PAIRS ? rp.positions[e >> PSH] : -1;
     }
     asm volatile("" ::: "memory");
@@ -1173,19 +1216,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     // wait for the rows must not be a wait for weights); wave w takes rows w, w + 4, ...: as many at a time as
     // there are (a slot without a row would fetch a row for nothing)
     if (wave < M) {
-      if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
-      else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
-      else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
-      else mid_norm_rows<4, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, voff_a, voff_b, steps, k_base);
+      if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else mid_norm_rows<4, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
     }
     if (wave >= M) {                                                   // a wave without rows still feeds the ring
 #pragma unroll
-      for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
+      for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
     }
     // rows past M stay as LDS holds them: their products are never stored
   } else {
 #pragma unroll
-    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
+    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
   }
   if constexpr (EPI == EPI_QKV_ROPE) {
     // These loads are younger than the ring's first stages: the loop's waits ("all but the last PENDING loads have
@@ -1194,7 +1237,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      const int e = threadIdx.x + j * 256;
+      const int e = threadIdx.x + j * THREADS;
       const int pos = r_pos[j];
       r_page[j] = 0;
       r_cos[j] = 1.f;
@@ -1212,35 +1255,41 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     __builtin_amdgcn_s_waitcnt(vmcnt_only(S::PENDING));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    mid_issue<EPI, NRB, NORM, NARROW>(mid_lds, rs_a, rs_b, voff_a, voff_b, wave, step + S::STAGES - 1, steps, k_base);   // into the stage worked on a step ago
+    mid_issue<EPI, NRB, NORM, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, step + S::STAGES - 1, steps, k_base);   // into the stage worked on a step ago
     const unsigned char* stage = mid_lds + (step % S::STAGES) * S::STAGE;
+    if (computing) {
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      u32x4 fa[NI], fb[NJ];
+      for (int sub = 0; sub < S::SUB; ++sub) {
+        const unsigned char* at = stage + sub * S::STEP_BYTES;         // this step of 64 along K
 #pragma unroll
-      for (int i = 0; i < NI; ++i)
-        fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + step * 2048 : stage) + (a_block0 + i) * 2048 + slot_off[kk]);
+        for (int kk = 0; kk < 2; ++kk) {
+          u32x4 fa[NI], fb[NJ];
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(stage + b_off0 + j * 4096 + slot_off[kk]);
+          for (int i = 0; i < NI; ++i)
+            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + step * 2048 : at) + (a_block0 + i) * 2048 + slot_off[kk]);
 #pragma unroll
-      for (int i = 0; i < NI; ++i)
+          for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(at + b_off0 + j * 4096 + slot_off[kk]);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
-    }
-    asm volatile("" ::: "memory");
-    if constexpr (!NORM) {
-      const int kn = (step + 1) * 64;
-      if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {            // a segment ends before the last: left to right
+          for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
+            for (int j = 0; j < NJ; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
+        }
+        if constexpr (!NORM) {
+          const int kn = (step * S::SUB + sub + 1) * 64;
+          if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {          // a segment ends before the last: left to right
 #pragma unroll
-          for (int j = 0; j < NJ; ++j) {
-            tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
-            acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+              for (int j = 0; j < NJ; ++j) {
+                tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
+                acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+              }
           }
+        }
       }
     }
+    asm volatile("" ::: "memory");
   }
   if constexpr (!NORM) {
     if (K > GEMM_SEG && gridDim.y == 1) {                               // the last segment joins the others
@@ -1266,7 +1315,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      const int e = threadIdx.x + j * 256;
+      const int e = threadIdx.x + j * THREADS;
       const int pos = r_pos[j];
       if (e >= M * PAIRS || pos < 0) continue;
       const int m = e >> PSH, ip = e & (PAIRS - 1), i = pair0 + ip;
@@ -1301,7 +1350,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
         // sums to the residual in segment order, every one of them read back from the scratch (its own too) with
         // device-scope loads issued after the barrier behind the count.  The counter is back at zero when the
         // kernel ends.
-        const int cell = 4 * NI * 1024;                              // bytes of a workgroup's sums: [wave][i][lane] x 16
+        const int cell = S::NW * NI * 1024;                          // bytes of a workgroup's sums: [wave][i][lane] x 16
         const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(
             (void*)((unsigned char*)sp.scratch + (size_t)blockIdx.x * nseg * cell), 0, nseg * cell, 0x00020000);
         const int mine = (wave * NI) * 1024 + lane * 16;
@@ -1345,20 +1394,31 @@ __global__ __launch_bounds__(256) void gemm_bf16_mid_kernel(
   }
 }
 
-template <int EPI, int NRB, bool NORM, bool NARROW = false>
-static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
-                      const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
-                      const MidSplitArgs& sp = MidSplitArgs{}) {
-  using S = MidShape<EPI, NRB, NORM, NARROW>;
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
+static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
+                            const MidNormArgs& na, const QkvRopeArgs& rp, int segments, const MidSplitArgs& sp) {
+  using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
   const int lds_bytes = S::RING + (NORM ? (K / 64) * 2048 : 0);
   if (lds_bytes > 160 * 1024) return -2;
   if (!allowed) {
-    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW>), dim3(wgs, segments), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>), dim3(wgs, segments), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
   return BW_LAUNCH_CHECK();
+}
+
+template <int EPI, int NRB, bool NORM, bool NARROW = false>
+static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
+                      const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
+                      const MidSplitArgs& sp = MidSplitArgs{}) {
+  // 17 rows or more, narrow or SwiGLU tiles, K in whole stages: the eight-wave variant (the same bits)
+  if constexpr (!NORM && NRB >= 2 && (NARROW || EPI == EPI_SWIGLU_BF16)) {
+    if (K % (64 * MidShape<EPI, NRB, NORM, NARROW, true>::SUB) == 0)
+      return launch_mid_waves<EPI, NRB, NORM, NARROW, true>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
+  }
+  return launch_mid_waves<EPI, NRB, NORM, NARROW, false>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
 }
 
 // RMSNorm of up to 16 rows of the residual stream + product with many columns in one kernel; -7: not this shape.
