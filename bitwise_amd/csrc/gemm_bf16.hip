@@ -999,24 +999,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // NARROW (plain epilogues, at least two blocks of rows): 32 columns a workgroup, the waves arranged as for SwiGLU
 // (strip s, half h of the row blocks), for products with so few columns that 64 a workgroup would leave most
 // compute units idle.
-// EIGHT (the narrow and the SwiGLU tiles of 17 rows or more): eight waves, wave (s, b) owns strip s for block b of
-// the rows (with two blocks of rows half the waves only load), and a stage is four steps of 64 along K (two of
-// SwiGLU): what a compute unit pulls grows with its waves and with the bytes between two barriers (64 rows of the
-// output projection: 29 KB a microsecond with four waves and a stage a step, 55 with eight and four steps).  K in
-// whole stages.
+// EIGHT (17 rows or more): eight waves, wave (s, b) owns strip s for one block of the rows (narrow and SwiGLU tiles;
+// with two blocks of rows half the waves only load) or for half of them (64 columns), and a stage is four steps of 64
+// along K (two where a step has 64 rows of W): what a compute unit pulls grows with its waves and with the bytes
+// between two barriers (64 rows of the output projection: 29 KB a microsecond with four waves and a stage a step,
+// 55 with eight and four steps).  K in whole stages.
 template <int EPI, int NRB, bool NORM, bool NARROW = false, bool EIGHT = false>
 struct MidShape {
   static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   static constexpr bool HALVES = GLU || NARROW;                     // waves are (strip, half of the row blocks)
   static constexpr int NW = EIGHT ? 8 : 4;                          // waves
-  static constexpr int SUB = EIGHT ? (GLU ? 2 : 4) : 1;             // steps of 64 along K a stage
   static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
   static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a step (SwiGLU: 32 gate, 32 up)
+  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? 2 : 4) : 1;    // steps of 64 along K a stage
+  static constexpr int STRIPS = COLS / 16, GROUPS = NW / STRIPS;    // wave = (strip of the columns, group of the row blocks)
   static constexpr int A_LOADS = NORM ? 0 : (SUB * 2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
   static constexpr int B_LOADS = SUB * B_ROWS / 8 / NW;             // 8 rows of W each
   static constexpr int LPW = A_LOADS + B_LOADS;
   static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STEP_BYTES = A_BYTES + B_ROWS * 128, STAGE = SUB * STEP_BYTES;
-  static constexpr int NI = EIGHT ? 1 : (HALVES ? (NRB >= 2 ? NRB / 2 : 1) : NRB); // blocks of rows a wave works on
+  static constexpr int NI = NRB >= GROUPS ? NRB / GROUPS : 1;       // blocks of rows a wave works on (fewer blocks than groups: waves that only load)
   static constexpr int NJ = GLU ? 2 : 1;
   static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
   static constexpr int FIT = 150 * 1024 / STAGE;
@@ -1028,7 +1029,7 @@ struct MidShape {
   static_assert(STAGES >= 3, "a stage at hand, one landing, one asked for");
   static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
   static_assert(!NARROW || (!GLU && (EPI == EPI_QKV_ROPE || NRB >= 2)), "narrow tiles: plain epilogues of 17 rows or more, or the rotary one");
-  static_assert(!EIGHT || (HALVES && !NORM && NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: the narrow and the SwiGLU tiles of 17 rows or more");
+  static_assert(!EIGHT || (!NORM && NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: 17 rows or more");
 };
 
 // Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
@@ -1189,10 +1190,10 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   int slot_off[2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
-  const int strip = S::HALVES ? (wave & 1) : wave;                    // of the tile's output columns
-  const int a_block0 = S::HALVES ? NI * (wave >> 1) : 0;              // first block of 16 rows this wave works on
+  const int strip = wave % S::STRIPS;                                 // of the tile's output columns
+  const int a_block0 = NI * (wave / S::STRIPS);                       // first block of 16 rows this wave works on
   const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
-  const bool computing = !EIGHT || a_block0 < NRB;                    // (eight waves, two blocks of rows: half the waves only load)
+  const bool computing = !EIGHT || a_block0 < NRB;                    // (eight waves, two blocks of rows, two strips: half the waves only load)
 
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's columns are a head, or 16 pairs of
   // one): what this thread's (row, pair) items need, cosine, sine and page, hangs on the row's position.
@@ -1413,8 +1414,8 @@ template <int EPI, int NRB, bool NORM, bool NARROW = false>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
                       const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
                       const MidSplitArgs& sp = MidSplitArgs{}) {
-  // 17 rows or more, narrow or SwiGLU tiles, K in whole stages: the eight-wave variant (the same bits)
-  if constexpr (!NORM && NRB >= 2 && (NARROW || EPI == EPI_SWIGLU_BF16)) {
+  // 17 rows or more, K in whole stages: the eight-wave variant (the same bits)
+  if constexpr (!NORM && NRB >= 2) {
     if (K % (64 * MidShape<EPI, NRB, NORM, NARROW, true>::SUB) == 0)
       return launch_mid_waves<EPI, NRB, NORM, NARROW, true>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
   }
