@@ -95,19 +95,13 @@ __device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_til
     if (tc[t].pos_c >= 0) kmin = min(kmin, tc[t].lo_c);
     // columns without a query do not count: what they compute is finite and never stored
     int hi = tc[t].pos_c >= 0 ? tc[t].pos_c : 0x7fffffff, lo = tc[t].pos_c >= 0 ? tc[t].lo_c : -1;
-#pragma unroll
-    for (int off = 8; off >= 1; off >>= 1) {
-      hi = min(hi, __shfl_xor(hi, off, BW_WAVE));
-      lo = max(lo, __shfl_xor(lo, off, BW_WAVE));
-    }
+    hi = row16_min(hi);                                    // (moves between registers, no trip through LDS)
+    lo = row16_max(lo);
     tc[t].all_hi = __builtin_amdgcn_readfirstlane(hi);   // the same in every lane: say so, branches on them are scalar then
     tc[t].all_lo = __builtin_amdgcn_readfirstlane(lo);
   }
-#pragma unroll
-  for (int off = 8; off >= 1; off >>= 1) {
-    kmax = max(kmax, __shfl_xor(kmax, off, BW_WAVE));
-    kmin = min(kmin, __shfl_xor(kmin, off, BW_WAVE));
-  }
+  kmax = row16_max(kmax);
+  kmin = row16_min(kmin);
   gc.kmax = __builtin_amdgcn_readfirstlane(kmax);
   gc.kmin = __builtin_amdgcn_readfirstlane(kmin);
   gc.table = a.block_table + (size_t)seq * a.table_stride;

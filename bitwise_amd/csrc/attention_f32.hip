@@ -399,10 +399,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
       if (key >= lo_q && key <= pos_q) mx = fmaxf(mx, dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR) * a.scale);
     }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 8, 16));
-  mx = fmaxf(mx, __shfl_xor(mx, 4, 16));
-  mx = fmaxf(mx, __shfl_xor(mx, 2, 16));
-  mx = fmaxf(mx, __shfl_xor(mx, 1, 16));
+  mx = row16_max(mx);
 
   // pass 2
   float acc[ND], sum = 0.0f;
@@ -661,7 +658,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 #undef ATT_PASS1
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  {
+    float lower, upper;
+    lane_halves<32>(mx, lower, upper);
+    mx = fmaxf(lower, upper);
+  }
 
   // pass 2: the keys of the next block are asked for when this block's scores are done, its values then too (for
   // heads of up to 64 elements, whose registers allow a second set), so both have a block's time to arrive.

@@ -71,18 +71,88 @@ __device__ __forceinline__ float bw_expf(float x) {
 // exp(x) through the hardware exp2; one fixed instruction sequence wherever it is used.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
-// Sum over the 64 lanes by xor butterflies.  Addition commutes, so every lane ends with
-// the same bits, and the order of additions is the same for every row of every launch.
+// Lane exchanges from register to register (no trip through LDS).  The halves and quarters of the wave by gfx950's
+// lane swaps: of (v, v) swapped, the first result holds in every lane the value of its partner or its own in the
+// lower half (32: lanes 0-31; 16: the even rows of 16 lanes), the second the one in the upper half; an operation
+// that commutes takes the two as they come.  Within a row of 16 lanes by data-parallel moves: l ^ 8 is a rotation
+// of the row by 8, l ^ 4 the mirror image of each 8 lanes followed by that of each 4, l ^ 2 and l ^ 1
+// permutations of each 4.
+template <int OFF>
+__device__ __forceinline__ void lane_halves(float v, float& lower, float& upper) {
+  static_assert(OFF == 32 || OFF == 16, "halves of the wave or of its halves");
+  typedef __attribute__((ext_vector_type(2))) unsigned u2;
+  const unsigned u = __float_as_uint(v);
+  const u2 r = OFF == 32 ? __builtin_amdgcn_permlane32_swap(u, u, false, false) : __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  lower = __uint_as_float(r[0]);
+  upper = __uint_as_float(r[1]);
+}
+
+template <int OFF>
+__device__ __forceinline__ float lane_xor(float v) {
+  const int u = (int)__float_as_uint(v);
+  if constexpr (OFF == 8) {
+    return __uint_as_float((unsigned)__builtin_amdgcn_mov_dpp(u, 0x128, 0xf, 0xf, true));                // row_ror:8
+  } else if constexpr (OFF == 4) {
+    const int h = __builtin_amdgcn_mov_dpp(u, 0x141, 0xf, 0xf, true);                                    // row_half_mirror: l ^ 7
+    return __uint_as_float((unsigned)__builtin_amdgcn_mov_dpp(h, 0x1b, 0xf, 0xf, true));                 // quad_perm [3,2,1,0]: ^ 3
+  } else if constexpr (OFF == 2) {
+    return __uint_as_float((unsigned)__builtin_amdgcn_mov_dpp(u, 0x4e, 0xf, 0xf, true));                 // quad_perm [2,3,0,1]
+  } else {
+    static_assert(OFF == 1, "1, 2, 4 or 8");
+    return __uint_as_float((unsigned)__builtin_amdgcn_mov_dpp(u, 0xb1, 0xf, 0xf, true));                 // quad_perm [1,0,3,2]
+  }
+}
+
+__device__ __forceinline__ int row16_min(int v) {
+  v = min(v, (int)__float_as_uint(lane_xor<8>(__uint_as_float((unsigned)v))));
+  v = min(v, (int)__float_as_uint(lane_xor<4>(__uint_as_float((unsigned)v))));
+  v = min(v, (int)__float_as_uint(lane_xor<2>(__uint_as_float((unsigned)v))));
+  v = min(v, (int)__float_as_uint(lane_xor<1>(__uint_as_float((unsigned)v))));
+  return v;
+}
+
+__device__ __forceinline__ int row16_max(int v) {
+  v = max(v, (int)__float_as_uint(lane_xor<8>(__uint_as_float((unsigned)v))));
+  v = max(v, (int)__float_as_uint(lane_xor<4>(__uint_as_float((unsigned)v))));
+  v = max(v, (int)__float_as_uint(lane_xor<2>(__uint_as_float((unsigned)v))));
+  v = max(v, (int)__float_as_uint(lane_xor<1>(__uint_as_float((unsigned)v))));
+  return v;
+}
+
+// Sum over a row of 16 lanes, and over the 64 lanes, by xor butterflies (offsets 32, 16, 8, 4, 2, 1).  Addition
+// commutes, so every lane ends with the same bits, and the order of additions is the same for every row of every launch.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += lane_xor<8>(v);
+  v += lane_xor<4>(v);
+  v += lane_xor<2>(v);
+  v += lane_xor<1>(v);
+  return v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, BW_WAVE);
+  float a, b;
+  lane_halves<32>(v, a, b);
+  v = a + b;
+  lane_halves<16>(v, a, b);
+  v = a + b;
+  return row16_sum(v);
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, lane_xor<8>(v));
+  v = fmaxf(v, lane_xor<4>(v));
+  v = fmaxf(v, lane_xor<2>(v));
+  v = fmaxf(v, lane_xor<1>(v));
   return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, BW_WAVE));
-  return v;
+  float a, b;
+  lane_halves<32>(v, a, b);
+  v = fmaxf(a, b);
+  lane_halves<16>(v, a, b);
+  v = fmaxf(a, b);
+  return row16_max(v);
 }
 
 // Sum of squares of one row given as 16-byte vectors: lane l owns vectors l, l+64, ... and runs

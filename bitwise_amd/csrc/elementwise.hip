@@ -58,10 +58,7 @@ __global__ void rmsnorm_f32_kernel(const float* __restrict__ x, const WT* __rest
   float acc = 0.0f;
   if (live)
     for (int i = sub; i < dim; i += 16) acc = fmaf(xr[i], xr[i], acc);
-  acc += __shfl_xor(acc, 8, 16);
-  acc += __shfl_xor(acc, 4, 16);
-  acc += __shfl_xor(acc, 2, 16);
-  acc += __shfl_xor(acc, 1, 16);
+  acc = row16_sum(acc);
   if (!live) return;
   const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
   float* yr = y + (size_t)row * dim;
@@ -89,10 +86,7 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_row_kernel(const float* __res
     float acc = 0.0f;
 #pragma unroll 8
     for (int i = threadIdx.x; i < dim; i += 16) acc = fmaf(row_lds[i], row_lds[i], acc);
-    acc += __shfl_xor(acc, 8, 16);
-    acc += __shfl_xor(acc, 4, 16);
-    acc += __shfl_xor(acc, 2, 16);
-    acc += __shfl_xor(acc, 1, 16);
+    acc = row16_sum(acc);
     if (threadIdx.x == 0) inv_lds = 1.0f / sqrtf(acc / (float)dim + eps);
   }
   __syncthreads();
