@@ -1011,7 +1011,7 @@ struct MidShape {
   static constexpr int NW = EIGHT ? 8 : 4;                          // waves
   static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
   static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a step (SwiGLU: 32 gate, 32 up)
-  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? 2 : 4) : 1;    // steps of 64 along K a stage
+  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? (NORM ? 1 : 2) : (NORM ? 2 : 4)) : 1;   // steps of 64 along K a stage (NORM: weights only)
   static constexpr int STRIPS = COLS / 16, GROUPS = NW / STRIPS;    // wave = (strip of the columns, group of the row blocks)
   static constexpr int A_LOADS = NORM ? 0 : (SUB * 2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
   static constexpr int B_LOADS = SUB * B_ROWS / 8 / NW;             // 8 rows of W each
@@ -1021,7 +1021,7 @@ struct MidShape {
   static constexpr int NJ = GLU ? 2 : 1;
   static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
   static constexpr int FIT = 150 * 1024 / STAGE;
-  static constexpr int STAGES = EIGHT ? (FIT > 6 ? 6 : FIT)
+  static constexpr int STAGES = EIGHT ? (NORM ? 8 : (FIT > 6 ? 6 : FIT))
                                       : (ROPE_NARROW && NRB <= 2 ? 16 : 8);   // (half the weights a stage: twice the stages, where they fit)
   static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
   static constexpr int RING = STAGES * STAGE + 1024;                // and 1 KB where padding loads put their zeros
@@ -1029,7 +1029,7 @@ struct MidShape {
   static_assert(STAGES >= 3, "a stage at hand, one landing, one asked for");
   static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
   static_assert(!NARROW || (!GLU && (EPI == EPI_QKV_ROPE || NRB >= 2)), "narrow tiles: plain epilogues of 17 rows or more, or the rotary one");
-  static_assert(!EIGHT || (!NORM && NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: 17 rows or more");
+  static_assert(!EIGHT || NORM || (NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: 17 rows or more, or rows normalised in the kernel");
 };
 
 // Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
@@ -1078,11 +1078,11 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
 
 // The NORM variant's rows: wave ``wave`` normalises rows wave, wave + 4, ... (RB of them at most) into LDS, the
 // ring's first stages asked for between the rows' loads and the arithmetic.
-template <int RB, int EPI, int NRB, bool NARROW>
+template <int RB, int EPI, int NRB, bool NARROW, bool EIGHT>
 __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int K, int wave, int lane, unsigned char* rows_lds,
                                               unsigned char* mid_lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                              const MidLoads<EPI, NRB, true, NARROW, false>& ld, int steps, int k_base) {
-  using S = MidShape<EPI, NRB, true, NARROW>;
+                                              const MidLoads<EPI, NRB, true, NARROW, EIGHT>& ld, int steps, int k_base) {
+  using S = MidShape<EPI, NRB, true, NARROW, EIGHT>;
   const int nvec = K >> 2;
   NormRows<RB> nr;
   const f32x4* nrows[RB];
@@ -1094,7 +1094,7 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW, false>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
+  for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
   __builtin_amdgcn_sched_barrier(0);
   unsigned char* rl = rows_lds;
   const int nw = S::NW;
@@ -1217,10 +1217,15 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     // wait for the rows must not be a wait for weights); wave w takes rows w, w + 4, ...: as many at a time as
     // there are (a slot without a row would fetch a row for nothing)
     if (wave < M) {
-      if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-      else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-      else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-      else mid_norm_rows<4, EPI, NRB, NARROW>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      if constexpr (EIGHT) {                                           // wave w takes rows w and w + 8
+        if (M <= 8) mid_norm_rows<1, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else mid_norm_rows<2, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      } else {
+        if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else mid_norm_rows<4, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      }
     }
     if (wave >= M) {                                                   // a wave without rows still feeds the ring
 #pragma unroll
@@ -1267,7 +1272,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
           u32x4 fa[NI], fb[NJ];
 #pragma unroll
           for (int i = 0; i < NI; ++i)
-            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + step * 2048 : at) + (a_block0 + i) * 2048 + slot_off[kk]);
+            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + (step * S::SUB + sub) * 2048 : at) + (a_block0 + i) * 2048 + slot_off[kk]);
 #pragma unroll
           for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(at + b_off0 + j * 4096 + slot_off[kk]);
 #pragma unroll
@@ -1414,8 +1419,9 @@ template <int EPI, int NRB, bool NORM, bool NARROW = false>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
                       const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
                       const MidSplitArgs& sp = MidSplitArgs{}) {
-  // 17 rows or more, K in whole stages: the eight-wave variant (the same bits)
-  if constexpr (!NORM && NRB >= 2) {
+  // 17 rows or more, or rows normalised in the kernel (a row a wave sooner done than two), K in whole stages: the
+  // eight-wave variant (the same bits)
+  if constexpr (NORM || NRB >= 2) {
     if (K % (64 * MidShape<EPI, NRB, NORM, NARROW, true>::SUB) == 0)
       return launch_mid_waves<EPI, NRB, NORM, NARROW, true>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
   }
