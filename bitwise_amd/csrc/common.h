@@ -199,25 +199,25 @@ __device__ __forceinline__ f32x4 load_norm_w4(const void* __restrict__ w, int is
   return norm_w_floats(load_norm_w_raw(w, is_bf16, c), is_bf16);
 }
 
-// RMSNorm of up to R rows of at most 2048 elements (a multiple of 4) by one wave, in two phases:
-// every load is issued in the first (vector indices past the row are clamped, missing rows read
+// RMSNorm of up to R rows of at most 256 NV elements (a multiple of 4; NV vectors of four a lane) by one wave, in
+// two phases: every load is issued in the first (vector indices past the row are clamped, missing rows read
 // the first row, so nothing is conditional), everything is computed in the second.  Between
 // them the caller may put other loads in flight: memory results are waited for in issue order,
 // so what is issued later does not hold the reductions up.  rows[0] must be a row; rows[j]
 // null skips row j.  The order is that of row_sumsq_vec and of the store loop of
 // rmsnorm_bf16_kernel: lane l owns vectors l, l+64, ...; ``store(j, c, packed)`` receives vector
 // c of row j as four bfloat16 in 8 bytes.
-template <int R>
+template <int R, int NV = 8>
 struct NormRows {
-  f32x4 v[R][8];
-  u32x4 w[8];
+  f32x4 v[R][NV];
+  u32x4 w[NV];
 };
 
-template <int R>
-__device__ __forceinline__ void norm_rows_load(NormRows<R>& nr, const f32x4* const (&rows)[R], const void* __restrict__ w,
+template <int R, int NV = 8>
+__device__ __forceinline__ void norm_rows_load(NormRows<R, NV>& nr, const f32x4* const (&rows)[R], const void* __restrict__ w,
                                                int w_is_bf16, int nvec, int lane) {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const int c = 64 * j + lane < nvec ? 64 * j + lane : nvec - 1;
     nr.w[j] = load_norm_w_raw(w, w_is_bf16, c);
 #pragma unroll
@@ -225,15 +225,15 @@ __device__ __forceinline__ void norm_rows_load(NormRows<R>& nr, const f32x4* con
   }
 }
 
-template <int R, typename Store>
-__device__ __forceinline__ void norm_rows_finish(const NormRows<R>& nr, const f32x4* const (&rows)[R], int w_is_bf16,
+template <int R, int NV = 8, typename Store>
+__device__ __forceinline__ void norm_rows_finish(const NormRows<R, NV>& nr, const f32x4* const (&rows)[R], int w_is_bf16,
                                                  int nvec, int dim, float eps, int lane, Store store) {
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     if (rows[i] == nullptr) continue;
     float acc = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NV; ++j) {
       const bool in = 64 * j + lane < nvec;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -244,7 +244,7 @@ __device__ __forceinline__ void norm_rows_finish(const NormRows<R>& nr, const f3
     acc = wave_sum(acc);
     const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NV; ++j) {
       const int c = 64 * j + lane;
       if (c < nvec) {
         const f32x4 wv = norm_w_floats(nr.w[j], w_is_bf16);

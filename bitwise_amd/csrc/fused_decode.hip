@@ -330,13 +330,14 @@ extern "C" int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, in
   DecodeGemmArgs a{};
   a.a = x; a.norm_w = norm_w; a.w = (const bf16_t*)w; a.out = out;
   a.M = M; a.N = N; a.K = K; a.lda = ldx; a.ldo = ldo; a.norm_w_is_bf16 = norm_w_is_bf16; a.eps = eps;
-  const int bad = check_decode_gemm(a);
-  if (bad) return bad;
-  if (ldo < N) return -2;
+  if (ldo < N || (ldx % 4) || ldx < K) return -2;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
-  // many columns: the kernel whose workgroups share the normalised rows among four strips and one ring
+  // many columns: the kernel whose workgroups share the normalised rows among their strips and one ring (it alone
+  // takes rows of two segments of K)
   const int mid = bw_norm_gemm_mid(x, ldx, norm_w, norm_w_is_bf16, eps, w, out, ldo, M, N, K, epilogue, stream);
   if (mid != -7) return mid;
+  const int bad = check_decode_gemm(a);
+  if (bad) return bad;
   const int waves = 4;                                   // strips per workgroup (their rings: 64 KB of LDS)
   const int strips = (N + 15) / 16;
   const int blocks = (strips + waves - 1) / waves;
@@ -369,8 +370,7 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.page_size = page_size;
   a.table_stride = table_stride; a.write_cache = write_cache;
   a.pairs = pairs;
-  const int bad = check_decode_gemm(a);
-  if (bad) return bad;
+  if ((a.lda % 4) || a.lda < K || K <= 0 || (K % 64) || M > 16) return -2;
   if ((reinterpret_cast<uintptr_t>(a.a) | reinterpret_cast<uintptr_t>(a.w)) & 15) return -3;
   if ((size_t)(pairs ? 32 : head_dim) * sizeof(float) > (size_t)(K + 8) * sizeof(bf16_t)) return -2;   // the epilogue reuses the LDS rows
   // many heads of 64: the kernel whose workgroups are a head each, four strips sharing the normalised rows and one ring
@@ -378,6 +378,8 @@ extern "C" int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w
                                        table_stride, cos_table, sin_table, k_cache, v_cache, M, heads, kv_heads, head_dim, K,
                                        page_size, write_cache, stream);
   if (mid != -7) return mid;
+  const int bad = check_decode_gemm(a);
+  if (bad) return bad;
   const int all_heads = heads + 2 * kv_heads;
   if (pairs) return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, 2, all_heads * pairs, (hipStream_t)stream);
   return launch_decode_gemm<DEPI_ROPE_KV, 10>(a, head_dim / 16, all_heads, (hipStream_t)stream);

@@ -1046,6 +1046,8 @@ struct MidNormArgs {
   const void* norm_w;    // [K]
   int ldx32, norm_w_is_bf16;
   float eps;
+  int row_step;          // bytes of LDS a step of 64 along K of the normalised rows takes: 2048 (16 rows), or 1024
+                         // (8 rows: rows of up to two segments of K, which are normalised a wave a row)
 };
 
 // Where a wave's loads of a stage go and come from.  A load is 8 rows of one step of 64 along K (1 KB): of x, block
@@ -1078,13 +1080,13 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
 
 // The NORM variant's rows: wave ``wave`` normalises rows wave, wave + 4, ... (RB of them at most) into LDS, the
 // ring's first stages asked for between the rows' loads and the arithmetic.
-template <int RB, int EPI, int NRB, bool NARROW, bool EIGHT>
+template <int RB, int NV, int EPI, int NRB, bool NARROW, bool EIGHT>
 __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int K, int wave, int lane, unsigned char* rows_lds,
                                               unsigned char* mid_lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
                                               const MidLoads<EPI, NRB, true, NARROW, EIGHT>& ld, int steps, int k_base) {
   using S = MidShape<EPI, NRB, true, NARROW, EIGHT>;
   const int nvec = K >> 2;
-  NormRows<RB> nr;
+  NormRows<RB, NV> nr;
   const f32x4* nrows[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
@@ -1097,11 +1099,11 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, true, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
   __builtin_amdgcn_sched_barrier(0);
   unsigned char* rl = rows_lds;
-  const int nw = S::NW;
+  const int nw = S::NW, row_step = na.row_step;
   norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
     // vector c = elements 4c..4c+3 of row m: step c / 16, 16-byte chunk (c % 16) / 2 of the step, its half c % 2
     const int m = wave + i * nw;
-    unsigned char* p = rl + (c >> 4) * 2048 + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ (m >> 1)) * 16) + (c & 1) * 8;
+    unsigned char* p = rl + (c >> 4) * row_step + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ ((m & 15) >> 1)) * 16) + (c & 1) * 8;
     *reinterpret_cast<u32x2*>(p) = pk;
   });
 }
@@ -1218,13 +1220,15 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     // there are (a slot without a row would fetch a row for nothing)
     if (wave < M) {
       if constexpr (EIGHT) {                                           // wave w takes rows w and w + 8
-        if (M <= 8) mid_norm_rows<1, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else mid_norm_rows<2, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        // (rows of two segments: sixteen vectors a lane, and by the launch no more than a row a wave)
+        if (K > GEMM_SEG) mid_norm_rows<1, 16, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else if (M <= 8) mid_norm_rows<1, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else mid_norm_rows<2, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
       } else {
-        if (M <= 4) mid_norm_rows<1, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else if (M <= 8) mid_norm_rows<2, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else if (M <= 12) mid_norm_rows<3, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else mid_norm_rows<4, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        if (M <= 4) mid_norm_rows<1, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else if (M <= 8) mid_norm_rows<2, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else if (M <= 12) mid_norm_rows<3, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+        else mid_norm_rows<4, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
       }
     }
     if (wave >= M) {                                                   // a wave without rows still feeds the ring
@@ -1272,7 +1276,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
           u32x4 fa[NI], fb[NJ];
 #pragma unroll
           for (int i = 0; i < NI; ++i)
-            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + (step * S::SUB + sub) * 2048 : at) + (a_block0 + i) * 2048 + slot_off[kk]);
+            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + (step * S::SUB + sub) * na.row_step : at) + (a_block0 + i) * 2048 + slot_off[kk]);
 #pragma unroll
           for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(at + b_off0 + j * 4096 + slot_off[kk]);
 #pragma unroll
@@ -1281,7 +1285,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
             for (int j = 0; j < NJ; ++j)
               acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb[j]), acc[i][j], 0, 0, 0);
         }
-        if constexpr (!NORM) {
+        if constexpr (!NORM || EIGHT) {
           const int kn = (step * S::SUB + sub + 1) * 64;
           if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {          // a segment ends before the last: left to right
 #pragma unroll
@@ -1297,7 +1301,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     }
     asm volatile("" ::: "memory");
   }
-  if constexpr (!NORM) {
+  if constexpr (!NORM || EIGHT) {
     if (K > GEMM_SEG && gridDim.y == 1) {                               // the last segment joins the others
 #pragma unroll
       for (int i = 0; i < NI; ++i)
@@ -1405,7 +1409,7 @@ static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, 
                             const MidNormArgs& na, const QkvRopeArgs& rp, int segments, const MidSplitArgs& sp) {
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
-  const int lds_bytes = S::RING + (NORM ? (K / 64) * 2048 : 0);
+  const int lds_bytes = S::RING + (NORM ? (K / 64) * na.row_step + (na.row_step == 1024 ? 1024 : 0) : 0);   // (8-row blocks: the reads of rows 8 to 15 end a block further)
   if (lds_bytes > 160 * 1024) return -2;
   if (!allowed) {
     (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1433,8 +1437,11 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
                      int ldo, int M, int N, int K, int epilogue, void* stream) {
   const int cols = epilogue == EPI_SWIGLU_BF16 ? 32 : 64;
   const int wgs = (N + cols - 1) / cols;
-  if (M > 16 || K > GEMM_SEG || K % 64 || wgs < 64) return -7;
-  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
+  if (M > 16 || K % 64 || wgs < 64) return -7;
+  // rows of two segments of K: eight of them at most (a row a wave, sixteen vectors a lane; LDS holds 8-row blocks)
+  const bool wide = K > GEMM_SEG;
+  if (wide && (M > 8 || K > 2 * GEMM_SEG || K % 128)) return -7;
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, wide ? 1024 : 2048};
   const bf16_t* wp = (const bf16_t*)w;
   hipStream_t s = (hipStream_t)stream;
   switch (epilogue) {
@@ -1444,6 +1451,11 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
     case EPI_SWIGLU_BF16: return launch_mid<EPI_SWIGLU_BF16, 1, true>(nullptr, wp, out, M, N, K, 0, ldo, wgs, s, na);
   }
   return -7;
+}
+
+// Whether bw_norm_gemm_mid takes rows of this width that the other fused kernels do not (wider than a segment of K).
+extern "C" int bw_norm_gemm_wide_supported(int M, int N, int K, int cols) {
+  return M > 0 && M <= 8 && K > GEMM_SEG && K <= 2 * GEMM_SEG && K % 128 == 0 && cols > 0 && (N + cols - 1) / cols >= 64;
 }
 
 #define ROPE_NARROW_BELOW 256
@@ -1475,9 +1487,11 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
                          int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream) {
   const int all_heads = heads + 2 * kv_heads;
   const int wide_tiles = all_heads * (head_dim / 64);
-  if (head_dim % 64 || M > 16 || K > GEMM_SEG || K % 64 || wide_tiles < 64)
+  if (head_dim % 64 || M > 16 || K % 64 || wide_tiles < 64)
     return -7;
-  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps};
+  const bool wide = K > GEMM_SEG;                       // as in bw_norm_gemm_mid
+  if (wide && (M > 8 || K > 2 * GEMM_SEG || K % 128)) return -7;
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, wide ? 1024 : 2048};
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
                  heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size), head_dim};

@@ -61,6 +61,7 @@ _SIGS = {
     "bw_attention_decode_scratch": [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_attention_fold_group_tiles": [c_int],
     "bw_norm_gemm_supported": [c_int, c_int],
+    "bw_norm_gemm_wide_supported": [c_int, c_int, c_int, c_int],
     "bw_norm_gemm_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
     "bw_norm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -308,11 +309,23 @@ def qkv_rope_head_dim_ok(head_dim: int, inner: int) -> bool:
     return (32 if head_dim % 32 == 0 else head_dim) * 4 <= (inner + 8) * 2
 
 
-def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor) -> bool:
-    """Whether RMSNorm + product can run as one kernel for this step."""
+def norm_gemm_wide_supported(rows: int, tiles_of: int, columns: int, inner: int) -> bool:
+    """Rows wider than a segment of K (2048): up to 8 of them, up to two segments, for products with at least 64
+    workgroups of ``columns`` output columns (``tiles_of`` columns in all)."""
+    key = (rows, tiles_of, columns, inner)
+    if key not in _decode_ok:
+        _decode_ok[key] = bool(_fn("bw_norm_gemm_wide_supported")(rows, tiles_of, inner, columns))
+    return _decode_ok[key]
+
+
+def can_fuse_norm(rows: int, weight: torch.Tensor, x: torch.Tensor, columns: int = 64, stacked: int = 1) -> bool:
+    """Whether RMSNorm + product can run as one kernel for this step.  ``columns``: output columns a workgroup of the
+    kernel for many columns (32 for SwiGLU and for heads in halves, else 64); ``stacked``: weights stacked in ``weight``
+    (2 for gate|up)."""
     K = weight.shape[1]
-    return (weight.dtype == torch.bfloat16 and x.dtype == torch.float32 and x.shape[1] == K
-            and x.stride(0) % 4 == 0 and norm_gemm_supported(rows, K))
+    if not (weight.dtype == torch.bfloat16 and x.dtype == torch.float32 and x.shape[1] == K and x.stride(0) % 4 == 0):
+        return False
+    return norm_gemm_supported(rows, K) or norm_gemm_wide_supported(rows, weight.shape[0] // stacked, columns, K)
 
 
 def norm_gemm_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
@@ -325,7 +338,8 @@ def norm_gemm_bf16(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: to
     if epilogue == EPI_SWIGLU_BF16:
         N //= 2
     _need(out, torch.bfloat16 if epilogue in (EPI_BF16, EPI_SWIGLU_BF16) else torch.float32, "out")
-    if not can_fuse_norm(rows, w, x) or norm_weight.numel() != K or not norm_weight.is_cuda:
+    glu = epilogue == EPI_SWIGLU_BF16
+    if not can_fuse_norm(rows, w, x, 32 if glu else 64, 2 if glu else 1) or norm_weight.numel() != K or not norm_weight.is_cuda:
         raise ValueError(f"norm_gemm_bf16: {rows} rows of width {x.shape[1]} against weight {tuple(w.shape)} cannot be fused")
     if out.shape[1] != N or out.shape[0] < rows or x.shape[0] < rows:
         raise ValueError("norm_gemm_bf16: out does not fit")

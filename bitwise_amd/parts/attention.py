@@ -117,8 +117,11 @@ class Attention(Mixer):
         """Decode steps of few rows: norm, q|k|v product, rotation and cache write are one kernel."""
         from .norm import RMSNorm
         rt, ws = self.rt, ctx.ws
-        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma
-                and ops.qkv_rope_head_dim_ok(self.head_dim, self.qkv.weight.shape[1])
+        inner = self.qkv.weight.shape[1]
+        # (rows wider than a segment of K: only the kernel with a workgroup per half head takes them)
+        takes_width = inner <= 2048 or ops.qkv_rope_gemm_ok(ctx.rows, self.head_dim, inner, self.heads + 2 * self.kv_heads)
+        if not (rt.bf16 and isinstance(norm, RMSNorm) and self.qkv.mfma and takes_width
+                and ops.qkv_rope_head_dim_ok(self.head_dim, inner)
                 and ops.can_fuse_norm(ctx.rows, self.qkv.weight, x)):
             return False
         q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)

@@ -47,7 +47,7 @@ class SwiGLU(FeedForward):
         from .norm import RMSNorm
         rt, ws = self.rt, ctx.ws
         if not (rt.bf16 and isinstance(norm, RMSNorm) and self.gate_up.mfma and self.down.mfma
-                and ops.can_fuse_norm(ctx.rows, self.gate_up.weight, x)):
+                and ops.can_fuse_norm(ctx.rows, self.gate_up.weight, x, columns=32, stacked=2)):
             return False
         act = ws.buffer("mlp_h", self.inter, torch.bfloat16)
         ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.gate_up.weight, act, ctx.rows, ops.EPI_SWIGLU_BF16)

@@ -748,7 +748,8 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
     must give the bits of the kernels run one after the other."""
     g = torch.Generator().manual_seed(14)
     for M, K, N in [(1, 64, 48), (5, 128, 500), (8, 2048, 6144), (16, 192, 112), (13, 1024, 72),
-                    (16, 192, 4100), (1, 64, 4096), (11, 2048, 4224)]:   # many columns: another kernel
+                    (16, 192, 4100), (1, 64, 4096), (11, 2048, 4224),    # many columns: another kernel
+                    (8, 4096, 4096), (5, 4096, 8200), (3, 2176, 4160), (1, 3968, 4224)]:   # rows of two segments of K, up to 8 of them
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
         nw = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().to(gpu)
         w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
@@ -766,13 +767,18 @@ def test_fused_norm_products_equal_the_separate_kernels(gpu):
             ops.norm_gemm_bf16(x, nw.float(), 1e-5, w, fused_s, M, ops.EPI_SWIGLU_BF16)
             assert torch.equal(fused_s, sep_s), (M, K, N)
     assert not ops.can_fuse_norm(17, w, x) and not ops.can_fuse_norm(4, torch.zeros(8, 4096, dtype=torch.bfloat16), x)
+    wide_x, wide_w = torch.zeros(9, 4096), torch.zeros(4096, 4096, dtype=torch.bfloat16)
+    assert ops.can_fuse_norm(8, wide_w, wide_x) and not ops.can_fuse_norm(9, wide_w, wide_x)           # wide rows: 8 at most,
+    assert not ops.can_fuse_norm(8, wide_w[:4032], wide_x) and ops.can_fuse_norm(8, wide_w[:4032], wide_x, columns=32, stacked=2) is False   # 64 workgroups,
+    assert not ops.can_fuse_norm(4, torch.zeros(4096, 4160, dtype=torch.bfloat16), torch.zeros(4, 4160))   # two segments
     assert not ops.can_fuse_norm(4, torch.zeros(8, 96, dtype=torch.bfloat16), torch.zeros(4, 96))   # steps of 64 along the rows
     assert not ops.qkv_rope_head_dim_ok(48, 64) and ops.qkv_rope_head_dim_ok(48, 192) and ops.qkv_rope_head_dim_ok(256, 64)   # the epilogue's LDS
 
     for heads, kvh, hd, page, K in [(4, 2, 16, 16, 64), (3, 1, 32, 8, 128), (32, 32, 64, 16, 2048), (6, 2, 48, 32, 192),
                                      (2, 1, 128, 16, 256), (3, 3, 96, 16, 128), (40, 12, 64, 32, 128),    # the last two: half a head a workgroup,
                                      (200, 28, 64, 16, 64),                                           # a head a workgroup
-                                     (24, 4, 128, 16, 128), (12, 2, 256, 8, 64), (100, 14, 128, 16, 64)]:     # larger heads: 16 or 32 pairs a workgroup
+                                     (24, 4, 128, 16, 128), (12, 2, 256, 8, 64), (100, 14, 128, 16, 64),      # larger heads: 16 or 32 pairs a workgroup
+                                     (32, 8, 128, 16, 4096), (40, 12, 64, 32, 2176)]:                 # rows of two segments of K
         M, pages = 7, 12
         cos, sin = rope_tables(10000.0, hd, 100, gpu)
         x = (torch.randn(M, K, generator=g) * 2).to(gpu)
