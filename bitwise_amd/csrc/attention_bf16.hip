@@ -696,6 +696,7 @@ __global__ __launch_bounds__(64 * FoldShape<HD>::NW) __attribute__((amdgpu_waves
 // workgroup then counts itself in, and the one that finds all others counted in folds all
 // partials, again in partition order from the first: the same statements on the same values.
 // The counter is back at zero when the kernel ends.
+
 // The fold of ``count`` parked partials, in partition order.  Often a single wave has all the output elements, and
 // a wave alone issues an instruction every four clocks whatever the instruction: the work is cut so that the serial
 // part is a few instructions a partition.  The factors of fold() for a partition depend only on the column's maxima
