@@ -44,20 +44,20 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return cfg["num_hidden_layers"] * (per_token * tokens + attn) + 2 * h * v      # the head runs for one row
 
 
-def make_engine(bw, model, batch: int, steps_total: int, dtype: str):
+def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT):
     block = 16
-    per_request = CONTEXT + steps_total + 2 * block
+    per_request = context + steps_total + 2 * block
     cfg = bw.EngineConfig(num_blocks=batch * ((per_request + block - 1) // block) + 8, max_batched_tokens=2048,
                           max_num_seqs=max(batch, 1), prefix_caching=False, fingerprint_logits=False,
-                          block_size=block, dtype=dtype, max_model_len=4096)
+                          block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024))
     return bw.Engine(model, None, cfg)
 
 
-def fill(engine, bw, torch, batch: int, vocab: int, new_tokens: int, seed: int):
-    """Admit ``batch`` requests with CONTEXT random tokens each and run their prompts."""
+def fill(engine, bw, torch, batch: int, vocab: int, new_tokens: int, seed: int, context: int = CONTEXT):
+    """Admit ``batch`` requests with ``context`` random tokens each and run their prompts."""
     g = torch.Generator().manual_seed(seed)
     for _ in range(batch):
-        prompt = torch.randint(0, vocab, (CONTEXT,), generator=g).tolist()
+        prompt = torch.randint(0, vocab, (context,), generator=g).tolist()
         engine.add_request(prompt, bw.SamplingParams(temperature=0.0, max_new_tokens=new_tokens, ignore_eos=True))
     while engine.num_waiting or any(s.computed < s.prompt_len for s in engine.sched.running):
         engine.step()
@@ -106,16 +106,19 @@ def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float) 
             "frac": round(flops / (ms * 1e-3) / peak_flops, 4)}
 
 
-def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int) -> dict:
-    """``steps`` decode steps of ``batch`` requests that each hold a 2,048-token context: tokens a second, and
-    the bytes a step has to read (every weight once, the cache of the live requests) over its time."""
+def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
+                   context: int = CONTEXT) -> dict:
+    """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
+    said otherwise): tokens a second, and the bytes a step has to read (every weight once, the cache of the live
+    requests) over its time."""
     torch.cuda.empty_cache()
-    # Requests admitted early decode while the later ones are still being prefilled (one prompt a
-    # step): every request gets enough new tokens to outlast the prefills, the warm-up and the
+    # Requests admitted early decode while the later ones are still being prefilled (2,048 prompt
+    # tokens a step): every request gets enough new tokens to outlast the prefills, the warm-up and the
     # timed steps, so that each timed step has all ``batch`` rows.
-    new_tokens = steps + warmup + batch + 8
-    eng = make_engine(bw, model, batch, new_tokens, dtype)
-    fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch)
+    chunks = (context + 2047) // 2048                  # steps a prompt takes under the 2,048-token budget
+    new_tokens = steps + warmup + batch * chunks + 8
+    eng = make_engine(bw, model, batch, new_tokens, dtype, context)
+    fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch, context=context)
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)
     assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
@@ -124,7 +127,7 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     ms = secs / steps * 1e3
     # keys a decoded token reads, on average: the prompt, what the request decoded while later
     # prompts were prefilled, the warm-up, and half the timed steps
-    avg_ctx = CONTEXT + (batch - 1) / 2 + warmup + (steps + 1) / 2
+    avg_ctx = context + chunks * (batch - 1) / 2 + warmup + (steps + 1) / 2
     step_bytes = model.weight_bytes + batch * avg_ctx * kv_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
     return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
@@ -204,9 +207,18 @@ def main() -> int:
             points[f"decode_b{b}"] = m["tok_s"]
             point_rooflines[f"decode_b{b}"] = m["roofline"]
         if args.dtype == "bf16":
-            # the true 32-bit path of the same model (the same bfloat16 weights, widened exactly; 32-bit caches)
+            # the same layers with 8,192-token contexts (position tables of 16,384; batch 8)
             del model
             torch.cuda.empty_cache()
+            long_cfg = dict(cfg, max_position_embeddings=16384)
+            model_long = bw.Model.random(long_cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+            m = measure_decode(bw, torch, model_long, long_cfg, dtype, 8, side_steps, 4, context=8192)
+            points["decode_b8_ctx8192"] = m["tok_s"]
+            point_rooflines["decode_b8_ctx8192"] = m["roofline"]
+            del model_long
+            model = None
+            torch.cuda.empty_cache()
+            # the true 32-bit path of the same model (the same bfloat16 weights, widened exactly; 32-bit caches)
             model32 = bw.Model.random(cfg, seed=0, dtype="float32", sigma=0.02, on_device=True)
             m = measure_decode(bw, torch, model32, cfg, "float32", args.batch, side_steps, 4)
             extra["fp32"] = {"decode_tok_s": m["tok_s"], "batch": args.batch, "ms_per_step": m["ms_per_step"],
