@@ -821,24 +821,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #define T128_STAGES 4
 
 __device__ __forceinline__ void t128_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_a, __amdgpu_buffer_rsrc_t rs_b,
-                                           const int* voff_a, const int* voff_b, int wave, int step, int steps) {
+                                           const int* voff_a, const int* voff_b, int wave, int step, int steps,
+                                           int k_base) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   unsigned char* dst = lds + (step % T128_STAGES) * T128_STAGE + (2 * wave) * 1024;
   const bool real = step < steps;                                     // scalar; past K: outside the descriptors
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, real ? voff_a[t] : 0x7ffffff0, step * 128, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + t * 1024), 16, real ? voff_a[t] : 0x7ffffff0,
+                                             k_base * 2 + step * 128, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 16 * 1024 + t * 1024), 16, real ? voff_b[t] : 0x7ffffff0,
-                                             step * 128, 0, 0);
+                                             k_base * 2 + step * 128, 0, 0);
   }
 }
 
 template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile128_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   constexpr bool ROPE = EPI == EPI_QKV_ROPE;           // waves of 32 x 64 outputs: a head's 64 columns in one wave
+  // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
+  // elements (a residual add's segments, joined in order by add_segments_kernel afterwards)
+  const int k_base = (int)blockIdx.y * GEMM_SEG;
+  if (gridDim.y > 1) out = (void*)((float*)out + (size_t)blockIdx.y * seg_stride);
   constexpr int NI = ROPE ? 2 : 4, NJ = ROPE ? 4 : 2;
   constexpr int COLS = GLU ? 64 : 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char t128_lds[];   // [4 stages][x 16 KB | W 16 KB]
@@ -884,14 +890,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int a_frag = (NI * wy) * 2048;
   const int b_frag = 16 * 1024 + (GLU ? wx : NJ * wx) * 2048;
   constexpr int b_step = GLU ? 4 * 2048 : 2048;                        // from the wave's first W block to its second
-  const int steps = K / 64;
+  const int steps = gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64;
 #pragma unroll
-  for (int st = 0; st < T128_STAGES - 1; ++st) t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps);
+  for (int st = 0; st < T128_STAGES - 1; ++st) t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, st, steps, k_base);
   for (int step = 0; step < steps; ++step) {
     __builtin_amdgcn_s_waitcnt(vmcnt_only(4 * (T128_STAGES - 2)));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, step + T128_STAGES - 1, steps);   // into the stage worked on a step ago
+    t128_issue(t128_lds, rs_a, rs_b, voff_a, voff_b, wave, step + T128_STAGES - 1, steps, k_base);   // into the stage worked on a step ago
     const unsigned char* stage = t128_lds + (step % T128_STAGES) * T128_STAGE;
     __builtin_amdgcn_sched_barrier(0);
     // 12 operand reads and 16 matrix instructions a step, the second half's reads under the first half's products
@@ -921,7 +927,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     asm volatile("" ::: "memory");
     if constexpr (EPI == EPI_ADD_F32) {
       const int kn = (step + 1) * 64;
-      if (kn % GEMM_SEG == 0 && kn < K) {              // a segment ends before the last: add it into the output now
+      if (kn % GEMM_SEG == 0 && step + 1 < steps) {    // a segment ends before the last: add it into the output now
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -936,7 +942,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     } else {
       const int kn = (step + 1) * 64;
-      if (kn % GEMM_SEG == 0 && kn < K) {              // a segment ends before the last: joined left to right
+      if (kn % GEMM_SEG == 0 && step + 1 < steps) {    // a segment ends before the last: joined left to right
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -947,7 +953,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
   }
-  if (EPI != EPI_ADD_F32 && K > GEMM_SEG) {
+  if (EPI != EPI_ADD_F32 && steps > GEMM_SEG / 64) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -1775,15 +1781,6 @@ __global__ __launch_bounds__(256) void add_segments_kernel(float* __restrict__ o
   *reinterpret_cast<f32x4*>(o) = y;
 }
 
-// A residual add of a prompt portion over several segments of K with 256 x 256 tiles, a workgroup per tile and
-// segment: for products whose 128 x 128 tiles would be bound by what a compute unit can fetch (half as many
-// bytes a flop here), if the caller brings scratch for the segments' sums.
-static bool big_add_shape(int M, int N, int K, int ldo) {
-  const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
-  const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
-  return S > 1 && K % 64 == 0 && M >= 2 * BIG_BM && bm * bn * S >= 128 && N % 4 == 0 && ldo % 4 == 0;
-}
-
 static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
   tiles = 0;
@@ -1792,6 +1789,42 @@ static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
   narrow = ((N + 63) / 64) * S < 256;
   tiles = narrow ? (N + 31) / 32 : (N + 63) / 64;
   if (tiles * S < 32) tiles = 0;
+}
+
+// How a residual add of more than 64 rows is laid out.  One workgroup of the tile kernels fits a compute unit, so
+// a product goes in rounds of 256 workgroups, and a workgroup that has all of K to itself takes K / 64 steps
+// whatever else is idle: an output of 2048 columns and 128 rows is 16 tiles (76 us for K = 8192).
+//   whole       128 x 128 tiles with all of K, each finished segment added into the output: needs no scratch.
+//   row blocks  the kernel for up to 64 rows once per block of 64 rows, with its workgroup per 32 or 64 columns and
+//               segment of K (its scratch if K has several segments): up to 128 rows and three segments, where a
+//               launch more costs less than the join below (K = 2048: 16 and 19 us at 65 and 128 rows, for 24).
+//   tile split  a 128 x 128 workgroup per tile and segment, the segments' sums whole in scratch and joined in order
+//               afterwards (128 rows of K = 8192: 25 us).
+//   big split   the same with 256 x 256 tiles, which fetch half as many bytes a flop: for 512 rows or more.
+// All four give the same bits.  The choice is by a count of steps: rounds times the steps of a workgroup (a step of
+// a 256 x 256 tile counts twice); the join moves 8 bytes an element and segment (about 500,000 elements in the
+// time of a step) and is a launch more (8 steps); a split has to win by a tenth.  tiles64: what the 64-row
+// kernel's scratch is sized by.
+enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT };
+
+static AddRoute add_route(int M, int N, int K, int ldo, int& tiles64) {
+  const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
+  tiles64 = 0;
+  if (M <= 64 || K % 64) return ADD_WHOLE;
+  bool narrow;
+  add_rows_shape(64, N, K, tiles64, narrow);
+  if (tiles64 && M <= 128 && S <= 3) return ADD_ROW_BLOCKS;
+  tiles64 = 0;
+  if (S < 2 || N % 4 || ldo % 4) return ADD_WHOLE;
+  const long long t128 = (long long)((M + 127) / 128) * ((N + 127) / 128);
+  const long long tbig = (long long)((M + BIG_BM - 1) / BIG_BM) * ((N + 255) / 256);
+  const long long join = (long long)S * M * N / 500000 + 8;
+  const long long whole = ((t128 + 255) / 256) * (K / 64);
+  const long long tile_split = ((t128 * S + 255) / 256) * (GEMM_SEG / 64) + join;
+  const long long big_split = M >= 2 * BIG_BM ? ((tbig * S + 255) / 256) * 2 * (GEMM_SEG / 64) + join : whole;
+  const long long split = tile_split <= big_split ? tile_split : big_split;
+  if (10 * split >= 9 * whole) return ADD_WHOLE;
+  return tile_split <= big_split ? ADD_TILE_SPLIT : ADD_BIG_SPLIT;
 }
 
 template <int EPI>
@@ -1871,6 +1904,52 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     }
 #undef BW_SKINNY
   } else {
+    if constexpr (EPI == EPI_ADD_F32) {
+      int tiles;
+      const AddRoute route = add_route(M, N, K, ldo, tiles);
+      if (route == ADD_ROW_BLOCKS && (size_t)M * ldx * 2 < ((size_t)1 << 31) &&
+          (S == 1 || (sp.scratch != nullptr && sp.counters != nullptr && scratch_floats >= (size_t)tiles * S * 4096 &&
+                      num_counters >= tiles))) {
+        for (int m0 = 0; m0 < M; m0 += 64) {
+          const int rc = launch_gemm_bf16<EPI>(x + (size_t)m0 * ldx, w, (float*)out + (size_t)m0 * ldo, M - m0 < 64 ? M - m0 : 64, N, K,
+                                               ldx, ldo, s, rp, sp, scratch_floats, num_counters);
+          if (rc) return rc;
+        }
+        return 0;
+      }
+      if (route == ADD_BIG_SPLIT && sp.scratch != nullptr && ((uintptr_t)out & 15) == 0) {
+        if (scratch_floats < (size_t)S * M * N) return -6;
+        const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
+        static bool allowed = false;                 // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<EPI_F32>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    BIG_SLOTS * BIG_SLOT);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI_F32>), dim3(bm * bn, S), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w,
+                           (void*)sp.scratch, M, N, K, ldx, N, bm, bn, rp, (size_t)M * N);
+        const size_t quads = (size_t)M * (N >> 2);
+        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+                           M, N, ldo);
+        return BW_LAUNCH_CHECK();
+      }
+      if (route == ADD_TILE_SPLIT && sp.scratch != nullptr && ((uintptr_t)out & 15) == 0) {
+        if (scratch_floats < (size_t)S * M * N) return -6;
+        const int mt = (M + 127) / 128, nt = (N + 127) / 128;
+        static bool allowed = false;
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_tile128_kernel<EPI_F32>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    T128_STAGES * T128_STAGE);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI_F32>), dim3(mt * nt, S), dim3(512), T128_STAGES * T128_STAGE, s, x, w,
+                           (void*)sp.scratch, M, N, K, ldx, N, mt, nt, rp, (size_t)M * N);
+        const size_t quads = (size_t)M * (N >> 2);
+        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+                           M, N, ldo);
+        return BW_LAUNCH_CHECK();
+      }
+    }
     if constexpr (EPI != EPI_ADD_F32) {
       // enough 256-row tiles to go round the compute units (a second round at least half full)
       constexpr int BIG_COLS = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
@@ -1887,24 +1966,6 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         return BW_LAUNCH_CHECK();
       }
     }
-    if constexpr (EPI == EPI_ADD_F32) {
-      if (sp.scratch != nullptr && big_add_shape(M, N, K, ldo) && ((uintptr_t)out & 15) == 0) {
-        if (scratch_floats < (size_t)S * M * N) return -6;
-        const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
-        static bool allowed = false;                 // more than 64 KB of dynamic LDS has to be asked for once
-        if (!allowed) {
-          (void)hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<EPI_F32>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    BIG_SLOTS * BIG_SLOT);
-          allowed = true;
-        }
-        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI_F32>), dim3(bm * bn, S), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w,
-                           (void*)sp.scratch, M, N, K, ldx, N, bm, bn, rp, (size_t)M * N);
-        const size_t quads = (size_t)M * (N >> 2);
-        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
-                           M, N, ldo);
-        return BW_LAUNCH_CHECK();
-      }
-    }
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
@@ -1918,7 +1979,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
           allowed = true;
         }
         hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI>), grid, dim3(512), T128_STAGES * T128_STAGE, s, x, w, out, M, N, K, ldx,
-                           ldo, m_tiles, n_tiles, rp);
+                           ldo, m_tiles, n_tiles, rp, (size_t)0);
         return BW_LAUNCH_CHECK();
       }
     }
@@ -1938,12 +1999,14 @@ extern "C" int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_float
   int tiles = 0;
   bool narrow = false;
   const int S = K > 0 ? (K + GEMM_SEG - 1) / GEMM_SEG : 0;
-  if (M > 64 && N > 0 && big_add_shape(M, N, K, 4)) {      // a prompt portion: the segments' sums, whole
+  const AddRoute route = M > 64 && N > 0 ? add_route(M, N, K, 4, tiles) : ADD_WHOLE;
+  if (route == ADD_TILE_SPLIT || route == ADD_BIG_SPLIT) {      // a prompt portion: the segments' sums, whole
     *scratch_floats = (long long)S * M * N;
     *counters = 1;                                          // (none is used)
     return 0;
   }
   if (M > 0 && M <= 64 && N > 0 && S > 1) add_rows_shape(M, N, K, tiles, narrow);
+  else if (S == 1) tiles = 0;                               // (blocks of 64 rows of one segment share nothing)
   *scratch_floats = (long long)tiles * S * 4096;
   *counters = tiles;
   return 0;

@@ -100,7 +100,16 @@ def _check(code: int, what: str) -> None:
         raise RuntimeError(f"{what}: {why}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    """The current stream's handle (the stream a graph capture has made current, too).  torch's own
+    ``current_stream()`` builds a Python object for it at some 8 us a call, which an eager step of a short
+    prompt pays 170 times; the raw handle costs a fraction of a microsecond."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 

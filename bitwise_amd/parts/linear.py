@@ -48,16 +48,15 @@ class Linear:
     def add_into(self, ws, x: torch.Tensor, residual: torch.Tensor, rows: int) -> None:
         """residual[:rows] += x[:rows] @ W.T, the sum in 32-bit (src/model.cpp:300, :305)."""
         if self.mfma:
-            # a long inner size and 17 to 64 rows: every 2048-segment of it gets workgroups of its own,
-            # which meet in device scratch
-            # (and a prompt portion of 512 rows or more: 256 x 256 tiles, a workgroup per tile and segment; its scratch
-            # is sized for the longest step, so that one buffer serves every portion)
+            # 17 rows or more and a long inner size: every 2048-segment of it gets workgroups of its own, which meet
+            # in device scratch.  For up to 64 rows (or a few blocks of 64) that is a fixed size; for a prompt portion
+            # it holds the segments' sums whole and is sized for the longest step, so that one buffer serves every
+            # portion.
             scratch = None
-            floats, counters = 0, 0
-            if 16 < rows <= 64:
-                floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features)
-            elif rows >= 512 and ops.gemm_add_scratch(rows, self.out_features, self.in_features)[0]:
-                floats, counters = ops.gemm_add_scratch(ws.max_rows, self.out_features, self.in_features)
+            floats, counters = ops.gemm_add_scratch(rows, self.out_features, self.in_features) if rows > 16 else (0, 0)
+            if floats and rows > 64:
+                longest = ops.gemm_add_scratch(ws.max_rows, self.out_features, self.in_features)
+                floats, counters = max(floats, longest[0]), max(counters, longest[1])
             if floats:
                 scratch = (ws.buffer("gemm_add_split", floats, torch.float32, rows=1),
                            ws.buffer("gemm_add_split_count", counters, torch.int32, rows=1))

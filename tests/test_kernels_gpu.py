@@ -189,24 +189,46 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             got = res.clone()
             ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
             assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
-    # a residual add of a prompt portion over several segments with scratch: 256 x 256 tiles, a workgroup per tile
-    # and segment, the segments joined in order afterwards: the bits of the add without scratch; ragged edges, a
-    # short last segment, scratch full of NaN and larger than needed
-    for M, N, K in [(700, 3000, 3 * 2048 + 128), (2048, 2048, 8192), (513, 8192, 4096)]:
+    # a residual add of more than 64 rows whose 128 x 128 tiles with all of K would leave compute units idle: up to
+    # 128 rows and three segments in blocks of 64 rows through that kernel (its scratch if K has several segments);
+    # else a workgroup per tile (128 x 128, or 256 x 256 from 512 rows) and segment, the segments' sums whole in
+    # scratch and joined in order afterwards.  The bits of the rows alone, 16 at a time, with and without scratch,
+    # twice on the same scratch (full of NaN at first, larger than needed); ragged edges, a short last segment
+    S = lambda K: (K + 2047) // 2048
+    for M, N, K, kind in [(65, 2048, 4096, "blocks"), (128, 1100, 2048 * 2 + 320, "blocks"), (100, 2048, 2048, "blocks"),
+                          (129, 2048, 2048, None), (81, 2048, 4096 + 72, None), (640, 4096, 4096, None),
+                          (65, 2048, 8192, "sums"), (145, 2048, 8192, "sums"), (300, 1000, 2 * 2048 + 192, "sums"),
+                          (768, 2048, 8192, "sums"), (700, 3000, 4 * 2048 + 128, "sums"), (2048, 2048, 8192, "sums"),
+                          (513, 8192, 4096, "sums")]:
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
         res = torch.randn(M, N, generator=g).to(gpu)
         want = res.clone()
-        ops.gemm_bf16(x, w, want, M, ops.EPI_ADD_F32)
-        floats, counters = ops.gemm_add_scratch(M, N, K)
-        assert floats == ((K + 2047) // 2048) * M * N and counters > 0
-        scratch = (torch.full((floats + 1000,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
+        for lo in range(0, M, 16):
+            n = min(16, M - lo)
+            part = res[lo:lo + n].clone()
+            ops.gemm_bf16(x[lo:lo + n].contiguous(), w, part, n, ops.EPI_ADD_F32)
+            want[lo:lo + n] = part
         got = res.clone()
-        ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
+        ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32)
         assert torch.equal(got, want), (M, N, K)
-        with pytest.raises(RuntimeError, match="scratch smaller"):
-            ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=(scratch[0][:floats - 8], scratch[1]))
-    assert ops.gemm_add_scratch(2048, 2048, 2048) == (0, 0) and ops.gemm_add_scratch(300, 2048, 8192) == (0, 0)
+        floats, counters = ops.gemm_add_scratch(M, N, K)
+        if kind == "sums":
+            assert (floats, counters) == (S(K) * M * N, 1), (M, N, K)
+        elif kind == "blocks" and K > 2048:
+            assert floats > 0 and (floats, counters) == ops.gemm_add_scratch(64, N, K), (M, N, K)
+        else:
+            assert (floats, counters) == (0, 0), (M, N, K)
+        if floats:
+            scratch = (torch.full((floats + 1000,), float("nan"), device=gpu), torch.zeros(counters, dtype=torch.int32, device=gpu))
+            for _ in range(2):
+                got = res.clone()
+                ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=scratch)
+                assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
+            if kind == "sums":
+                with pytest.raises(RuntimeError, match="scratch smaller"):
+                    ops.gemm_bf16(x, w, got, M, ops.EPI_ADD_F32, scratch=(scratch[0][:floats - 8], scratch[1]))
+    assert ops.gemm_add_scratch(2048, 2048, 2048) == (0, 0)
     # SwiGLU with many columns (x shared through LDS; one, two or four blocks of 16 rows): the plain result, and
     # the bits of the same rows inside a prompt portion's product (another kernel)
     for inter, K in ((2100, 128), (2100, 2048 + 128)):             # the second: two segments of K
