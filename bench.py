@@ -3,6 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
+                    [--prefill-tokens T] [--no-points]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -85,14 +86,15 @@ LLAMA3_8B = {
 }
 
 
-def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float) -> dict:
-    """One 2,048-token prompt in one step (model, head for the last row, sampling); the best of six after two
-    untimed ones (the shader clock takes some milliseconds of load to rise from its idle 2.1 GHz to 2.4)."""
+def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float, tokens: int = PREFILL_TOKENS) -> dict:
+    """One prompt of ``tokens`` tokens (2,048 unless said otherwise) in one step (model, head for the last row,
+    sampling); the best of six after two untimed ones (the shader clock takes some milliseconds of load to rise
+    from its idle 2.1 GHz to 2.4)."""
     engine = make_engine(bw, model, 1, 8, dtype)
     g = torch.Generator().manual_seed(99)
     times = []
     for _ in range(8):
-        prompt = torch.randint(0, cfg["vocab_size"], (PREFILL_TOKENS,), generator=g).tolist()
+        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
         engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -101,8 +103,8 @@ def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float) 
         times.append((time.perf_counter() - t0) * 1e3)
         assert engine.idle()
     ms = min(times[2:])
-    flops = prefill_flops(cfg, PREFILL_TOKENS)
-    return {"value": round(PREFILL_TOKENS / ms * 1e3, 1), "tokens": PREFILL_TOKENS, "ms": round(ms, 3),
+    flops = prefill_flops(cfg, tokens)
+    return {"value": round(tokens / ms * 1e3, 1), "tokens": tokens, "ms": round(ms, 3),
             "frac": round(flops / (ms * 1e-3) / peak_flops, 4)}
 
 
@@ -177,6 +179,8 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (named in config)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="the length of the headline prefill's prompt (for profiles of shorter prompts; up to 2048)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -197,7 +201,10 @@ def main() -> int:
     vocab = cfg["vocab_size"]
     side_steps = max(16, args.steps // 2)
 
-    prefill = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype])
+    if not 1 <= args.prefill_tokens <= PREFILL_TOKENS:
+        print(f"bench.py: --prefill-tokens {args.prefill_tokens} is outside 1..{PREFILL_TOKENS}")
+        return 2
+    prefill = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype], args.prefill_tokens)
     head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup)
     points, point_rooflines = {}, {}
     extra = {}
@@ -206,6 +213,8 @@ def main() -> int:
             m = measure_decode(bw, torch, model, cfg, dtype, b, side_steps, 4)
             points[f"decode_b{b}"] = m["tok_s"]
             point_rooflines[f"decode_b{b}"] = m["roofline"]
+        for t in (128, 512):                          # shorter prompts, one step each: tokens a second
+            points[f"prefill_t{t}"] = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype], t)["value"]
         if args.dtype == "bf16":
             # the same layers with 8,192-token contexts (position tables of 16,384; batch 8)
             del model
