@@ -257,13 +257,13 @@ __device__ __forceinline__ void norm_rows_finish(const NormRows<R, NV>& nr, cons
 }
 
 // One row at once: the whole of rmsnorm_bf16_kernel for rows that fit a wave's registers.
-template <typename Store>
+template <int NV = 8, typename Store>
 __device__ __forceinline__ void rmsnorm_row_small(const f32x4* __restrict__ xv, const void* __restrict__ w,
                                                   int w_is_bf16, int nvec, int dim, float eps, int lane, Store store) {
-  NormRows<1> nr;
+  NormRows<1, NV> nr;
   const f32x4* rows[1] = {xv};
-  norm_rows_load<1>(nr, rows, w, w_is_bf16, nvec, lane);
-  norm_rows_finish<1>(nr, rows, w_is_bf16, nvec, dim, eps, lane, [&](int, int c, u32x2 pk) { store(c, pk); });
+  norm_rows_load<1, NV>(nr, rows, w, w_is_bf16, nvec, lane);
+  norm_rows_finish<1, NV>(nr, rows, w_is_bf16, nvec, dim, eps, lane, [&](int, int c, u32x2 pk) { store(c, pk); });
 }
 
 // The operand of s_waitcnt that waits for all but the last n memory loads of the wave and for nothing else.

@@ -125,6 +125,11 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16_kernel(const float* __restri
                         [&](int c, u32x2 pk) { *reinterpret_cast<u32x2*>(yr + 4 * c) = pk; });
       return;
     }
+    if (dim <= 4096) {      // sixteen vectors a lane: still one round of loads (two cost a second trip to memory)
+      rmsnorm_row_small<16>(xv, w, sizeof(WT) == 2, nvec, dim, eps, lane,
+                            [&](int c, u32x2 pk) { *reinterpret_cast<u32x2*>(yr + 4 * c) = pk; });
+      return;
+    }
     acc = row_sumsq_vec(xv, nvec, lane);
     const float inv = 1.0f / sqrtf(acc / (float)dim + eps);
     // eight vectors of the row and of the weight asked for before the first is used (a loop of one load and its

@@ -353,6 +353,23 @@ def test_rmsnorm(gpu):
                 inv = np.float32(1.0) / np.sqrt(np.float32(ss / np.float32(dim) + np.float32(eps)), dtype=np.float32)
                 want = (xr * inv) * w.numpy()
                 assert np.array_equal(o32[r].cpu().numpy().view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # bfloat16 out (rows as 16-byte vectors, a row a wave): lane l owns vectors l, l + 64, ... and runs one chain over
+    # their elements in ascending order; the lanes are joined by xor butterflies 32, 16, ..., 1.  The three routes
+    # (a row in eight vectors a lane, in sixteen, in two passes) against that order spelled out, bit for bit
+    for dim in (2048, 2052, 4096, 4100):
+        x, w = torch.randn(2, dim, generator=g) * 3, torch.randn(dim, generator=g)
+        ob = torch.zeros(2, dim, device=gpu, dtype=torch.bfloat16)
+        ops.rmsnorm(x.to(gpu), w.to(gpu), ob, 2, 1e-5)
+        xr, nvec = x[1].numpy(), dim // 4
+        lanes = [np.float32(0.0)] * 64
+        for c in range(nvec):
+            for e in range(4):
+                lanes[c % 64] = fma32(xr[4 * c + e], xr[4 * c + e], lanes[c % 64])
+        for off in (32, 16, 8, 4, 2, 1):
+            lanes = [np.float32(lanes[l] + lanes[l ^ off]) for l in range(64)]
+        inv = np.float32(1.0) / np.sqrt(np.float32(lanes[0] / np.float32(dim) + np.float32(1e-5)), dtype=np.float32)
+        want = torch.from_numpy(((xr * inv) * w.numpy()).astype(np.float32)).bfloat16()
+        assert torch.equal(ob[1].cpu(), want), dim
     z = torch.zeros(2, 64, device=gpu)
     out = torch.ones(2, 64, device=gpu)
     ops.rmsnorm(z, torch.ones(64, device=gpu), out, 2, 1e-5)
