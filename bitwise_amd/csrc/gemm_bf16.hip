@@ -1017,7 +1017,7 @@ struct MidShape {
   static constexpr int NW = EIGHT ? 8 : 4;                          // waves
   static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
   static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a step (SwiGLU: 32 gate, 32 up)
-  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? (NORM ? 1 : 2) : (NORM ? 2 : 4)) : 1;   // steps of 64 along K a stage (NORM: weights only)
+  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? (NORM || NRB == 4 ? 1 : 2) : (NORM ? 2 : 4)) : 1;   // steps of 64 along K a stage (NORM: weights only)
   static constexpr int STRIPS = COLS / 16, GROUPS = NW / STRIPS;    // wave = (strip of the columns, group of the row blocks)
   static constexpr int A_LOADS = NORM ? 0 : (SUB * 2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
   static constexpr int B_LOADS = SUB * B_ROWS / 8 / NW;             // 8 rows of W each
@@ -1026,7 +1026,11 @@ struct MidShape {
   static constexpr int NI = NRB >= GROUPS ? NRB / GROUPS : 1;       // blocks of rows a wave works on (fewer blocks than groups: waves that only load)
   static constexpr int NJ = GLU ? 2 : 1;
   static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
-  static constexpr int FIT = 150 * 1024 / STAGE;
+  // 17 rows or more: a ring of at most 72 KB, so that two workgroups share a compute unit and one's first loads
+  // and epilogue lie under the other's steps (products with more workgroups than compute units: gate|up 17.2 ->
+  // 16.0 us, the 8B shape's 53 -> 50 and its down projection 37 -> 35; the others unchanged); never fewer than 3
+  static constexpr int FIT0 = (NORM || NRB < 2 ? 150 : 72) * 1024 / STAGE;
+  static constexpr int FIT = FIT0 < 3 ? 3 : FIT0;
   static constexpr int STAGES = EIGHT ? (NORM ? 8 : (FIT > 6 ? 6 : FIT))
                                       : (ROPE_NARROW && NRB <= 2 ? 16 : 8);   // (half the weights a stage: twice the stages, where they fit)
   static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
