@@ -250,7 +250,7 @@ def main() -> int:
 
     value = head["tok_s"]
     line = {
-        "metric": "decode tok/s at batch 8, SmolLM2-1.7B shape, 2048-token contexts",
+        "metric": f"decode tok/s at batch {args.batch}, SmolLM2-1.7B shape, 2048-token contexts",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / BASELINE_TOK_S, 1), "dtype": args.dtype, "data": "synthetic",
