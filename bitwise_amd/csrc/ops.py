@@ -6,6 +6,7 @@ stream.  There is no fallback: without the compiled library every call raises.
 from __future__ import annotations
 
 import ctypes
+import functools
 from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
 from typing import Optional, Tuple
 
@@ -256,9 +257,11 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, acc
                               x.stride(0), out.stride(0), int(accumulate), _stream()), "gemm_f32")
 
 
+@functools.lru_cache(maxsize=None)
 def gemm_add_scratch(rows: int, N: int, K: int) -> Tuple[int, int]:
     """(float32 elements, int32 counters) that a residual add of this shape wants as ``scratch``
-    to give every 2048-segment of K workgroups of its own; (0, 0): it would not."""
+    to give every 2048-segment of K workgroups of its own; (0, 0): it would not.  (A function of the
+    three sizes alone: asked once for each.)"""
     floats, counters = ctypes.c_longlong(0), ctypes.c_int(0)
     _check(_fn("bw_gemm_add_scratch")(rows, N, K, ctypes.addressof(floats), ctypes.addressof(counters)), "gemm_add_scratch")
     return int(floats.value), int(counters.value)
