@@ -125,9 +125,18 @@ class ModelRunner:
                  max_logit_rows: Optional[int] = None, use_graphs: bool = True):
         self.model, self.storage = model, storage
         self.rt = model.rt
-        self.ws = Workspace(model.rt.device, max_rows, storage.page_size, max_logit_rows)
-        self.max_model_len = min(int(max_model_len), model.spec.max_positions)
         self.use_graphs = bool(use_graphs) and model.graph_safe
+        # the limits a step is checked against are the caller's; the workspace holds the rows of the graph bucket
+        # above them, so that a step of that many decoded tokens still replays a graph (48 requests: the bucket of 64)
+        self.max_rows = int(max_rows)
+        self.max_logit_rows = int(max_logit_rows if max_logit_rows is not None else max_rows)
+        ws_rows, ws_logit_rows = self.max_rows, self.max_logit_rows
+        if self.use_graphs:
+            bucket = next((b for b in GRAPH_BUCKETS if b >= min(self.max_rows, self.max_logit_rows)), None)
+            if bucket is not None:
+                ws_rows, ws_logit_rows = max(ws_rows, bucket), max(ws_logit_rows, bucket)
+        self.ws = Workspace(model.rt.device, ws_rows, storage.page_size, ws_logit_rows)
+        self.max_model_len = min(int(max_model_len), model.spec.max_positions)
         self._graphs: Dict[int, tuple] = {}
         self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
         self.last_graph_rows = 0      # requests of the last step if it was replayed from a graph, else 0
@@ -146,10 +155,10 @@ class ModelRunner:
             return None
         rows = sum(len(s.tokens) for s in segments)
         wanted = sum(len(s.want) for s in segments)
-        if rows > self.ws.max_rows:
-            raise ValueError(f"a step of {rows} tokens exceeds the engine's {self.ws.max_rows}")
-        if wanted > self.ws.max_logit_rows:
-            raise ValueError(f"logits wanted at {wanted} places, the engine allows {self.ws.max_logit_rows}")
+        if rows > self.max_rows:
+            raise ValueError(f"a step of {rows} tokens exceeds the engine's {self.max_rows}")
+        if wanted > self.max_logit_rows:
+            raise ValueError(f"logits wanted at {wanted} places, the engine allows {self.max_logit_rows}")
         for s in segments:
             if not len(s.tokens):
                 raise ValueError("a request without tokens in a step")

@@ -82,7 +82,7 @@ class Replayer:
         from .sampling.rng import FINGERPRINT_BASIS
         from .sampling.sampler import Sampler
         if self._sampler is None:
-            self._sampler = Sampler(logits.device, self.runner.ws.max_logit_rows)
+            self._sampler = Sampler(logits.device, self.runner.max_logit_rows)
         waves: List[List[int]] = []
         seen: Dict[str, int] = {}
         for row, rid in enumerate(owners):
@@ -98,7 +98,7 @@ class Replayer:
                 self.fingerprints[owners[r]] = h
 
     def _run(self, segments: List[Segment], owners: Sequence[str] = ()) -> Optional[np.ndarray]:
-        limit = self.runner.ws.max_rows
+        limit = self.runner.max_rows
         if sum(len(s.tokens) for s in segments) <= limit:
             lg = self.runner.step(segments)
             if lg is not None and self.fingerprint_logits:
