@@ -106,6 +106,44 @@ def test_long_decoding_with_and_without_graphs(folders):
     assert outs[0].tokens == want
 
 
+def test_many_requests_decode_from_the_large_graph_buckets(gpu):
+    """100 and then 200 requests decoding at once (the graph buckets of 128 and 256 rows, where the residual adds
+    take their layouts for 65 rows and more inside a captured graph) at SmolLM2's layer widths, one layer: every
+    request's tokens and fingerprint are those of the same request run alone, with graphs and without."""
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "num_hidden_layers": 1,
+           "rms_norm_eps": 1e-5, "max_position_embeddings": 256, "bos_token_id": 1, "eos_token_id": 2,
+           "vocab_size": 1000, "hidden_size": 2048, "num_attention_heads": 32, "num_key_value_heads": 32, "head_dim": 64,
+           "intermediate_size": 8192, "rope_theta": 130000.0, "tie_word_embeddings": True}
+    model = bw.Model.random(cfg, seed=5, dtype="bfloat16", sigma=0.05, on_device=True)
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, 1000, (int(n),), generator=g).tolist() for n in torch.randint(3, 20, (200,), generator=g)]
+    sp = [bw.SamplingParams(max_new_tokens=6, ignore_eos=True, temperature=0.8 if i % 3 else 0.0, seed=i) for i in range(200)]
+
+    replayed = []
+
+    def run(which, graphs, seqs):
+        ecfg = bw.EngineConfig(num_blocks=seqs * 4 + 8, max_batched_tokens=2048, max_num_seqs=seqs, prefix_caching=False,
+                               block_size=16, dtype="bfloat16", max_model_len=256, use_graphs=graphs)
+        eng = bw.Engine(model, None, ecfg)
+        ids = [eng.add_request(prompts[i], sp[i]) for i in which]
+        most = 0
+        while not eng.idle():
+            eng.step()
+            most = max(most, eng.exec.runner.last_graph_rows)
+        replayed.append((seqs, graphs, most))
+        return [eng.result(i) for i in ids]
+
+    solo = {i: run([i], False, 1)[0] for i in (0, 1, 57, 99, 100, 199)}
+    for count in (100, 200):
+        for graphs in (True, False):
+            outs = run(range(count), graphs, count)
+            assert all(len(o.tokens) == 6 for o in outs)
+            for i, want in solo.items():
+                if i < count:
+                    assert outs[i].tokens == want.tokens and outs[i].logits_fingerprint == want.logits_fingerprint, (count, graphs, i)
+    assert (100, True, 100) in replayed and (200, True, 200) in replayed and (200, False, 0) in replayed, replayed
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_randomized_traces(gpu, dtype):
     """The reference's simulator (sim/simulate.cpp) on the real engine: 0 token or logit
