@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -181,6 +181,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (named in config)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="the length of the headline prefill's prompt (for profiles of shorter prompts; up to 2048)")
+    ap.add_argument("--shape", choices=["smollm2", "llama3_8b"], default="smollm2",
+                    help="the layer sizes of the headline run (llama3_8b: for profiles of that shape; implies --no-points)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -192,7 +194,10 @@ def main() -> int:
     import bitwise_amd as bw
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
-    cfg = dict(SMOLLM2_1_7B)
+    cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B)
+    shape_name = "SmolLM2-1.7B" if args.shape == "smollm2" else "Llama-3-8B"
+    if args.shape != "smollm2":
+        args.no_points = True
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -250,15 +255,16 @@ def main() -> int:
 
     value = head["tok_s"]
     line = {
-        "metric": f"decode tok/s at batch {args.batch}, SmolLM2-1.7B shape, 2048-token contexts",
+        "metric": f"decode tok/s at batch {args.batch}, {shape_name} shape, 2048-token contexts",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": round(value / BASELINE_TOK_S, 1), "dtype": args.dtype, "data": "synthetic",
+        "vs_baseline": round(value / BASELINE_TOK_S, 1) if args.shape == "smollm2" else None, "dtype": args.dtype,
+        "data": "synthetic",
         "config": {
-            "model": "SmolLM2-1.7B shape, random weights", "layers": cfg["num_hidden_layers"],
+            "model": f"{shape_name} shape, random weights", "layers": cfg["num_hidden_layers"],
             "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"], "ffn": cfg["intermediate_size"],
-            "vocab": vocab, "tied": True, "global_batch": args.batch, "seq_len": CONTEXT, "max_context": 4096,
+            "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]), "global_batch": args.batch, "seq_len": CONTEXT, "max_context": 4096,
             "page_size": 16, "parallelism": "single GPU", "weights": "bf16" if args.dtype == "bf16" else "bf16 widened",
             "baseline": "reference CPU decode, one stream, 7.26 tok/s",
         },
