@@ -32,8 +32,11 @@
 //     into the output as they end), and for products with at least 128 tiles of 256 x 256 the "big" kernel,
 //     which computes twice as much per byte it fetches (a ring of five 32 KB slots, operand reads pipelined
 //     under the matrix instructions; one segment, or for a residual add with scratch a workgroup per tile and
-//     segment, the segments' sums joined in order by a second kernel); the "wide" kernel (128 x 128 tiles staged
-//     through registers by four waves) takes what those do not: K no multiple of 64.
+//     segment, the segments' sums joined in order by a second kernel); 128 x 256 tiles ("tile256": eight waves of
+//     64 x 64, room in the registers for the sums of the segments before) where they make fewer rounds of the compute
+//     units than the 128 x 128 ones by enough, which is where K has several segments and the big kernel does not
+//     run; the "wide" kernel (128 x 128 tiles staged through registers by four waves) takes what those do not: K no
+//     multiple of 64.
 //
 // Epilogues: store 32-bit, store bfloat16, add into a 32-bit residual (each output owned
 // by one lane: no atomics), SwiGLU of two products (gate rows n, up rows N+n of a
@@ -980,6 +983,135 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
   }
+}
+
+// ------------------------------------------------------------------------------ 128 x 256 tiles through an LDS ring
+
+// 128 rows x 256 columns a workgroup (128 of SwiGLU: 128 gate and 128 up rows of W), eight waves of 64 x 64 outputs:
+// a step pulls 48 KB for twice the 128 x 128 tile's products (which pulls 32), and a wave's 64 accumulators leave room
+// for the sums of the segments before, so that a K of several segments, which the 256 x 256 kernel does not take,
+// runs on these where there are enough of them.  Three stages of 48 KB (x 16 KB | W 32 KB); a wave issues six loads a
+// stage.  Plain and SwiGLU epilogues; segments joined left to right in registers.  K a multiple of 64.
+#define T256_STAGE (48 * 1024)
+#define T256_STAGES 3
+
+template <int EPI>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile256_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
+    int ldo, int m_tiles, int n_tiles) {
+  static_assert(EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16, "plain and SwiGLU epilogues");
+  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr int COLS = GLU ? 128 : 256;
+  extern __shared__ __attribute__((aligned(16))) unsigned char t256_lds[];   // [3 stages][x 16 KB | W 32 KB]
+  const int wave = wave_index(), lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int wy = wave >> 2, wx = wave & 3;
+  int bid = blockIdx.x;
+  const int nblocks = m_tiles * n_tiles;
+  if (nblocks % 8 == 0) bid = (bid % 8) * (nblocks / 8) + bid / 8;      // an n tile's workgroups share an XCD
+  const int m0 = (bid % m_tiles) * 128;
+  const int n0 = (bid / m_tiles) * COLS;
+  // this wave's loads of a stage: rows 16*wave .. 16*wave + 15 of x's 128 and rows 32*wave .. 32*wave + 31 of W's 256
+  // (SwiGLU: W rows 0-127 of the tile are gate rows n0.., 128-255 the up rows N + n0..)
+  const int a_rows = min(128, M - m0), b_rows = min(COLS, N - n0);
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+  const bool up = GLU && wave >= 4;
+  const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+  const int b_row0 = GLU ? 32 * (wave & 3) : 32 * wave;
+  const int lrow = lane >> 3, lslot = lane & 7;
+  int voff_a[2], voff_b[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int r16 = (8 * t + lrow) & 15;                    // the row within its block of 16
+    const int chunk = lslot ^ (r16 >> 1);
+    if (t < 2) voff_a[t] = ((16 * wave + 8 * t + lrow) * ldx + 8 * chunk) * 2;
+    voff_b[t] = ((b_row0 + 8 * t + lrow) * K + 8 * chunk) * 2;
+  }
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const int steps = K / 64;
+  auto issue = [&](int step) {
+    unsigned char* dst = t256_lds + (step % T256_STAGES) * T256_STAGE;
+    const bool real = step < steps;                                     // scalar; past K: outside the descriptors
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + (2 * wave + t) * 1024), 16, real ? voff_a[t] : 0x7ffffff0,
+                                               step * 128, 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 16 * 1024 + (4 * wave + t) * 1024), 16,
+                                               real ? voff_b[t] : 0x7ffffff0, step * 128, 0, 0);
+  };
+  f32x4 acc[4][4], tot[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+  // operands: x row blocks 4*wy + i; W row blocks 4*wx + j, or in SwiGLU mode gate blocks 2*wx, 2*wx + 1 (j = 0, 1)
+  // and up blocks 8 + 2*wx, 8 + 2*wx + 1 (j = 2, 3)
+  const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
+  int slot_off[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
+  const int a_frag = (4 * wy) * 2048;
+  const int b_frag = 16 * 1024 + (GLU ? 2 * wx : 4 * wx) * 2048;
+  auto b_off = [&](int j) { return GLU ? ((j & 1) + 8 * (j >> 1)) * 2048 : j * 2048; };
+#pragma unroll
+  for (int st = 0; st < T256_STAGES - 1; ++st) issue(st);
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(6 * (T256_STAGES - 2)));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    issue(step + T256_STAGES - 1);                                      // into the stage worked on a step ago
+    const unsigned char* stage = t256_lds + (step % T256_STAGES) * T256_STAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    // 16 operand reads and 32 matrix instructions a step, the second half's reads under the first half's products
+    u32x4 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fb[kk][j] = *reinterpret_cast<const u32x4*>(stage + b_frag + b_off(j) + slot_off[kk]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) fa[kk][i] = *reinterpret_cast<const u32x4*>(stage + a_frag + i * 2048 + slot_off[kk]);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk][i]), as_bf16x8(fb[kk][j]), acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    const int kn = (step + 1) * 64;
+    if (kn % GEMM_SEG == 0 && kn < K) {                // a segment ends before the last: joined left to right
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
+          acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+    }
+  }
+  if (K > GEMM_SEG) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] + acc[i][j];
+  }
+  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, QkvRopeArgs{});
 }
 
 // ------------------------------------------------------------------------------ up to 64 rows, through LDS
@@ -1967,6 +2099,25 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         }
         hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI>), dim3(bm * bn), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w, out, M, N, K, ldx,
                            ldo, bm, bn, rp, (size_t)0);
+        return BW_LAUNCH_CHECK();
+      }
+    }
+    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16) {
+      // 128 x 256 tiles where they go round the compute units (the 256 x 256 kernel above took what it takes: one
+      // segment of K and enough of its tiles)
+      constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+      const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
+      // (in rounds of 256 workgroups; a step of these takes 1.0 us where a 128 x 128 tile's takes 0.58)
+      const int rounds256 = (mt * nt + 255) / 256, rounds128 = (mt * ((N + COLS256 / 2 - 1) / (COLS256 / 2)) + 255) / 256;
+      if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) {
+        static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
+        if (!allowed) {
+          (void)hipFuncSetAttribute((const void*)gemm_bf16_tile256_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    T256_STAGES * T256_STAGE);
+          allowed = true;
+        }
+        hipLaunchKernelGGL((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K,
+                           ldx, ldo, mt, nt);
         return BW_LAUNCH_CHECK();
       }
     }

@@ -243,6 +243,26 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             hb = torch.zeros(M, inter, device=gpu, dtype=torch.bfloat16)
             ops.gemm_bf16(xl[100:100 + M].contiguous(), wgu, hb, M, ops.EPI_SWIGLU_BF16)
             assert torch.equal(hb, big[100:100 + M]), (M, K)
+    # enough 128 x 128 tiles for two rounds of the compute units and few enough 128 x 256 tiles for one: those run
+    # (plain and SwiGLU epilogues, two segments of K joined in registers, ragged last tiles of rows and columns);
+    # the plain result, and the bits of the rows 16 at a time (other kernels)
+    M, N, K = 300, 11000, 2048 + 192
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
+    xl = torch.randn(M, K, generator=g).bfloat16().to(gpu)
+    for dt, e, cols in ((torch.float32, ops.EPI_F32, N), (torch.bfloat16, ops.EPI_BF16, N), (torch.bfloat16, ops.EPI_SWIGLU_BF16, N // 2)):
+        y = torch.zeros(M, cols, device=gpu, dtype=dt)
+        ops.gemm_bf16(xl, w, y, M, e)
+        for lo in (0, 64, 128, 250, 288):
+            n = min(16, M - lo)
+            part = torch.zeros(n, cols, device=gpu, dtype=dt)
+            ops.gemm_bf16(xl[lo:lo + n].contiguous(), w, part, n, e)
+            assert torch.equal(part, y[lo:lo + n]), (lo, e)
+        if e == ops.EPI_SWIGLU_BF16:
+            gate, up = xl.double() @ w[:N // 2].double().T, xl.double() @ w[N // 2:].double().T
+            ref = gate * torch.sigmoid(gate) * up
+        else:
+            ref = xl.double() @ w.double().T
+        assert (y.double() - ref).abs().max() <= 2 ** -7 * ref.abs().max() + 1e-3, e
     M, inter, K = 19, 56, 96
     x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
     wgu = torch.randn(2 * inter, K, generator=g).bfloat16().to(gpu)
