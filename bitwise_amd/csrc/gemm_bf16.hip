@@ -991,7 +991,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // a step pulls 48 KB for twice the 128 x 128 tile's products (which pulls 32), and a wave's 64 accumulators leave room
 // for the sums of the segments before, so that a K of several segments, which the 256 x 256 kernel does not take,
 // runs on these where there are enough of them.  Three stages of 48 KB (x 16 KB | W 32 KB); a wave issues six loads a
-// stage.  Plain and SwiGLU epilogues; segments joined left to right in registers.  K a multiple of 64.
+// stage.  Plain, residual and SwiGLU epilogues; segments joined left to right in registers (a residual add's chain
+// starts at the residual, which is read when the first segment ends).  K a multiple of 64.
 #define T256_STAGE (48 * 1024)
 #define T256_STAGES 3
 
@@ -999,7 +1000,7 @@ template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile256_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
     int ldo, int m_tiles, int n_tiles) {
-  static_assert(EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16, "plain and SwiGLU epilogues");
+  static_assert(EPI != EPI_QKV_ROPE, "plain, residual and SwiGLU epilogues");
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char t256_lds[];   // [3 stages][x 16 KB | W 32 KB]
@@ -1096,11 +1097,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     asm volatile("" ::: "memory");
     const int kn = (step + 1) * 64;
     if (kn % GEMM_SEG == 0 && kn < K) {                // a segment ends before the last: joined left to right
+      if (EPI == EPI_ADD_F32 && kn == GEMM_SEG) {      // the chain of a residual add starts at the residual
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + 64 * wy + 16 * i + 4 * g + q, n = n0 + 64 * wx + 16 * j + r;
+              tot[i][j][q] = (m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;
+            }
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          tot[i][j] = kn == GEMM_SEG ? acc[i][j] : tot[i][j] + acc[i][j];
+          tot[i][j] = (EPI != EPI_ADD_F32 && kn == GEMM_SEG) ? acc[i][j] : tot[i][j] + acc[i][j];
           acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
     }
@@ -1111,7 +1123,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] + acc[i][j];
   }
-  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, QkvRopeArgs{});
+  // (a residual add of several segments has the residual in its sums; of one segment the epilogue adds it)
+  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g,
+                        EPI == EPI_ADD_F32 && K > GEMM_SEG, QkvRopeArgs{});
+}
+
+template <int EPI>
+static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s) {
+  constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+  const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
+  static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_tile256_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              T256_STAGES * T256_STAGE);
+    allowed = true;
+  }
+  hipLaunchKernelGGL((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
+                     ldo, mt, nt);
+  return BW_LAUNCH_CHECK();
 }
 
 // ------------------------------------------------------------------------------ up to 64 rows, through LDS
@@ -1937,11 +1966,12 @@ static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
 //   tile split  a 128 x 128 workgroup per tile and segment, the segments' sums whole in scratch and joined in order
 //               afterwards (128 rows of K = 8192: 25 us).
 //   big split   the same with 256 x 256 tiles, which fetch half as many bytes a flop: for 512 rows or more.
-// All four give the same bits.  The choice is by a count of steps: rounds times the steps of a workgroup (a step of
+//   tile256     128 x 256 tiles with all of K, the segments joined in registers: needs no scratch.
+// All five give the same bits.  The choice is by a count of steps: rounds times the steps of a workgroup (a step of
 // a 256 x 256 tile counts twice); the join moves 8 bytes an element and segment (about 500,000 elements in the
 // time of a step) and is a launch more (8 steps); a split has to win by a tenth.  tiles64: what the 64-row
 // kernel's scratch is sized by.
-enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT };
+enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT, ADD_TILE256 };
 
 static AddRoute add_route(int M, int N, int K, int ldo, int& tiles64) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
@@ -1959,6 +1989,11 @@ static AddRoute add_route(int M, int N, int K, int ldo, int& tiles64) {
   const long long tile_split = ((t128 * S + 255) / 256) * (GEMM_SEG / 64) + join;
   const long long big_split = M >= 2 * BIG_BM ? ((tbig * S + 255) / 256) * 2 * (GEMM_SEG / 64) + join : whole;
   const long long split = tile_split <= big_split ? tile_split : big_split;
+  // 128 x 256 tiles with all of K, the segments joined in registers: no scratch, no join; a step of theirs takes
+  // 1.0 us (1.6 of the 128 x 128 tile's)
+  const long long t256 = (long long)((M + 127) / 128) * ((N + 255) / 256);
+  const long long whole256 = ((t256 + 255) / 256) * (K / 64) * 8 / 5;
+  if (whole256 < whole && whole256 <= split) return ADD_TILE256;
   if (10 * split >= 9 * whole) return ADD_WHOLE;
   return tile_split <= big_split ? ADD_TILE_SPLIT : ADD_BIG_SPLIT;
 }
@@ -2053,6 +2088,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         }
         return 0;
       }
+      if (route == ADD_TILE256) return launch_tile256<EPI>(x, w, out, M, N, K, ldx, ldo, s);
       if (route == ADD_BIG_SPLIT && sp.scratch != nullptr && ((uintptr_t)out & 15) == 0) {
         if (scratch_floats < (size_t)S * M * N) return -6;
         const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + 255) / 256;
@@ -2109,17 +2145,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
       // (in rounds of 256 workgroups; a step of these takes 1.0 us where a 128 x 128 tile's takes 0.58)
       const int rounds256 = (mt * nt + 255) / 256, rounds128 = (mt * ((N + COLS256 / 2 - 1) / (COLS256 / 2)) + 255) / 256;
-      if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) {
-        static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
-        if (!allowed) {
-          (void)hipFuncSetAttribute((const void*)gemm_bf16_tile256_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    T256_STAGES * T256_STAGE);
-          allowed = true;
-        }
-        hipLaunchKernelGGL((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K,
-                           ldx, ldo, mt, nt);
-        return BW_LAUNCH_CHECK();
-      }
+      if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) return launch_tile256<EPI>(x, w, out, M, N, K, ldx, ldo, s);
     }
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;

@@ -192,11 +192,14 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     # a residual add of more than 64 rows whose 128 x 128 tiles with all of K would leave compute units idle: up to
     # 128 rows and three segments in blocks of 64 rows through that kernel (its scratch if K has several segments);
     # else a workgroup per tile (128 x 128, or 256 x 256 from 512 rows) and segment, the segments' sums whole in
-    # scratch and joined in order afterwards.  The bits of the rows alone, 16 at a time, with and without scratch,
+    # scratch and joined in order afterwards; or 128 x 256 tiles with all of K where those go round the compute units
+    # once (no scratch).  The bits of the rows alone, 16 at a time, with and without scratch,
     # twice on the same scratch (full of NaN at first, larger than needed); ragged edges, a short last segment
     S = lambda K: (K + 2047) // 2048
     for M, N, K, kind in [(65, 2048, 4096, "blocks"), (128, 1100, 2048 * 2 + 320, "blocks"), (100, 2048, 2048, "blocks"),
                           (129, 2048, 2048, None), (81, 2048, 4096 + 72, None), (640, 4096, 4096, None),
+                          (2048, 4096, 4096, None),       # 128 x 256 tiles, the two segments joined in registers
+
                           (65, 2048, 8192, "sums"), (145, 2048, 8192, "sums"), (300, 1000, 2 * 2048 + 192, "sums"),
                           (768, 2048, 8192, "sums"), (700, 3000, 4 * 2048 + 128, "sums"), (2048, 2048, 8192, "sums"),
                           (513, 8192, 4096, "sums")]:
