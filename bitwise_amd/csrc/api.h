@@ -2,7 +2,8 @@
 // returns 0, a HIP error code (> 0), or a negative code for arguments it refuses:
 //   -2 sizes or strides out of range, -3 misaligned pointer or stride,
 //   -4 head size not compiled in, -5 page size not supported, -6 scratch smaller than asked for,
-//   -7 sizes beyond what the library's own static scratch holds.
+//   -7 sizes beyond what the library's own static scratch holds (inside the library also: not this kernel's shape),
+//   -8 a decode attention whose partials do not fit a workgroup's LDS (a context too long for the kernel).
 // All pointers are device pointers.  Nothing here allocates.
 #pragma once
 #include <stdint.h>
@@ -60,6 +61,8 @@ int bw_attention_decode_scratch(int num_tiles, int heads, int kv_heads, int head
                                 int page_size, long long* scratch_floats, int* counters);
 int bw_attention_fold_group_tiles(int head_dim);
 int bw_norm_gemm_supported(int M, int K);
+// rows wider than one 2048-segment of K: whether the fused norm + product kernel with ``cols`` columns a workgroup takes them
+int bw_norm_gemm_wide_supported(int M, int N, int K, int cols);
 int bw_norm_gemm_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps, const void* w,
                       void* out, int ldo, int M, int N, int K, int epilogue, void* stream);
 int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w, int norm_w_is_bf16, float eps,

@@ -22,11 +22,15 @@ from .runtime import Runtime
 from .weights import loader
 
 
+def model_spec(config: Mapping[str, Any]):
+    """The ``ModelSpec`` its architecture makes of a configuration (a config.json dictionary)."""
+    arch = registry.architecture_of(config)
+    return arch.spec_from_config(arch.config_from_dict(config))
+
+
 def describe(config: Mapping[str, Any]) -> Dict[str, TensorSpec]:
     """Names and shapes of the checkpoint tensors a configuration needs (no GPU involved)."""
-    arch = registry.architecture_of(config)
-    spec = arch.spec_from_config(arch.config_from_dict(config))
-    return AssembledModel(spec, Runtime("float32", device=None)).tensor_specs()
+    return AssembledModel(model_spec(config), Runtime("float32", device=None)).tensor_specs()
 
 
 def write_random_model(folder: str | Path, config: Mapping[str, Any], seed: int, sigma: float = 0.02,
@@ -36,7 +40,7 @@ def write_random_model(folder: str | Path, config: Mapping[str, Any], seed: int,
     model's tensor order from one generator seeded with ``seed``."""
     arch = registry.architecture_of(config)
     typed = arch.config_from_dict(config)
-    torch_dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
+    torch_dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}[dtype]
     return loader.write_model_folder(folder, typed.to_dict(), describe(config), seed, sigma, torch_dtype)
 
 
@@ -54,8 +58,9 @@ class Model:
         arch = registry.architecture_of(raw)
         typed = arch.config_from_dict(raw)
         rt = Runtime(dtype, device)
-        assembled = AssembledModel(arch.spec_from_config(typed), rt)
-        tensors = loader.load_folder(path, assembled.tensor_specs())
+        spec = arch.spec_from_config(typed)
+        assembled = AssembledModel(spec, rt)
+        tensors = loader.load_folder(path, assembled.tensor_specs(), spec.ignored_tensor_suffixes, spec.unused_tensors)
         assembled.bind_tensors(tensors)
         return cls(typed, assembled)
 

@@ -38,4 +38,8 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         max_positions=cfg.max_position_embeddings,
         bos_token_id=cfg.bos_token_id,
         eos_token_id=cfg.eos_token_id,
+        # exporters store the rotary frequencies as a buffer; a tied checkpoint may still carry the
+        # head's matrix, which the reference never reads then (src/model.cpp:170-171)
+        ignored_tensor_suffixes=("rotary_emb.inv_freq",),
+        unused_tensors=("lm_head.weight",) if cfg.tie_word_embeddings else (),
     )

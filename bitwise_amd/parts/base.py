@@ -79,6 +79,11 @@ class ModelSpec:
     max_positions: int
     bos_token_id: int = -1
     eos_token_id: int = -1
+    # Checkpoint tensors the model does not read and the loader lets pass: names that end in one of
+    # ``ignored_tensor_suffixes`` are exporters' buffers without learned values (no word is said);
+    # a name in ``unused_tensors`` holds values this configuration has no use for (a warning).
+    ignored_tensor_suffixes: Tuple[str, ...] = ()
+    unused_tensors: Tuple[str, ...] = ()
 
 
 @dataclass(frozen=True)

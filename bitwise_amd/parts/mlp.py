@@ -64,7 +64,9 @@ class SwiGLU(FeedForward):
             self.gate_up.store(ws, h, gu, rows)
             act32 = ws.buffer("mlp_h32", self.inter, torch.float32)
             ops.swiglu_f32(gu, act32, rows)
-            if rt.bf16 and self.down.mfma:
+            if rt.bf16:
+                # bfloat16 mode rounds the activation here whatever dtype the weights are stored in, so that
+                # the mode has one set of rounding points (a 32-bit down projection widens it again)
                 act = ws.buffer("mlp_h", self.inter, torch.bfloat16)
                 ops.convert(act32, act, rows)
             else:

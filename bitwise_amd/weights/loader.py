@@ -12,7 +12,7 @@ from __future__ import annotations
 import json
 import warnings
 from pathlib import Path
-from typing import Dict, Iterator, Mapping, Tuple
+from typing import Dict, Iterator, Mapping, Sequence, Tuple
 
 import torch
 
@@ -24,14 +24,21 @@ class WeightError(ValueError):
     """One error for everything wrong with a checkpoint: missing, unexpected, misshapen."""
 
 
-# Buffers some exporters store beside the weights; they carry no learned values.
-_IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
+class UnusedTensorWarning(UserWarning):
+    """A checkpoint tensor that the architecture knows of and this configuration does not read."""
 
 
 def check_and_convert(specs: Mapping[str, TensorSpec], found: Mapping[str, torch.Tensor],
-                      source: str = "checkpoint") -> Dict[str, torch.Tensor]:
+                      source: str = "checkpoint", ignored_suffixes: Sequence[str] = (),
+                      unused: Sequence[str] = ()) -> Dict[str, torch.Tensor]:
+    """``ignored_suffixes`` and ``unused`` come from the architecture (``ModelSpec``): tensors it
+    knows to carry nothing (passed over in silence) or nothing this configuration reads (passed
+    over with an ``UnusedTensorWarning``).  Any other tensor the model has no use for is an error."""
     missing = [n for n in specs if n not in found]
-    unexpected = [n for n in found if n not in specs and not n.endswith(_IGNORED_SUFFIXES)]
+    ignored = tuple(ignored_suffixes)
+    extra = [n for n in found if n not in specs and not (ignored and n.endswith(ignored))]
+    unexpected = [n for n in extra if n not in unused]
+    tolerated = [n for n in extra if n in unused]
     wrong = []
     out: Dict[str, torch.Tensor] = {}
     for name, spec in specs.items():
@@ -62,14 +69,18 @@ def check_and_convert(specs: Mapping[str, TensorSpec], found: Mapping[str, torch
             lines.append(f"  wrong shape or dtype ({len(wrong)}):")
             lines.extend("    " + w for w in wrong)
         raise WeightError("\n".join(lines))
+    if tolerated:
+        warnings.warn(f"{source}: tensors stored and not used by this configuration: " + ", ".join(tolerated),
+                      UnusedTensorWarning, stacklevel=2)
     return out
 
 
-def load_folder(folder: str | Path, specs: Mapping[str, TensorSpec]) -> Dict[str, torch.Tensor]:
+def load_folder(folder: str | Path, specs: Mapping[str, TensorSpec], ignored_suffixes: Sequence[str] = (),
+                unused: Sequence[str] = ()) -> Dict[str, torch.Tensor]:
     with warnings.catch_warnings():
         warnings.simplefilter("ignore")       # read-only memory maps viewed as tensors
         found = safetensors_io.read_folder(folder)
-    return check_and_convert(specs, found, source=str(folder))
+    return check_and_convert(specs, found, str(folder), ignored_suffixes, unused)
 
 
 def random_tensors(specs: Mapping[str, TensorSpec], seed: int, sigma: float = 0.02,

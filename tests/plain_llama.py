@@ -82,11 +82,17 @@ def rope(v: torch.Tensor, positions: Sequence[int], inv_freq: np.ndarray) -> tor
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rnd: Callable = identity,
-              window: Optional[int] = None) -> torch.Tensor:
+              window: Optional[int] = None, partition: Optional[int] = None, first_position: int = 0) -> torch.Tensor:
     """Causal grouped-query attention over one whole sequence (src/kernels.cpp:312-368).
     q: [T, heads, hd]; k, v: [T, kv_heads, hd].  Head h reads kv head h // group; the score
     is dot(q, k) * (1/sqrt(hd)) (scale after the dot); the query at position p sees keys
-    0..p; weights are exp(s - max) and the output is sum(e*v) * (1/sum(e))."""
+    0..p; weights are exp(s - max) and the output is sum(e*v) * (1/sum(e)).
+
+    ``partition`` (with a rounding ``rnd``; the reference has neither): where a weight is rounded.  The engine's
+    bfloat16 path cuts the keys at absolute positions into partitions of that many and rounds a weight against
+    the maximum of its own partition's visible scores, rnd(exp(s - m_partition)); the partitions are then
+    weighed against each other by exp(m_partition - max) unrounded.  Without rounding this is the formula
+    above, term for term."""
     T, heads, hd = q.shape
     group = heads // k.shape[1]
     scale = 1.0 / math.sqrt(hd)
@@ -96,8 +102,15 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rnd: Callable =
         for p in range(T):
             lo = 0 if window is None else max(0, p - window + 1)
             s = (kh[lo:p + 1] @ q[p, h]) * scale
-            e = torch.exp(s - s.max())
-            out[p, h] = (rnd(e)[:, None] * vh[lo:p + 1]).sum(0) * (1.0 / rnd(e).sum())
+            if partition is None:
+                e = rnd(torch.exp(s - s.max()))
+            else:
+                part = (torch.arange(lo, p + 1) + first_position) // partition
+                part = part - part[0]
+                maxima = torch.full((int(part[-1]) + 1,), -math.inf, dtype=F64).scatter_reduce(0, part, s, "amax")
+                local = maxima[part]                                                   # each key's partition's maximum
+                e = rnd(torch.exp(s - local)) * torch.exp(local - s.max())
+            out[p, h] = (e[:, None] * vh[lo:p + 1]).sum(0) * (1.0 / e.sum())
     return out
 
 
@@ -106,7 +119,7 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return gate * (1.0 / (1.0 + torch.exp(-gate))) * up
 
 
-def attention_block(x, w, pre, c, positions, rnd, window=None):
+def attention_block(x, w, pre, c, positions, rnd, window=None, partition=None):
     """Steps 3-8 of the layer (src/model.cpp:281-300): norm, q/k/v projections (the engine's
     stacked QKV GEMM is the three projections side by side, src/model.cpp:150-153), rotary
     on q and k, attention, output projection."""
@@ -117,7 +130,7 @@ def attention_block(x, w, pre, c, positions, rnd, window=None):
     v = linear(xn, w[pre + "self_attn.v_proj.weight"]).view(T, c["kv_heads"], c["head_dim"])
     inv_freq = rope_inv_freq(c["theta"], c["head_dim"])
     q, k, v = rnd(rope(q, positions, inv_freq)), rnd(rope(k, positions, inv_freq)), rnd(v)
-    a = rnd(attention(q, k, v, rnd, window)).reshape(T, -1)
+    a = rnd(attention(q, k, v, rnd, window, partition, positions[0])).reshape(T, -1)
     return linear(a, w[pre + "self_attn.o_proj.weight"])
 
 
@@ -129,17 +142,19 @@ def mlp_block(x, w, pre, c, rnd):
 
 
 def forward(config: Mapping[str, object], w: Mapping[str, torch.Tensor], tokens: Sequence[int],
-            rnd: Callable = identity, first_position: int = 0, windows: Optional[Sequence[Optional[int]]] = None) -> torch.Tensor:
+            rnd: Callable = identity, first_position: int = 0, windows: Optional[Sequence[Optional[int]]] = None,
+            partition: Optional[int] = None) -> torch.Tensor:
     """Logits [T, vocab] (float64) at every position of one whole sequence
     (src/model.cpp:267-322 with every row wanted, as python/bindings.cpp:35-52 does).
     ``first_position`` shifts all positions (only distances matter to rotary attention).
-    ``windows``: per layer, how many keys a query sees (None: all; the reference has no window)."""
+    ``windows``: per layer, how many keys a query sees (None: all; the reference has no window).
+    ``partition``: see ``attention``."""
     c = read_config(config)
     positions = [first_position + i for i in range(len(tokens))]
     x = embed(tokens, w["model.embed_tokens.weight"])
     for layer in range(c["layers"]):
         pre = f"model.layers.{layer}."
-        x = x + attention_block(x, w, pre, c, positions, rnd, None if windows is None else windows[layer])
+        x = x + attention_block(x, w, pre, c, positions, rnd, None if windows is None else windows[layer], partition)
         x = x + mlp_block(x, w, pre, c, rnd)
     x = rnd(rmsnorm(x, w["model.norm.weight"], c["eps"]))
     head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]
@@ -221,14 +236,14 @@ def block_hash(parent: int, tokens: Sequence[int]) -> int:
 
 
 def generate(config, w, prompt: List[int], max_new_tokens: int, temperature: float = 0.0, seed: int = 0,
-             ignore_eos: bool = False, rnd: Callable = identity) -> List[int]:
+             ignore_eos: bool = False, rnd: Callable = identity, partition: Optional[int] = None) -> List[int]:
     """Whole-sequence recomputation for every new token; sampling position is the number of
     tokens held before the new one (src/engine.cpp:467-476), stop rules of :250-254."""
     c = read_config(config)
     toks = list(prompt)
     out: List[int] = []
     for _ in range(max_new_tokens):
-        row = forward(config, w, toks, rnd)[-1].to(torch.float32).numpy()
+        row = forward(config, w, toks, rnd, partition=partition)[-1].to(torch.float32).numpy()
         if temperature <= 0:
             t = argmax_row(row)
         else:

@@ -8,6 +8,7 @@ import torch
 import bitwise_amd as bw
 from bitwise_amd import registry
 from bitwise_amd.config.llama import ConfigError, LlamaConfig
+from bitwise_amd.model import model_spec
 from bitwise_amd.weights import loader, safetensors_io
 from tiny import TINY_A, TINY_B
 
@@ -96,16 +97,33 @@ def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
     tensors = dict(loader.random_tensors(specs, 0))
     del tensors["model.layers.1.mlp.down_proj.weight"]
     del tensors["model.norm.weight"]
-    tensors["lm_head.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)               # tied model: not wanted
+    tensors["model.layers.0.self_attn.bias"] = torch.zeros(64, dtype=torch.bfloat16)     # nothing reads it
     tensors["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 32, dtype=torch.bfloat16)
     tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)             # exporter's buffer: ignored
     safetensors_io.write_file(tmp_path / "model.safetensors", tensors.items())
+    spec = model_spec(TINY_A)
     with pytest.raises(bw.WeightError) as e:
-        loader.load_folder(tmp_path, specs)
+        loader.load_folder(tmp_path, specs, spec.ignored_tensor_suffixes, spec.unused_tensors)
     msg = str(e.value)
     assert "missing tensors (2)" in msg and "model.norm.weight" in msg and "model.layers.1.mlp.down_proj.weight" in msg
-    assert "unexpected tensors (1): lm_head.weight" in msg and "inv_freq" not in msg
+    assert "unexpected tensors (1): model.layers.0.self_attn.bias" in msg and "inv_freq" not in msg
     assert "model.layers.0.self_attn.q_proj.weight: stored (64, 32), the configuration needs (64, 64)" in msg
+
+
+def test_a_tied_checkpoint_that_stores_the_head_loads_with_a_warning(tmp_path):
+    """The reference reads lm_head.weight only when the head is not tied (src/model.cpp:170-171); a tied
+    checkpoint that stores it anyway is used without it, and says so.  An untied model still needs it, and a
+    tensor that no configuration of the architecture reads is still an error."""
+    specs, spec = bw.describe(TINY_A), model_spec(TINY_A)
+    assert spec.unused_tensors == ("lm_head.weight",) and model_spec(TINY_B).unused_tensors == ()
+    tensors = dict(loader.random_tensors(specs, 0))
+    tensors["lm_head.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)
+    safetensors_io.write_file(tmp_path / "model.safetensors", tensors.items())
+    with pytest.warns(loader.UnusedTensorWarning, match="lm_head.weight"):
+        w = loader.load_folder(tmp_path, specs, spec.ignored_tensor_suffixes, spec.unused_tensors)
+    assert set(w) == set(specs)
+    with pytest.raises(bw.WeightError, match="unexpected tensors \\(1\\): lm_head.weight"):
+        loader.load_folder(tmp_path, specs)                      # an architecture that does not know the name
 
 
 def test_broken_files(tmp_path):

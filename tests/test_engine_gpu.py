@@ -40,7 +40,6 @@ def test_generation_equals_plain(folders, name, dtype):
     implementation, which recomputes the whole sequence for every token."""
     cfg, w = tiny.read_config(folders[name]), tiny.read_weights(folders[name])
     model = bw.Model.load(folders[name], dtype)
-    rnd = pl.round_bf16 if dtype == "bfloat16" else pl.identity
     g = torch.Generator().manual_seed(4)
     prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (1, 7, 19, 33)]
     params = [bw.SamplingParams(max_new_tokens=16, ignore_eos=True),
@@ -48,7 +47,7 @@ def test_generation_equals_plain(folders, name, dtype):
               bw.SamplingParams(max_new_tokens=16), bw.SamplingParams(max_new_tokens=10, temperature=1.3, seed=9)]
     results = bw.generate(model, prompts, params, engine_config(name, dtype, max_batched_tokens=24))
     for p, sp, r in zip(prompts, params, results):
-        want = pl.generate(cfg, w, p, sp.max_new_tokens, sp.temperature, sp.seed, sp.ignore_eos, rnd)
+        want = pl.generate(cfg, w, p, sp.max_new_tokens, sp.temperature, sp.seed, sp.ignore_eos, **tiny.plain_mode(dtype))
         assert r.tokens == want and r.finished
     assert model.config.num_key_value_heads == cfg["num_key_value_heads"] and model.weight_bytes > 0
 
@@ -102,7 +101,7 @@ def test_long_decoding_with_and_without_graphs(folders):
         (r,) = bw.generate(model, [prompt], sp, engine_config(name, dtype, use_graphs=graphs))
         outs.append(r)
     assert outs[0].tokens == outs[1].tokens and outs[0].logits_fingerprint == outs[1].logits_fingerprint
-    want = pl.generate(cfg_long, tiny.read_weights(folder), prompt, 100, 0.9, 3, True, pl.round_bf16)
+    want = pl.generate(cfg_long, tiny.read_weights(folder), prompt, 100, 0.9, 3, True, **tiny.plain_mode(dtype))
     assert outs[0].tokens == want
 
 

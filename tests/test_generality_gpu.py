@@ -291,9 +291,9 @@ def test_windowed_groups_end_to_end(gpu, tmp_path, dtype):
     g = torch.Generator().manual_seed(14)
     x = torch.randint(0, 500, (150,), generator=g).tolist()
     y = torch.randint(0, 500, (70,), generator=g).tolist()
-    rnd = pl.round_bf16 if dtype == "bfloat16" else pl.identity
-    refs = {"x": pl.forward(cfg, w, x, rnd, windows=windows).numpy(), "y": pl.forward(cfg, w, y, rnd, windows=windows).numpy()}
-    tol = 2e-2 if dtype == "bfloat16" else 2e-5
+    mode = tiny.plain_mode(dtype)
+    refs = {"x": pl.forward(cfg, w, x, windows=windows, **mode).numpy(), "y": pl.forward(cfg, w, y, windows=windows, **mode).numpy()}
+    tol = 1e-2 if dtype == "bfloat16" else 2e-5
 
     def run(steps, max_tokens, **kw):
         rp = Replayer("", dtype, max_tokens, block_size=8, model=model, poison_freed_pages=True, **kw)

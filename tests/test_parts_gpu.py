@@ -23,6 +23,16 @@ F64 = torch.float64
 TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
 
 
+def check_rows(got, ref, mode, what):
+    """Maximum over all rows within TOL, and the median over rows at 32-bit accuracy: in bfloat16 mode part and
+    plain code round at the same places, so a row differs by more only where a value fell so close to the
+    middle between two bfloat16 numbers that the two roundings parted."""
+    scale = ref.abs().max()
+    per_row = ((got - ref).abs().amax(dim=1) / scale).numpy()
+    print(f"{what} {mode}: max {per_row.max():.2e} (bound {TOL[mode]:.1e}), median over rows {np.median(per_row):.2e} (bound 1e-6)")
+    assert per_row.max() <= TOL[mode] and np.median(per_row) <= 1e-6, what
+
+
 def rnd_for(mode):
     return pl.round_bf16 if mode == "bfloat16" else pl.identity
 
@@ -64,7 +74,7 @@ def test_feed_forward_part(gpu, mode):
     hd = h[:n].cpu().double()
     act = rnd_for(mode)(pl.swiglu(pl.linear(hd, w["gate_proj.weight"]), pl.linear(hd, w["up_proj.weight"])))
     ref = before[:n].cpu().double() + pl.linear(act, w["down_proj.weight"])
-    assert (res[:n].cpu().double() - ref).abs().max() <= TOL[mode] * ref.abs().max()
+    check_rows(res[:n].cpu().double(), ref, mode, "feed-forward part")
     assert torch.equal(res[n:], before[n:])                         # rows beyond the step are not touched
 
 
@@ -105,8 +115,9 @@ def test_attention_part(gpu, mode, heads, kvh, hd, window):
     q = rnd(pl.rope(pl.linear(x, w["q_proj.weight"]).view(n, heads, hd), range(n), inv))
     k = rnd(pl.rope(pl.linear(x, w["k_proj.weight"]).view(n, kvh, hd), range(n), inv))
     v = rnd(pl.linear(x, w["v_proj.weight"]).view(n, kvh, hd))
-    ref = pl.linear(rnd(pl.attention(q, k, v, rnd, window)).reshape(n, -1), w["o_proj.weight"])
-    assert (got - ref).abs().max() <= TOL[mode] * ref.abs().max()
+    ref = pl.linear(rnd(pl.attention(q, k, v, rnd, window, partition=64 if mode == "bfloat16" else None)).reshape(n, -1),
+                    w["o_proj.weight"])
+    check_rows(got, ref, mode, f"attention part {heads}/{kvh}x{hd} window {window}")
 
 
 # ----------------------------------------------------------------------------- a toy mixer with state

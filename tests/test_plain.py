@@ -89,6 +89,35 @@ def test_attention_groups_causality_and_window():
     assert torch.allclose(w[6, 0], pl.attention(q[4:7, :1], k[4:7, :1], v[4:7, :1])[2, 0], rtol=1e-12)
 
 
+def test_rounding_in_partitions_changes_only_where_a_weight_is_rounded():
+    """Without rounding, partitions of keys are the plain formula term for term (any partition size, any shift
+    of the positions, with a window); with a rounding, a sequence within one partition is the unpartitioned
+    formula, and a partition whose maximum is far below the row's keeps the relative precision of its weights
+    (rounded against the row's maximum they would lose it)."""
+    torch.manual_seed(2)
+    T, heads, hd = 150, 2, 8
+    q, k, v = (torch.randn(T, heads, hd, dtype=F64) for _ in range(3))
+    base = pl.attention(q, k, v)
+    for part, first, window in ((64, 0, None), (64, 37, None), (16, 5, 40), (1, 0, None), (1000, 0, 7)):
+        ref = base if window is None else pl.attention(q, k, v, window=window)
+        got = pl.attention(q, k, v, window=window, partition=part, first_position=first)
+        assert torch.allclose(got, ref, rtol=1e-11, atol=1e-13), (part, first, window)
+    short = pl.attention(q[:60], k[:60], v[:60], pl.round_bf16, partition=64)
+    assert torch.equal(short, pl.attention(q[:60], k[:60], v[:60], pl.round_bf16))
+    assert not torch.equal(pl.attention(q[:60], k[:60], v[:60], pl.round_bf16, partition=64, first_position=30), short)
+    # two keys in two partitions, the second score 20 above the first: the first key's weight is e^-20, which the
+    # fold applies unrounded to a weight of exactly 1
+    q1 = torch.zeros(2, 1, 1, dtype=F64)
+    q1[1] = 1.0
+    k1 = torch.tensor([0.0, 20.0], dtype=F64).view(2, 1, 1)
+    v1 = torch.tensor([1.0, 0.0], dtype=F64).view(2, 1, 1)
+    out = pl.attention(q1, k1, v1, pl.round_bf16, partition=1)[1, 0, 0].item()
+    exact = math.exp(-20.0) / (1.0 + math.exp(-20.0))
+    assert abs(out - exact) < 1e-15 * exact + 1e-22
+    rough = pl.attention(q1, k1, v1, pl.round_bf16)[1, 0, 0].item()
+    assert abs(rough - exact) > 1e-4 * exact
+
+
 def test_swiglu():
     g, u = torch.tensor([0.0, 40.0, -40.0, 1.5], dtype=F64), torch.tensor([3.0, 2.0, 2.0, -1.0], dtype=F64)
     out = pl.swiglu(g, u)

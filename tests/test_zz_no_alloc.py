@@ -27,6 +27,26 @@ def _library():
     return lib
 
 
+def _hip_runtime() -> ctypes.CDLL:
+    """The HIP runtime this process has already loaded (the one torch and the kernel library call), by the path
+    the process maps it from; a second copy of the runtime would count its own allocations only."""
+    with open("/proc/self/maps") as f:
+        paths = {line.split()[-1] for line in f if "libamdhip64.so" in line}
+    assert len(paths) == 1, f"one HIP runtime is expected in the process, found {sorted(paths)}"
+    return ctypes.CDLL(paths.pop())
+
+
+def _free_device_memory() -> int:
+    """Free bytes on the current device as the HIP runtime itself counts them: any hipMalloc or hipFree, by
+    whomever, moves it; torch's own counters see only torch's allocator."""
+    hip = _hip_runtime()
+    hip.hipMemGetInfo.argtypes = [c_void_p, c_void_p]
+    hip.hipMemGetInfo.restype = c_int
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.addressof(free), ctypes.addressof(total)) == 0
+    return free.value
+
+
 def _scratch_need(lib, M, N, K):
     floats, counters = c_longlong(0), c_int(0)
     assert lib.bw_gemm_add_scratch(M, N, K, ctypes.addressof(floats), ctypes.addressof(counters)) == 0
@@ -52,16 +72,38 @@ def test_static_scratch_residual_add_matches_the_workspace_one(gpu):
                                   count.data_ptr(), counters, stream)
         assert rc == 0
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated(gpu)
+        # a first call on a copy of the output (it may load the kernels' code and takes the array's address), then
+        # the call that is measured: the runtime's free memory must not move, whoever might have allocated
+        warm = res.clone()
+        assert lib.bw_gemm_add_bf16_static(x.data_ptr(), w.data_ptr(), warm.data_ptr(), M, N, K, K, N, stream) == 0
+        torch.cuda.synchronize()
+        before, before_torch = _free_device_memory(), torch.cuda.memory_allocated(gpu)
         rc = lib.bw_gemm_add_bf16_static(x.data_ptr(), w.data_ptr(), got.data_ptr(), M, N, K, K, N, stream)
         assert rc == 0
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated(gpu) == before
+        assert _free_device_memory() == before and torch.cuda.memory_allocated(gpu) == before_torch
+        assert torch.equal(warm, got)
         assert not torch.equal(got, res), "the product must have been added"
         assert torch.equal(got.view(torch.int32), want.view(torch.int32)), (M, N, K)
         # and against the plain sum, so that two equal wrong results do not pass
         ref = res.double() + x.double() @ w.double().T
         assert (got.double() - ref).abs().max().item() < 2e-3 * max(1.0, ref.abs().max().item())
+
+
+def test_the_free_memory_figure_sees_an_allocation(gpu):
+    """The measure the test above relies on can fail: an allocation behind torch's back moves it."""
+    hip = _hip_runtime()
+    hip.hipMalloc.argtypes = [c_void_p, ctypes.c_size_t]
+    hip.hipMalloc.restype = c_int
+    hip.hipFree.argtypes = [c_void_p]
+    hip.hipFree.restype = c_int
+    torch.cuda.synchronize()
+    before, before_torch = _free_device_memory(), torch.cuda.memory_allocated(gpu)
+    ptr = c_void_p(0)
+    assert hip.hipMalloc(ctypes.addressof(ptr), 64 << 20) == 0
+    held = _free_device_memory()
+    assert hip.hipFree(ptr) == 0
+    assert held < before and torch.cuda.memory_allocated(gpu) == before_torch
 
 
 def test_static_scratch_refuses_what_it_cannot_hold(gpu):

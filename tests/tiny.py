@@ -57,3 +57,13 @@ def read_weights(folder: Path) -> Dict[str, torch.Tensor]:
 
 def read_config(folder: Path) -> dict:
     return json.loads((Path(folder) / "config.json").read_text())
+
+
+def plain_mode(dtype: str) -> dict:
+    """Keyword arguments that make the plain float64 model the counterpart of a precision mode: in bfloat16
+    mode activations are rounded to bfloat16 where the engine stores them so, and attention weights are rounded
+    within partitions of 64 keys at absolute positions (the engine's definition of that mode); the 32-bit mode
+    rounds nothing."""
+    import plain_llama as pl
+
+    return {"rnd": pl.round_bf16, "partition": 64} if dtype == "bfloat16" else {"rnd": pl.identity}
