@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "layout.h"
+
 typedef uint16_t bf16_t;  // raw bfloat16 bits
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -218,7 +220,7 @@ __device__ __forceinline__ void norm_rows_load(NormRows<R, NV>& nr, const f32x4*
                                                int w_is_bf16, int nvec, int lane) {
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int c = 64 * j + lane < nvec ? 64 * j + lane : nvec - 1;
+    const int c = norm_vec_index(j, lane, nvec);
     nr.w[j] = load_norm_w_raw(w, w_is_bf16, c);
 #pragma unroll
     for (int i = 0; i < R; ++i) nr.v[i][j] = (rows[i] != nullptr ? rows[i] : rows[0])[c];
@@ -234,7 +236,7 @@ __device__ __forceinline__ void norm_rows_finish(const NormRows<R, NV>& nr, cons
     float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const bool in = 64 * j + lane < nvec;
+      const bool in = norm_vec_in_row(j, lane, nvec);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float x = in ? nr.v[i][j][e] : 0.0f;
@@ -246,7 +248,7 @@ __device__ __forceinline__ void norm_rows_finish(const NormRows<R, NV>& nr, cons
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int c = 64 * j + lane;
-      if (c < nvec) {
+      if (norm_vec_in_row(j, lane, nvec)) {
         const f32x4 wv = norm_w_floats(nr.w[j], w_is_bf16);
         u32x2 pk = {pack_bf16x2((nr.v[i][j][0] * inv) * wv[0], (nr.v[i][j][1] * inv) * wv[1]),
                     pack_bf16x2((nr.v[i][j][2] * inv) * wv[2], (nr.v[i][j][3] * inv) * wv[3])};

@@ -39,7 +39,7 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
 
 enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI_ROPE_KV = 4 };
 
-#define DEC_SEG 2048
+// (DEC_SEG, the LDS layout of the rows and the rings, and what the launchers admit: layout.h)
 
 struct DecodeGemmArgs {
   const float* a;          // [M, lda] rows of the 32-bit residual stream
@@ -110,7 +110,7 @@ __device__ __forceinline__ void decode_norm_rows(const DecodeGemmArgs& a, int wa
   __builtin_amdgcn_sched_barrier(0);
   for (int m0 = wave; m0 < M;) {
     norm_rows_finish<RB>(nr, nrows, a.norm_w_is_bf16, nvec, K, a.eps, lane, [&](int i, int c, u32x2 pk) {
-      *reinterpret_cast<u32x2*>(xs + (size_t)(m0 + i * nwaves) * lds_row + 4 * c) = pk;
+      *reinterpret_cast<u32x2*>(xs + decode_norm_store_elem(m0 + i * nwaves, c, K)) = pk;
     });
     m0 += RB * nwaves;
     if (m0 >= M) break;
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   constexpr int NB = SH::NB;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int K = a.K, M = a.M;
-  const int lds_row = K + 8;                      // bf16 elements; +16 bytes keeps operand reads conflict-free
+  const int lds_row = decode_lds_row(K);          // bf16 elements; +16 bytes keeps operand reads conflict-free
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);   // [M][lds_row], then the waves' rings
   const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
 #pragma unroll
   for (int t = 0; t < 2; ++t) voff_w[t] = ((8 * t + lrow) * K + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
   const int steps = K / 64;
-  unsigned char* ring = smem + (((size_t)M * lds_row * sizeof(bf16_t) + 15) & ~(size_t)15) + (size_t)wave * SH::STAGES * SH::STAGE;
+  unsigned char* ring = smem + decode_ring_offset(M, K, wave, SH::STAGES, SH::STAGE);
 
   // 1. Everything but weights is asked for before the ring (see the head of the file).  The rotary
   // epilogue's items first: what this thread's (row, pair) items need (at most 2 items a thread).
@@ -202,10 +202,10 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
 
   // 3. the product: A from the rows in LDS (rows past M read row 0; their results are thrown away), B from
   // the wave's ring.
-  const bf16_t* ap = xs + (size_t)(r < M ? r : 0) * lds_row + 8 * g;
+  const bf16_t* ap = xs + decode_operand_elem(r, M, g, 0, 0, K);
   int off_w[2];
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) off_w[kk] = (r >> 3) * 1024 + (r & 7) * 128 + (((4 * kk + g) ^ (r >> 1)) * 16);
+  for (int kk = 0; kk < 2; ++kk) off_w[kk] = decode_ring_operand_offset(r, g, kk);
   f32x4 acc[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -292,13 +292,13 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
   }
 }
 
-static const size_t kMaxLds = 160 * 1024 - 1024;
+static const size_t kMaxLds = DEC_MAX_LDS;
 
 template <int EPI, int ST>
 static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hipStream_t s) {
   static bool raised = false;
   using SH = DecodeShape<EPI, ST>;
-  const size_t lds = (((size_t)a.M * (a.K + 8) * sizeof(bf16_t) + 15) & ~(size_t)15) + (size_t)waves * SH::STAGES * SH::STAGE;
+  const size_t lds = decode_lds_bytes(a.M, a.K, waves, SH::STAGES, SH::STAGE);
   if (lds > kMaxLds) return -2;
   if (!raised) {   // more than 64 KB of dynamic LDS has to be asked for once
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gemm_kernel<EPI, ST>),
@@ -312,10 +312,7 @@ static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hi
 
 // Can the rows (M of them, K wide) live in LDS, and do the waves of a strip fit a workgroup?
 static int check_decode_gemm(const DecodeGemmArgs& a) {
-  if (a.M <= 0 || a.M > 16 || a.N <= 0 || a.K <= 0 || (a.K % 64)) return -2;
-  if (a.K > DEC_SEG || (a.lda % 4) || a.lda < a.K) return -2;      // a row is normalised from a wave's registers
-  if ((size_t)a.M * (a.K + 8) * sizeof(bf16_t) + 64 * 1024 > kMaxLds) return -2;      // the rows and the waves' rings
-  return 0;
+  return decode_gemm_admits(a.M, a.N, a.K, a.lda) ? 0 : -2;      // (a row is normalised from a wave's registers)
 }
 
 extern "C" int bw_norm_gemm_supported(int M, int K) {

@@ -47,8 +47,7 @@
 
 #include "common.h"
 #include "api.h"
-
-enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3, EPI_QKV_ROPE = 4 };
+#include "layout.h"        // the epilogues' numbers, GEMM_SEG, MidShape and the LDS layout of the rows normalised in the kernel
 
 // What the rotary epilogue of the stacked q|k|v product needs: the statements of
 // rope_kvwrite_bf16_kernel on the 32-bit products while they are still in registers.
@@ -64,8 +63,6 @@ struct QkvRopeArgs {
   int page_shift;              // page_size is a power of two: positions are split by shift and mask, not by division
   int head_dim = 64;           // (the kernels for up to 64 rows take multiples of 64; the tiled ones 64)
 };
-
-#define GEMM_SEG 2048
 
 template <int EPI>
 __device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o, float v, float u) {
@@ -1171,37 +1168,7 @@ static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, in
 // along K (two where a step has 64 rows of W): what a compute unit pulls grows with its waves and with the bytes
 // between two barriers (64 rows of the output projection: 29 KB a microsecond with four waves and a stage a step,
 // 55 with eight and four steps).  K in whole stages.
-template <int EPI, int NRB, bool NORM, bool NARROW = false, bool EIGHT = false>
-struct MidShape {
-  static constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
-  static constexpr bool HALVES = GLU || NARROW;                     // waves are (strip, half of the row blocks)
-  static constexpr int NW = EIGHT ? 8 : 4;                          // waves
-  static constexpr int COLS = HALVES ? 32 : 64;                     // output columns a workgroup
-  static constexpr int B_ROWS = NARROW ? 32 : 64;                   // rows of W a step (SwiGLU: 32 gate, 32 up)
-  static constexpr int SUB = EIGHT ? (B_ROWS == 64 ? (NORM || NRB == 4 ? 1 : 2) : (NORM ? 2 : 4)) : 1;   // steps of 64 along K a stage (NORM: weights only)
-  static constexpr int STRIPS = COLS / 16, GROUPS = NW / STRIPS;    // wave = (strip of the columns, group of the row blocks)
-  static constexpr int A_LOADS = NORM ? 0 : (SUB * 2 * NRB + NW - 1) / NW; // per wave and stage: 8 rows of x each
-  static constexpr int B_LOADS = SUB * B_ROWS / 8 / NW;             // 8 rows of W each
-  static constexpr int LPW = A_LOADS + B_LOADS;
-  static constexpr int A_BYTES = NORM ? 0 : NRB * 2048, STEP_BYTES = A_BYTES + B_ROWS * 128, STAGE = SUB * STEP_BYTES;
-  static constexpr int NI = NRB >= GROUPS ? NRB / GROUPS : 1;       // blocks of rows a wave works on (fewer blocks than groups: waves that only load)
-  static constexpr int NJ = GLU ? 2 : 1;
-  static constexpr bool ROPE_NARROW = NARROW && EPI == EPI_QKV_ROPE;  // a workgroup = 16 rotary pairs of a head
-  // 17 rows or more: a ring of at most 72 KB, so that two workgroups share a compute unit and one's first loads
-  // and epilogue lie under the other's steps (products with more workgroups than compute units: gate|up 17.2 ->
-  // 16.0 us, the 8B shape's 53 -> 50 and its down projection 37 -> 35; the others unchanged); never fewer than 3
-  static constexpr int FIT0 = (NORM || NRB < 2 ? 150 : 72) * 1024 / STAGE;
-  static constexpr int FIT = FIT0 < 3 ? 3 : FIT0;
-  static constexpr int STAGES = EIGHT ? (NORM ? 8 : (FIT > 6 ? 6 : FIT))
-                                      : (ROPE_NARROW && NRB <= 2 ? 16 : 8);   // (half the weights a stage: twice the stages, where they fit)
-  static constexpr int PENDING = LPW * (STAGES - 2);                // loads that may still be in flight at a step's start
-  static constexpr int RING = STAGES * STAGE + 1024;                // and 1 KB where padding loads put their zeros
-  static_assert(PENDING < 64, "the wait count has six bits");
-  static_assert(STAGES >= 3, "a stage at hand, one landing, one asked for");
-  static_assert(!NORM || NRB == 1, "rows are normalised in the kernel only up to 16 of them");
-  static_assert(!NARROW || (!GLU && (EPI == EPI_QKV_ROPE || NRB >= 2)), "narrow tiles: plain epilogues of 17 rows or more, or the rotary one");
-  static_assert(!EIGHT || NORM || (NRB >= 2 && (SUB * 2 * NRB) % NW == 0), "eight waves: 17 rows or more, or rows normalised in the kernel");
-};
+// (MidShape, the numbers that follow from these choices, is in layout.h)
 
 // Residual add over several segments of K, a workgroup per tile and segment (gridDim.y segments): where the
 // segments' sums meet (device scratch, [tile][segment][wave][block of rows][lane] x 16 bytes) and the tiles'
@@ -1237,12 +1204,12 @@ __device__ __forceinline__ void mid_issue(unsigned char* lds, __amdgpu_buffer_rs
                                           const MidLoads<EPI, NRB, NORM, NARROW, EIGHT>& ld, int step, int steps, int k_base) {
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
-  unsigned char* dst = lds + (step % S::STAGES) * S::STAGE;
+  unsigned char* dst = lds + mid_stage_offset<S>(step);
   const bool real = step < steps;                                     // scalar
   const int k_off = (k_base + step * S::SUB * 64) * 2;
 #pragma unroll
   for (int t = 0; t < S::A_LOADS; ++t)                                // (a padding load's zeros go behind the ring)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(ld.dst_a[t] >= 0 ? dst + ld.dst_a[t] : lds + S::STAGES * S::STAGE), 16,
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(ld.dst_a[t] >= 0 ? dst + ld.dst_a[t] : lds + mid_padding_offset<S>()), 16,
                                              real ? ld.voff_a[t] : 0x7ffffff0, k_off, 0, 0);
 #pragma unroll
   for (int t = 0; t < S::B_LOADS; ++t)
@@ -1261,7 +1228,7 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   const f32x4* nrows[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    const int m = wave + i * S::NW;
+    const int m = mid_norm_row_of(wave, i, S::NW);
     nrows[i] = m < M ? reinterpret_cast<const f32x4*>(na.x32 + (size_t)m * na.ldx32) : nullptr;
   }
   norm_rows_load<RB>(nr, nrows, na.norm_w, na.norm_w_is_bf16, nvec, lane);
@@ -1273,9 +1240,8 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   const int nw = S::NW, row_step = na.row_step;
   norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
     // vector c = elements 4c..4c+3 of row m: step c / 16, 16-byte chunk (c % 16) / 2 of the step, its half c % 2
-    const int m = wave + i * nw;
-    unsigned char* p = rl + (c >> 4) * row_step + (m >> 3) * 1024 + (m & 7) * 128 + ((((c & 15) >> 1) ^ ((m & 15) >> 1)) * 16) + (c & 1) * 8;
-    *reinterpret_cast<u32x2*>(p) = pk;
+    const int m = mid_norm_row_of(wave, i, nw);
+    *reinterpret_cast<u32x2*>(rl + mid_norm_store_offset(c, m, row_step)) = pk;
   });
 }
 
@@ -1305,18 +1271,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   // SwiGLU: W rows 0-31 of the tile are gate rows n0.., 32-63 the up rows N + n0..; a wave's loads are all of one kind
   const int lrow = lane >> 3, lslot = lane & 7;
   // which 1 KB of a stage this wave's t-th load of W is: block ``blk`` (8 rows) of step ``sub`` of the stage
-  auto b_load = [&](int t, int& sub, int& blk) {
-    constexpr int PER_STEP = S::B_ROWS / 8;
-    if constexpr (EIGHT && GLU) {                                    // waves 0-3: the gate rows, 4-7: the up rows
-      const int id = (wave & 3) * S::B_LOADS + t;
-      sub = id / (PER_STEP / 2);
-      blk = id % (PER_STEP / 2) + (PER_STEP / 2) * (wave >> 2);
-    } else {
-      const int id = wave * S::B_LOADS + t;
-      sub = id / PER_STEP;
-      blk = id % PER_STEP;
-    }
-  };
+  auto b_load = [&](int t, int& sub, int& blk) { mid_b_load<S>(wave, t, sub, blk); };
   int sub0, blk0;
   b_load(0, sub0, blk0);
   const bool up = GLU && blk0 >= 4;                                  // (all of a wave's loads are of one kind)
@@ -1325,12 +1280,12 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   MidLoads<EPI, NRB, NORM, NARROW, EIGHT> ld;
 #pragma unroll
   for (int t = 0; t < S::A_LOADS; ++t) {
-    const int id = wave * S::A_LOADS + t, sub = id / (2 * NRB), block = id % (2 * NRB);
+    int sub, block;
+    const bool is_load = mid_a_load<S, NRB>(wave, t, sub, block);    // past the stage's blocks: a padding load
     const int row = block * 8 + lrow;                                // of the NRB * 16 rows of x
     const int chunk = lslot ^ ((row & 15) >> 1);
-    const bool is_load = id < S::SUB * 2 * NRB;                      // past them: a padding load
     ld.voff_a[t] = is_load ? (row * ldx + 8 * chunk + 64 * sub) * 2 : 0x7ffffff0;
-    ld.dst_a[t] = is_load ? sub * S::STEP_BYTES + block * 1024 : -1;
+    ld.dst_a[t] = is_load ? mid_a_dst<S>(sub, block) : -1;
   }
   if constexpr (S::A_LOADS == 0) {
     ld.voff_a[0] = 0;
@@ -1344,7 +1299,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     const int chunk = lslot ^ ((row & 15) >> 1);
     const int w_row = ROPE ? (row < PAIRS ? pair0 + row : half + pair0 + row - PAIRS) : (GLU ? row & 31 : row);
     ld.voff_b[t] = (w_row * K + 8 * chunk + 64 * sub) * 2;
-    ld.dst_b[t] = sub * S::STEP_BYTES + S::A_BYTES + blk * 1024;
+    ld.dst_b[t] = mid_b_dst<S>(sub, blk);
   }
   // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
   // segment after segment, each segment's sums joined to those before it when it ends
@@ -1359,14 +1314,12 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
       tot[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
   // lane (g, r) wants row r of a block of 16 rows (2 KB), chunk 4*kk + g: slot (4*kk + g) ^ (r >> 1) of that row
-  const int row_off = (r >> 3) * 1024 + (r & 7) * 128;
   int slot_off[2];
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = row_off + (((4 * kk + g) ^ (r >> 1)) * 16);
+  for (int kk = 0; kk < 2; ++kk) slot_off[kk] = mid_operand_offset(r, g, kk);
   const int strip = wave % S::STRIPS;                                 // of the tile's output columns
-  const int a_block0 = NI * (wave / S::STRIPS);                       // first block of 16 rows this wave works on
-  const int b_off0 = S::A_BYTES + strip * 2048;                       // its (gate) strip; the up strip lies 4 KB further
-  const bool computing = !EIGHT || a_block0 < NRB;                    // (eight waves, two blocks of rows, two strips: half the waves only load)
+  const int a_block0 = mid_first_block<S>(wave);                      // first block of 16 rows this wave works on
+  const bool computing = a_block0 < NRB;                              // (more groups of waves than blocks of rows: the others only load)
 
   // Rotary epilogue (the stacked q|k|v product, heads of 64: the workgroup's columns are a head, or 16 pairs of
   // one): what this thread's (row, pair) items need, cosine, sine and page, hangs on the row's position.
@@ -1390,15 +1343,13 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     // wait for the rows must not be a wait for weights); wave w takes rows w, w + 4, ...: as many at a time as
     // there are (a slot without a row would fetch a row for nothing)
     if (wave < M) {
-      if constexpr (EIGHT) {                                           // wave w takes rows w and w + 8
-        // (rows of two segments: sixteen vectors a lane, and by the launch no more than a row a wave)
-        if (K > GEMM_SEG) mid_norm_rows<1, 16, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else if (M <= 8) mid_norm_rows<1, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else mid_norm_rows<2, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-      } else {
-        if (M <= 4) mid_norm_rows<1, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else if (M <= 8) mid_norm_rows<2, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
-        else if (M <= 12) mid_norm_rows<3, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      const int rows_a_wave = mid_norm_rows_a_wave(M, S::NW);         // EIGHT: at most 2 (rows w and w + 8), else at most 4
+      if (mid_norm_vectors_a_lane(K) == 16)                           // (rows of two segments: by the launch no more than a row a wave)
+        mid_norm_rows<1, 16, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else if (rows_a_wave == 1) mid_norm_rows<1, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else if (rows_a_wave == 2) mid_norm_rows<2, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
+      else if constexpr (!EIGHT) {
+        if (rows_a_wave == 3) mid_norm_rows<3, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
         else mid_norm_rows<4, 8, EPI, NRB, NARROW, EIGHT>(na, M, K, wave, lane, rows_lds, mid_lds, rs_a, rs_b, ld, steps, k_base);
       }
     }
@@ -1437,7 +1388,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     mid_issue<EPI, NRB, NORM, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, step + S::STAGES - 1, steps, k_base);   // into the stage worked on a step ago
-    const unsigned char* stage = mid_lds + (step % S::STAGES) * S::STAGE;
+    const unsigned char* stage = mid_lds + mid_stage_offset<S>(step);
     if (computing) {
 #pragma unroll
       for (int sub = 0; sub < S::SUB; ++sub) {
@@ -1447,9 +1398,10 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
           u32x4 fa[NI], fb[NJ];
 #pragma unroll
           for (int i = 0; i < NI; ++i)
-            fa[i] = *reinterpret_cast<const u32x4*>((NORM ? rows_lds + (step * S::SUB + sub) * na.row_step : at) + (a_block0 + i) * 2048 + slot_off[kk]);
+            fa[i] = *reinterpret_cast<const u32x4*>(NORM ? rows_lds + mid_norm_read_offset(step * S::SUB + sub, a_block0 + i, na.row_step, r, g, kk)
+                                                         : at + (a_block0 + i) * 2048 + slot_off[kk]);
 #pragma unroll
-          for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(at + b_off0 + j * 4096 + slot_off[kk]);
+          for (int j = 0; j < NJ; ++j) fb[j] = *reinterpret_cast<const u32x4*>(at + mid_b_read_offset<S>(strip, j, r, g, kk));
 #pragma unroll
           for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -1580,8 +1532,8 @@ static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, 
                             const MidNormArgs& na, const QkvRopeArgs& rp, int segments, const MidSplitArgs& sp) {
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
-  const int lds_bytes = S::RING + (NORM ? (K / 64) * na.row_step + (na.row_step == 1024 ? 1024 : 0) : 0);   // (8-row blocks: the reads of rows 8 to 15 end a block further)
-  if (lds_bytes > 160 * 1024) return -2;
+  const int lds_bytes = NORM ? mid_norm_lds_bytes(S::RING, K, na.row_step) : S::RING;
+  if (lds_bytes > BW_LDS_LIMIT) return -2;
   if (!allowed) {
     (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
@@ -1608,11 +1560,9 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
                      int ldo, int M, int N, int K, int epilogue, void* stream) {
   const int cols = epilogue == EPI_SWIGLU_BF16 ? 32 : 64;
   const int wgs = (N + cols - 1) / cols;
-  if (M > 16 || K % 64 || wgs < 64) return -7;
-  // rows of two segments of K: eight of them at most (a row a wave, sixteen vectors a lane; LDS holds 8-row blocks)
-  const bool wide = K > GEMM_SEG;
-  if (wide && (M > 8 || K > 2 * GEMM_SEG || K % 128)) return -7;
-  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, wide ? 1024 : 2048};
+  // (rows of two segments of K: eight of them at most, a row a wave, sixteen vectors a lane; LDS holds 8-row blocks)
+  if (!mid_norm_admits(M, K, wgs)) return -7;
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, mid_norm_row_step(K)};
   const bf16_t* wp = (const bf16_t*)w;
   hipStream_t s = (hipStream_t)stream;
   switch (epilogue) {
@@ -1626,7 +1576,7 @@ int bw_norm_gemm_mid(const float* x32, int ldx32, const void* norm_w, int norm_w
 
 // Whether bw_norm_gemm_mid takes rows of this width that the other fused kernels do not (wider than a segment of K).
 extern "C" int bw_norm_gemm_wide_supported(int M, int N, int K, int cols) {
-  return M > 0 && M <= 8 && K > GEMM_SEG && K <= 2 * GEMM_SEG && K % 128 == 0 && cols > 0 && (N + cols - 1) / cols >= 64;
+  return cols > 0 && K > GEMM_SEG && mid_norm_admits(M, K, (N + cols - 1) / cols);
 }
 
 #define ROPE_NARROW_BELOW 256
@@ -1658,11 +1608,8 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
                          int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream) {
   const int all_heads = heads + 2 * kv_heads;
   const int wide_tiles = all_heads * (head_dim / 64);
-  if (head_dim % 64 || M > 16 || K % 64 || wide_tiles < 64)
-    return -7;
-  const bool wide = K > GEMM_SEG;                       // as in bw_norm_gemm_mid
-  if (wide && (M > 8 || K > 2 * GEMM_SEG || K % 128)) return -7;
-  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, wide ? 1024 : 2048};
+  if (head_dim % 64 || !mid_norm_admits(M, K, wide_tiles)) return -7;        // as in bw_norm_gemm_mid
+  MidNormArgs na{x32, norm_w, ldx32, norm_w_is_bf16, eps, mid_norm_row_step(K)};
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
                  heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size), head_dim};

@@ -135,8 +135,9 @@ class ModelRunner:
             bucket = next((b for b in GRAPH_BUCKETS if b >= min(self.max_rows, self.max_logit_rows)), None)
             if bucket is not None:
                 ws_rows, ws_logit_rows = max(ws_rows, bucket), max(ws_logit_rows, bucket)
-        self.ws = Workspace(model.rt.device, ws_rows, storage.page_size, ws_logit_rows)
         self.max_model_len = min(int(max_model_len), model.spec.max_positions)
+        self.ws = Workspace(model.rt.device, ws_rows, storage.page_size, ws_logit_rows,
+                            max_table_width=(self.max_model_len + storage.page_size - 1) // storage.page_size)
         self._graphs: Dict[int, tuple] = {}
         self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
         self.last_graph_rows = 0      # requests of the last step if it was replayed from a graph, else 0

@@ -176,6 +176,22 @@ class Attention(Mixer):
                     ops.attention_f32_tiles(qkv, ctx.positions, table, plan.decode_tiles, plan.decode_count, False, *common)
             self.o.add_into(ws, out, residual, rows)
 
+    def _split_scratch(self, ws, tiles: int, table_width: int):
+        """(floats, counters) of the split decode's scratch for this workspace: the worst case over the launches it
+        can see, or (0, 0) if this launch would not split."""
+        if not ops.attention_decode_scratch(tiles, self.heads, self.kv_heads, self.head_dim, table_width, ws.page_size)[0]:
+            return 0, 0
+        width = max(table_width, ws.max_table_width or 0)
+        key = ("attn_split_size", self.heads, self.kv_heads, self.head_dim, width)
+        sizes = ws.notes.get(key)
+        if sizes is None:
+            floats = counters = 0
+            for t in range(1, min(ws.max_rows, 128) + 1):            # (from 128 workgroups on nothing splits)
+                f, c = ops.attention_decode_scratch(t, self.heads, self.kv_heads, self.head_dim, width, ws.page_size)
+                floats, counters = max(floats, f), max(counters, c)
+            sizes = ws.notes[key] = (floats, counters)
+        return sizes
+
     def _attend(self, ctx, call, q, residual) -> None:
         """bfloat16 attention over the cache for rotated queries ``q``, then the output projection."""
         ws, rows = ctx.ws, ctx.rows
@@ -188,9 +204,10 @@ class Attention(Mixer):
         if plan.fold_count:
             ops.attention_bf16(q, ctx.positions, table, plan.fold_tiles, plan.fold_count, *common)
         if plan.decode_count:
-            # few decoded tokens: several workgroups a tile, meeting in device scratch
-            floats, counters = ops.attention_decode_scratch(plan.decode_count, self.heads, self.kv_heads, self.head_dim,
-                                                            table.stride(0), ws.page_size)
+            # few decoded tokens: several workgroups a tile, meeting in device scratch.  One buffer a workspace, sized
+            # for the worst launch it can see (the most tiles that still split, the widest table), whatever this
+            # step's shape: tables grow by a page every few steps, and a buffer per width would pile up.
+            floats, counters = self._split_scratch(ws, plan.decode_count, table.stride(0))
             scratch = None
             if floats:
                 scratch = (ws.buffer("attn_split", floats, torch.float32, rows=1),

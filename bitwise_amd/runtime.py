@@ -47,16 +47,21 @@ class Workspace:
     ``Model.logits`` call).  Buffers are made once per name for ``max_rows`` rows and never
     move, so HIP graphs captured over them stay valid; two workspaces share nothing."""
 
-    def __init__(self, device: torch.device, max_rows: int, page_size: int, max_logit_rows: int | None = None):
+    def __init__(self, device: torch.device, max_rows: int, page_size: int, max_logit_rows: int | None = None,
+                 max_table_width: int | None = None):
         self.device = torch.device(device)
         self.max_rows = int(max_rows)
         self.page_size = int(page_size)
         self.max_logit_rows = int(max_logit_rows if max_logit_rows is not None else max_rows)
+        # the widest block table a step of this engine can bring (pages of its longest request), if the owner
+        # knows it: a part that sizes scratch by the table's width asks once for the widest, not once per width
+        self.max_table_width = None if max_table_width is None else int(max_table_width)
         if self.max_rows < 1 or self.max_logit_rows < 1:
             raise ValueError("a workspace needs room for at least one row")
         if self.page_size < 1 or self.page_size & (self.page_size - 1):
             raise ValueError(f"page size must be a power of two, got {self.page_size}")
         self._buffers: Dict[Any, torch.Tensor] = {}
+        self.notes: Dict[Any, Any] = {}       # what parts have worked out for this workspace (sizes of their scratch)
 
     def buffer(self, name: str, cols: int, dtype: torch.dtype, rows: int | None = None) -> torch.Tensor:
         """A persistent zero-initialised [rows or max_rows, cols] scratch tensor by name."""

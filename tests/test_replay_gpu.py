@@ -226,6 +226,34 @@ def test_peaked_attention_whole_model(gpu, tmp_path, name, dtype):
         assert np.array_equal(got[rid], whole[rid]), f"{rid}: the mixed trace differs from the whole prompt"
 
 
+def test_the_workspace_stops_growing_while_contexts_grow(folders, tmp_path):
+    """Steps launched kernel by kernel bring block tables as wide as the step needs, and decoded tokens of few
+    requests split their attention over workgroups that meet in scratch sized by that width: the scratch is made
+    once for the widest table the engine can see, so a long run's memory stays where the first such step put it."""
+    from bitwise_amd.model import Model, write_random_model
+    from bitwise_amd.replay import Replayer
+
+    cfg = dict(tiny.CONFIGS["LONG"][0], max_position_embeddings=2048)
+    folder = write_random_model(tmp_path / "long2k", cfg, 6, 0.05)
+    model = Model.load(folder, "bfloat16")
+    toks = ru.requests_for(cfg["vocab_size"], 8, [900])["r0"]
+    other = ru.requests_for(cfg["vocab_size"], 9, [500])["r0"]
+    rp = Replayer("", "bfloat16", 2048, block_size=16, model=model, use_graphs=False)
+    rp.step([{"id": "a", "tokens": toks[:520], "want": []}])
+    sizes, widths = [], set()
+    for i in range(520, 900):
+        entries = [{"id": "a", "tokens": [toks[i]], "want": [0]}]
+        if i >= 600:                              # a second request comes and decodes beside the first
+            j = i - 600
+            entries.append({"id": "b", "tokens": other[:200] if j == 0 else [other[199 + j]], "want": []})
+        rp.step(entries)
+        sizes.append(rp.runner.ws.nbytes())
+        widths.add(len(rp.live["a"].tables[0]))
+    assert len(widths) > 20, "the block table must have grown page by page"
+    assert len([k for k in rp.runner.ws._buffers if k[0] == "attn_split"]) == 1, "the split route must have run, on one buffer"
+    assert sizes[-1] == sizes[0], f"the workspace grew from {sizes[0]} to {sizes[-1]} bytes"
+
+
 def test_first_tokens_of_a_sequence(folders):
     """Positions 0 and 1: one key, no rotation at position 0."""
     for name in ("A", "B"):
