@@ -16,6 +16,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence
 
+from ..config.engine import Fault
 from .pages import PagePool, StateSlots, block_hash
 
 
@@ -34,8 +35,9 @@ class RequestCache:
 
 class CacheManager:
     def __init__(self, groups: Sequence[GroupSpec], num_pages: int, page_size: int, num_slots: int,
-                 prefix_caching: bool = True, has_state: bool = False):
+                 prefix_caching: bool = True, has_state: bool = False, fault: int = 0):
         self.groups = list(groups)
+        self.fault = int(fault)            # a test-only bug for the simulator to catch (config.engine.Fault)
         self.page_size = page_size
         self.num_pages = num_pages
         self.prefix_caching = (bool(prefix_caching) and not has_state and len(self.groups) == 1
@@ -81,7 +83,7 @@ class CacheManager:
         if not self.prefix_caching or rc.tables[0]:
             return rc.computed
         ps = self.page_size
-        full = (len(tokens) - 1) // ps
+        full = (len(tokens) - (0 if self.fault == Fault.PREFIX_COVERS_LAST_TOKEN else 1)) // ps
         parent = 0
         pool = self.pools[0]
         for i in range(full):
@@ -145,7 +147,10 @@ class CacheManager:
         ps = self.page_size
         if self.prefix_caching:
             pool, table = self.pools[0], rc.tables[0]
-            for i in range(len(rc.hashes), computed // ps):
+            full = computed // ps
+            if self.fault == Fault.REGISTER_UNFINISHED_PAGE:        # (the page's tokens are known, its keys not yet there)
+                full = min(len(table), (computed + ps - 1) // ps, len(tokens) // ps)
+            for i in range(len(rc.hashes), full):
                 toks = tokens[i * ps:(i + 1) * ps]
                 h = block_hash(rc.hashes[i - 1] if i else 0, toks)
                 pool.register_full(table[i], h, toks)

@@ -19,6 +19,18 @@ class SamplingParams:
     ignore_eos: bool = False
 
 
+class Fault:
+    """Bugs the simulator must catch, switched on by ``EngineConfig.fault`` (src/engine.h:52-62: each a slip of one
+    line that an implementation could plausibly make; 3 belongs to speculative decoding, which is not here)."""
+    NONE = 0
+    PREFIX_COVERS_LAST_TOKEN = 1     # a prefix hit may take the page that holds the request's last known token
+    RNG_KEYED_BY_STEP = 2            # a draw is keyed by the engine's step instead of the request's position
+    REGISTER_UNFINISHED_PAGE = 4     # a page enters the prefix cache while a portion of its prompt is still to come
+    CANCEL_KEEPS_PAGES = 5           # a cancelled request's pages are not given back
+    NAMES = {1: "prefix hit covers the last token", 2: "randomness keyed by the engine's step",
+             4: "page registered before it is full", 5: "cancel keeps the pages"}
+
+
 @dataclass
 class EngineConfig:
     num_blocks: int = 512            # pages in every cache group's pool
@@ -31,6 +43,7 @@ class EngineConfig:
     max_model_len: int = 0           # 0: the model's max_position_embeddings
     use_graphs: bool = True          # replay pure-decode steps from captured HIP graphs
     run_ahead: bool = True           # launch the next pure-decode step before the last one's tokens are read back
+    fault: int = 0                   # a test-only bug (``Fault``) for the simulator to catch; 0: none
 
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
@@ -39,3 +52,5 @@ class EngineConfig:
             raise ValueError(f"block_size must be 8, 16, 32 or 64, got {self.block_size}")
         if self.num_blocks < 1 or self.max_batched_tokens < 1 or self.max_num_seqs < 1:
             raise ValueError("num_blocks, max_batched_tokens and max_num_seqs must be positive")
+        if self.fault and self.fault not in Fault.NAMES:
+            raise ValueError(f"fault must be 0 or one of {sorted(Fault.NAMES)}, got {self.fault}")

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, GroupSpec
-from ..config.engine import EngineConfig, SamplingParams
+from ..config.engine import EngineConfig, Fault, SamplingParams
 from ..csrc import ops
 from ..sampling.rng import FINGERPRINT_BASIS
 from .batch import Segment
@@ -183,7 +183,8 @@ class Engine:
         self.cfg.validate()
         self.exec = executor if executor is not None else GpuExecutor(target, self.cfg)
         self.manager = CacheManager(self.exec.group_specs, self.cfg.num_blocks, self.cfg.block_size,
-                                    self.cfg.max_num_seqs, self.cfg.prefix_caching, self.exec.has_state)
+                                    self.cfg.max_num_seqs, self.cfg.prefix_caching, self.exec.has_state,
+                                    fault=self.cfg.fault)
         self.sched = Scheduler(self.manager, self.cfg, on_open=self.exec.reset_slot)
         self._seqs: Dict[int, Sequence] = {}
         self._results: Dict[int, RequestResult] = {}
@@ -305,6 +306,8 @@ class Engine:
         records = [self.manager.record(w.seq.cache) for w in sampled]
         draw = ([w.seq.params.temperature for w in sampled], [r.seed for r in records],
                 [r.position + w.n for r, w in zip(records, sampled)])
+        if self.cfg.fault == Fault.RNG_KEYED_BY_STEP:
+            draw = (draw[0], draw[1], [self._stats.steps] * len(sampled))
         prints = [self._results[w.seq.id].logits_fingerprint for w in sampled] if self.cfg.fingerprint_logits else None
         t0 = self.now()
         return _Flight(plan, sampled, self._exec_launch(segments, draw, prints), t0)
@@ -344,6 +347,8 @@ class Engine:
         segments = [Segment([AHEAD_TOKEN], len(s.tokens), s.cache.tables, s.cache.slot, [0]) for s in running]
         records = [self.manager.record(s.cache) for s in running]
         draw = ([s.params.temperature for s in running], [r.seed for r in records], [len(s.tokens) + 1 for s in running])
+        if cfg.fault == Fault.RNG_KEYED_BY_STEP:
+            draw = (draw[0], draw[1], [self._stats.steps + 1] * len(running))
         t0 = self.now()
         pending = ex.launch(segments, draw, None, after=flight.pending if cfg.fingerprint_logits else None)
         self._stats.decode_rows += len(running)
@@ -393,7 +398,7 @@ class Engine:
         return False
 
     def _finish(self, s: Sequence, cancelled: bool) -> None:
-        self.sched.remove(s)
+        self.sched.remove(s, cancelled)
         r = self._results[s.id]
         r.finished = True
         r.cancelled = cancelled

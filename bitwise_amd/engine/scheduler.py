@@ -25,7 +25,7 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
 from ..cache.manager import CacheManager, RequestCache
-from ..config.engine import EngineConfig, SamplingParams
+from ..config.engine import EngineConfig, Fault, SamplingParams
 
 
 @dataclass
@@ -94,8 +94,10 @@ class Scheduler:
         self.stats.preemptions += 1
         self.preempted_ids.append(seq.id)
 
-    def remove(self, seq: Sequence) -> None:
+    def remove(self, seq: Sequence, cancelled: bool = False) -> None:
         """Finish or cancel: give back everything and leave the queues."""
+        if cancelled and self.cfg.fault == Fault.CANCEL_KEEPS_PAGES and seq.cache is not None:
+            seq.cache.tables = [[] for _ in seq.cache.tables]         # (the injected bug: the pages are forgotten)
         self._drop_cache(seq)
         if seq.running:
             self.running.remove(seq)

@@ -1,0 +1,141 @@
+"""Measuring the engine: decode steps, prefills and serving workloads with seeded synthetic tokens, each with
+the bytes or flops it has to move against the MI355X's published peaks (HBM 8 TB/s; dense matrix peaks 2.5 PFLOP/s
+in bfloat16 and 157.3 TFLOP/s in 32-bit).  ``bench.py`` and ``python -m bitwise_amd bench`` both call these."""
+
+from __future__ import annotations
+
+import time
+
+CONTEXT = 2048                      # tokens each request holds when decoding starts
+PREFILL_TOKENS = 2048
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12, "bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def prefill_flops(cfg: dict, tokens: int) -> float:
+    h, inter, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    qd = cfg["num_attention_heads"] * cfg["head_dim"]
+    kvd = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_token = 2 * (h * (qd + 2 * kvd) + qd * h + 2 * h * inter + inter * h)
+    attn = 2 * 2 * cfg["num_attention_heads"] * cfg["head_dim"] * tokens * (tokens + 1) / 2
+    return cfg["num_hidden_layers"] * (per_token * tokens + attn) + 2 * h * v      # the head runs for one row
+
+
+def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT):
+    block = 16
+    per_request = context + steps_total + 2 * block
+    cfg = bw.EngineConfig(num_blocks=batch * ((per_request + block - 1) // block) + 8, max_batched_tokens=2048,
+                          max_num_seqs=max(batch, 1), prefix_caching=False, fingerprint_logits=False,
+                          block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024))
+    return bw.Engine(model, None, cfg)
+
+
+def fill(engine, bw, torch, batch: int, vocab: int, new_tokens: int, seed: int, context: int = CONTEXT):
+    """Admit ``batch`` requests with ``context`` random tokens each and run their prompts."""
+    g = torch.Generator().manual_seed(seed)
+    for _ in range(batch):
+        prompt = torch.randint(0, vocab, (context,), generator=g).tolist()
+        engine.add_request(prompt, bw.SamplingParams(temperature=0.0, max_new_tokens=new_tokens, ignore_eos=True))
+    while engine.num_waiting or any(s.computed < s.prompt_len for s in engine.sched.running):
+        engine.step()
+
+
+def time_decode(engine, torch, steps: int, warmup: int):
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+
+
+def measure_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops: float, tokens: int = PREFILL_TOKENS) -> dict:
+    """One prompt of ``tokens`` tokens (2,048 unless said otherwise) in one step (model, head for the last row,
+    sampling): the median of six after two untimed ones (the shader clock takes some milliseconds of load to rise
+    from its idle 2.1 GHz to 2.4); the best of the six is given beside it."""
+    engine = make_engine(bw, model, 1, 8, dtype)
+    g = torch.Generator().manual_seed(99)
+    times = []
+    for _ in range(8):
+        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
+        engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+        assert engine.idle()
+    timed = sorted(times[2:])
+    ms, best = (timed[2] + timed[3]) / 2, timed[0]
+    flops = prefill_flops(cfg, tokens)
+    return {"value": round(tokens / ms * 1e3, 1), "tokens": tokens, "ms": round(ms, 3),
+            "frac": round(flops / (ms * 1e-3) / peak_flops, 4), "ms_best": round(best, 3), "runs": len(timed)}
+
+
+def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
+                   context: int = CONTEXT) -> dict:
+    """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
+    said otherwise): tokens a second, and the bytes a step has to read (every weight once, the cache of the live
+    requests) over its time."""
+    torch.cuda.empty_cache()
+    # Requests admitted early decode while the later ones are still being prefilled (2,048 prompt
+    # tokens a step): every request gets enough new tokens to outlast the prefills, the warm-up and the
+    # timed steps, so that each timed step has all ``batch`` rows.
+    chunks = (context + 2047) // 2048                  # steps a prompt takes under the 2,048-token budget
+    new_tokens = steps + warmup + batch * chunks + 8
+    eng = make_engine(bw, model, batch, new_tokens, dtype, context)
+    fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch, context=context)
+    assert len(eng.sched.running) == batch
+    secs = time_decode(eng, torch, steps, warmup)
+    assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
+    kv_token = eng.exec.storage.bytes_per_token()
+    del eng
+    ms = secs / steps * 1e3
+    # keys a decoded token reads, on average: the prompt, what the request decoded while later
+    # prompts were prefilled, the warm-up, and half the timed steps
+    avg_ctx = context + chunks * (batch - 1) / 2 + warmup + (steps + 1) / 2
+    step_bytes = model.weight_bytes + batch * avg_ctx * kv_token
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+    return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(achieved / PEAK_HBM_GBS, 4)}}
+
+
+def measure_serving(bw, torch, model, cfg: dict, dtype: str, requests: int = 64, seed: int = 5) -> dict:
+    """The continuous-batching workload of the reference's load generator (bench/loadgen.py:170-207) with synthetic
+    tokens: ``requests`` requests at once, prompt lengths uniform in [128, 2048], generation lengths uniform in
+    [64, 512], greedy, prompts cut into portions under a budget of 2,048 tokens a step, decoded beside each other."""
+    import random
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    work = []
+    for _ in range(requests):
+        n, new = rng.randint(128, 2048), rng.randint(64, 512)
+        work.append((torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), new))
+    block = 16
+    pages = sum((len(p) + new + 2 * block) // block + 1 for p, new in work)
+    ecfg = bw.EngineConfig(num_blocks=pages, max_batched_tokens=2048, max_num_seqs=requests, prefix_caching=False,
+                           fingerprint_logits=False, block_size=block, dtype=dtype, max_model_len=4096)
+    eng = bw.Engine(model, None, ecfg)
+    for p, new in work:
+        eng.add_request(p, bw.SamplingParams(max_new_tokens=new, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while not eng.idle():
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    generated = eng.stats.generated_tokens
+    prompt_tokens = sum(len(p) for p, _ in work)
+    assert generated == sum(new for _, new in work)
+    return {"requests": requests, "prompt_tokens": prompt_tokens, "generated_tokens": generated, "steps": steps,
+            "seconds": round(secs, 3), "generated_tok_s": round(generated / secs, 1),
+            "all_tok_s": round((generated + prompt_tokens) / secs, 1), "preemptions": eng.stats.preemptions}
+
+

@@ -9,6 +9,17 @@ from ..config.llama import LlamaConfig
 from ..parts.base import LayerCall, LayerSpec, ModelSpec, PartSpec
 
 
+# The sizes of the reference simulator's tiny model (sim/simulate.cpp:64-79) as a Llama (no biases): small enough
+# that a solo run of every request of a randomized scenario takes milliseconds, a vocabulary small enough that
+# an end-of-sequence token is drawn now and then.
+TINY_LLAMA = {
+    "architectures": ["LlamaForCausalLM"], "vocab_size": 97, "hidden_size": 64, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 512,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 256,
+    "eos_token_id": 3,
+}
+
+
 def llama_spec(cfg: LlamaConfig) -> ModelSpec:
     position = PartSpec("rope", {"theta": cfg.rope_theta, "head_dim": cfg.head_dim,
                                  "max_positions": cfg.max_position_embeddings})

@@ -7,10 +7,10 @@ from __future__ import annotations
 import json
 from dataclasses import dataclass
 from pathlib import Path
-from typing import Any, Callable, Dict, Mapping
+from typing import Any, Callable, Dict, Mapping, Optional
 
 from .config.llama import ConfigError, LlamaConfig
-from .models.llama import llama_spec
+from .models.llama import TINY_LLAMA, llama_spec
 from .parts.base import ModelSpec
 
 
@@ -19,15 +19,16 @@ class Architecture:
     name: str
     config_from_dict: Callable[[Mapping[str, Any]], Any]
     spec_from_config: Callable[[Any], ModelSpec]
+    tiny_config: Optional[Mapping[str, Any]] = None     # a small config.json of this architecture for simulations and smoke runs
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, spec_from_config) -> None:
+def register_architecture(name: str, config_from_dict, spec_from_config, tiny_config=None) -> None:
     if name in ARCHITECTURES:
         raise ValueError(f"architecture '{name}' is already registered")
-    ARCHITECTURES[name] = Architecture(name, config_from_dict, spec_from_config)
+    ARCHITECTURES[name] = Architecture(name, config_from_dict, spec_from_config, tiny_config)
 
 
 def architecture_of(config: Mapping[str, Any]) -> Architecture:
@@ -47,4 +48,4 @@ def read_config(folder: str | Path) -> Dict[str, Any]:
     return json.loads(path.read_text())
 
 
-register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec)
+register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec, TINY_LLAMA)

@@ -4,6 +4,7 @@ randomized scheduling traces (the reference's engine test and simulator,
 tests/test_main.cpp:241-302, sim/simulate.cpp)."""
 
 import json
+import os
 import subprocess
 import sys
 from pathlib import Path
@@ -144,15 +145,43 @@ def test_many_requests_decode_from_the_large_graph_buckets(gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_randomized_traces(gpu, dtype):
-    """The reference's simulator (sim/simulate.cpp) on the real engine: 0 token or logit
-    mismatches, no hang, no leaked page, and the traces must reach preemption and prefix hits."""
-    from bitwise_amd.cli import TINY_SIM_CONFIG
+def test_randomized_scenarios(gpu, dtype):
+    """The scenario simulator on the real engine: page sizes, graphs, steps launched ahead, model lengths, pools
+    and budgets drawn per scenario, every request against its solo run with pages of 16 and none of that: no
+    wrong token, no other logits, no hang, no page lost; and the scenarios reach preemption, prefix hits,
+    requests that end at an end-of-sequence token and cancellations."""
+    from bitwise_amd.registry import ARCHITECTURES
 
-    model = bw.Model.random(TINY_SIM_CONFIG, 42, dtype, sigma=0.08)
-    out = Simulator(model, dtype, block_size=16).run(traces=12, seed=1)
-    assert out.violations() == 0, "\n".join(out.notes[:10])
-    assert out.requests_checked > 20 and out.preemptions > 0 and out.prefix_hits > 0
+    model = bw.Model.random(ARCHITECTURES["LlamaForCausalLM"].tiny_config, 42, dtype, sigma=0.08)
+    tally = Simulator(model, dtype).run(24, seed=1)
+    print(tally.line(dtype))
+    assert tally.violations() == 0, "\n".join(tally.notes[:10])
+    assert tally.requests_compared > 60 and tally.preemptions > 0 and tally.prefix_hit_tokens > 0
+    assert tally.ended_by_eos > 0 and tally.cancelled > 0
+    assert len(tally.knobs_seen["block_size"]) >= 3 and tally.knobs_seen["use_graphs"] == {True, False}
+    assert tally.knobs_seen["run_ahead"] == {True, False}
+
+
+def test_the_simulator_program_catches_every_injected_fault(gpu):
+    """python -m bitwise_amd sim --sweep-faults on the GPU: the run without a fault is clean, each of the engine's
+    test-only bugs is reported, exit status 0; --fault alone exits with 1; an unknown fault with 2
+    (sim/simulate.cpp:239-240, :283-300)."""
+    import subprocess
+    import sys as _sys
+
+    env = dict(os.environ, PYTHONPATH=str(ROOT))
+    base = [_sys.executable, "-m", "bitwise_amd", "sim", "--seed", "3"]
+    p = subprocess.run(base + ["--traces", "40", "--sweep-faults"], capture_output=True, text=True, env=env, timeout=900)
+    print(p.stdout)
+    assert p.returncode == 0, p.stdout[-3000:] + p.stderr[-3000:]
+    lines = p.stdout.strip().splitlines()
+    assert lines[0].startswith("no fault: 40 scenarios") and "wrong tokens 0" in lines[0]
+    assert len(lines) == 6 and lines[-1].startswith("caught 4 of 4 injected faults; violations of the run without a fault: 0")
+    assert all("first failing scenario" in l for l in lines[1:5])
+    p = subprocess.run(base + ["--traces", "40", "--fault", "5"], capture_output=True, text=True, env=env, timeout=600)
+    assert p.returncode == 1 and "pages or slots lost 0" not in p.stdout
+    p = subprocess.run(base + ["--fault", "3"], capture_output=True, text=True, env=env, timeout=600)
+    assert p.returncode == 2 and "speculative" in p.stderr
 
 
 def test_long_shared_prefix_trace_at_real_layer_sizes_equals_solo(gpu):
@@ -223,6 +252,26 @@ def test_command_line(folders):
     p = subprocess.run([sys.executable, "-m", "bitwise_amd", "generate", "--nonsense"], capture_output=True, text=True,
                        cwd=str(ROOT), timeout=120)
     assert p.returncode == 2
+
+
+def test_command_line_random_config_and_bench(folders, tmp_path):
+    """--random-config: a config.json run with seeded random weights, the tokens of the same seed's folder; the
+    bench subcommand: one JSON line with a decode rate, its roofline and a prefill; both need one model source."""
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(tiny.TINY_B))
+    common = ["--dtype", "bfloat16", "--block-size", "8", "--prompt-tokens", "7,8,9,10", "--max-new-tokens", "5", "--ignore-eos"]
+    run = lambda extra: subprocess.run([sys.executable, "-m", "bitwise_amd", "generate", *extra, *common], capture_output=True,
+                                       text=True, cwd=str(ROOT), timeout=300)
+    a = run(["--random-config", str(cfg_file), "--weights-seed", "1", "--sigma", "0.05"])
+    b = run(["--model", str(folders["B"])])                        # tiny B's folder: seed 1, sigma 0.05
+    assert a.returncode == 0 and b.returncode == 0, a.stderr[-2000:] + b.stderr[-2000:]
+    assert json.loads(a.stdout)["tokens"] == json.loads(b.stdout)["tokens"]
+    assert run([]).returncode == 2 and run(["--model", str(folders["B"]), "--random-config", str(cfg_file)]).returncode == 2
+    p = subprocess.run([sys.executable, "-m", "bitwise_amd", "bench", "--model", str(tiny.make_folder(tmp_path, "LONG")), "--batch", "3", "--context", "200",
+                        "--steps", "8", "--warmup", "2", "--prefill-tokens", "150"], capture_output=True, text=True, cwd=str(ROOT), timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    line = json.loads(p.stdout.strip().splitlines()[-1])
+    assert line["decode"]["tok_s"] > 0 and line["decode"]["roofline"]["bound"] == "hbm" and line["prefill"]["tokens"] == 150
 
 
 def test_model_errors(folders, tmp_path):

@@ -3,6 +3,7 @@ to library routines, invariants, and known constants, each chosen so that a plau
 mistake (a wrong sign or pairing, a norm in the wrong place, a transposed weight) fails."""
 
 import math
+from pathlib import Path
 
 import numpy as np
 import pytest
@@ -248,3 +249,47 @@ def test_scalar_primitives():
     assert ps.swiglu([0.0], [5.0])[0] == 0.0 and ps.swiglu([30.0], [2.0])[0] == np.float32(60.0)
     y = ps.rmsnorm(np.full((1, 8), 3.0, np.float32), np.ones(8, np.float32), 0.5)
     assert np.allclose(y, 3.0 / math.sqrt(9.5), rtol=1e-6)
+
+
+def test_the_scalar_decoder_under_the_compilers_memory_and_arithmetic_checks(tmp_path):
+    """plain_scalar.cpp built as a program with -fsanitize=address,undefined (the reference builds its own C++
+    so for its sanitizer job: CMakeLists.txt:19-22, .github/workflows/ci.yml:29-40) and run on both tiny
+    configurations, one with windows: no report, and the bits of the optimised library."""
+    import subprocess
+    import numpy as np
+    import plain_scalar as ps
+    from bitwise_amd.model import describe
+    from bitwise_amd.weights.loader import random_tensors
+    from tiny import TINY_A, TINY_B
+
+    exe = tmp_path / "plain_scalar_checked"
+    here = Path(__file__).resolve().parent
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-ffp-contract=off", "-fno-fast-math", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=undefined", str(here / "plain_scalar_main.cpp"), "-o", str(exe)], check=True)
+    for cfg, seed, sigma, windows in ((TINY_A, 0, 0.02, [0, 0]), (TINY_B, 1, 0.05, [7, 0, 12])):
+        w = dict(random_tensors(describe(cfg), seed, sigma))
+        toks = [(i * 31 + 5) % cfg["vocab_size"] for i in range(23)]
+        want = ps.forward(cfg, w, toks, window=windows)
+        heads, H, L = cfg["num_attention_heads"], cfg["hidden_size"], cfg["num_hidden_layers"]
+        hd, kvh, I, V = cfg["head_dim"], cfg["num_key_value_heads"], cfg["intermediate_size"], cfg["vocab_size"]
+        cos, sin = ps.rope_tables(cfg["rope_theta"], hd, range(len(toks)))
+        names = ["model.embed_tokens.weight"]
+        for l in range(L):
+            pre = f"model.layers.{l}."
+            names += [pre + n for n in ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight",
+                                        "self_attn.v_proj.weight", "self_attn.o_proj.weight", "post_attention_layernorm.weight",
+                                        "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight")]
+        names += ["model.norm.weight", "model.embed_tokens.weight" if cfg["tie_word_embeddings"] else "lm_head.weight"]
+        case = tmp_path / "case.bin"
+        with open(case, "wb") as f:
+            f.write(np.asarray([len(toks), V, H, L, heads, kvh, hd, I], np.int32).tobytes())
+            f.write(np.float32(cfg["rms_norm_eps"]).tobytes())
+            f.write(np.asarray(windows, np.int32).tobytes() + np.asarray(toks, np.int32).tobytes())
+            f.write(np.ascontiguousarray(cos, np.float32).tobytes() + np.ascontiguousarray(sin, np.float32).tobytes())
+            for n in names:
+                f.write(w[n].float().numpy().astype("<f4").tobytes())
+        out = tmp_path / "logits.bin"
+        p = subprocess.run([str(exe), str(case), str(out)], capture_output=True, text=True, timeout=300)
+        assert p.returncode == 0 and not p.stderr.strip(), (p.returncode, p.stderr[-3000:])
+        got = np.fromfile(out, dtype="<f4").reshape(len(toks), V)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
