@@ -6,9 +6,13 @@ given back when it ends, is preempted or cancelled, and, in a windowed group, as
 window has passed them; cached full pages of a finished request stay until the space is
 needed (reference: src/engine.cpp:146-220, src/block_manager.cpp).
 
-Prefix reuse (src/engine.cpp:176-205) is only sound when the reused pages hold everything
-the request has computed: it is on for models with one group that keeps all keys and no
-per-request state outside the pages, and switched off otherwise.
+Prefix reuse (src/engine.cpp:176-205) is only sound when the reused pages hold everything the
+request has computed for its first tokens.  That is decided group by group: every group
+registers its full pages under the request's hash chain; a request may start behind n cached
+pages if every group still has the pages a query at position n * page_size reads there: all n
+in a group that keeps all keys, the pages under the window in a windowed group (pages the
+window has passed are given back, and stay findable until their space is needed).  State that
+a mixer keeps in a slot is in no page, so a model with such a mixer has no prefix reuse.
 """
 
 from __future__ import annotations
@@ -40,8 +44,7 @@ class CacheManager:
         self.fault = int(fault)            # a test-only bug for the simulator to catch (config.engine.Fault)
         self.page_size = page_size
         self.num_pages = num_pages
-        self.prefix_caching = (bool(prefix_caching) and not has_state and len(self.groups) == 1
-                               and self.groups[0].window is None)
+        self.prefix_caching = bool(prefix_caching) and not has_state and len(self.groups) > 0
         self.pools = [PagePool(num_pages, page_size, self.prefix_caching) for _ in self.groups]
         self.slots = StateSlots(num_slots)
         # called with (group, page) whenever a page becomes free (tests fill such pages with NaN, so that a
@@ -80,22 +83,34 @@ class CacheManager:
     def admit_prefix(self, rc: RequestCache, tokens: Sequence[int]) -> int:
         """Take cached pages holding a prefix of ``tokens``.  The page holding the last token
         is never reused, so that its logits are computed (src/engine.cpp:178-179)."""
-        if not self.prefix_caching or rc.tables[0]:
+        if not self.prefix_caching or any(rc.tables):
             return rc.computed
         ps = self.page_size
         full = (len(tokens) - (0 if self.fault == Fault.PREFIX_COVERS_LAST_TOKEN else 1)) // ps
+        chain: List[int] = []                       # the hash chain of the request's full pages
         parent = 0
-        pool = self.pools[0]
         for i in range(full):
-            toks = tokens[i * ps:(i + 1) * ps]
-            h = block_hash(parent, toks)
-            page = pool.lookup(h, toks)
-            if page is None:
-                break
-            rc.tables[0].append(page)
-            rc.hashes.append(h)
-            parent = h
-        rc.computed = len(rc.tables[0]) * ps
+            parent = block_hash(parent, tokens[i * ps:(i + 1) * ps])
+            chain.append(parent)
+
+        def has(g: int, i: int) -> bool:
+            return self.pools[g].peek(chain[i], tokens[i * ps:(i + 1) * ps]) is not None
+
+        # groups that keep all keys need pages 0..n-1: n is at most their common run of hits from the start
+        n = full
+        for g, spec in enumerate(self.groups):
+            if spec.window is None:
+                n = next((i for i in range(n) if not has(g, i)), n)
+        # windowed groups need the pages under the window of the next position: the longest n they all still hold
+        while n > 0 and not all(has(g, i) for g, spec in enumerate(self.groups) if spec.window is not None
+                                for i in range(self.first_needed_page(g, n * ps), n)):
+            n -= 1
+        for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
+            lo = self.first_needed_page(g, n * ps)
+            for i in range(n):
+                table.append(pool.lookup(chain[i], tokens[i * ps:(i + 1) * ps]) if i >= lo else -1)
+        rc.hashes.extend(chain[:n])
+        rc.computed = n * ps
         self.slots.records[rc.slot].position = rc.computed
         return rc.computed
 
@@ -146,14 +161,15 @@ class CacheManager:
         self.slots.records[rc.slot].position = computed
         ps = self.page_size
         if self.prefix_caching:
-            pool, table = self.pools[0], rc.tables[0]
             full = computed // ps
             if self.fault == Fault.REGISTER_UNFINISHED_PAGE:        # (the page's tokens are known, its keys not yet there)
-                full = min(len(table), (computed + ps - 1) // ps, len(tokens) // ps)
+                full = min(min(len(t) for t in rc.tables), (computed + ps - 1) // ps, len(tokens) // ps)
             for i in range(len(rc.hashes), full):
                 toks = tokens[i * ps:(i + 1) * ps]
                 h = block_hash(rc.hashes[i - 1] if i else 0, toks)
-                pool.register_full(table[i], h, toks)
+                for pool, table in zip(self.pools, rc.tables):
+                    if table[i] >= 0:                               # (a page before the window was never held)
+                        pool.register_full(table[i], h, toks)
                 rc.hashes.append(h)
         for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
             if self.groups[g].window is None:

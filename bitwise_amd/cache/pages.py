@@ -84,12 +84,19 @@ class PagePool:
         self._free.append(page)
         return True
 
-    def lookup(self, hash_: int, tokens: Sequence[int]) -> Optional[int]:
-        """A cached full page with this hash AND these tokens; takes a reference on a hit."""
+    def peek(self, hash_: int, tokens: Sequence[int]) -> Optional[int]:
+        """The page ``lookup`` would give, without taking it."""
         if not self.prefix_caching:
             return None
         page = self._by_hash.get(hash_)
         if page is None or self._tokens_of[page] != tuple(tokens):
+            return None
+        return page
+
+    def lookup(self, hash_: int, tokens: Sequence[int]) -> Optional[int]:
+        """A cached full page with this hash AND these tokens; takes a reference on a hit."""
+        page = self.peek(hash_, tokens)
+        if page is None:
             return None
         self._evictable.pop(page, None)
         self._ref[page] += 1

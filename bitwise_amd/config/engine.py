@@ -48,8 +48,8 @@ class EngineConfig:
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
-        if self.block_size not in (8, 16, 32, 64):
-            raise ValueError(f"block_size must be 8, 16, 32 or 64, got {self.block_size}")
+        if self.block_size < 1 or self.block_size & (self.block_size - 1):
+            raise ValueError(f"block_size must be a power of two, got {self.block_size}")   # (which ones a model takes: its mixers say)
         if self.num_blocks < 1 or self.max_batched_tokens < 1 or self.max_num_seqs < 1:
             raise ValueError("num_blocks, max_batched_tokens and max_num_seqs must be positive")
         if self.fault and self.fault not in Fault.NAMES:

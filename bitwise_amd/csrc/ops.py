@@ -23,6 +23,7 @@ def fold_group_tiles(head_dim: int) -> int:
     to one sequence, so the host pads every sequence's tile list to a multiple of this."""
     return int(_fn("bw_attention_fold_group_tiles")(int(head_dim)))
 HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
+PAGE_SIZES = (8, 16, 32, 64)       # tokens in a page that the attention kernels and the cache writes take
 
 _ERRORS = {
     -2: "sizes or strides out of the kernel's range",

@@ -127,6 +127,8 @@ class GpuExecutor:
         self._prints_in = torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device)
         self.group_specs = [GroupSpec(g.window) for g in asm.group_specs]
         self.has_state = bool(asm.state_specs)
+        self.prefix_reusable = asm.prefix_reusable      # every mixer keeps what it computed in its pages
+        self.run_ahead_safe = asm.run_ahead_safe        # no mixer minds a row that runs for a request that has ended
         self.vocab_size = asm.spec.vocab_size
         self.eos_token_id = asm.spec.eos_token_id
 
@@ -169,8 +171,8 @@ class GpuExecutor:
     def can_run_ahead(self, pend: "_Pending", rows: int) -> bool:
         """Whether the next decode step of the same ``rows`` requests may be launched before this one's
         tokens are read: it was replayed from a graph that sampled them (the next replay of that graph finds
-        them on the device) and no mixer keeps state that a step thrown away would have advanced."""
-        return pend.graph_rows == rows and pend.n == rows and not self.has_state
+        them on the device) and every mixer says that a row may run for a request that has just ended."""
+        return pend.graph_rows == rows and pend.n == rows and self.run_ahead_safe
 
 class Engine:
     def __init__(self, target, draft=None, config: Optional[EngineConfig] = None, executor=None):
@@ -183,8 +185,8 @@ class Engine:
         self.cfg.validate()
         self.exec = executor if executor is not None else GpuExecutor(target, self.cfg)
         self.manager = CacheManager(self.exec.group_specs, self.cfg.num_blocks, self.cfg.block_size,
-                                    self.cfg.max_num_seqs, self.cfg.prefix_caching, self.exec.has_state,
-                                    fault=self.cfg.fault)
+                                    self.cfg.max_num_seqs, self.cfg.prefix_caching,
+                                    not getattr(self.exec, "prefix_reusable", not self.exec.has_state), fault=self.cfg.fault)
         self.sched = Scheduler(self.manager, self.cfg, on_open=self.exec.reset_slot)
         self._seqs: Dict[int, Sequence] = {}
         self._results: Dict[int, RequestResult] = {}

@@ -22,11 +22,14 @@ class CacheStorage:
     def __init__(self, model: AssembledModel, num_pages: int, num_slots: int, page_size: int):
         rt = model.rt
         self.num_pages, self.num_slots, self.page_size = int(num_pages), int(num_slots), int(page_size)
+        model.check_page_size(self.page_size)
         self.keys: List[torch.Tensor] = []
         self.values: List[torch.Tensor] = []
         for spec, caches in zip(model.group_specs, model.group_caches):
             for pool, elems in ((self.keys, spec.key_elements(self.page_size)), (self.values, spec.value_elements(self.page_size))):
-                pool.append(torch.zeros((len(caches), self.num_pages, elems), dtype=rt.act_dtype, device=rt.device))
+                # (a mixer may page something else than activations: its cache spec names the pools' dtype then)
+                dtype = rt.act_dtype if spec.dtype is None else _TORCH_DTYPE[spec.dtype]
+                pool.append(torch.zeros((len(caches), self.num_pages, elems), dtype=dtype, device=rt.device))
         self.states: Dict[int, torch.Tensor] = {}
         for idx, ss in model.state_specs.items():
             self.states[idx] = torch.zeros((self.num_slots, *ss.shape), dtype=_TORCH_DTYPE[ss.dtype], device=rt.device)
@@ -59,5 +62,5 @@ class CacheStorage:
         handed out again must be written before it is read)."""
         if len(pages):
             idx = torch.as_tensor(list(pages), dtype=torch.long, device=self.keys[group].device)
-            self.keys[group][:, idx] = float("nan")
-            self.values[group][:, idx] = float("nan")
+            for pool in (self.keys[group], self.values[group]):
+                pool[:, idx] = float("nan") if pool.dtype.is_floating_point else -(2 ** 31)

@@ -52,6 +52,17 @@ class AssembledModel:
         self._plan_caches(spec.schedule)
         every = [self.embedding, self.final_norm, self.lm_head] + [p for b in self.layers for p in (b, *b.parts.values())]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
+        # each mixer's own word on what the engine may do around it (parts.base.Mixer)
+        mixers = [self.layers[c.layer].mixer for c in spec.schedule]
+        self.prefix_reusable = all(m.prefix_reusable for m in mixers)
+        self.run_ahead_safe = all(m.run_ahead_safe for m in mixers)
+
+    def check_page_size(self, page_size: int) -> None:
+        """Refuse a page size that one of the mixers' kernels does not take."""
+        for i, block in enumerate(self.layers):
+            sizes = block.mixer.page_sizes()
+            if sizes is not None and page_size not in sizes:
+                raise ValueError(f"layer {i}: its mixer takes pages of {sorted(sizes)} tokens, not of {page_size}")
 
     # ------------------------------------------------------------------ caches and state
     def _plan_caches(self, schedule: List[LayerCall]) -> None:

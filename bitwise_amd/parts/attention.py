@@ -81,7 +81,11 @@ class Attention(Mixer):
         self.scale = 1.0 / math.sqrt(float(self.head_dim))     # 1.0f / sqrtf(float(hd)), src/kernels.cpp:347
         pos = p["position"]
         self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+        if int(getattr(self.position, "rotary_dim", 0)) != self.head_dim:
+            raise ValueError(f"attention: this part rotates whole heads of {self.head_dim}; position encoding '{pos.kind}' "
+                             f"rotates {getattr(self.position, 'rotary_dim', 0)} elements of a head and needs a mixer of its own")
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))    # the tables must be device tensors
+        self.cos = self.sin = None
         self.qkv: Optional[Linear] = None
         self.o: Optional[Linear] = None
         group = self.heads // self.kv_heads
@@ -96,7 +100,24 @@ class Attention(Mixer):
             "o_proj.weight": TensorSpec((self.width, self.q_dim)),
         }
 
+    def _tables(self):
+        """The position encoding's tables, checked once against what the kernels index: [positions, head size / 2],
+        32-bit, contiguous, on the device."""
+        if self.cos is None:
+            cos, sin = self.position.tables()
+            for name, t in (("cos", cos), ("sin", sin)):
+                if (not isinstance(t, torch.Tensor) or t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != self.head_dim // 2
+                        or not t.is_contiguous() or t.device != self.rt.device or t.shape != cos.shape):
+                    raise ValueError(f"attention: the position encoding's {name} table must be a contiguous float32 "
+                                     f"[positions, {self.head_dim // 2}] tensor on {self.rt.device}")
+            self.cos, self.sin = cos, sin
+        return self.cos, self.sin
+
+    def page_sizes(self):
+        return ops.PAGE_SIZES
+
     def bind(self, tensors) -> None:
+        self._tables()
         q, k, v = tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]
         if not (q.dtype == k.dtype == v.dtype):
             raise ValueError("q, k and v projections must be stored in one dtype to be stacked")
@@ -126,7 +147,7 @@ class Attention(Mixer):
             return False
         q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
         ops.norm_qkv_rope_bf16(x, norm.weight, norm.eps, self.qkv.weight, q, ctx.positions, ctx.row_seq,
-                               ctx.block_tables[call.group], self.position.cos, self.position.sin, call.k_cache,
+                               ctx.block_tables[call.group], self.cos, self.sin, call.k_cache,
                                call.v_cache, ctx.rows, self.heads, self.kv_heads, self.head_dim, ws.page_size,
                                call.writes_cache)
         self._attend(ctx, call, q, residual)
@@ -140,8 +161,8 @@ class Attention(Mixer):
                                                               self.heads + 2 * self.kv_heads):
             # rotation and cache write ride in the product's epilogue
             q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
-            ops.gemm_qkv_rope_bf16(h, self.qkv.weight, q, ctx.positions, ctx.row_seq, table, self.position.cos,
-                                   self.position.sin, call.k_cache, call.v_cache, rows, self.heads, self.kv_heads,
+            ops.gemm_qkv_rope_bf16(h, self.qkv.weight, q, ctx.positions, ctx.row_seq, table, self.cos,
+                                   self.sin, call.k_cache, call.v_cache, rows, self.heads, self.kv_heads,
                                    self.head_dim, ws.page_size, call.writes_cache)
             self._attend(ctx, call, q, residual)
             return
@@ -149,12 +170,12 @@ class Attention(Mixer):
         self.qkv.store(ws, h, qkv, rows)
         if rt.bf16:
             q = ws.buffer("q_rot", self.q_dim, torch.bfloat16)
-            ops.rope_kvwrite(qkv, q, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
+            ops.rope_kvwrite(qkv, q, ctx.positions, ctx.row_seq, table, self.cos, self.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              ws.page_size, call.writes_cache)
             self._attend(ctx, call, q, residual)
         else:
-            ops.rope_kvwrite(qkv, None, ctx.positions, ctx.row_seq, table, self.position.cos, self.position.sin,
+            ops.rope_kvwrite(qkv, None, ctx.positions, ctx.row_seq, table, self.cos, self.sin,
                              call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.head_dim,
                              ws.page_size, call.writes_cache)
             out = ws.buffer("attn_out", self.q_dim, torch.float32)

@@ -101,6 +101,7 @@ class CacheSpec:
     window: Optional[int] = None
     key_width: Optional[int] = None        # elements per token; None: kv_heads * head_dim
     value_width: Optional[int] = None
+    dtype: Optional[str] = None            # "float32" / "bfloat16" / "int32" of the pools; None: the mode's activation dtype
 
     def key_elements(self, page_size: int) -> int:
         return page_size * (self.kv_heads * self.head_dim if self.key_width is None else self.key_width)
@@ -164,7 +165,26 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Owns its table(s); mixers apply it through the kernels they call."""
+    """Owns its tables; mixers apply it through the kernels they call.
+
+    What a mixer that rotates pairs of elements by a position's angles may rely on (the attention part refuses a
+    position encoding that does not keep it):
+    * ``rotary_dim``: how many leading elements of a head are rotated; even, at most the head size.  Element i is
+      paired with element i + rotary_dim / 2 (the rotate-half layout).
+    * ``tables()`` -> (cos, sin): two contiguous 32-bit tensors [positions, rotary_dim / 2] on the runtime's
+      device, row p holding the cosines and sines of position p's angles; they do not move or change once made
+      (captured graphs read them).
+    * ``shared(params, runtime)``: the instance for these parameters (mixers of several layers may share one).
+    What the angles are (base, scaling, stretching, learned) is the part's own business."""
+
+    rotary_dim: int = 0
+
+    def tables(self):
+        raise NotImplementedError
+
+    @classmethod
+    def shared(cls, params, runtime):
+        return cls(params, runtime)
 
 
 class Mixer(Part):
@@ -173,6 +193,24 @@ class Mixer(Part):
 
     def state_spec(self) -> Optional[StateSpec]:
         return None
+
+    def page_sizes(self) -> Optional[Tuple[int, ...]]:
+        """Page sizes (tokens) this mixer's kernels take for its paged cache; None: any."""
+        return None
+
+    @property
+    def prefix_reusable(self) -> bool:
+        """Whether a request may start behind cached pages of another request with the same first tokens: true
+        if everything this mixer has computed for those tokens lies in its pages.  State in a slot does not."""
+        return self.state_spec() is None
+
+    @property
+    def run_ahead_safe(self) -> bool:
+        """Whether a decode step may be launched before the step before it is known to have been the last of a
+        request (that request's row of the new step is then thrown away, after it has run).  By default a mixer
+        with state of its own says no; one whose state may be advanced once more for a request that has ended
+        (the slot is reset when it is taken again) overrides this."""
+        return self.state_spec() is None
 
     def forward(self, ctx, call, h, residual) -> None:
         """h: normed rows [rows, width]; adds the mixer's output into ``residual`` in place.

@@ -27,6 +27,7 @@ class RotaryTable(PositionEncoding):
         self.max_positions = int(params["max_positions"])
         if self.head_dim % 2:
             raise ValueError("rotary encoding needs an even head size")
+        self.rotary_dim = self.head_dim          # whole heads are rotated
         self._cos = self._sin = None
 
     def _build(self) -> None:
@@ -40,17 +41,10 @@ class RotaryTable(PositionEncoding):
         self._cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(runtime.device).contiguous()
         self._sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(runtime.device).contiguous()
 
-    @property
-    def cos(self) -> torch.Tensor:
+    def tables(self):
         if self._cos is None:
             self._build()
-        return self._cos
-
-    @property
-    def sin(self) -> torch.Tensor:
-        if self._sin is None:
-            self._build()
-        return self._sin
+        return self._cos, self._sin
 
     @classmethod
     def shared(cls, params, runtime) -> "RotaryTable":

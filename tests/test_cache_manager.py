@@ -110,7 +110,6 @@ def test_random_orders_lose_nothing(seed):
 
 def test_window_pages_are_given_back_as_the_window_passes():
     mgr = CacheManager([GroupSpec(None), GroupSpec(20)], num_pages=16, page_size=8, num_slots=2)
-    assert not mgr.prefix_caching                                  # two groups: no prefix reuse
     rc = mgr.open()
     toks = list(range(100))
     assert mgr.ensure(rc, 30)
@@ -127,6 +126,48 @@ def test_window_pages_are_given_back_as_the_window_passes():
         assert all(p == -1 for p in rc.tables[1][:first]) and all(p >= 0 for p in rc.tables[1][first:])
     assert len([p for p in rc.tables[0] if p >= 0]) == 13
     mgr.close(rc)
+    assert mgr.all_free()
+
+
+def test_prefix_reuse_is_decided_group_by_group():
+    """A group that keeps all keys and one with a window of 20 keys, pages of 8: a second request with the same
+    tokens starts behind as many pages as every group can still serve: all of them in the first group, the pages
+    under the window in the second (found again although the first request gave them back when its window had
+    passed them).  Once those have been evicted the prefix is not reused in either group."""
+    mgr = CacheManager([GroupSpec(None), GroupSpec(20)], num_pages=12, page_size=8, num_slots=3)
+    assert mgr.prefix_caching
+    toks = [(i * 7 + 3) % 50 for i in range(60)]
+    a = mgr.open()
+    for upto in (13, 29, 30, 47, 60):
+        assert mgr.ensure(a, upto)
+        mgr.advance(a, toks, upto)
+        mgr.check()
+    assert a.tables[1][:5] == [-1] * 5 and all(p >= 0 for p in a.tables[1][5:]) and len(a.hashes) == 7
+    b = mgr.open()
+    assert mgr.admit_prefix(b, toks) == 56                         # 7 full pages; the last token's page is computed
+    assert b.tables[0] == a.tables[0][:7]
+    assert b.tables[1][:4] == [-1] * 4 and all(p >= 0 for p in b.tables[1][4:7])     # position 56 reads keys 37..: pages 4, 5, 6
+    assert b.tables[1][5:7] == a.tables[1][5:7] and mgr.pools[1].refcount(b.tables[1][4]) == 1     # page 4: a had given it back
+    # a shorter prompt with the same start: 3 full pages, the window of position 24 starts in page 0
+    c = mgr.open()
+    assert mgr.admit_prefix(c, toks[:30]) == 24 and all(p >= 0 for p in c.tables[1]) and c.tables[0] == a.tables[0][:3]
+    for rc in (a, b, c):
+        mgr.close(rc)
+    mgr.check()
+    assert mgr.all_free()
+    # everything is still cached; now the windowed group's pool is filled by someone else: its cached pages are evicted
+    d = mgr.open()
+    other = [49 - t for t in toks] + list(range(40))
+    assert mgr.ensure(d, 96)
+    assert mgr.pools[1].evictions > 0 and mgr.pools[0].evictions > 0
+    mgr.close(d)
+    e = mgr.open()
+    hit = mgr.admit_prefix(e, toks)
+    assert hit % 8 == 0 and hit < 56
+    lo = mgr.first_needed_page(1, hit)
+    assert all(p >= 0 for p in e.tables[0]) and all(p >= 0 for p in e.tables[1][lo:]) and len(e.tables[0]) == len(e.tables[1]) == hit // 8
+    mgr.close(e)
+    mgr.check()
     assert mgr.all_free()
 
 

@@ -346,3 +346,90 @@ def test_windowed_groups_end_to_end(gpu, tmp_path, dtype):
             assert same.all(), f"{rid}: first differing position {int(np.argmin(same))} (graphs={graphs})"
         # in the windowed groups y was served from pages that x had given back
         assert taken[("y", 0)] & taken[("x", 0)] and taken[("y", 2)] & taken[("x", 2)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefix_reuse_with_windowed_groups_in_the_engine(gpu, tmp_path, dtype):
+    """Three cache groups (windows of 24 and 40 keys beside all keys) in the engine with the prefix cache on:
+    requests that share a 40-token start, and one that repeats another's prompt, arrive one after the other
+    in a pool that forces preemption; later ones start behind cached pages in every group (for the windowed
+    groups only the pages under the window are taken), and everyone's tokens and logits are those of a solo run
+    without any of that."""
+    folder = tiny.make_folder(tmp_path, "B")
+    model = windowed_model(folder, dtype, [24, None, 40])
+    g = torch.Generator().manual_seed(21)
+    stem = torch.randint(0, 500, (40,), generator=g).tolist()
+    prompts = [stem + torch.randint(0, 500, (n,), generator=g).tolist() for n in (9, 30, 3, 17)]
+    prompts.append(list(prompts[1]))
+    sp = [bw.SamplingParams(max_new_tokens=24, ignore_eos=True, temperature=0.8 if i % 2 else 0.0, seed=i) for i in range(5)]
+    solo = [bw.generate(model, [p], s, bw.EngineConfig(num_blocks=32, block_size=8, dtype=dtype, prefix_caching=False,
+                                                       use_graphs=False, run_ahead=False))[0] for p, s in zip(prompts, sp)]
+    for graphs in (True, False):
+        eng = bw.Engine(model, None, bw.EngineConfig(num_blocks=26, block_size=8, max_batched_tokens=32, max_num_seqs=3,
+                                                     dtype=dtype, use_graphs=graphs))
+        assert eng.manager.prefix_caching and len(eng.manager.pools) == 3
+        ids, guard = [], 0
+        while len(ids) < len(prompts) or not eng.idle():
+            if guard % 4 == 0 and len(ids) < len(prompts):
+                ids.append(eng.add_request(prompts[len(ids)], sp[len(ids)]))
+            eng.step()
+            eng.manager.check()
+            guard += 1
+            assert guard < 3000, eng.debug_state()
+        assert eng.stats.prefix_hit_tokens >= 40 and eng.manager.all_free()
+        for i, ref in zip(ids, solo):
+            assert eng.result(i).tokens == ref.tokens, (graphs, i)
+            assert eng.result(i).logits_fingerprint == ref.logits_fingerprint, (graphs, i)
+        assert eng.result(ids[4]).prefix_cached_tokens >= 64      # the repeated prompt: every full page but the last token's
+
+
+def test_a_mixer_names_its_caches_dtype_and_page_sizes(gpu):
+    """A toy mixer that pages 32-bit integers (token ids) in bfloat16 mode and takes pages of 4 or 8 tokens only:
+    the storage gives its group pools of that dtype, a page size it does not take is refused by name, and a
+    position encoding that rotates part of a head is refused by the attention part."""
+    from bitwise_amd.engine.storage import CacheStorage
+    from bitwise_amd.parts import base
+    from bitwise_amd.parts.base import CacheSpec, LayerCall, LayerSpec, ModelSpec, PartSpec
+
+    @base.register_mixer("toy_token_pager")
+    class TokenPager(base.Mixer):
+        graph_safe = False
+
+        def cache_spec(self):
+            return CacheSpec(1, 1, None, key_width=1, value_width=0, dtype="int32")
+
+        def page_sizes(self):
+            return (4, 8)
+
+        def forward(self, ctx, call, h, residual):
+            pass
+
+    width = 32
+    norm = PartSpec("rmsnorm", {"width": width, "eps": 1e-5}, "n.")
+    layers = [LayerSpec.prenorm(PartSpec("toy_token_pager", {}, "m."), PartSpec("swiglu", {"width": width, "inter": 16}, "f."), norm, norm),
+              LayerSpec.prenorm(PartSpec("attention", {"width": width, "heads": 2, "kv_heads": 1, "head_dim": 16, "window": None,
+                                                       "position": PartSpec("rope", {"theta": 1e4, "head_dim": 16, "max_positions": 32})},
+                                         "a."), PartSpec("swiglu", {"width": width, "inter": 16}, "f."), norm, norm)]
+    spec = ModelSpec("ToyPager", 20, width, PartSpec("embedding", {"vocab": 20, "width": width}, "e."), layers,
+                     [LayerCall(0, 0), LayerCall(1, 1)], norm, PartSpec("lm_head", {"vocab": 20, "width": width, "tied": True}, "h."), 32)
+    asm = AssembledModel(spec, Runtime("bfloat16", "cuda:0"))
+    assert len(asm.group_specs) == 2
+    storage = CacheStorage(asm, num_pages=6, num_slots=2, page_size=8)
+    assert storage.keys[0].dtype == torch.int32 and storage.keys[0].shape == (1, 6, 8) and storage.values[0].shape == (1, 6, 0)
+    assert storage.keys[1].dtype == torch.bfloat16
+    storage.poison_pages(0, [2])
+    assert int(storage.keys[0][0, 2, 0]) == -(2 ** 31) and int(storage.keys[0][0, 1, 0]) == 0
+    with pytest.raises(ValueError, match="layer 0: its mixer takes pages of \\[4, 8\\] tokens, not of 16"):
+        CacheStorage(asm, num_pages=6, num_slots=2, page_size=16)
+    with pytest.raises(ValueError, match="layer 1: its mixer takes pages of \\[8, 16, 32, 64\\] tokens, not of 4"):
+        CacheStorage(asm, num_pages=6, num_slots=2, page_size=4)
+
+    @base.register_position_encoding("toy_partial_rope")
+    class PartialRotary(base.PositionEncoding):
+        def __init__(self, params, runtime):
+            super().__init__(params, runtime)
+            self.rotary_dim = 8
+
+    with pytest.raises(ValueError, match="rotates 8 elements of a head and needs a mixer of its own"):
+        base.MIXERS["attention"]({"width": width, "heads": 2, "kv_heads": 1, "head_dim": 16, "window": None,
+                                  "position": PartSpec("toy_partial_rope", {})}, Runtime("bfloat16", "cuda:0"))

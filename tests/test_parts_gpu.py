@@ -293,12 +293,12 @@ class StretchedRotary(base.PositionEncoding):
         inv = pl.rope_inv_freq(float(params["theta"]), hd)
         places = (np.arange(n, dtype=np.float32) / np.float32(params["stretch"]))[:, None]
         angle = (places * inv[None, :]).astype(np.float32).astype(np.float64)
+        self.rotary_dim = hd
         self.cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(runtime.device).contiguous()
         self.sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(runtime.device).contiguous()
 
-    @classmethod
-    def shared(cls, params, runtime):
-        return cls(params, runtime)
+    def tables(self):
+        return self.cos, self.sin
 
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
