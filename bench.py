@@ -9,8 +9,9 @@ A step is one decode step of the whole engine (scheduler, graph replay of the mo
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
 decoded tokens per second.  One JSON line is printed; it also carries the 2,048-token prefill,
 the decode step's HBM roofline, decode at batch 1 and 64 with their rooflines, the same model's true
-32-bit path (decode and prefill) and, at Llama-3-8B's sizes, decode, prefill and a continuous-batching workload
-of 64 requests.
+32-bit path (decode and prefill) and, at Llama-3-8B's sizes, decode, prefill, a continuous-batching workload
+of 64 requests and a trace of 128 requests with shared prefixes, cancellations and preemption whose sampled requests
+are checked against solo runs.
 """
 
 from __future__ import annotations
@@ -66,7 +67,7 @@ def main() -> int:
 
     import torch
     import bitwise_amd as bw
-    from bitwise_amd.measure import CONTEXT, PEAK_FLOPS, measure_decode, measure_prefill, measure_serving
+    from bitwise_amd.measure import CONTEXT, PEAK_FLOPS, measure_decode, measure_prefill, measure_serving, measure_trace
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B)
@@ -124,7 +125,10 @@ def main() -> int:
                                   "decode_tok_s": m["tok_s"], "batch": 8, "ms_per_step": m["ms_per_step"],
                                   "roofline": m["roofline"],
                                   "prefill": measure_prefill(bw, torch, model8, big, "bfloat16", PEAK_FLOPS["bf16"]),
-                                  "serving": measure_serving(bw, torch, model8, big, "bfloat16")}
+                                  "serving": measure_serving(bw, torch, model8, big, "bfloat16"),
+                                  # 128 requests, four shared 1,024-token starts, contexts up to 6,144, a tenth cancelled, a pool
+                                  # that forces preemption; 16 of them checked against solo runs
+                                  "trace8k": measure_trace(bw, torch, model8, big, "bfloat16")}
             del model8
             model = None
 

@@ -139,3 +139,90 @@ def measure_serving(bw, torch, model, cfg: dict, dtype: str, requests: int = 64,
             "all_tok_s": round((generated + prompt_tokens) / secs, 1), "preemptions": eng.stats.preemptions}
 
 
+
+
+def shared_prefix_trace(vocab: int, requests: int, seed: int, prefixes: int = 4, prefix_tokens: int = 1024,
+                        suffix=(16, 4096), outputs=(32, 1024), rate: float = 40.0, cancel_share: float = 0.1):
+    """The randomized trace of the hardest workload the reference's simulator and load generator describe
+    (sim/simulate.cpp:120-210, bench/loadgen.py:170-207) at serving sizes, with synthetic tokens: ``requests``
+    requests with exponential gaps between their arrivals (``rate`` a second); every prompt is one of ``prefixes``
+    shared starts of ``prefix_tokens`` tokens and a suffix of its own, uniform in ``suffix``; new tokens uniform in
+    ``outputs``; greedy or temperature 0.7 with a seed of its own; a share of them is given up by the client some
+    time after it arrived.  Returns a list of dicts: prompt, params (temperature, seed, max_new_tokens), at (seconds),
+    cancel_at (seconds or None)."""
+    import random
+    rng = random.Random(seed)
+    stems = [[rng.randrange(vocab) for _ in range(prefix_tokens)] for _ in range(prefixes)]
+    out, t = [], 0.0
+    for i in range(requests):
+        t += rng.expovariate(rate)
+        prompt = list(rng.choice(stems)) + [rng.randrange(vocab) for _ in range(rng.randint(*suffix))]
+        out.append({"prompt": prompt, "temperature": 0.0 if rng.random() < 0.5 else 0.7, "seed": rng.getrandbits(48),
+                    "max_new_tokens": rng.randint(*outputs), "at": t,
+                    "cancel_at": t + rng.uniform(0.0, 3.0) if rng.random() < cancel_share else None})
+    return out
+
+
+def measure_trace(bw, torch, model, cfg: dict, dtype: str, requests: int = 128, seed: int = 7, pool_tokens: int = 96 * 1024,
+                  max_num_seqs: int = 64, check: int = 16, trace=None, clock=None) -> dict:
+    """Run ``shared_prefix_trace`` through an engine whose page pool (``pool_tokens`` tokens) is smaller than what its
+    running requests come to hold, so that some are preempted and recomputed, with the prefix cache on and logits
+    fingerprints kept; then run a seeded sample of ``check`` requests that were not cancelled alone (no prefix cache, a
+    pool of their own) and compare tokens and fingerprints.  Arrivals and cancellations follow the wall clock (or
+    ``clock``, a function of the engine's step count, for a run that does not depend on the machine's speed)."""
+    import random
+    trace = trace if trace is not None else shared_prefix_trace(cfg["vocab_size"], requests, seed)
+    block = 16
+    longest = max(len(r["prompt"]) + r["max_new_tokens"] for r in trace)
+    ecfg = bw.EngineConfig(num_blocks=pool_tokens // block, max_batched_tokens=2048, max_num_seqs=max_num_seqs, prefix_caching=True,
+                           fingerprint_logits=True, block_size=block, dtype=dtype, max_model_len=longest + block)
+    eng = bw.Engine(model, None, ecfg)
+    params = [bw.SamplingParams(temperature=r["temperature"], seed=r["seed"], max_new_tokens=r["max_new_tokens"], ignore_eos=True)
+              for r in trace]
+    ids = [None] * len(trace)
+    cancelled = set()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps, nxt = 0, 0
+    while nxt < len(trace) or not eng.idle():
+        now = clock(steps) if clock is not None else time.perf_counter() - t0
+        while nxt < len(trace) and trace[nxt]["at"] <= now:
+            ids[nxt] = eng.add_request(trace[nxt]["prompt"], params[nxt])
+            nxt += 1
+        for i, r in enumerate(trace[:nxt]):
+            if r["cancel_at"] is not None and r["cancel_at"] <= now and i not in cancelled:
+                cancelled.add(i)
+                eng.cancel(ids[i])
+        if eng.idle():
+            if clock is None:
+                time.sleep(min(0.001, max(0.0, trace[nxt]["at"] - now)))      # nothing to do before the next arrival
+            steps += 1
+            continue
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    results = [eng.result(i) for i in ids]
+    really_cancelled = [i for i in cancelled if results[i].cancelled]
+    done = [i for i in range(len(trace)) if not results[i].cancelled]
+    generated = eng.stats.generated_tokens
+    stats = eng.stats
+    leaked = not eng.manager.all_free()
+    del eng
+    torch.cuda.empty_cache()
+    # a seeded sample of the finished requests, each alone on an engine of its own
+    sample = random.Random(seed + 1).sample(done, min(check, len(done)))
+    wrong = []
+    for i in sample:
+        need = len(trace[i]["prompt"]) + trace[i]["max_new_tokens"]
+        solo_cfg = bw.EngineConfig(num_blocks=need // block + 2, max_batched_tokens=2048, max_num_seqs=1, prefix_caching=False,
+                                   fingerprint_logits=True, block_size=block, dtype=dtype, max_model_len=need + block)
+        (ref,) = bw.generate(model, [trace[i]["prompt"]], params[i], solo_cfg)
+        if ref.tokens != results[i].tokens or ref.logits_fingerprint != results[i].logits_fingerprint:
+            wrong.append(i)
+    return {"requests": len(trace), "cancelled": len(really_cancelled), "prompt_tokens": sum(len(r["prompt"]) for r in trace),
+            "generated_tokens": generated, "steps": stats.steps, "seconds": round(secs, 3),
+            "generated_tok_s": round(generated / secs, 1), "preemptions": stats.preemptions,
+            "prefix_hit_tokens": stats.prefix_hit_tokens, "evictions": stats.evictions, "pool_tokens": pool_tokens,
+            "checked_against_solo": len(sample), "differ_from_solo": len(wrong), "pages_lost": bool(leaked),
+            "longest_request": longest}

@@ -184,60 +184,29 @@ def test_the_simulator_program_catches_every_injected_fault(gpu):
     assert p.returncode == 2 and "speculative" in p.stderr
 
 
-def test_long_shared_prefix_trace_at_real_layer_sizes_equals_solo(gpu):
-    """A reduced form of the reference's hardest workload: layers of Llama-3-8B's sizes (width 4096, 32 query heads on
-    8 key heads of 128, feed-forward 14336; two layers, a small vocabulary), contexts up to 8,192; requests that
-    arrive over time, share one of two 1,024-token prefixes, add suffixes of 16 to 3,000 tokens, generate 24 to 72 tokens
-    greedily or at temperature 0.7 with seeds of their own; one is cancelled; the page pool is so small that requests are
-    preempted and recomputed.  Every request's tokens and logits fingerprints equal its solo run."""
-    import random
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_shared_prefix_trace_of_128_requests_at_real_layer_sizes_equals_solo(gpu, dtype):
+    """The hardest workload the reference describes (sim/simulate.cpp:120-210 at the sizes of bench/loadgen.py), whole:
+    layers of Llama-3-8B's sizes (width 4096, 32 query heads on 8 key heads of 128, feed-forward 14336, the whole
+    vocabulary; two layers), 128 requests with exponential gaps between arrivals, four shared 1,024-token starts and
+    suffixes of 16 to 4,096 tokens, 32 to 1,024 new tokens, greedy or temperature 0.7, a tenth given up by the client,
+    contexts up to 6,144 in a pool of 96k tokens for up to 64 running requests, so that requests are preempted and
+    recomputed; in bfloat16 and in 32-bit.  A seeded sample of 16 finished requests (8 in 32-bit) must have the tokens
+    and the logits fingerprints of the same requests run alone."""
+    from bitwise_amd import measure
 
-    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "vocab_size": 4096,
-           "hidden_size": 4096, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8,
-           "head_dim": 128, "intermediate_size": 14336, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
-           "tie_word_embeddings": False, "max_position_embeddings": 8192, "bos_token_id": 1, "eos_token_id": 2}
-    model = bw.Model.random(cfg, seed=9, dtype="bfloat16", sigma=0.02, on_device=True)
-    rng = random.Random(4)
-    g = torch.Generator().manual_seed(4)
-    prefixes = [torch.randint(3, 4096, (1024,), generator=g).tolist() for _ in range(2)]
-    reqs, step_of = [], 0
-    for i in range(10):
-        suffix = torch.randint(3, 4096, (rng.choice([16, 200, 700, 1500, 3000]),), generator=g).tolist()
-        sp = bw.SamplingParams(temperature=0.0 if i % 2 else 0.7, seed=50 + i, max_new_tokens=rng.randint(24, 72),
-                               ignore_eos=i % 3 != 0)
-        step_of += int(rng.expovariate(1 / 3.0))
-        reqs.append((prefixes[i % 2] + suffix, sp, step_of))
-    cancelled = 7
-    solo = []
-    for p, sp, _ in reqs:
-        (r,) = bw.generate(model, [p], sp, bw.EngineConfig(num_blocks=(len(p) + 80) // 16 + 2, max_batched_tokens=2048,
-                                                          prefix_caching=False, max_model_len=8192))
-        solo.append(r)
-    longest = max(len(p) + sp.max_new_tokens for p, sp, _ in reqs)
-    ecfg = bw.EngineConfig(num_blocks=(longest + 16) // 16 + 150, max_batched_tokens=2048, max_num_seqs=6,
-                           prefix_caching=True, max_model_len=8192)
-    eng = bw.Engine(model, None, ecfg)
-    ids = [None] * len(reqs)
-    for step in range(20000):
-        for i, (p, sp, at) in enumerate(reqs):
-            if at == step:
-                ids[i] = eng.add_request(p, sp)
-        if step == reqs[cancelled][2] + 6:
-            eng.cancel(ids[cancelled])
-        if all(i is not None for i in ids) and eng.idle():
-            break
-        eng.step()
-    else:
-        raise AssertionError(eng.debug_state())
-    assert eng.free_blocks == ecfg.num_blocks and eng.manager.all_free()
-    assert eng.stats.preemptions > 0 and eng.stats.prefix_hit_tokens >= 1024
-    for i, ref in enumerate(solo):
-        got = eng.result(ids[i])
-        if i == cancelled:
-            assert got.cancelled and got.tokens == ref.tokens[:len(got.tokens)]
-            continue
-        assert got.tokens == ref.tokens, f"request {i}"
-        assert got.logits_fingerprint == ref.logits_fingerprint, f"request {i}"
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "num_hidden_layers": 2,
+           "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "bos_token_id": 1, "eos_token_id": 2,
+           "vocab_size": 128256, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+           "intermediate_size": 14336, "rope_theta": 500000.0, "tie_word_embeddings": False}
+    model = bw.Model.random(cfg, seed=9, dtype=dtype, sigma=0.02, on_device=True)
+    # arrivals and cancellations by the engine's step count (20 ms a step), so that the run is the same on any machine
+    check = 16 if dtype == "bfloat16" else 8                  # (solo runs decode one token a step: the slow part)
+    out = measure.measure_trace(bw, torch, model, cfg, dtype, requests=128, seed=7, check=check, clock=lambda steps: steps * 0.02)
+    print(dtype, out)
+    assert out["differ_from_solo"] == 0 and out["checked_against_solo"] == check and not out["pages_lost"]
+    assert out["preemptions"] > 0 and out["prefix_hit_tokens"] >= 64 * 1024 and out["cancelled"] >= 5
+    assert out["longest_request"] > 5000 and out["requests"] == 128
 
 
 def test_command_line(folders):
