@@ -145,31 +145,74 @@ extern "C" int bw_sample(const float* logits, int vocab, int ld, int rows, const
 
 // Fingerprint chain of the reference (src/engine.cpp:18-29): h = (h ^ word) * 1099511628211
 // over the row's 8-byte words, single trailing bytes likewise, then the splitmix64 finaliser.
-// The chain is sequential by construction; one lane per row.
-__global__ void fingerprint_kernel(const float* __restrict__ logits, int vocab, int ld, int rows,
-                                   const uint64_t* __restrict__ h_in, uint64_t* __restrict__ h_out) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+// The chain is sequential by construction (an exclusive or, then a product modulo 2^64: no algebra in which both
+// are linear), so a row's time is its number of words times the latency of one link.  A wave takes a row: the row's
+// address is the same for every lane, so the words arrive through the scalar unit, sixteen of them a load and the
+// next sixteen asked for before these are used, and the chain runs in scalar registers, a link every dozen clocks;
+// rows run beside each other on as many compute units.  (One lane a row with loads of its own, as this kernel
+// was first written, spent a memory latency a word: 6.4 ms for 64 rows of 128,256 logits.)
+#define FP_BLOCK 16        // words of 8 bytes a block
+__device__ __forceinline__ uint64_t fp_link(uint64_t h, uint32_t lo, uint32_t hi) {
+  return (h ^ ((uint64_t)lo | ((uint64_t)hi << 32))) * 1099511628211ull;
+}
+
+struct FpBlock {
+  uint32_t d[2 * FP_BLOCK];
+};
+
+__device__ __forceinline__ void fp_load(FpBlock& blk, const uint32_t* __restrict__ p) {
+#pragma unroll
+  for (int j = 0; j < 2 * FP_BLOCK; ++j) blk.d[j] = p[j];
+}
+
+__device__ __forceinline__ uint64_t fp_chain(uint64_t h, const FpBlock& blk) {
+#pragma unroll
+  for (int j = 0; j < FP_BLOCK; ++j) h = fp_link(h, blk.d[2 * j], blk.d[2 * j + 1]);
+  return h;
+}
+
+__global__ __launch_bounds__(64) void fingerprint_kernel(const float* __restrict__ logits, int vocab, int ld, int rows,
+                                                         const uint64_t* __restrict__ h_in, uint64_t* __restrict__ h_out) {
+  const int row = blockIdx.x;                                         // the same for every lane: scalar from here on
   if (row >= rows) return;
-  const uint32_t* p = reinterpret_cast<const uint32_t*>(logits + (size_t)row * ld);
+  const uint32_t* __restrict__ p = reinterpret_cast<const uint32_t*>(logits + (size_t)row * ld);
   uint64_t h = h_in[row];
-  int i = 0;
-  for (; i + 2 <= vocab; i += 2) {
-    const uint64_t wd = (uint64_t)p[i] | ((uint64_t)p[i + 1] << 32);
-    h = (h ^ wd) * 1099511628211ull;
+  const int words = vocab >> 1;
+  const int blocks = words / FP_BLOCK;
+  // two blocks in turn: while one is chained the other is on its way (scalar loads come back in any order, so a
+  // wait is for all of them; each block is asked for a whole chain of sixteen links before it is needed)
+  FpBlock even, odd;
+  if (blocks > 0) fp_load(even, p);
+  int b = 0;
+  for (; b + 2 <= blocks; b += 2) {
+    __builtin_amdgcn_s_waitcnt(0xc07f);                                // lgkmcnt(0): the block to be chained now is there ...
+    __builtin_amdgcn_sched_barrier(0);
+    fp_load(odd, p + (size_t)(b + 1) * 2 * FP_BLOCK);                  // ... before the next one is asked for
+    __builtin_amdgcn_sched_barrier(0);
+    h = fp_chain(h, even);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_sched_barrier(0);
+    fp_load(even, p + (size_t)(b + 2 < blocks ? b + 2 : b) * 2 * FP_BLOCK);      // (past the end: a block once more, unused)
+    __builtin_amdgcn_sched_barrier(0);
+    h = fp_chain(h, odd);
+    __builtin_amdgcn_sched_barrier(0);
   }
-  if (i < vocab) {
-    const uint32_t t = p[i];
-    for (int b = 0; b < 4; ++b) h = (h ^ ((t >> (8 * b)) & 0xffu)) * 1099511628211ull;
+  if (b < blocks) h = fp_chain(h, even);                               // an odd number of blocks: the last one
+  for (int i = blocks * FP_BLOCK; i < words; ++i) h = fp_link(h, p[2 * i], p[2 * i + 1]);
+  if (vocab & 1) {
+    const uint32_t t = p[vocab - 1];
+    for (int k = 0; k < 4; ++k) h = (h ^ ((t >> (8 * k)) & 0xffu)) * 1099511628211ull;
   }
   h = (h ^ (h >> 30)) * 0xBF58476D1CE4E5B9ull;
   h = (h ^ (h >> 27)) * 0x94D049BB133111EBull;
-  h_out[row] = h ^ (h >> 31);
+  if (threadIdx.x == 0) h_out[row] = h ^ (h >> 31);
 }
 
 extern "C" int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out,
                               void* stream) {
   if (rows <= 0) return 0;
-  hipLaunchKernelGGL(fingerprint_kernel, dim3((rows + 63) / 64), dim3(64), 0, (hipStream_t)stream, logits, vocab, ld,
+  hipLaunchKernelGGL(fingerprint_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, logits, vocab, ld,
                      rows, (const uint64_t*)h_in, (uint64_t*)h_out);
   return BW_LAUNCH_CHECK();
 }

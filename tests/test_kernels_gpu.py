@@ -772,7 +772,9 @@ def test_sampling_and_fingerprint(gpu):
     for r in range(9):
         want = pl.argmax_row(host[r]) if temps[r] <= 0 else pl.sample_row(host[r], temps[r], us[r])
         assert got[r] == want, f"row {r}"
-    for Vv in (500, 501, 6):
+    # (blocks of 16 words chained in turn from two sets of registers: none, one, two, three, many, with words and an
+    # odd element left over; rows that start on an odd element)
+    for Vv in (500, 501, 6, 1, 2, 31, 32, 33, 64, 65, 96, 97, 128, 1000, 49152):
         rows = torch.randn(3, Vv, generator=g).to(gpu)
         basis = [1469598103934665603, 12345, 2 ** 64 - 1]
         h_in = torch.from_numpy(np.asarray(basis, np.uint64).view(np.int64)).to(gpu)
