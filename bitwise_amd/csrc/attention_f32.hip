@@ -59,13 +59,23 @@ __device__ __forceinline__ float dot_canonical(const float* __restrict__ q_lds, 
 }
 
 #define ATT32_THREADS 256
+
+// A workgroup barrier for data that meets in LDS: this wave's LDS writes are done, then the barrier.  (The
+// language's own barrier also waits for every load from memory that is still on its way, which would end the
+// fetching ahead of the values across the chunks' barriers.)
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xc07f);                    // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
 #define ATT32_TABLE 2048            // entries of a block table's row that the workgroup keeps in LDS
 
 // Keys of a chunk of pass 2: as many as 32 KB of value rows hold, at most one a thread.
 template <int HD>
 struct Att32Shape {
   static constexpr int T = ATT32_THREADS;
-  static constexpr int KC = (8192 / HD) < T ? (8192 / HD) : T;
+  static constexpr int KC = ((8192 / HD) < T ? (8192 / HD) : T) & ~3;   // (a multiple of 4: the values of four keys lie side by side in LDS)
   static constexpr int SEGS = HD / 4;                              // 16-byte pieces of a key's row
   static constexpr int VJ = (KC * SEGS + T - 1) / T;               // pieces of a chunk's value rows a thread
   static constexpr int LDS_BYTES = 2 * KC * HD * (int)sizeof(float);
@@ -142,29 +152,52 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
   // element offset of key j (clamped to the last key: loads past it stay inside the sequence and go unused)
   auto offset_of = [&](int j) -> size_t {
     j = j < pos ? j : pos;
-    const int page = a.page_shift >= 0 ? j >> a.page_shift : j / a.page_size;
-    const int slot = a.page_shift >= 0 ? j & (a.page_size - 1) : j % a.page_size;
-    const int id = table_fits ? table_lds[page] : table[page];
+    // (KEEP: the launcher has seen to it that pages are a power of two and the table's row fits: no branch, no division)
+    const int page = (KEEP || a.page_shift >= 0) ? j >> a.page_shift : j / a.page_size;
+    const int slot = (KEEP || a.page_shift >= 0) ? j & (a.page_size - 1) : j % a.page_size;
+    // (KEEP: the launcher has seen to it that the row fits.  A lookup in memory here, even one that is never
+    // taken, makes the compiler wait for every load that is on its way before the next one is issued.)
+    int id;
+    if constexpr (KEEP) id = table_lds[page];
+    else id = table_fits ? table_lds[page] : table[page];
     return (size_t)id * page_stride + head_off + (size_t)slot * HD;
   };
 
-  // pass 1: the maximum (exact whatever the order), a key a thread at a time, the next key's row on its way
-  // while this one's score is computed (two sets of registers in turn)
+  // pass 1: the scores and their maximum (exact whatever the order).  Sixteen lanes take a key: lane t holds the
+  // elements t, t + 16, ... of the query and loads those of the key (the sixteen lanes' loads are 64 bytes side by
+  // side), so chain t of the canonical dot is its own, and the tree is the butterflies of a row of sixteen lanes
+  // (l ^ 8, ^ 4, ^ 2, ^ 1: lane[i] + lane[i + 8], then + 4, then (s4[0] + s4[2]) + (s4[1] + s4[3]); an addition
+  // gives the same bits whichever side a lane's own value stands on).  Four keys a group are on their way while
+  // one is worked on.
   float mx = -INFINITY;
   {
-    KeyRow<HD> ka, kb;
-    int j = lo + tid;
-    load_row<HD>(ka, a.k_cache + offset_of(j));
-    for (; j <= pos; j += 2 * T) {
-      load_row<HD>(kb, a.k_cache + offset_of(j + T));
-      const float s0 = dot_canonical<HD>(q_lds, ka) * a.scale;
-      if constexpr (KEEP) scores[j - lo] = s0;
-      mx = fmaxf(mx, s0);
-      load_row<HD>(ka, a.k_cache + offset_of(j + 2 * T));
-      if (j + T <= pos) {
-        const float s1 = dot_canonical<HD>(q_lds, kb) * a.scale;
-        if constexpr (KEEP) scores[j + T - lo] = s1;
-        mx = fmaxf(mx, s1);
+    constexpr int NC = HD / 16, G = T / 16, DEPTH = 4;
+    const int grp = tid >> 4, t = tid & 15;
+    float qr[NC], kr[DEPTH][NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) qr[c] = q_lds[16 * c + t];
+    auto fetch_key = [&](float (&dst)[NC], int j) {
+      const float* kp = a.k_cache + offset_of(j) + t;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) dst[c] = kp[16 * c];
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) fetch_key(kr[d], lo + grp + d * G);
+    for (int base = lo; base <= pos; base += DEPTH * G) {          // (the same trips for every thread)
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int j = base + grp + d * G;
+        float chain = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) chain = fmaf(qr[c], kr[d][c], chain);
+        fetch_key(kr[d], j + DEPTH * G);                           // (past the last key: the last key again, unused)
+        const float sc = row16_sum(chain) * a.scale;
+        if (j <= pos) {
+          if constexpr (KEEP) {
+            if (t == 0) scores[j - lo] = sc;
+          }
+          mx = fmaxf(mx, sc);
+        }
       }
     }
   }
@@ -225,47 +258,121 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
     // Values only.  Three chunks of them are on their way at any time (three sets of registers in turn; a chunk in
     // flight is what keeps a compute unit's share of the memory system busy across a trip to memory), the first
     // three asked for before the scores turn into e_j.  Chunks past the last key fetch the last key again.
-    f32x4 r0[VJ], r1[VJ], r2[VJ];
-    auto fetch_into = [&](f32x4 (&reg)[VJ], int j0) {
+    // Where the walk leaves two waves or more without an element (head sizes up to 128), those waves alone fetch
+    // and stash, and the walking waves only walk: a chunk then costs the longer of the two, not their sum.
+    constexpr int WW = (HD + 63) / 64, LW = T / 64 - WW;     // waves that walk, waves that do not
+    constexpr bool APART = LW >= 2;
+    constexpr int LT = APART ? 64 * LW : T;                  // threads that fetch and stash
+    constexpr int VL = (KC * SEGS + LT - 1) / LT;            // pieces of a chunk's value rows for each of them
+    const int lt = APART ? tid - 64 * WW : tid;              // (negative: this thread walks only)
+    const bool loads = lt >= 0;
+    f32x4 r0[VL], r1[VL], r2[VL];
+    auto fetch_into = [&](f32x4 (&reg)[VL], int j0) {
+      size_t off[VL];                                        // (all the pages looked up before the first load goes out)
 #pragma unroll
-      for (int i = 0; i < VJ; ++i) {
-        const int c = tid + T * i;
+      for (int i = 0; i < VL; ++i) {
+        const int c = lt + LT * i;
         const int cc = c < KC * SEGS ? c : KC * SEGS - 1;
-        reg[i] = *reinterpret_cast<const f32x4*>(a.v_cache + offset_of(j0 + cc / SEGS) + 4 * (cc % SEGS));
+        off[i] = offset_of(j0 + cc / SEGS) + 4 * (cc % SEGS);
       }
-    };
-    auto stash_from = [&](int buf, const f32x4 (&reg)[VJ]) {
 #pragma unroll
-      for (int i = 0; i < VJ; ++i) {
-        const int c = tid + T * i;
-        if (c < KC * SEGS) *reinterpret_cast<f32x4*>(v_lds + buf * KC * HD + 4 * c) = reg[i];
+      for (int i = 0; i < VL; ++i) reg[i] = *reinterpret_cast<const f32x4*>(a.v_cache + off[i]);
+    };
+    // The values of four keys lie side by side in LDS, [key / 4][place of d][key % 4], so that the walking thread
+    // reads four keys' values of its element with one instruction; d's place is (d % 4) * HD / 4 + d / 4, which
+    // spreads the stores of a wave (four keys, sixteen pieces each) over the banks.
+    auto stash_from = [&](int buf, const f32x4 (&reg)[VL]) {
+#pragma unroll
+      for (int i = 0; i < VL; ++i) {
+        const int c = lt + LT * i;                           // piece c = key c / SEGS, elements 4 * (c % SEGS)..
+        if (c < KC * SEGS) {
+          const int kk = c / SEGS, seg = c % SEGS;
+          float* dst = v_lds + buf * KC * HD + (kk >> 2) * HD * 4 + seg * 4 + (kk & 3);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[e * SEGS * 4] = reg[i][e];
+        }
       }
     };
-    fetch_into(r0, lo);
-    fetch_into(r1, lo + KC);
-    fetch_into(r2, lo + 2 * KC);
-    // every thread turns the scores it wrote itself into e_j; the barrier behind the first chunk's values publishes them
+    const int my_place = (tid & 3) * SEGS + (tid >> 2);      // (of element ``tid``, for the threads that walk)
+    auto walk4 = [&](int j0, int buf) {                      // thread d < HD: the chunk's keys in key order, four a read
+      if (tid >= HD) return;
+      const int cnt = (pos - j0 + 1) < KC ? (pos - j0 + 1) : KC;
+      const float* vb = v_lds + buf * KC * HD + my_place * 4;
+      const float* eb = scores + (j0 - lo);
+      if (cnt == KC) {
+        // a whole chunk: KC / 4 reads of four e_j and of four values, written out so that the reads of the next
+        // four quads are on their way while these four are chained (no condition, no register handed on)
+        constexpr int NQ = KC / 4, BQ = 4;
+        f32x4 ev[2][BQ], vv[2][BQ];
+#pragma unroll
+        for (int u = 0; u < BQ; ++u) {
+          ev[0][u] = *reinterpret_cast<const f32x4*>(eb + 4 * u);
+          vv[0][u] = *reinterpret_cast<const f32x4*>(vb + u * HD * 4);
+        }
+#pragma unroll
+        for (int q0 = 0; q0 < NQ; q0 += BQ) {
+          const int cur = (q0 / BQ) & 1;
+          if (q0 + BQ < NQ) {
+#pragma unroll
+            for (int u = 0; u < BQ; ++u)
+              if (q0 + BQ + u < NQ) {
+                ev[cur ^ 1][u] = *reinterpret_cast<const f32x4*>(eb + 4 * (q0 + BQ + u));
+                vv[cur ^ 1][u] = *reinterpret_cast<const f32x4*>(vb + (q0 + BQ + u) * HD * 4);
+              }
+          }
+#pragma unroll
+          for (int u = 0; u < BQ; ++u)
+            if (q0 + u < NQ) {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                sum += ev[cur][u][i];
+                acc = fmaf(ev[cur][u][i], vv[cur][u][i], acc);
+              }
+            }
+        }
+      } else {
+#pragma unroll 4
+        for (int jj = 0; jj < cnt; ++jj) {                   // the sequence's last keys
+          const float ej = eb[jj];
+          sum += ej;
+          acc = fmaf(ej, vb[(jj >> 2) * HD * 4 + (jj & 3)], acc);
+        }
+      }
+    };
+    // one chunk's turn: the chunk three ahead is asked for into ``next``, the chunk in ``buf`` is walked, the
+    // chunk one ahead goes from ``ready`` into the other buffer; the barrier publishes it
+    auto turn = [&](f32x4 (&next)[VL], const f32x4 (&ready)[VL], int j0, int buf) {
+      if constexpr (APART) {
+        if (loads) {
+          fetch_into(next, j0 + 3 * KC);
+          stash_from(buf ^ 1, ready);
+        } else {
+          walk4(j0, buf);
+        }
+      } else {
+        fetch_into(next, j0 + 3 * KC);
+        walk4(j0, buf);
+        stash_from(buf ^ 1, ready);
+      }
+      lds_barrier();
+    };
+    if (loads) {
+      fetch_into(r0, lo);
+      fetch_into(r1, lo + KC);
+      fetch_into(r2, lo + 2 * KC);
+    }
+    // the scores turn into e_j (the barrier behind the maximum has published them; the one behind the first chunk's
+    // values publishes the e_j)
     for (int j = lo + tid; j <= pos; j += T) scores[j - lo] = bw_expf(scores[j - lo] - mx);
-    stash_from(0, r0);
-    __syncthreads();
+    if (loads) stash_from(0, r0);
+    lds_barrier();
     int buf = 0;
     for (int j0 = lo; j0 <= pos; j0 += 3 * KC) {           // (pos is the same for the whole workgroup: so are the exits)
-      fetch_into(r0, j0 + 3 * KC);
-      walk(j0, buf);
-      stash_from(buf ^ 1, r1);
-      __syncthreads();
-      buf ^= 1;
+      turn(r0, r1, j0, buf);
       if (j0 + KC > pos) break;
-      fetch_into(r1, j0 + 4 * KC);
-      walk(j0 + KC, buf);
-      stash_from(buf ^ 1, r2);
-      __syncthreads();
-      buf ^= 1;
+      turn(r1, r2, j0 + KC, buf ^ 1);
       if (j0 + 2 * KC > pos) break;
-      fetch_into(r2, j0 + 5 * KC);
-      walk(j0 + 2 * KC, buf);
-      stash_from(buf ^ 1, r0);
-      __syncthreads();
+      turn(r2, r0, j0 + 2 * KC, buf);
       buf ^= 1;
     }
   } else {
@@ -803,7 +910,7 @@ static void launch_attention_f32(const AttnF32Args& a, dim3 grid, hipStream_t s)
   long long capacity = (long long)a.table_stride * a.page_size;
   if (a.window > 0 && a.window < capacity) capacity = a.window;
   const long long keep_bytes = Att32Shape<HD>::LDS_BYTES + ((capacity + 3) & ~3ll) * (long long)sizeof(float);
-  if (keep_bytes <= ATT32_KEEP_LDS)
+  if (keep_bytes <= ATT32_KEEP_LDS && a.table_stride <= ATT32_TABLE && a.page_shift >= 0)   // (and the table's row fits the kernel's copy of it)
     hipLaunchKernelGGL((attention_f32_kernel<HD, true>), grid, dim3(ATT32_THREADS), (size_t)keep_bytes, s, a);
   else
     hipLaunchKernelGGL((attention_f32_kernel<HD, false>), grid, dim3(ATT32_THREADS), Att32Shape<HD>::LDS_BYTES, s, a);
