@@ -466,6 +466,236 @@ static void launch_lanes(const float* x, const WT* w, float* y, int M, int N, in
   }
 }
 
+// ------------------------------------------------------------------------------ a wave a row, the row four elements a register
+
+// Decoded tokens once more: a wave is a row and 64 columns, lane l the chain of (row, column n0 + l), weights and
+// rows in an LDS ring as above (weights packed).  What is new is how a row's elements reach the multiply-adds.
+// x[row][k] is the same number for every lane of the wave; read as such from LDS it costs what any read costs (LDS
+// returns 128 bytes a clock whatever the addresses: above, the rows took two thirds of what LDS returned).  Here lane
+// l reads the 16 bytes at element 4 * (l % 4) of a run of sixteen, so that a register holds four elements of the row,
+// the same four in every quad of lanes, and the multiply-add picks its element with the quad permutation of its
+// first operand (v_fmac_f32 with quad_perm [i,i,i,i]: the same fused multiply-add, the operand routed on the way
+// in): sixteen elements a read instead of four.
+// A workgroup is 64 columns and all rows (a chain wave a row, sharing the ring).  A block is 64 bytes of a row of W
+// (four 16-byte chunks: 32 bfloat16 or 16 32-bit elements), a stage two blocks; the next block's operands are read
+// from LDS while this block's chains run.  (A chain is bound by its own links: a multiply-add that waits for the one
+// before it issues every 3.8 ns, and 5.3 ns with one other vector instruction a link, such as the widening of a
+// bfloat16 weight, wherever that instruction stands.)
+#define F32C_W (64 * 128)                                             // 64 rows of W, 128 bytes each
+#define F32C_X (8 * 256)                                              // 8 rows of x, up to 64 elements each
+#define F32C_STAGE (F32C_W + F32C_X)
+
+template <int KB>
+struct ChainBlock {
+  f32x4 x[KB / 16];                                                   // register j of x[a]: element 16 a + 4 (lane % 4) + j of the block
+  u32x4 w[4];
+};
+
+template <typename WT>
+__device__ __forceinline__ void chain_read(ChainBlock<64 / (int)sizeof(WT)>& b, const unsigned char* stage, int half, int my, int swz,
+                                           const unsigned char* xs) {
+  constexpr int KB = 64 / (int)sizeof(WT);
+#pragma unroll
+  for (int a = 0; a < KB / 16; ++a) b.x[a] = *reinterpret_cast<const f32x4*>(xs + (half * KB + 16 * a) * 4);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b.w[j] = *reinterpret_cast<const u32x4*>(stage + my + (((4 * half + j) ^ swz) * 16));
+}
+
+// acc = fma(x of quad lane I, w, acc): v_fmac_f32 with its first operand routed through the quad permutation
+// [I,I,I,I] (written out: the compiler keeps a move of its own in front of the multiply-add otherwise, which costs
+// what the multiply-add costs).  The operand comes from an LDS read, never from a vector instruction just before
+// (which would want two idle states in between).
+template <int I>
+__device__ __forceinline__ float fma_quad(float xq, float w, float acc) {
+  static_assert(I >= 0 && I < 4, "a quad has four lanes");
+  if constexpr (I == 0) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(xq), "v"(w));
+  else if constexpr (I == 1) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(xq), "v"(w));
+  else if constexpr (I == 2) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(xq), "v"(w));
+  else asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(xq), "v"(w));
+  return acc;
+}
+
+// element k of the block: register k % 4 of x[k / 16], quad lane (k / 4) % 4
+template <int K16>
+__device__ __forceinline__ float chain_step(float acc, const f32x4& x, float w) {
+  constexpr int I = (K16 >> 2) & 3, J = K16 & 3;
+  return fma_quad<I>(x[J], w, acc);
+}
+
+// Element e of 16-byte chunk ``c`` as a 32-bit float (bfloat16: the bits, shifted: exact).
+template <typename WT, int E>
+__device__ __forceinline__ float chain_weight(const u32x4& c) {
+  if constexpr (sizeof(WT) == 2) return __uint_as_float((E & 1) ? (c[E >> 1] & 0xffff0000u) : (c[E >> 1] << 16));
+  else return __uint_as_float(c[E]);
+}
+
+// The block's chains.  A multiply-add that depends on the one before it can issue every other slot, and one whose
+// weight was widened in the slot before it waits for that as well: so chunk j + 1 is widened between the multiply-adds
+// of chunk j (``f`` comes in with the block's chunk 0 widened, and leaves with chunk 0 of the next block).
+template <typename WT>
+__device__ __forceinline__ float chain_run(float acc, const ChainBlock<64 / (int)sizeof(WT)>& b, const ChainBlock<64 / (int)sizeof(WT)>& nxt,
+                                           float (&f)[16 / (int)sizeof(WT)]) {
+  constexpr int EPC = 16 / (int)sizeof(WT);                           // elements a chunk
+  float g[EPC];
+#define BW_CHAIN_STEP(J, E, FROM, TO, SRC)                                                \
+  TO[E] = chain_weight<WT, E>(SRC);                                                       \
+  acc = chain_step<(EPC * J + E) & 15>(acc, b.x[(EPC * J + E) >> 4], FROM[E]);
+#define BW_CHAIN_CHUNK(J, FROM, TO, SRC)                                                  \
+  BW_CHAIN_STEP(J, 0, FROM, TO, SRC) BW_CHAIN_STEP(J, 1, FROM, TO, SRC) BW_CHAIN_STEP(J, 2, FROM, TO, SRC) BW_CHAIN_STEP(J, 3, FROM, TO, SRC) \
+  if constexpr (EPC == 8) {                                                               \
+    BW_CHAIN_STEP(J, (EPC == 8 ? 4 : 0), FROM, TO, SRC) BW_CHAIN_STEP(J, (EPC == 8 ? 5 : 1), FROM, TO, SRC)                                   \
+    BW_CHAIN_STEP(J, (EPC == 8 ? 6 : 2), FROM, TO, SRC) BW_CHAIN_STEP(J, (EPC == 8 ? 7 : 3), FROM, TO, SRC)                                   \
+  }
+  BW_CHAIN_CHUNK(0, f, g, b.w[1])
+  BW_CHAIN_CHUNK(1, g, f, b.w[2])
+  BW_CHAIN_CHUNK(2, f, g, b.w[3])
+  BW_CHAIN_CHUNK(3, g, f, nxt.w[0])
+#undef BW_CHAIN_CHUNK
+#undef BW_CHAIN_STEP
+  return acc;
+}
+
+template <typename WT>
+__device__ __forceinline__ void chain_first(const ChainBlock<64 / (int)sizeof(WT)>& b, float (&f)[16 / (int)sizeof(WT)]) {
+  f[0] = chain_weight<WT, 0>(b.w[0]);
+  f[1] = chain_weight<WT, 1>(b.w[0]);
+  f[2] = chain_weight<WT, 2>(b.w[0]);
+  f[3] = chain_weight<WT, 3>(b.w[0]);
+  if constexpr (sizeof(WT) == 2) {
+    f[4] = chain_weight<WT, 4>(b.w[0]);
+    f[5] = chain_weight<WT, 5>(b.w[0]);
+    f[6] = chain_weight<WT, 6>(b.w[0]);
+    f[7] = chain_weight<WT, 7>(b.w[0]);
+  }
+}
+
+// The loads are not the chain waves' business.  A buffer load with LDS as destination holds the wave that issues it
+// for some hundred clocks (ten of them a stage were more than the stage's chains), so a workgroup has two waves more
+// that do nothing else: they ask for the stages, wait for them and meet the chain waves at the stage's barrier.  A
+// loader issues five loads a stage: the ten are the eight blocks of 8 rows of W and two blocks of 4 rows of x,
+// dealt in turn (loads for rows the workgroup does not have go outside the descriptor: no traffic, zeros into a
+// spare KB behind the ring, so that both loaders count alike).
+#define F32C_LOADERS 2
+#define F32C_LPL 5                                                    // loads a loader and stage
+
+template <int STAGES>
+__device__ __forceinline__ void chain_issue(unsigned char* lds, __amdgpu_buffer_rsrc_t rs_w, __amdgpu_buffer_rsrc_t rs_x, const int* voff,
+                                            int loader, int step, int steps, int x_step) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  unsigned char* dst = lds + (step % STAGES) * F32C_STAGE;
+  const bool real = step < steps;                                     // scalar
+#pragma unroll
+  for (int t = 0; t < F32C_LPL; ++t) {
+    const int q = loader + F32C_LOADERS * t;                          // 0..7: W; 8, 9: x
+    if (q < 8) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + q * 1024), 16, real ? voff[t] : 0x7ffffff0, step * 128, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + F32C_W + (q - 8) * 1024), 16, real ? voff[t] : 0x7ffffff0,
+                                                  step * x_step, 0, 0);
+  }
+}
+
+template <typename WT, int STAGES>
+__global__ __launch_bounds__(64 * (8 + F32C_LOADERS)) void gemm_f32_chain_kernel(const float* __restrict__ x, const WT* __restrict__ w,
+                                                                                 float* __restrict__ y, int M, int N, int K, int ldx,
+                                                                                 int ldy, int accumulate) {
+  constexpr int KB = 64 / (int)sizeof(WT);                            // elements of k a block
+  extern __shared__ __attribute__((aligned(16))) unsigned char chain_lds[];   // [stages][W: 64 rows of 128 B | x: 8 rows of 256 B]
+  const int wave = wave_index(), lane = threadIdx.x & 63, rw = (int)(blockDim.x >> 6) - F32C_LOADERS;
+  const int n0 = blockIdx.x * 64;
+  const int m0 = blockIdx.y * rw;                                     // the workgroup's first row
+  const int steps = K / (2 * KB);
+  if (wave >= rw) {
+    // ---- a loader
+    const int loader = wave - rw;
+    const int w_rows = min(64, N - n0), x_rows = min(rw, M - m0);
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void*)(w + (size_t)n0 * K), 0,
+                                                                          (int)((size_t)w_rows * K * sizeof(WT)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void*)(x + (size_t)m0 * ldx), 0,
+                                                                          (int)((((size_t)x_rows - 1) * ldx + K) * 4), 0x00020000);
+    // W: lane l of a load fetches row l / 8 of its 8 rows, chunk (l % 8) ^ (row within 16 >> 1) of the row's 128 bytes;
+    // x: lane l fetches row 4 (q - 8) + l / 16 of the workgroup's, chunk l % 16 of the stage's elements (with 32-bit
+    // weights a stage is 32 elements: the chunks past them lie outside)
+    int voff[F32C_LPL];
+#pragma unroll
+    for (int t = 0; t < F32C_LPL; ++t) {
+      const int q = loader + F32C_LOADERS * t;
+      if (q < 8) {
+        const int r = 8 * q + (lane >> 3);
+        voff[t] = (int)((r * K) * (int)sizeof(WT) + 16 * ((lane & 7) ^ ((r & 15) >> 1)));
+      } else {
+        const int xrow = 4 * (q - 8) + (lane >> 4), xchunk = lane & 15;
+        voff[t] = (xrow < x_rows && 4 * xchunk < 2 * KB) ? (xrow * ldx + 4 * xchunk) * 4 : 0x7ffffff0;
+      }
+    }
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) chain_issue<STAGES>(chain_lds, rs_w, rs_x, voff, loader, st, steps, 2 * KB * 4);
+    for (int step = 0; step < steps; ++step) {
+      // this stage and the next have landed (the next stage's first block is read during this one's second); behind
+      // the barrier every chain wave is done with the stage before, which the new loads overwrite
+      __builtin_amdgcn_s_waitcnt(vmcnt_only(F32C_LPL * (STAGES - 3)));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      chain_issue<STAGES>(chain_lds, rs_w, rs_x, voff, loader, step + STAGES - 1, steps, 2 * KB * 4);
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                        // the padding loads too, before the wave ends
+    return;
+  }
+  // ---- a chain wave: row m0 + wave
+  const int row = m0 + wave;
+  // this lane's row of the tile: chunk j lies in slot j ^ (row within 16 >> 1); its four elements of the wave's row
+  const int my = (lane >> 3) * 1024 + (lane & 7) * 128, swz = (lane & 15) >> 1;
+  const int mine = F32C_W + wave * 256 + (lane & 3) * 16;
+  ChainBlock<KB> even, odd;
+  float f[16 / (int)sizeof(WT)];                                      // a chunk of W, widened
+  float acc = 0.0f;
+  for (int step = 0; step < steps; ++step) {
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const unsigned char* stage = chain_lds + (step % STAGES) * F32C_STAGE;
+    const unsigned char* next = chain_lds + ((step + 1) % STAGES) * F32C_STAGE;
+    if (step == 0) {
+      chain_read<WT>(even, stage, 0, my, swz, stage + mine);
+      chain_first<WT>(even, f);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    chain_read<WT>(odd, stage, 1, my, swz, stage + mine);
+    __builtin_amdgcn_sched_barrier(0);
+    acc = chain_run<WT>(acc, even, odd, f);
+    __builtin_amdgcn_sched_barrier(0);
+    chain_read<WT>(even, next, 0, my, swz, next + mine);              // (past the last stage: whatever the ring holds, unused)
+    __builtin_amdgcn_sched_barrier(0);
+    acc = chain_run<WT>(acc, odd, even, f);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+  }
+  const int n = n0 + lane;
+  if (n >= N || row >= M) return;
+  float* o = y + (size_t)row * ldy + n;
+  *o = accumulate ? (*o + acc) : acc;
+}
+
+// For products with at least as many blocks of 64 columns as there are compute units and up to 8 rows: a workgroup
+// a block of columns with all the rows (there it is faster than the kernels above: gate|up of 16,384 columns
+// at 8 rows 26.6 us against 29.1, a head of 49,152 columns 65 against 85; with fewer columns a chain wave has a
+// compute unit to itself in either kernel and both take what the chain takes).
+#define F32C_STAGES 7
+#define F32C_MAX_ROWS 8
+
+template <typename WT>
+static void launch_chain(const float* x, const WT* w, float* y, int M, int N, int K, int ldx, int ldy, int accumulate, hipStream_t s) {
+  constexpr int lds_bytes = F32C_STAGES * F32C_STAGE + 1024;
+  static_assert(F32C_LPL * (F32C_STAGES - 3) < 64, "the wait count has six bits");
+  static_assert(F32C_LPL * F32C_LOADERS == 10, "eight loads of W and two of x a stage");
+  static bool allowed = false;                       // 64 KB of dynamic LDS and more has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_f32_chain_kernel<WT, F32C_STAGES>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    allowed = true;
+  }
+  int rw = 1;
+  while (rw < M) rw *= 2;                            // (1, 2, 4 or 8 chain waves)
+  hipLaunchKernelGGL((gemm_f32_chain_kernel<WT, F32C_STAGES>), dim3((N + 63) / 64, 1), dim3(64 * (rw + F32C_LOADERS)), lds_bytes, s, x, w, y,
+                     M, N, K, ldx, ldy, accumulate);
+}
+
 // ------------------------------------------------------------------------------ up to 64 rows on the matrix cores
 
 // v_mfma_f32_4x4x1_16b_f32 computes, for 16 blocks of 4 x 4 outputs at once, D[r][j] = fma(A[r], B[j], D[r][j]):
@@ -861,6 +1091,13 @@ extern "C" int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* 
       (size_t)M * ldx * 4 < ((size_t)1 << 31) && (size_t)64 * K * 4 < ((size_t)1 << 31)) {
     if (w_is_bf16) launch_f32_mfma_rows<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
     else launch_f32_mfma_rows<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    return BW_LAUNCH_CHECK();
+  }
+  // up to 8 rows, many columns, K in whole stages: a wave a row, the row four elements a register, loader waves
+  if (M <= F32C_MAX_ROWS && (N + 63) / 64 >= F32L_MIN_BLOCKS && K % (w_is_bf16 ? 64 : 32) == 0 && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0 &&
+      ((uintptr_t)w & 15) == 0 && (size_t)64 * K * 4 < ((size_t)1 << 31) && (size_t)M * ldx * 4 < ((size_t)1 << 31)) {
+    if (w_is_bf16) launch_chain<bf16_t>(x, (const bf16_t*)w, y, M, N, K, ldx, ldy, accumulate, s);
+    else launch_chain<float>(x, (const float*)w, y, M, N, K, ldx, ldy, accumulate, s);
     return BW_LAUNCH_CHECK();
   }
   // up to 16 rows, many columns, K in whole stages: a wave a row, weights packed in LDS

@@ -99,9 +99,11 @@ def test_gemm_f32_grid_rows_and_accumulate(gpu):
             before = batch.clone()
             ops.gemm_f32(x, weight, batch, M, accumulate=True)
             assert torch.equal(batch, before + before)
-    # many columns and up to 16 rows (a wave a row, weights packed in LDS): the bits of the same rows inside a product of
-    # 20 rows (matrix cores) and of the chain-per-thread kernel (K + 8 is no whole stage of the first)
-    for M, N, K in [(1, 16400, 64), (8, 16384, 2048), (16, 20000, 128), (5, 16385, 192), (13, 16500, 96)]:
+    # many columns and up to 16 rows (a wave a row, weights packed in LDS; up to 8 rows with loader waves and the row
+    # four elements a register): the bits of the same rows inside a product of 20 rows (matrix cores) and of the
+    # chain-per-thread kernel (K + 8 is no whole stage of the first)
+    for M, N, K in [(1, 16400, 64), (8, 16384, 2048), (16, 20000, 128), (5, 16385, 192), (13, 16500, 96), (3, 16390, 128),
+                    (7, 16384, 320), (2, 17000, 64), (9, 16384, 64)]:
         x, w = torch.randn(20, K + 8, generator=g).to(gpu), (torch.randn(N, K + 8, generator=g) * 0.1).to(gpu)
         for weight in (w, w.bfloat16()):
             xs, ws = x[:, :K].contiguous(), weight[:, :K].contiguous()
