@@ -67,7 +67,8 @@ def main() -> int:
 
     import torch
     import bitwise_amd as bw
-    from bitwise_amd.measure import CONTEXT, PEAK_FLOPS, measure_decode, measure_prefill, measure_serving, measure_trace
+    from bitwise_amd.measure import (CONTEXT, PEAK_FLOPS, measure_chunked_prefill, measure_decode, measure_prefill, measure_serving,
+                                     measure_trace)
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B)
@@ -112,32 +113,45 @@ def main() -> int:
             model32 = bw.Model.random(cfg, seed=0, dtype="float32", sigma=0.02, on_device=True)
             m = measure_decode(bw, torch, model32, cfg, "float32", args.batch, side_steps, 4)
             extra["fp32"] = {"decode_tok_s": m["tok_s"], "batch": args.batch, "ms_per_step": m["ms_per_step"],
-                             "roofline": m["roofline"],
+                             "roofline": m["roofline"], "weights_stored_as": "bfloat16, widened exactly where they are used",
                              "prefill": measure_prefill(bw, torch, model32, cfg, "float32", PEAK_FLOPS["fp32"])}
             del model32
             torch.cuda.empty_cache()
-            # Llama-3-8B's sizes, all 32 layers, bfloat16: decode at batch 8 with 2,048-token contexts, one prefill
-            big = dict(LLAMA3_8B)
+            # Llama-3-8B's sizes, all 32 layers, bfloat16 (position tables of 16,384 for the 8,192-token contexts): decode at
+            # batch 8, 1 and 64 with 2,048-token contexts and at batch 8 with 8,192-token contexts, a prefill of 2,048 tokens
+            # in one step and one of 8,192 in portions of 2,048
+            big = dict(LLAMA3_8B, max_position_embeddings=16384)
             model8 = bw.Model.random(big, seed=1, dtype="bfloat16", sigma=0.02, on_device=True)
             m = measure_decode(bw, torch, model8, big, "bfloat16", 8, side_steps, 4)
+            points8, rooflines8 = {}, {}
+            for name, b, ctx in (("decode_b1", 1, CONTEXT), ("decode_b64", 64, CONTEXT), ("decode_b8_ctx8192", 8, 8192)):
+                mp = measure_decode(bw, torch, model8, big, "bfloat16", b, side_steps, 4, context=ctx)
+                points8[name] = mp["tok_s"]
+                rooflines8[name] = mp["roofline"]["frac"]
             extra["llama3_8b"] = {"layers": big["num_hidden_layers"], "hidden": big["hidden_size"], "heads": 32, "kv_heads": 8,
                                   "head_dim": 128, "ffn": big["intermediate_size"], "vocab": big["vocab_size"],
                                   "decode_tok_s": m["tok_s"], "batch": 8, "ms_per_step": m["ms_per_step"],
-                                  "roofline": m["roofline"],
+                                  "roofline": m["roofline"], "points": points8, "point_roofline_fracs": rooflines8,
                                   "prefill": measure_prefill(bw, torch, model8, big, "bfloat16", PEAK_FLOPS["bf16"]),
+                                  "prefill_8192_in_portions": measure_chunked_prefill(bw, torch, model8, big, "bfloat16",
+                                                                                      PEAK_FLOPS["bf16"]),
                                   "serving": measure_serving(bw, torch, model8, big, "bfloat16"),
                                   # 128 requests, four shared 1,024-token starts, contexts up to 6,144, a tenth cancelled, a pool
-                                  # that forces preemption; 16 of them checked against solo runs
-                                  "trace8k": measure_trace(bw, torch, model8, big, "bfloat16")}
+                                  # that forces preemption; 8 of them checked against solo runs
+                                  "trace8k": measure_trace(bw, torch, model8, big, "bfloat16", check=8)}
             del model8
             model = None
 
     value = head["tok_s"]
+    # The reference's figure is one stream on a CPU: like for like is this engine's rate at batch 1, where it is measured.
+    one_stream = points.get("decode_b1", value if args.batch == 1 else None)
     line = {
         "metric": f"decode tok/s at batch {args.batch}, {shape_name} shape, 2048-token contexts",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": round(value / BASELINE_TOK_S, 1) if args.shape == "smollm2" else None, "dtype": args.dtype,
+        "vs_baseline": round(value / BASELINE_TOK_S, 1) if args.shape == "smollm2" else None,
+        "vs_baseline_one_stream": round(one_stream / BASELINE_TOK_S, 1) if args.shape == "smollm2" and one_stream else None,
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {
             "model": f"{shape_name} shape, random weights", "layers": cfg["num_hidden_layers"],
@@ -145,7 +159,7 @@ def main() -> int:
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"], "ffn": cfg["intermediate_size"],
             "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]), "global_batch": args.batch, "seq_len": CONTEXT, "max_context": 4096,
             "page_size": 16, "parallelism": "single GPU", "weights": "bf16" if args.dtype == "bf16" else "bf16 widened",
-            "baseline": "reference CPU decode, one stream, 7.26 tok/s",
+            "baseline": f"reference CPU decode, one stream, 7.26 tok/s (vs_baseline: batch {args.batch} over it)",
         },
         "prefill": prefill,
         "roofline": head["roofline"],
