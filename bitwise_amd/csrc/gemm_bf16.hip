@@ -2073,7 +2073,14 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       // enough 256-row tiles to go round the compute units (a second round at least half full)
       constexpr int BIG_COLS = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
       const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + BIG_COLS - 1) / BIG_COLS;
-      if (S == 1 && K % 64 == 0 && M >= 2 * BIG_BM && bm * bn >= 128) {
+      // (fewer of these tiles than compute units while the 128-row tiles below would fill the chip in one round: a step
+      // of those takes half as long, so they win: gate|up of 512 rows 62 us here, half the chip idle)
+      bool half_tiles_win = false;
+      if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16) {
+        const int t256 = ((M + 127) / 128) * bn;
+        half_tiles_win = (t256 + 255) / 256 < 2 * ((bm * bn + 255) / 256);
+      }
+      if (S == 1 && K % 64 == 0 && M >= 2 * BIG_BM && bm * bn >= 128 && !half_tiles_win) {
         static bool allowed = false;                 // more than 64 KB of dynamic LDS has to be asked for once
         if (!allowed) {
           (void)hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
