@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -58,6 +58,8 @@ def main() -> int:
                     help="the length of the headline prefill's prompt (for profiles of shorter prompts; up to 2048)")
     ap.add_argument("--shape", choices=["smollm2", "llama3_8b"], default="smollm2",
                     help="the layer sizes of the headline run (llama3_8b: for profiles of that shape; implies --no-points)")
+    ap.add_argument("--trace-only", action="store_true",
+                    help="run nothing but the 128-request shared-prefix trace at Llama-3-8B's sizes and print its figures (for profiles)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -71,6 +73,11 @@ def main() -> int:
                                      measure_trace)
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    if args.trace_only:
+        big = dict(LLAMA3_8B, max_position_embeddings=16384)
+        model8 = bw.Model.random(big, seed=1, dtype=dtype, sigma=0.02, on_device=True)
+        print(json.dumps({"llama3_8b.trace8k": measure_trace(bw, torch, model8, big, dtype, check=8), "dtype": args.dtype}))
+        return 0
     cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B)
     shape_name = "SmolLM2-1.7B" if args.shape == "smollm2" else "Llama-3-8B"
     if args.shape != "smollm2":
