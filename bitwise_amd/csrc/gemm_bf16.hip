@@ -1252,6 +1252,24 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   constexpr bool GLU = S::GLU;
   constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ, THREADS = 64 * S::NW;
+  if constexpr (!NORM) {
+    // gridDim.z > 1: a prompt portion of a few blocks of 16 * NRB rows in one launch, workgroup (tile, segment, z) the
+    // rows of block z (the launcher sees to it that blocks share no scratch)
+    if (gridDim.z > 1) {
+      const int first = (int)blockIdx.z * 16 * NRB;
+      x += (size_t)first * ldx;
+      if constexpr (EPI == EPI_QKV_ROPE) {
+        rp.positions += first;
+        rp.row_seq += first;
+        out = (void*)((bf16_t*)out + (size_t)first * rp.heads * rp.head_dim);
+      } else if constexpr (EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16) {
+        out = (void*)((bf16_t*)out + (size_t)first * ldo);
+      } else {
+        out = (void*)((float*)out + (size_t)first * ldo);
+      }
+      M = min(16 * NRB, M - first);
+    }
+  }
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];   // [8 stages][x: NRB * 2 KB | W: 8 KB], 1 KB for padding loads; NORM: then the rows, 2 KB a step
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
@@ -1529,7 +1547,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
 
 template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
 static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
-                            const MidNormArgs& na, const QkvRopeArgs& rp, int segments, const MidSplitArgs& sp) {
+                            const MidNormArgs& na, const QkvRopeArgs& rp, int segments, const MidSplitArgs& sp, int row_blocks) {
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
   const int lds_bytes = NORM ? mid_norm_lds_bytes(S::RING, K, na.row_step) : S::RING;
@@ -1538,21 +1556,21 @@ static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, 
     (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>), dim3(wgs, segments), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
+  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>), dim3(wgs, segments, row_blocks), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
   return BW_LAUNCH_CHECK();
 }
 
 template <int EPI, int NRB, bool NORM, bool NARROW = false>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
                       const MidNormArgs& na = MidNormArgs{}, const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1,
-                      const MidSplitArgs& sp = MidSplitArgs{}) {
+                      const MidSplitArgs& sp = MidSplitArgs{}, int row_blocks = 1) {
   // 17 rows or more, or rows normalised in the kernel (a row a wave sooner done than two), K in whole stages: the
   // eight-wave variant (the same bits)
   if constexpr (NORM || NRB >= 2) {
     if (K % (64 * MidShape<EPI, NRB, NORM, NARROW, true>::SUB) == 0)
-      return launch_mid_waves<EPI, NRB, NORM, NARROW, true>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
+      return launch_mid_waves<EPI, NRB, NORM, NARROW, true>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp, row_blocks);
   }
-  return launch_mid_waves<EPI, NRB, NORM, NARROW, false>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp);
+  return launch_mid_waves<EPI, NRB, NORM, NARROW, false>(x, w, out, M, N, K, ldx, ldo, wgs, s, na, rp, segments, sp, row_blocks);
 }
 
 // RMSNorm of up to 16 rows of the residual stream + product with many columns in one kernel; -7: not this shape.
@@ -1587,9 +1605,17 @@ static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, vo
                                hipStream_t s) {
   const int all_heads = rp.heads + 2 * rp.kv_heads, hd = rp.head_dim;
   const int wide_tiles = all_heads * (hd / 64);         // workgroups with 32 pairs each
-  if (M > 64 || K % 64 || hd % 64 || wide_tiles < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31))
-    return -7;
+  if (K % 64 || hd % 64 || wide_tiles < 64 || (size_t)M * ldx * 2 >= ((size_t)1 << 31)) return -7;
   const int N = all_heads * hd, ldo = rp.heads * hd;
+  if (M > 64) {
+    // a short prompt portion: blocks of 64 rows in one launch, while all of them fit the chip at once
+    const int zb = (M + 63) / 64;
+    if (wide_tiles * zb > 512) return -7;
+    if (2 * wide_tiles * zb <= 512 && wide_tiles < ROPE_NARROW_BELOW)
+      return launch_mid<EPI_QKV_ROPE, 4, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp, 1,
+                                                      MidSplitArgs{}, zb);
+    return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, wide_tiles, s, MidNormArgs{}, rp, 1, MidSplitArgs{}, zb);
+  }
   if (wide_tiles < ROPE_NARROW_BELOW) {                // fewer workgroups than compute units: 16 pairs a workgroup
     if (M <= 16) return launch_mid<EPI_QKV_ROPE, 1, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp);
     if (M <= 32) return launch_mid<EPI_QKV_ROPE, 2, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp);
@@ -1914,6 +1940,10 @@ static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
 //               afterwards (128 rows of K = 8192: 25 us).
 //   big split   the same with 256 x 256 tiles, which fetch half as many bytes a flop: for 512 rows or more.
 //   tile256     128 x 256 tiles with all of K, the segments joined in registers: needs no scratch.
+//   blocks at once  one segment of K only: the kernel for up to 64 rows with all blocks of 64 rows in one launch (its
+//               grid's third dimension), while the workgroups fit the chip at once (512): the output projection of
+//               2048 columns takes 8.4 us at 128 rows and 13.3 at 512, where 128 x 128 tiles took 16.4 and 21.6.  The
+//               q|k|v product with rotation and cache write goes the same way (launch_qkv_rope_mid).
 // All five give the same bits.  The choice is by a count of steps: rounds times the steps of a workgroup (a step of
 // a 256 x 256 tile counts twice); the join moves 8 bytes an element and segment (about 500,000 elements in the
 // time of a step) and is a launch more (8 steps); a split has to win by a tenth.  tiles64: what the 64-row
@@ -2023,6 +2053,20 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
 #undef BW_SKINNY
   } else {
     if constexpr (EPI == EPI_ADD_F32) {
+      // One segment of K and few columns (the output projection of a short prompt: 16 tiles of 128 x 128 for 128 rows and
+      // 2048 columns, whatever is idle): the kernel for up to 64 rows, a workgroup per block of 64 rows and 64 or 32
+      // columns, all blocks in one launch, while they fit the chip at once (two workgroups a compute unit).
+      if (S == 1 && K % 64 == 0 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        const int zb = (M + 63) / 64, wide = (N + 63) / 64;
+        const bool narrow = wide * zb < 192;
+        const int tiles = narrow ? (N + 31) / 32 : wide;
+        if (tiles * zb >= 32 && tiles * zb <= 512 && zb <= 65535) {
+          const MidNormArgs na{};
+          const QkvRopeArgs no{};
+          if (narrow) return launch_mid<EPI, 4, false, true>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, 1, MidSplitArgs{}, zb);
+          return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, 1, MidSplitArgs{}, zb);
+        }
+      }
       int tiles;
       const AddRoute route = add_route(M, N, K, ldo, tiles);
       if (route == ADD_ROW_BLOCKS && (size_t)M * ldx * 2 < ((size_t)1 << 31) &&
@@ -2193,6 +2237,10 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
   if (M <= 64) {
     const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
     return mid == -7 ? -2 : mid;
+  }
+  {
+    const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
+    if (mid != -7) return mid;
   }
   const int N = (heads + 2 * kv_heads) * 64;
   return launch_gemm_bf16<EPI_QKV_ROPE>((const bf16_t*)x, (const bf16_t*)w_qkv, q_out, M, N, K, ldx, heads * 64,
