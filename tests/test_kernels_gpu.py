@@ -129,6 +129,7 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
                     (7, 200, 4160), (16, 5000, 4096), (3, 40, 128), (12, 4104, 6144),   # up to 16 rows streaming through LDS, several segments
                     (50, 1030, 128), (20, 2048, 256),   # 17 to 64 rows, one segment, few columns: narrow tiles for the residual add
                     (130, 96, 256), (200, 300, 1024), (129, 130, 2048),   # wide tiles, K in whole double steps
+                    (130, 2048, 256), (500, 2100, 128), (65, 1030, 64), (320, 1024, 2048),   # a residual add of one segment: all blocks of 64 rows in one launch
                     (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
                     (129, 96, 6144)]:                                     # several 2048-segments of K
@@ -884,6 +885,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
                                    (40, 10, 128, 2100, 32),        # enough 256 x 256 tiles for the big-tile kernel
                                    (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16),   # up to 64 rows, half a head a workgroup
                                    (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32),   # a head a workgroup
+                                   (40, 12, 128, 130, 16), (72, 12, 192, 300, 16), (64, 16, 2048, 190, 32),   # blocks of 64 rows in one launch
                                    (40, 12, 4160, 16, 16),                                 # several segments of K
                                    (32, 8, 4096, 8, 16, 128), (24, 4, 128, 40, 8, 128), (100, 14, 64, 12, 16, 128),
                                    (16, 8, 2112, 20, 16, 256)]:                            # larger heads, up to 64 rows
