@@ -1254,7 +1254,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ, THREADS = 64 * S::NW;
   if constexpr (!NORM) {
     // gridDim.z > 1: a prompt portion of a few blocks of 16 * NRB rows in one launch, workgroup (tile, segment, z) the
-    // rows of block z (the launcher sees to it that blocks share no scratch)
+    // rows of block z (a residual add's segments meet in scratch cells of their own for every block and tile)
     if (gridDim.z > 1) {
       const int first = (int)blockIdx.z * 16 * NRB;
       x += (size_t)first * ldx;
@@ -1502,8 +1502,9 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         // device-scope loads issued after the barrier behind the count.  The counter is back at zero when the
         // kernel ends.
         const int cell = S::NW * NI * 1024;                          // bytes of a workgroup's sums: [wave][i][lane] x 16
+        const int tile_id = (int)(blockIdx.z * gridDim.x + blockIdx.x);   // (block of rows, tile of columns)
         const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(
-            (void*)((unsigned char*)sp.scratch + (size_t)blockIdx.x * nseg * cell), 0, nseg * cell, 0x00020000);
+            (void*)((unsigned char*)sp.scratch + (size_t)tile_id * nseg * cell), 0, nseg * cell, 0x00020000);
         const int mine = (wave * NI) * 1024 + lane * 16;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
@@ -1511,10 +1512,10 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                   // this wave's stores have been acknowledged
         __syncthreads();                                             // also: every wave is done with the ring, whose first word is the flag now
         int* is_last = reinterpret_cast<int*>(mid_lds);
-        if (threadIdx.x == 0) *is_last = atomicAdd(&sp.counters[blockIdx.x], 1) == nseg - 1;
+        if (threadIdx.x == 0) *is_last = atomicAdd(&sp.counters[tile_id], 1) == nseg - 1;
         __syncthreads();
         if (!*is_last) return;
-        if (threadIdx.x == 0) sp.counters[blockIdx.x] = 0;
+        if (threadIdx.x == 0) sp.counters[tile_id] = 0;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
           f32x4 y;
@@ -1950,6 +1951,22 @@ static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
 // kernel's scratch is sized by.
 enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT, ADD_TILE256 };
 
+// "Blocks at once" for a residual add of more than 64 rows: how many blocks of 64 rows, tiles of 64 or (narrow) 32
+// columns; tiles 0: it does not run that way (more than 512 workgroups, or too few to matter).  Several segments of K
+// meet in scratch: 4096 floats a workgroup, a counter a (block, tile).
+#define ADD_BLOCKS_MAX_WGS 512
+static void add_blocks_shape(int M, int N, int K, int& tiles, bool& narrow, int& zb) {
+  const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
+  tiles = 0;
+  narrow = false;
+  zb = (M + 63) / 64;
+  if (M <= 64 || K % 64 || N <= 0) return;
+  const int wide = (N + 63) / 64;
+  narrow = wide * zb * S < 192;
+  const int t = narrow ? (N + 31) / 32 : wide;
+  if (t * zb * S >= 32 && t * zb * S <= ADD_BLOCKS_MAX_WGS) tiles = t;
+}
+
 static AddRoute add_route(int M, int N, int K, int ldo, int& tiles64) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
   tiles64 = 0;
@@ -2053,18 +2070,20 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
 #undef BW_SKINNY
   } else {
     if constexpr (EPI == EPI_ADD_F32) {
-      // One segment of K and few columns (the output projection of a short prompt: 16 tiles of 128 x 128 for 128 rows and
-      // 2048 columns, whatever is idle): the kernel for up to 64 rows, a workgroup per block of 64 rows and 64 or 32
-      // columns, all blocks in one launch, while they fit the chip at once (two workgroups a compute unit).
-      if (S == 1 && K % 64 == 0 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
-        const int zb = (M + 63) / 64, wide = (N + 63) / 64;
-        const bool narrow = wide * zb < 192;
-        const int tiles = narrow ? (N + 31) / 32 : wide;
-        if (tiles * zb >= 32 && tiles * zb <= 512 && zb <= 65535) {
+      // Few enough workgroups to be on the chip at once (the output projection of a short prompt is 16 tiles of 128 x 128
+      // for 128 rows and 2048 columns, whatever is idle): the kernel for up to 64 rows, a workgroup per block of 64 rows,
+      // 64 or 32 columns and segment of K, all blocks in one launch.
+      if ((size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        int tiles, zb;
+        bool narrow;
+        add_blocks_shape(M, N, K, tiles, narrow, zb);
+        const bool scratch_ok = S == 1 || (sp.scratch != nullptr && sp.counters != nullptr &&
+                                           scratch_floats >= (size_t)tiles * zb * S * 4096 && num_counters >= tiles * zb);
+        if (tiles && scratch_ok) {
           const MidNormArgs na{};
           const QkvRopeArgs no{};
-          if (narrow) return launch_mid<EPI, 4, false, true>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, 1, MidSplitArgs{}, zb);
-          return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, 1, MidSplitArgs{}, zb);
+          if (narrow) return launch_mid<EPI, 4, false, true>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp, zb);
+          return launch_mid<EPI, 4, false>(x, w, out, M, N, K, ldx, ldo, tiles, s, na, no, S, sp, zb);
         }
       }
       int tiles;
@@ -2178,6 +2197,15 @@ extern "C" int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_float
   int tiles = 0;
   bool narrow = false;
   const int S = K > 0 ? (K + GEMM_SEG - 1) / GEMM_SEG : 0;
+  if (M > 64 && N > 0 && S > 1) {                           // a few blocks of 64 rows at once: a cell a workgroup
+    int zb;
+    add_blocks_shape(M, N, K, tiles, narrow, zb);
+    if (tiles) {
+      *scratch_floats = (long long)ADD_BLOCKS_MAX_WGS * 4096;   // (the same for every shape: one buffer serves all)
+      *counters = ADD_BLOCKS_MAX_WGS;
+      return 0;
+    }
+  }
   const AddRoute route = M > 64 && N > 0 ? add_route(M, N, K, 4, tiles) : ADD_WHOLE;
   if (route == ADD_TILE_SPLIT || route == ADD_BIG_SPLIT) {      // a prompt portion: the segments' sums, whole
     *scratch_floats = (long long)S * M * N;

@@ -199,11 +199,13 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
     # once (no scratch).  The bits of the rows alone, 16 at a time, with and without scratch,
     # twice on the same scratch (full of NaN at first, larger than needed); ragged edges, a short last segment
     S = lambda K: (K + 2047) // 2048
-    for M, N, K, kind in [(65, 2048, 4096, "blocks"), (128, 1100, 2048 * 2 + 320, "blocks"), (100, 2048, 2048, "blocks"),
+    # ("at once": up to 512 workgroups of the 64-row kernel, a block of 64 rows, a tile of columns and a segment each, in
+    # one launch; their scratch is the same size whatever the shape)
+    for M, N, K, kind in [(65, 2048, 4096, "at once"), (128, 1100, 2048 * 2 + 320, "at once"), (100, 2048, 2048, None),
                           (129, 2048, 2048, None), (81, 2048, 4096 + 72, None), (640, 4096, 4096, None),
                           (2048, 4096, 4096, None),       # 128 x 256 tiles, the two segments joined in registers
-
-                          (65, 2048, 8192, "sums"), (145, 2048, 8192, "sums"), (300, 1000, 2 * 2048 + 192, "sums"),
+                          (65, 2048, 8192, "at once"), (145, 2048, 8192, "at once"), (300, 1000, 2 * 2048 + 192, "at once"),
+                          (256, 2048, 8192, "at once"), (320, 2048, 8192, "sums"),
                           (768, 2048, 8192, "sums"), (700, 3000, 4 * 2048 + 128, "sums"), (2048, 2048, 8192, "sums"),
                           (513, 8192, 4096, "sums")]:
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
@@ -221,8 +223,8 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
         floats, counters = ops.gemm_add_scratch(M, N, K)
         if kind == "sums":
             assert (floats, counters) == (S(K) * M * N, 1), (M, N, K)
-        elif kind == "blocks" and K > 2048:
-            assert floats > 0 and (floats, counters) == ops.gemm_add_scratch(64, N, K), (M, N, K)
+        elif kind == "at once":
+            assert (floats, counters) == (512 * 4096, 512), (M, N, K)
         else:
             assert (floats, counters) == (0, 0), (M, N, K)
         if floats:
