@@ -1612,7 +1612,7 @@ static int launch_qkv_rope_mid(const bf16_t* x, int ldx, const bf16_t* w_qkv, vo
     // a short prompt portion: blocks of 64 rows in one launch, while all of them fit the chip at once
     const int zb = (M + 63) / 64;
     if (wide_tiles * zb > 512) return -7;
-    if (2 * wide_tiles * zb <= 512 && wide_tiles < ROPE_NARROW_BELOW)
+    if (2 * wide_tiles * zb <= 256 && wide_tiles < ROPE_NARROW_BELOW)      // (half heads only while they leave compute units idle)
       return launch_mid<EPI_QKV_ROPE, 4, false, true>(x, w_qkv, q_out, M, N, K, ldx, ldo, 2 * wide_tiles, s, MidNormArgs{}, rp, 1,
                                                       MidSplitArgs{}, zb);
     return launch_mid<EPI_QKV_ROPE, 4, false>(x, w_qkv, q_out, M, N, K, ldx, ldo, wide_tiles, s, MidNormArgs{}, rp, 1, MidSplitArgs{}, zb);
