@@ -2263,20 +2263,18 @@ extern "C" int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, 
                                      int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                                      int write_cache, void* stream) {
   if (M <= 0) return 0;
-  if (head_dim != 64 && (M > 64 || head_dim % 64)) return -4;     // the tiled kernels' epilogue: heads of 64
-  if (K <= 0 || (K > GEMM_SEG && M > 64) || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
+  if (head_dim % 64) return -4;
+  if (K <= 0 || (K % 8) || (ldx % 8) || ldx < K || page_size <= 0) return -2;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_qkv)) & 15) return -3;
   if (page_size <= 0 || (page_size & (page_size - 1))) return -5;
   QkvRopeArgs rp{positions, row_seq, block_table, cos_table, sin_table, (bf16_t*)k_cache, (bf16_t*)v_cache,
                  heads, kv_heads, page_size, table_stride, write_cache, __builtin_ctz((unsigned)page_size), head_dim};
-  if (M <= 64) {
-    const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
-    return mid == -7 ? -2 : mid;
-  }
-  {
-    const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
-    if (mid != -7) return mid;
-  }
+  // up to 64 rows, or a few blocks of 64 rows at once: a workgroup per 32 or 16 rotary pairs of a head
+  const int mid = launch_qkv_rope_mid((const bf16_t*)x, ldx, (const bf16_t*)w_qkv, q_out, M, K, rp, (hipStream_t)stream);
+  if (mid != -7) return mid;
+  if (M <= 64) return -2;
+  if (head_dim != 64) return -4;                                   // the tiled kernels' epilogue: heads of 64 ...
+  if (K > GEMM_SEG) return -2;                                     // ... and one segment of K
   const int N = (heads + 2 * kv_heads) * 64;
   return launch_gemm_bf16<EPI_QKV_ROPE>((const bf16_t*)x, (const bf16_t*)w_qkv, q_out, M, N, K, ldx, heads * 64,
                                         (hipStream_t)stream, rp);

@@ -518,12 +518,16 @@ def attention_decode_scratch(num_tiles: int, heads: int, kv_heads: int, head_dim
 
 def qkv_rope_gemm_ok(rows: int, head_dim: int, inner: int, all_heads: int = 0) -> bool:
     """Whether the q|k|v product of normalised rows can take rotation and cache write into its
-    epilogue.  More than 64 rows: heads of 64 and one segment of K.  Up to 64 rows (a workgroup per 32 or 16
-    rotary pairs of a head): head sizes in multiples of 64, K in steps of 64, and enough heads (q, k and v
-    heads together) for 64 workgroups."""
+    epilogue.  Up to 64 rows (a workgroup per 32 or 16 rotary pairs of a head), or a few blocks of 64 rows whose
+    workgroups are 512 at most: head sizes in multiples of 64, K in steps of 64, and enough heads (q, k and v
+    heads together) for 64 workgroups.  More rows: heads of 64 and one segment of K."""
+    tiles = all_heads * (head_dim // 64)
+    small = head_dim % 64 == 0 and inner % 64 == 0 and tiles >= 64
     if rows > 64:
-        return head_dim == 64 and inner <= 2048 and inner % 8 == 0
-    return head_dim % 64 == 0 and inner % 64 == 0 and all_heads * (head_dim // 64) >= 64
+        # (a few blocks of 64 rows at once, while their workgroups fit the chip together: any head size the small kernel takes)
+        at_once = small and tiles * ((rows + 63) // 64) <= 512
+        return at_once or (head_dim == 64 and inner <= 2048 and inner % 8 == 0)
+    return small
 
 
 def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,

@@ -888,6 +888,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
                                    (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16),   # up to 64 rows, half a head a workgroup
                                    (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32),   # a head a workgroup
                                    (40, 12, 128, 130, 16), (72, 12, 192, 300, 16), (64, 16, 2048, 190, 32),   # blocks of 64 rows in one launch
+                                   (32, 8, 4096, 130, 16, 128), (24, 4, 128, 200, 16, 128), (40, 12, 4160, 200, 16),   # ... with larger heads, several segments of K
                                    (40, 12, 4160, 16, 16),                                 # several segments of K
                                    (32, 8, 4096, 8, 16, 128), (24, 4, 128, 40, 8, 128), (100, 14, 64, 12, 16, 128),
                                    (16, 8, 2112, 20, 16, 256)]:                            # larger heads, up to 64 rows
@@ -921,7 +922,8 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
         assert torch.equal(outs[0][0][live], outs[1][0][live]), (heads, kvh, K, M)
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), (heads, kvh, K, M)
     assert not ops.qkv_rope_gemm_ok(64, 64, 256, 63) and not ops.qkv_rope_gemm_ok(200, 128, 256, 96)
-    assert not ops.qkv_rope_gemm_ok(64, 64, 96, 96) and not ops.qkv_rope_gemm_ok(8, 96, 128, 200) and not ops.qkv_rope_gemm_ok(200, 64, 4096, 96)
+    assert not ops.qkv_rope_gemm_ok(64, 64, 96, 96) and not ops.qkv_rope_gemm_ok(8, 96, 128, 200) and not ops.qkv_rope_gemm_ok(700, 64, 4096, 96)
+    assert ops.qkv_rope_gemm_ok(200, 64, 4096, 96) and ops.qkv_rope_gemm_ok(320, 128, 4096, 48) and not ops.qkv_rope_gemm_ok(384, 128, 4096, 48)
 
 
 def test_decode_attention_beyond_one_pass_of_partials(gpu):
