@@ -1355,6 +1355,22 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
   }
+  // A residual add without a meeting of segments: the outputs' old values are asked for before the ring (older than its
+  // loads, so the loop's waits cover them); asked for at the end they were one more trip to memory.
+  constexpr bool OLD_FIRST = EPI == EPI_ADD_F32 && !NORM;
+  float old_out[OLD_FIRST ? NI : 1][4];
+  if constexpr (OLD_FIRST) {
+    const int n = n0 + 16 * strip + r;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = 16 * (a_block0 + i) + 4 * g + q;
+        old_out[i][q] = (gridDim.y == 1 && computing && m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;
+      }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
   unsigned char* rows_lds = mid_lds + S::RING;
   if constexpr (NORM) {
     // the rows to normalise are asked for before the ring (loads complete in the order they are issued: the
@@ -1541,7 +1557,9 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int m = 16 * (a_block0 + i) + 4 * g + q;
-        if (m < M) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
+        if (m >= M) continue;
+        if constexpr (OLD_FIRST) ((float*)out)[(size_t)m * ldo + n] = old_out[i][q] + acc[i][0][q];
+        else epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
       }
   }
 }
@@ -1718,6 +1736,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
   }
   unsigned char* ring = stream_lds + wave * SH::RING;
   float* red = reinterpret_cast<float*>(stream_lds + nwaves * SH::RING);
+  // A residual add: the wave that stores asks for its outputs' old values before anything else (loads older than
+  // the ring's, so every wait below covers them); asked for at the end they were one more trip to memory.
+  float old_out[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (EPI == EPI_ADD_F32) {
+    if (wave == 0 && n_ok) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = 4 * g + q;
+        if (m < M) old_out[q] = ((const float*)out)[(size_t)m * ldo + n0 + c];
+      }
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int s = wave; s < S; s += nwaves) {
     const int k_begin = s * GEMM_SEG;
@@ -1756,7 +1788,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
       float y = red[q * 64 + lane];
       if constexpr (EPI == EPI_ADD_F32) {            // the chain of additions starts at the residual
         const int m = 4 * g + q;
-        if (n_ok && m < M) y = ((const float*)out)[(size_t)m * ldo + n0 + c] + y;
+        if (n_ok && m < M) y = old_out[q] + y;
       }
       for (int s = 1; s < S; ++s) y += red[(s * 4 + q) * 64 + lane];
       acc[q] = y;
@@ -1767,8 +1799,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
   for (int q = 0; q < 4; ++q) {
     const int m = 4 * g + q;
     if (m >= M) continue;
-    if (EPI == EPI_ADD_F32 && S > 1) ((float*)out)[(size_t)m * ldo + n0 + c] = acc[q];   // the residual is in already
-    else epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+    if constexpr (EPI == EPI_ADD_F32) {
+      // (several segments: the residual is in already; one: old + sum, the addition of the store that reads)
+      ((float*)out)[(size_t)m * ldo + n0 + c] = S > 1 ? acc[q] : old_out[q] + acc[q];
+    } else {
+      epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+    }
   }
 }
 
@@ -1829,6 +1865,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __re
   for (int t = 0; t < 2; ++t) voff_x[t] = ((8 * t + lrow) * ldx + 8 * (lslot ^ ((8 * t + lrow) >> 1))) * 2;
   const int voff_w = (lrow * K + 8 * (lslot ^ (lrow >> 1))) * 2;
   const int steps = K / 64;
+  // A residual add: the wave that stores asks for its outputs' old values before anything else (older than its loads
+  // of the steps, so every wait below covers them); asked for at the end they were one more trip to memory.
+  float old_out[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (EPI == EPI_ADD_F32) {
+    if (wave == 0 && n_ok) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = 4 * g + q;
+        if (m < M) old_out[q] = ((const float*)out)[(size_t)m * ldo + n0 + c];
+      }
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // eight steps a wave, whatever K: those past K are asked for outside the descriptors (no traffic, zeros), so
   // that the counts below are the same for every wave
 #pragma unroll
@@ -1885,7 +1935,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __re
   for (int q = 0; q < 4; ++q) {
     const int m = 4 * g + q;
     if (m >= M) continue;
-    epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+    if constexpr (EPI == EPI_ADD_F32) ((float*)out)[(size_t)m * ldo + n0 + c] = old_out[q] + acc[q];
+    else epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
   }
 }
 
