@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -60,6 +60,8 @@ def main() -> int:
                     help="the layer sizes of the headline run (llama3_8b: for profiles of that shape; implies --no-points)")
     ap.add_argument("--trace-only", action="store_true",
                     help="run nothing but the 128-request shared-prefix trace at Llama-3-8B's sizes and print its figures (for profiles)")
+    ap.add_argument("--decode-phases", action="store_true",
+                    help="the headline decode with EngineConfig.decode_phases (its products as phases of a few launches; for profiles)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -94,7 +96,7 @@ def main() -> int:
         print(f"bench.py: --prefill-tokens {args.prefill_tokens} is outside 1..{PREFILL_TOKENS}")
         return 2
     prefill = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype], args.prefill_tokens)
-    head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup)
+    head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup, decode_phases=args.decode_phases)
     points, point_rooflines = {}, {}
     extra = {}
     if not args.no_points:

@@ -43,6 +43,9 @@ class EngineConfig:
     max_model_len: int = 0           # 0: the model's max_position_embeddings
     use_graphs: bool = True          # replay pure-decode steps from captured HIP graphs
     run_ahead: bool = True           # launch the next pure-decode step before the last one's tokens are read back
+    decode_phases: bool = False      # captured decode steps of up to 16 rows run their products as phases of a few
+                                     # launches that wait for each other inside the kernel (ops.chain): the same
+                                     # bits; on MI355X some 5 % slower than a launch each, so off
     fault: int = 0                   # a test-only bug (``Fault``) for the simulator to catch; 0: none
 
     def validate(self) -> None:

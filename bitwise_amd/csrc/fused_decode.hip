@@ -37,6 +37,8 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
                          int table_stride, const float* cos_table, const float* sin_table, void* k_cache, void* v_cache, int M,
                          int heads, int kv_heads, int head_dim, int K, int page_size, int write_cache, void* stream);
 
+int bw_chain_flush_open(void* stream);
+
 enum { DEPI_F32 = 0, DEPI_BF16 = 1, DEPI_ADD_F32 = 2, DEPI_SWIGLU_BF16 = 3, DEPI_ROPE_KV = 4 };
 
 // (DEC_SEG, the LDS layout of the rows and the rings, and what the launchers admit: layout.h)
@@ -306,6 +308,7 @@ static int launch_decode_gemm(const DecodeGemmArgs& a, int waves, int blocks, hi
       return (int)hipGetLastError();
     raised = true;
   }
+  (void)bw_chain_flush_open((void*)s);              // phases that wait in an open chain go first
   hipLaunchKernelGGL((decode_gemm_kernel<EPI, ST>), dim3(blocks), dim3(64 * waves), lds, s, a);
   return BW_LAUNCH_CHECK();
 }

@@ -64,13 +64,90 @@ struct QkvRopeArgs {
   int head_dim = 64;           // (the kernels for up to 64 rows take multiples of 64; the tiled ones 64)
 };
 
-template <int EPI>
-__device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o, float v, float u) {
-  if constexpr (EPI == EPI_F32) ((float*)out)[o] = v;
-  else if constexpr (EPI == EPI_BF16) ((bf16_t*)out)[o] = f32_to_bf16(v);
-  else if constexpr (EPI == EPI_ADD_F32) ((float*)out)[o] += v;
-  else if constexpr (EPI == EPI_SWIGLU_BF16) ((bf16_t*)out)[o] = f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * u);
+// ------------------------------------------------------------------------------ phases of one launch
+//
+// A decode step is a row of small kernels, each of which has to wait for the one before it, and the end of one
+// kernel and the start of the next cost as much as many of them take to stream their weights.  The kernels for up
+// to 16 rows can therefore also run as phases of ONE launch: the workgroups of phase 0 come first in block order, then
+// those of phase 1, and so on.  Workgroups are handed to the compute units in block order, so when a workgroup runs
+// every workgroup of the phases before it is running or done; it asks for its weights at once (they depend on
+// nothing), then waits until the phase before it has counted all of its workgroups in (a flag that the last of them
+// sets; the wait is bounded: a wave that gives up sets a bit of an error word and goes on, nothing hangs), and only
+// then reads what that phase wrote.  What one phase writes and a later one reads travels with stores and loads
+// of device scope: the dies' L2s are not coherent with each other, a plain load could hit a stale line.  The
+// arithmetic of a phase is the statements of its kernel: the same bits.
+struct ChainCtx {
+  int bx, by, bz, gx, gy, gz;      // the workgroup's place in its phase's grid, and that grid
+  int waves;                       // waves of a workgroup of this phase
+  const int* wait_flag;            // null: this phase waits for nothing
+  int* err;                        // a word that gets bit err_bit when a wait gives up
+  int err_bit, spin_limit;
+};
+
+__device__ __forceinline__ ChainCtx launch_ctx() {
+  return ChainCtx{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, (int)gridDim.x, (int)gridDim.y, (int)gridDim.z,
+                  (int)(blockDim.x >> 6), nullptr, nullptr, 0, 0};
 }
+
+// The workgroup waits for the phase before its own (every wave of the workgroup calls this).
+template <bool CH>
+__device__ __forceinline__ void chain_wait(const ChainCtx& cc) {
+  if constexpr (CH) {
+    if (cc.wait_flag == nullptr) return;
+    if (threadIdx.x == 0) {
+      int spins = 0;
+      while (__hip_atomic_load(cc.wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+        if (++spins > cc.spin_limit) {
+          atomicOr(cc.err, 1 << cc.err_bit);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    __syncthreads();
+    asm volatile("" ::: "memory");
+  }
+}
+
+// Loads and stores of what another phase of the same launch wrote or will read (DEV), else plain ones.
+template <bool DEV>
+__device__ __forceinline__ float ld_f32(const float* p) {
+  if constexpr (DEV) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *p;
+}
+template <bool DEV>
+__device__ __forceinline__ void st_f32(float* p, float v) {
+  if constexpr (DEV) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+template <bool DEV>
+__device__ __forceinline__ void st_bf16(bf16_t* p, bf16_t v) {
+  if constexpr (DEV) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+
+template <int EPI, bool DEV = false>
+__device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o, float v, float u) {
+  if constexpr (EPI == EPI_F32) st_f32<DEV>((float*)out + o, v);
+  else if constexpr (EPI == EPI_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v));
+  else if constexpr (EPI == EPI_ADD_F32) st_f32<DEV>((float*)out + o, ld_f32<DEV>((const float*)out + o) + v);
+  else if constexpr (EPI == EPI_SWIGLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * u));
+}
+
+// (host) The phases asked for while a chain is open wait in a list and leave as one launch (further down).
+struct MidCall;
+struct RowsCall;
+static bool chain_is_open();
+static int chain_flush(hipStream_t s);
+static int chain_record_mid(int kind, const MidCall& c, int wgs, int lds_bytes, hipStream_t s);
+static int chain_record_rows(int kind, const RowsCall& c, int wgs, int waves, int lds_bytes, hipStream_t s);
+
+// Every other launch of this file: what waits in an open chain goes first.
+#define BW_LAUNCH(kernel, grid, block, lds, stream, ...)                \
+  do {                                                                  \
+    if (chain_is_open()) (void)chain_flush(stream);                     \
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);  \
+  } while (0)
 
 // ------------------------------------------------------------------------------ skinny
 
@@ -1135,7 +1212,7 @@ static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, in
                               T256_STAGES * T256_STAGE);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
+  BW_LAUNCH((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
                      ldo, mt, nt);
   return BW_LAUNCH_CHECK();
 }
@@ -1187,6 +1264,42 @@ struct MidNormArgs {
   int row_step;          // bytes of LDS a step of 64 along K of the normalised rows takes: 2048 (16 rows), or 1024
                          // (8 rows: rows of up to two segments of K, which are normalised a wave a row)
 };
+
+// What a phase of a chain is asked with: the operands of bw_norm_gemm_mid / bw_norm_qkv_rope_mid, or of the kernels for
+// up to 16 rows and few columns.
+struct MidCall {
+  const bf16_t* w;
+  void* out;
+  int M, N, K, ldo;
+  MidNormArgs na;
+  QkvRopeArgs rp;
+};
+struct RowsCall {
+  const bf16_t* x;
+  const bf16_t* w;
+  void* out;
+  int M, N, K, ldx, ldo, S;
+};
+enum ChainKind {
+  CK_QKV_NARROW, CK_QKV_WIDE, CK_GLU, CK_F32, CK_BURST_ADD, CK_STREAM_ADD_8_8, CK_STREAM_ADD_8_16, CK_STREAM_ADD_16_8,
+  CK_STREAM_ADD_16_16
+};
+// Which phase a variant of the kernel for up to 64 rows is; -1: it does not run as a phase.
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
+constexpr int mid_chain_kind() {
+  if (!NORM || !EIGHT || NRB != 1) return -1;
+  if (EPI == EPI_QKV_ROPE) return NARROW ? CK_QKV_NARROW : CK_QKV_WIDE;
+  if (NARROW) return -1;
+  if (EPI == EPI_SWIGLU_BF16) return CK_GLU;
+  if (EPI == EPI_F32) return CK_F32;
+  return -1;
+}
+template <int EPI, int CW, int XR>
+constexpr int stream_chain_kind() {
+  if (EPI != EPI_ADD_F32) return -1;
+  if (CW == 8) return XR == 8 ? CK_STREAM_ADD_8_8 : CK_STREAM_ADD_8_16;
+  return XR == 8 ? CK_STREAM_ADD_16_8 : CK_STREAM_ADD_16_16;
+}
 
 // Where a wave's loads of a stage go and come from.  A load is 8 rows of one step of 64 along K (1 KB): of x, block
 // ``id % (2 NRB)`` of step ``id / (2 NRB)`` of the stage for the wave's id-th load; of W likewise (SwiGLU with eight
@@ -1245,18 +1358,52 @@ __device__ __forceinline__ void mid_norm_rows(const MidNormArgs& na, int M, int 
   });
 }
 
-template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
-__global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW)) void gemm_bf16_mid_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-    MidNormArgs na, QkvRopeArgs rp, MidSplitArgs sp) {
+// The same for a workgroup that is a phase of a launch of several: the rows were written earlier in this launch,
+// maybe on another die, so they are loaded at device scope (through a descriptor over all rows), after the ring's
+// first stages and after the wait for the phase that wrote them.  The statements that follow the loads are the same.
+template <int RB, int NV, int NW>
+__device__ __forceinline__ void mid_norm_rows_dev(const MidNormArgs& na, int M, int K, int wave, int lane, unsigned char* rows_lds) {
+  const int nvec = K >> 2;
+  NormRows<RB, NV> nr;
+  const f32x4* nrows[RB];
+  int row_off[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int m = mid_norm_row_of(wave, i, NW);
+    nrows[i] = m < M ? reinterpret_cast<const f32x4*>(na.x32 + (size_t)m * na.ldx32) : nullptr;
+    row_off[i] = (m < M ? m : mid_norm_row_of(wave, 0, NW)) * na.ldx32 * 4;
+  }
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)na.x32, 0, (int)((((size_t)M - 1) * na.ldx32 + K) * 4), 0x00020000);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = norm_vec_index(j, lane, nvec);
+    nr.w[j] = load_norm_w_raw(na.norm_w, na.norm_w_is_bf16, c);
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+      nr.v[i][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, row_off[i] + 16 * c, 0, 16));
+  }
+  unsigned char* rl = rows_lds;
+  const int row_step = na.row_step;
+  norm_rows_finish<RB>(nr, nrows, na.norm_w_is_bf16, nvec, K, na.eps, lane, [=](int i, int c, u32x2 pk) {
+    const int m = mid_norm_row_of(wave, i, NW);
+    *reinterpret_cast<u32x2*>(rl + mid_norm_store_offset(c, m, row_step)) = pk;
+  });
+}
+
+// CH: the workgroup is one of a phase of a launch of several (ChainCtx): the ring's first stages are asked for before
+// the wait for the phase before, the rows to normalise after it, and rows and outputs travel at device scope.
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT, bool CH>
+__device__ __forceinline__ void mid_body(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
+                                         int K, int ldx, int ldo, MidNormArgs na, QkvRopeArgs rp, MidSplitArgs sp, const ChainCtx& cc) {
+  static_assert(!CH || NORM, "as a phase: the variants that normalise their rows");
   using S = MidShape<EPI, NRB, NORM, NARROW, EIGHT>;
   constexpr bool GLU = S::GLU;
   constexpr int COLS = S::COLS, NI = S::NI, NJ = S::NJ, THREADS = 64 * S::NW;
   if constexpr (!NORM) {
-    // gridDim.z > 1: a prompt portion of a few blocks of 16 * NRB rows in one launch, workgroup (tile, segment, z) the
+    // cc.gz > 1: a prompt portion of a few blocks of 16 * NRB rows in one launch, workgroup (tile, segment, z) the
     // rows of block z (a residual add's segments meet in scratch cells of their own for every block and tile)
-    if (gridDim.z > 1) {
-      const int first = (int)blockIdx.z * 16 * NRB;
+    if (cc.gz > 1) {
+      const int first = cc.bz * 16 * NRB;
       x += (size_t)first * ldx;
       if constexpr (EPI == EPI_QKV_ROPE) {
         rp.positions += first;
@@ -1280,9 +1427,9 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
   constexpr int PAIRS = RN ? 16 : 32, PSH = RN ? 4 : 5;              // rotary pairs of a row in this tile
   const int hd = ROPE ? rp.head_dim : 64, half = hd >> 1;
   const int tiles_per_head = half / PAIRS;
-  const int head = ROPE ? (int)blockIdx.x / tiles_per_head : 0;
-  const int pair0 = ROPE ? PAIRS * ((int)blockIdx.x % tiles_per_head) : 0;   // the tile's first pair within the head
-  const int n0 = ROPE ? head * hd : blockIdx.x * COLS;
+  const int head = ROPE ? cc.bx / tiles_per_head : 0;
+  const int pair0 = ROPE ? PAIRS * (cc.bx % tiles_per_head) : 0;   // the tile's first pair within the head
+  const int n0 = ROPE ? head * hd : cc.bx * COLS;
   const int b_rows = ROPE ? hd : min(COLS, N - n0);
   const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)x, 0, NORM ? 0 : (int)((((size_t)M - 1) * ldx + K) * 2), 0x00020000);
@@ -1319,10 +1466,10 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     ld.voff_b[t] = (w_row * K + 8 * chunk + 64 * sub) * 2;
     ld.dst_b[t] = mid_b_dst<S>(sub, blk);
   }
-  // gridDim.y > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
+  // cc.gy > 1: this workgroup works on one segment of K (the residual add's split, below); else on all of K,
   // segment after segment, each segment's sums joined to those before it when it ends
-  const int k_base = blockIdx.y * GEMM_SEG;
-  const int steps = (gridDim.y > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64) / S::SUB;   // stages
+  const int k_base = cc.by * GEMM_SEG;
+  const int steps = (cc.gy > 1 ? ((K - k_base) < GEMM_SEG ? K - k_base : GEMM_SEG) / 64 : K / 64) / S::SUB;   // stages
   f32x4 acc[NI][NJ], tot[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -1366,13 +1513,26 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int m = 16 * (a_block0 + i) + 4 * g + q;
-        old_out[i][q] = (gridDim.y == 1 && computing && m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;
+        old_out[i][q] = (cc.gy == 1 && computing && m < M && n < N) ? ((const float*)out)[(size_t)m * ldo + n] : 0.0f;
       }
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
   }
   unsigned char* rows_lds = mid_lds + S::RING;
-  if constexpr (NORM) {
+  if constexpr (NORM && CH) {
+    // as a phase: the weights depend on nothing, the rows on the phase before
+#pragma unroll
+    for (int st = 0; st < S::STAGES - 1; ++st) mid_issue<EPI, NRB, NORM, NARROW, EIGHT>(mid_lds, rs_a, rs_b, ld, st, steps, k_base);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    chain_wait<CH>(cc);
+    if (wave < M) {
+      const int rows_a_wave = mid_norm_rows_a_wave(M, S::NW);
+      if (mid_norm_vectors_a_lane(K) == 16) mid_norm_rows_dev<1, 16, S::NW>(na, M, K, wave, lane, rows_lds);
+      else if (rows_a_wave == 1) mid_norm_rows_dev<1, 8, S::NW>(na, M, K, wave, lane, rows_lds);
+      else mid_norm_rows_dev<2, 8, S::NW>(na, M, K, wave, lane, rows_lds);
+    }
+  } else if constexpr (NORM) {
     // the rows to normalise are asked for before the ring (loads complete in the order they are issued: the
     // wait for the rows must not be a wait for weights); wave w takes rows w, w + 4, ...: as many at a time as
     // there are (a slot without a row would fetch a row for nothing)
@@ -1444,7 +1604,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         }
         if constexpr (!NORM || EIGHT) {
           const int kn = (step * S::SUB + sub + 1) * 64;
-          if (kn % GEMM_SEG == 0 && kn < K && gridDim.y == 1) {          // a segment ends before the last: left to right
+          if (kn % GEMM_SEG == 0 && kn < K && cc.gy == 1) {          // a segment ends before the last: left to right
 #pragma unroll
             for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -1459,7 +1619,7 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
     asm volatile("" ::: "memory");
   }
   if constexpr (!NORM || EIGHT) {
-    if (K > GEMM_SEG && gridDim.y == 1) {                               // the last segment joins the others
+    if (K > GEMM_SEG && cc.gy == 1) {                               // the last segment joins the others
 #pragma unroll
       for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -1496,20 +1656,20 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         else if (rp.write_cache)
           dst = rp.k_cache + (((size_t)r_page[j] * rp.kv_heads + (head - rp.heads)) * rp.page_size + (pos & (rp.page_size - 1))) * hd;
         if (dst != nullptr) {
-          dst[i] = f32_to_bf16(o1);
-          dst[i + half] = f32_to_bf16(o2);
+          st_bf16<CH>(dst + i, f32_to_bf16(o1));
+          st_bf16<CH>(dst + i + half, f32_to_bf16(o2));
         }
       } else if (rp.write_cache) {
         bf16_t* dst = rp.v_cache + ((size_t)r_page[j] * rp.kv_heads + (head - rp.heads - rp.kv_heads)) * hd * rp.page_size +
                       (pos & (rp.page_size - 1));
-        dst[(size_t)i * rp.page_size] = f32_to_bf16(x1);
-        dst[(size_t)(i + half) * rp.page_size] = f32_to_bf16(x2);
+        st_bf16<CH>(dst + (size_t)i * rp.page_size, f32_to_bf16(x1));
+        st_bf16<CH>(dst + (size_t)(i + half) * rp.page_size, f32_to_bf16(x2));
       }
     }
   } else {
     const int n = n0 + 16 * strip + r;
     if constexpr (EPI == EPI_ADD_F32 && !NORM) {
-      const int nseg = gridDim.y;
+      const int nseg = cc.gy;
       if (nseg > 1) {
         // Every segment's workgroup leaves its sums in device scratch (stores of device scope: they write through,
         // and each wave waits below until its own are acknowledged, so they are in memory, not in this die's L2,
@@ -1518,13 +1678,13 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         // device-scope loads issued after the barrier behind the count.  The counter is back at zero when the
         // kernel ends.
         const int cell = S::NW * NI * 1024;                          // bytes of a workgroup's sums: [wave][i][lane] x 16
-        const int tile_id = (int)(blockIdx.z * gridDim.x + blockIdx.x);   // (block of rows, tile of columns)
+        const int tile_id = (int)(cc.bz * cc.gx + cc.bx);   // (block of rows, tile of columns)
         const __amdgpu_buffer_rsrc_t rs_s = __builtin_amdgcn_make_buffer_rsrc(
             (void*)((unsigned char*)sp.scratch + (size_t)tile_id * nseg * cell), 0, nseg * cell, 0x00020000);
         const int mine = (wave * NI) * 1024 + lane * 16;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][0]), rs_s, mine + i * 1024, (int)blockIdx.y * cell, 16);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][0]), rs_s, mine + i * 1024, cc.by * cell, 16);
         __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                   // this wave's stores have been acknowledged
         __syncthreads();                                             // also: every wave is done with the ring, whose first word is the flag now
         int* is_last = reinterpret_cast<int*>(mid_lds);
@@ -1559,10 +1719,18 @@ __global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW))
         const int m = 16 * (a_block0 + i) + 4 * g + q;
         if (m >= M) continue;
         if constexpr (OLD_FIRST) ((float*)out)[(size_t)m * ldo + n] = old_out[i][q] + acc[i][0][q];
-        else epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
+        else epilogue_store<EPI, CH>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][NJ - 1][q]);
       }
   }
 }
+
+template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
+__global__ __launch_bounds__((64 * MidShape<EPI, NRB, NORM, NARROW, EIGHT>::NW)) void gemm_bf16_mid_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+    MidNormArgs na, QkvRopeArgs rp, MidSplitArgs sp) {
+  mid_body<EPI, NRB, NORM, NARROW, EIGHT, false>(x, w, out, M, N, K, ldx, ldo, na, rp, sp, launch_ctx());
+}
+
 
 template <int EPI, int NRB, bool NORM, bool NARROW, bool EIGHT>
 static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int wgs, hipStream_t s,
@@ -1575,7 +1743,14 @@ static int launch_mid_waves(const bf16_t* x, const bf16_t* w, void* out, int M, 
     (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>), dim3(wgs, segments, row_blocks), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
+  if (chain_is_open()) {
+    constexpr int kind = mid_chain_kind<EPI, NRB, NORM, NARROW, EIGHT>();
+    if constexpr (kind >= 0) {
+      if (segments == 1 && row_blocks == 1 && (size_t)M * na.ldx32 * 4 < ((size_t)1 << 31))
+        return chain_record_mid(kind, MidCall{w, out, M, N, K, ldo, na, rp}, wgs, lds_bytes, s);
+    }
+  }
+  BW_LAUNCH((gemm_bf16_mid_kernel<EPI, NRB, NORM, NARROW, EIGHT>), dim3(wgs, segments, row_blocks), dim3(64 * S::NW), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, na, rp, sp);
   return BW_LAUNCH_CHECK();
 }
 
@@ -1687,7 +1862,9 @@ struct StreamShape {
 
 // A wave's loads of one stage of its ring (a device function rather than a lambda in the kernel: the
 // host pass drops, without a word, kernel templates whose lambdas capture arrays of dependent size).
-template <int CW, int XR>
+// DO_X, DO_W: which of the stage's loads (a phase of a launch of several asks for the weights of its first stages
+// before the rows); DEV: x at device scope.
+template <int CW, int XR, bool DO_X = true, bool DO_W = true, bool DEV = false>
 __device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
                                              const int* voff_x, const int* voff_w, int step, int steps, int k_begin) {
   using SH = StreamShape<CW, XR>;
@@ -1695,24 +1872,31 @@ __device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffe
   unsigned char* dst = ring + (step % SH::STAGES) * SH::STAGE;
   const bool real = step < steps;                                  // scalar; past the segment: outside the descriptors
   const int soff = (k_begin + step * 64) * 2;
+  if constexpr (DO_X) {
 #pragma unroll
-  for (int t = 0; t < SH::A_LOADS; ++t)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, soff, 0, 0);
+    for (int t = 0; t < SH::A_LOADS; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, soff, 0, DEV ? 16 : 0);
+  }
+  if constexpr (DO_W) {
 #pragma unroll
-  for (int t = 0; t < SH::B_LOADS; ++t)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + SH::A_BYTES + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0, soff, 0, 0);
+    for (int t = 0; t < SH::B_LOADS; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + SH::A_BYTES + t * 1024), 16, real ? voff_w[t] : 0x7ffffff0, soff, 0, 0);
+  }
 }
 
-template <int EPI, int CW, int XR = 16>
-__global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                               void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                               int S) {
+// CH: as a phase of a launch of several (ChainCtx): x and the outputs' old values were written by the phase before, so a
+// wave asks for the weights of its first segment's first stages, waits, and asks for their rows of x then (loads
+// complete in the order they are issued: until the ring has turned once the wait for a stage lets fewer loads stay in
+// flight); x, old values and outputs travel at device scope.
+template <int EPI, int CW, int XR, bool CH>
+__device__ __forceinline__ void stream_body(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
+                                            int K, int ldx, int ldo, int S, const ChainCtx& cc) {
   using SH = StreamShape<CW, XR>;
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];   // [waves][ring], then [S][4][64] floats when S > 1
-  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = cc.waves;
   const int r = lane & 15, g = lane >> 4;
   const int c = r % CW;
-  const int n0 = blockIdx.x * CW;
+  const int n0 = cc.bx * CW;
   const bool n_ok = r < CW && n0 + c < N;
   const int w_rows = min(CW, N - n0);
   const __amdgpu_buffer_rsrc_t rs_w =
@@ -1739,26 +1923,44 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
   // A residual add: the wave that stores asks for its outputs' old values before anything else (loads older than
   // the ring's, so every wait below covers them); asked for at the end they were one more trip to memory.
   float old_out[4] = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (EPI == EPI_ADD_F32) {
-    if (wave == 0 && n_ok) {
+  auto ask_old = [&]() {
+    if constexpr (EPI == EPI_ADD_F32) {
+      if (wave == 0 && n_ok) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int m = 4 * g + q;
-        if (m < M) old_out[q] = ((const float*)out)[(size_t)m * ldo + n0 + c];
+        for (int q = 0; q < 4; ++q) {
+          const int m = 4 * g + q;
+          if (m < M) old_out[q] = ld_f32<CH>((const float*)out + (size_t)m * ldo + n0 + c);
+        }
       }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
     }
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  }
+  };
+  if constexpr (!CH) ask_old();
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int s = wave; s < S; s += nwaves) {
     const int k_begin = s * GEMM_SEG;
     const int steps = ((K - k_begin) < GEMM_SEG ? K - k_begin : GEMM_SEG) / 64;
     acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const bool first_turn = CH && s == wave;                       // (scalar) the segment whose x had to wait
+    if (first_turn) {
 #pragma unroll
-    for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, false, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      chain_wait<CH>(cc);
+      ask_old();
+#pragma unroll
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, false, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+    } else {
+#pragma unroll
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+    }
     for (int step = 0; step < steps; ++step) {
-      __builtin_amdgcn_s_waitcnt(0x4f78);                          // vmcnt(24): the stage at hand has landed
+      // the stage at hand has landed when all but the loads of the stages after it have: 24, or, while x of the
+      // first stages was asked for behind their weights, what is left of x (B_LOADS fewer a stage) and what came since
+      if (first_turn && step < SH::STAGES - 2) __builtin_amdgcn_s_waitcnt(vmcnt_only(SH::A_LOADS * (SH::STAGES - 2)));
+      else __builtin_amdgcn_s_waitcnt(0x4f78);                     // vmcnt(24)
       asm volatile("" ::: "memory");
       const unsigned char* stage = ring + (step % SH::STAGES) * SH::STAGE;
       u32x4 fa[2], fb[2];
@@ -1772,7 +1974,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk]), acc, 0, 0, 0);
       // the reads above are done (their values were used) before the stage is asked for again
       asm volatile("" ::: "memory");
-      stream_issue<CW, XR>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
+      stream_issue<CW, XR, true, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);                            // the padding loads too, before the ring is reused
     if (S > 1) {
@@ -1801,11 +2003,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __r
     if (m >= M) continue;
     if constexpr (EPI == EPI_ADD_F32) {
       // (several segments: the residual is in already; one: old + sum, the addition of the store that reads)
-      ((float*)out)[(size_t)m * ldo + n0 + c] = S > 1 ? acc[q] : old_out[q] + acc[q];
+      st_f32<CH>((float*)out + (size_t)m * ldo + n0 + c, S > 1 ? acc[q] : old_out[q] + acc[q]);
     } else {
-      epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+      epilogue_store<EPI, CH>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
     }
   }
+}
+
+template <int EPI, int CW, int XR = 16>
+__global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                               void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                               int S) {
+  stream_body<EPI, CW, XR, false>(x, w, out, M, N, K, ldx, ldo, S, launch_ctx());
 }
 
 template <int EPI, int CW, int XR>
@@ -1819,7 +2028,11 @@ static int launch_stream_rows(const bf16_t* x, const bf16_t* w, void* out, int M
     (void)hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<EPI, CW, XR>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_stream_kernel<EPI, CW, XR>), dim3((N + CW - 1) / CW), dim3(64 * waves), lds_bytes, s, x, w, out, M, N,
+  if (chain_is_open()) {
+    constexpr int kind = stream_chain_kind<EPI, CW, XR>();
+    if constexpr (kind >= 0) return chain_record_rows(kind, RowsCall{x, w, out, M, N, K, ldx, ldo, S}, (N + CW - 1) / CW, waves, (int)lds_bytes, s);
+  }
+  BW_LAUNCH((gemm_bf16_stream_kernel<EPI, CW, XR>), dim3((N + CW - 1) / CW), dim3(64 * waves), lds_bytes, s, x, w, out, M, N,
                      K, ldx, ldo, S);
   return BW_LAUNCH_CHECK();
 }
@@ -1844,15 +2057,17 @@ static int launch_stream(const bf16_t* x, const bf16_t* w, void* out, int M, int
 #define BURST_STEPS 32
 #define BURST_STAGE 3072                                           // x: 16 rows of 128 bytes, then 8 rows of W
 
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                              void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+// CH: as a phase of a launch of several (ChainCtx): all the weights are asked for, then the wait for the phase before,
+// then the old values and x at device scope; a wave's q-th step is there when all but its last 2 * (7 - q) loads are.
+template <int EPI, bool CH>
+__device__ __forceinline__ void burst_body(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
+                                           int K, int ldx, int ldo, const ChainCtx& cc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char burst_lds[];   // [BURST_STEPS][BURST_STAGE]
   typedef __attribute__((address_space(3))) void* lds_ptr;
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int c = r & 7;
-  const int n0 = blockIdx.x * 8;
+  const int n0 = cc.bx * 8;
   const bool n_ok = r < 8 && n0 + c < N;
   const int w_rows = min(8, N - n0);
   const __amdgpu_buffer_rsrc_t rs_w =
@@ -1868,28 +2083,51 @@ __global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __re
   // A residual add: the wave that stores asks for its outputs' old values before anything else (older than its loads
   // of the steps, so every wait below covers them); asked for at the end they were one more trip to memory.
   float old_out[4] = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (EPI == EPI_ADD_F32) {
-    if (wave == 0 && n_ok) {
+  auto ask_old = [&]() {
+    if constexpr (EPI == EPI_ADD_F32) {
+      if (wave == 0 && n_ok) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int m = 4 * g + q;
-        if (m < M) old_out[q] = ((const float*)out)[(size_t)m * ldo + n0 + c];
+        for (int q = 0; q < 4; ++q) {
+          const int m = 4 * g + q;
+          if (m < M) old_out[q] = ld_f32<CH>((const float*)out + (size_t)m * ldo + n0 + c);
+        }
       }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // eight steps a wave, whatever K: those past K are asked for outside the descriptors (no traffic, zeros), so
+  // that the counts below are the same for every wave
+  if constexpr (CH) {
+#pragma unroll
+    for (int i = 0; i < BURST_STEPS / 4; ++i) {
+      const int st = wave + 4 * i;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(burst_lds + st * BURST_STAGE + 2048), 16, st < steps ? voff_w : 0x7ffffff0, st * 128, 0, 0);
     }
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-  }
-  // eight steps a wave, whatever K: those past K are asked for outside the descriptors (no traffic, zeros), so
-  // that the counts below are the same for every wave
+    chain_wait<CH>(cc);
+    ask_old();
 #pragma unroll
-  for (int i = 0; i < BURST_STEPS / 4; ++i) {
-    const int st = wave + 4 * i;
-    const bool real = st < steps;                                  // scalar
-    unsigned char* dst = burst_lds + st * BURST_STAGE;
+    for (int i = 0; i < BURST_STEPS / 4; ++i) {
+      const int st = wave + 4 * i;
+      const bool real = st < steps;                                // scalar
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, st * 128, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + 2048), 16, real ? voff_w : 0x7ffffff0, st * 128, 0, 0);
+      for (int t = 0; t < 2; ++t)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(burst_lds + st * BURST_STAGE + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, st * 128, 0, 16);
+    }
+  } else {
+    ask_old();
+#pragma unroll
+    for (int i = 0; i < BURST_STEPS / 4; ++i) {
+      const int st = wave + 4 * i;
+      const bool real = st < steps;                                  // scalar
+      unsigned char* dst = burst_lds + st * BURST_STAGE;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr)(dst + t * 1024), 16, real ? voff_x[t] : 0x7ffffff0, st * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(dst + 2048), 16, real ? voff_w : 0x7ffffff0, st * 128, 0, 0);
+    }
   }
   int off_x[2], off_w[2];
 #pragma unroll
@@ -1920,13 +2158,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __re
     asm volatile("" ::: "memory");                             \
     if (wave == 0) run_steps(Q);                               \
   }
-  BURST_ROUND(0, vmcnt_only(21))
-  BURST_ROUND(1, vmcnt_only(18))
-  BURST_ROUND(2, vmcnt_only(15))
-  BURST_ROUND(3, vmcnt_only(12))
-  BURST_ROUND(4, vmcnt_only(9))
-  BURST_ROUND(5, vmcnt_only(6))
-  BURST_ROUND(6, vmcnt_only(3))
+  BURST_ROUND(0, vmcnt_only(CH ? 14 : 21))
+  BURST_ROUND(1, vmcnt_only(CH ? 12 : 18))
+  BURST_ROUND(2, vmcnt_only(CH ? 10 : 15))
+  BURST_ROUND(3, vmcnt_only(CH ? 8 : 12))
+  BURST_ROUND(4, vmcnt_only(CH ? 6 : 9))
+  BURST_ROUND(5, vmcnt_only(CH ? 4 : 6))
+  BURST_ROUND(6, vmcnt_only(CH ? 2 : 3))
   BURST_ROUND(7, vmcnt_only(0))
 #undef BURST_ROUND
   __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                        // the padding loads too, before the wave ends
@@ -1935,9 +2173,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __re
   for (int q = 0; q < 4; ++q) {
     const int m = 4 * g + q;
     if (m >= M) continue;
-    if constexpr (EPI == EPI_ADD_F32) ((float*)out)[(size_t)m * ldo + n0 + c] = old_out[q] + acc[q];
-    else epilogue_store<EPI>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
+    if constexpr (EPI == EPI_ADD_F32) st_f32<CH>((float*)out + (size_t)m * ldo + n0 + c, old_out[q] + acc[q]);
+    else epilogue_store<EPI, CH>(out, (size_t)m * ldo + n0 + c, acc[q], acc[q]);
   }
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_burst_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              void* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+  burst_body<EPI, false>(x, w, out, M, N, K, ldx, ldo, launch_ctx());
 }
 
 template <int EPI>
@@ -1947,9 +2191,186 @@ static int launch_burst(const bf16_t* x, const bf16_t* w, void* out, int M, int 
     (void)hipFuncSetAttribute((const void*)gemm_bf16_burst_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     allowed = true;
   }
-  hipLaunchKernelGGL((gemm_bf16_burst_kernel<EPI>), dim3((N + 7) / 8), dim3(256), BURST_STEPS * BURST_STAGE, s, x, w, out, M, N, K,
+  if (chain_is_open()) {
+    if constexpr (EPI == EPI_ADD_F32) return chain_record_rows(CK_BURST_ADD, RowsCall{x, w, out, M, N, K, ldx, ldo, 1}, (N + 7) / 8, 4, BURST_STEPS * BURST_STAGE, s);
+  }
+  BW_LAUNCH((gemm_bf16_burst_kernel<EPI>), dim3((N + 7) / 8), dim3(256), BURST_STEPS * BURST_STAGE, s, x, w, out, M, N, K,
                      ldx, ldo);
   return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ several phases, one launch
+
+#define CHAIN_MAX_PHASES 6
+#define CHAIN_SYNC_WORDS 4096          // 32-bit words the caller brings, zero before the first launch: phase p counts its
+#define CHAIN_FLAGS_AT 2048            // workgroups in at word 64 p and raises its flag at word 2048 + 64 p
+#define CHAIN_LDS_BYTES (160 * 1024 - 256)
+
+struct ChainPhase {
+  int kind, first, gx, waves;          // which kernel's statements, the phase's first block, its workgroups and their waves
+  MidCall mid;
+  RowsCall rows;
+};
+struct ChainArgs {
+  int n, spin_limit;
+  int* sync;
+  int* err;
+  ChainPhase ph[CHAIN_MAX_PHASES];
+};
+
+// Workgroups in block order, phase after phase.  A workgroup runs its phase's statements (waves the phase has no use
+// for end at once), then counts itself in: every wave waits until its own device-scope stores are acknowledged, a
+// barrier, and the first thread adds one to the phase's counter.  The last one to arrive puts the counter back to
+// zero, takes down the flag its own phase waited for (every workgroup of the phase is past that wait) and raises the
+// flag the next phase waits for: after the launch every word is zero again.
+// (The statements are for the device pass only: they name types that the host pass does not know, and unlike those of
+// the other kernels they do not all hang on a template parameter.  CH is true.)
+template <bool CH>
+__global__ __launch_bounds__(512) void gemm_bf16_chain_kernel(const ChainArgs c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  int p = 0;
+#pragma unroll
+  for (int i = 1; i < CHAIN_MAX_PHASES; ++i)
+    if (i < c.n && (int)blockIdx.x >= c.ph[i].first) p = i;
+  const ChainPhase& P = c.ph[p];
+  if (wave_index() >= P.waves) return;
+  const ChainCtx cc{(int)blockIdx.x - P.first, 0, 0, P.gx, 1, 1, P.waves, p > 0 ? c.sync + CHAIN_FLAGS_AT + 64 * (p - 1) : nullptr,
+                    c.err, p, c.spin_limit};
+  const MidCall& m = P.mid;
+  const RowsCall& r = P.rows;
+  switch (P.kind) {
+    case CK_QKV_NARROW:
+      mid_body<EPI_QKV_ROPE, 1, true, true, true, CH>(nullptr, m.w, m.out, m.M, m.N, m.K, 0, m.ldo, m.na, m.rp, MidSplitArgs{}, cc);
+      break;
+    case CK_QKV_WIDE:
+      mid_body<EPI_QKV_ROPE, 1, true, false, true, CH>(nullptr, m.w, m.out, m.M, m.N, m.K, 0, m.ldo, m.na, m.rp, MidSplitArgs{}, cc);
+      break;
+    case CK_GLU:
+      mid_body<EPI_SWIGLU_BF16, 1, true, false, true, CH>(nullptr, m.w, m.out, m.M, m.N, m.K, 0, m.ldo, m.na, m.rp, MidSplitArgs{}, cc);
+      break;
+    case CK_F32:
+      mid_body<EPI_F32, 1, true, false, true, CH>(nullptr, m.w, m.out, m.M, m.N, m.K, 0, m.ldo, m.na, m.rp, MidSplitArgs{}, cc);
+      break;
+    case CK_BURST_ADD: burst_body<EPI_ADD_F32, CH>(r.x, r.w, r.out, r.M, r.N, r.K, r.ldx, r.ldo, cc); break;
+    case CK_STREAM_ADD_8_8: stream_body<EPI_ADD_F32, 8, 8, CH>(r.x, r.w, r.out, r.M, r.N, r.K, r.ldx, r.ldo, r.S, cc); break;
+    case CK_STREAM_ADD_8_16: stream_body<EPI_ADD_F32, 8, 16, CH>(r.x, r.w, r.out, r.M, r.N, r.K, r.ldx, r.ldo, r.S, cc); break;
+    case CK_STREAM_ADD_16_8: stream_body<EPI_ADD_F32, 16, 8, CH>(r.x, r.w, r.out, r.M, r.N, r.K, r.ldx, r.ldo, r.S, cc); break;
+    case CK_STREAM_ADD_16_16: stream_body<EPI_ADD_F32, 16, 16, CH>(r.x, r.w, r.out, r.M, r.N, r.K, r.ldx, r.ldo, r.S, cc); break;
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int blocks = (p + 1 < c.n ? c.ph[p + 1].first : (int)gridDim.x) - P.first;
+    int* counter = c.sync + 64 * p;
+    if (__hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == blocks - 1) {
+      __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (p > 0) __hip_atomic_store(c.sync + CHAIN_FLAGS_AT + 64 * (p - 1), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (p + 1 < c.n) __hip_atomic_store(c.sync + CHAIN_FLAGS_AT + 64 * p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+#endif
+}
+
+// (host) The chain that is open in this thread, if any: what bw_chain_begin was given, and the phases that wait.
+struct ChainState {
+  bool open = false;
+  int* sync = nullptr;
+  int* err = nullptr;
+  int spin_limit = 0;
+  int n = 0, blocks = 0, lds = 0;
+  hipStream_t stream = nullptr;
+  ChainPhase ph[CHAIN_MAX_PHASES];
+};
+static thread_local ChainState g_chain;
+
+static bool chain_is_open() { return g_chain.open; }
+
+static int chain_flush(hipStream_t s) {
+  ChainState& g = g_chain;
+  if (g.n == 0) return 0;
+  ChainArgs a;
+  a.n = g.n;
+  a.spin_limit = g.spin_limit;
+  a.sync = g.sync;
+  a.err = g.err;
+  for (int i = 0; i < g.n; ++i) a.ph[i] = g.ph[i];
+  for (int i = g.n; i < CHAIN_MAX_PHASES; ++i) a.ph[i] = ChainPhase{};
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_chain_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    allowed = true;
+  }
+  const int blocks = g.blocks, lds = g.lds;
+  hipStream_t stream = g.stream;
+  g.n = g.blocks = g.lds = 0;
+  (void)s;                                           // (the phases were asked for on g.stream; a caller on another stream has flushed)
+  hipLaunchKernelGGL(gemm_bf16_chain_kernel<true>, dim3(blocks), dim3(512), lds, stream, a);
+  return BW_LAUNCH_CHECK();
+}
+
+static int chain_append(const ChainPhase& ph, int wgs, int lds_bytes, hipStream_t s) {
+  ChainState& g = g_chain;
+  if (lds_bytes > CHAIN_LDS_BYTES || wgs <= 0) return -2;
+  if (g.n > 0 && (g.stream != s || g.n == CHAIN_MAX_PHASES)) {
+    const int rc = chain_flush(g.stream);
+    if (rc) return rc;
+  }
+  g.stream = s;
+  g.ph[g.n] = ph;
+  g.ph[g.n].first = g.blocks;
+  g.ph[g.n].gx = wgs;
+  g.blocks += wgs;
+  if (lds_bytes > g.lds) g.lds = lds_bytes;
+  ++g.n;
+  return 0;
+}
+
+static int chain_record_mid(int kind, const MidCall& c, int wgs, int lds_bytes, hipStream_t s) {
+  ChainPhase ph{};
+  ph.kind = kind;
+  ph.waves = 8;
+  ph.mid = c;
+  return chain_append(ph, wgs, lds_bytes, s);
+}
+
+static int chain_record_rows(int kind, const RowsCall& c, int wgs, int waves, int lds_bytes, hipStream_t s) {
+  if ((size_t)c.M * c.ldo * 4 >= ((size_t)1 << 31)) return -2;
+  ChainPhase ph{};
+  ph.kind = kind;
+  ph.waves = waves;
+  ph.rows = c;
+  return chain_append(ph, wgs, lds_bytes, s);
+}
+
+// From bw_chain_begin to bw_chain_end (in the calling thread) the products of up to 16 rows that can run as phases
+// (RMSNorm + product with SwiGLU, with a 32-bit store or with rotation and cache write; residual adds of few columns)
+// are not launched when they are asked for but wait, and leave as one launch when anything else is launched through this
+// library, at bw_chain_flush or at the end.  sync: CHAIN_SYNC_WORDS 32-bit words, zero before the first chain (every
+// launch leaves them zero; after an error word that is not zero the caller clears them).  err: a word that gets a bit
+// for every phase one of whose waits gave up after spin_limit looks.  Launches that do not come through this library
+// (another library's kernels on the same stream) must not be made while phases wait: they would overtake them.
+extern "C" int bw_chain_sync_words() { return CHAIN_SYNC_WORDS; }
+
+extern "C" int bw_chain_begin(void* sync, int sync_words, void* err, int spin_limit) {
+  if (g_chain.open || sync == nullptr || err == nullptr || sync_words < CHAIN_SYNC_WORDS || spin_limit < 0) return -2;
+  g_chain = ChainState{};
+  g_chain.open = true;
+  g_chain.sync = (int*)sync;
+  g_chain.err = (int*)err;
+  g_chain.spin_limit = spin_limit;
+  return 0;
+}
+
+extern "C" int bw_chain_flush(void* stream) { return g_chain.open ? chain_flush((hipStream_t)stream) : 0; }
+
+// (for the launches of this library's other source files)
+int bw_chain_flush_open(void* stream) { return bw_chain_flush(stream); }
+
+extern "C" int bw_chain_end(void* stream) {
+  if (!g_chain.open) return -2;
+  const int rc = chain_flush((hipStream_t)stream);
+  g_chain.open = false;
+  return rc;
 }
 
 // ------------------------------------------------------------------------------ launch
@@ -2106,9 +2527,9 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     if ((size_t)M * ldx * 2 >= ((size_t)1 << 31) || (size_t)16 * K * 2 >= ((size_t)1 << 31)) return -2;   // offsets within x, within a strip of W
 #define BW_SKINNY(WMV, DV, CWV)                                                                                    \
   if (K % 32)                                                                                                      \
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, true, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S); \
+    BW_LAUNCH((gemm_bf16_skinny_kernel<WMV, EPI, DV, true, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S); \
   else                                                                                                             \
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<WMV, EPI, DV, false, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S);
+    BW_LAUNCH((gemm_bf16_skinny_kernel<WMV, EPI, DV, false, CWV>), grid, block, lds, s, x, w, out, M, N, K, ldx, ldo, S);
     switch (wm) {
       case 1:
         if (half) { BW_SKINNY(1, 16, 8) }
@@ -2159,10 +2580,10 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                                     BIG_SLOTS * BIG_SLOT);
           allowed = true;
         }
-        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI_F32>), dim3(bm * bn, S), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w,
+        BW_LAUNCH((gemm_bf16_big_kernel<EPI_F32>), dim3(bm * bn, S), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w,
                            (void*)sp.scratch, M, N, K, ldx, N, bm, bn, rp, (size_t)M * N);
         const size_t quads = (size_t)M * (N >> 2);
-        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+        BW_LAUNCH(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
                            M, N, ldo);
         return BW_LAUNCH_CHECK();
       }
@@ -2175,10 +2596,10 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                                     T128_STAGES * T128_STAGE);
           allowed = true;
         }
-        hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI_F32>), dim3(mt * nt, S), dim3(512), T128_STAGES * T128_STAGE, s, x, w,
+        BW_LAUNCH((gemm_bf16_tile128_kernel<EPI_F32>), dim3(mt * nt, S), dim3(512), T128_STAGES * T128_STAGE, s, x, w,
                            (void*)sp.scratch, M, N, K, ldx, N, mt, nt, rp, (size_t)M * N);
         const size_t quads = (size_t)M * (N >> 2);
-        hipLaunchKernelGGL(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+        BW_LAUNCH(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
                            M, N, ldo);
         return BW_LAUNCH_CHECK();
       }
@@ -2208,7 +2629,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                                     BIG_SLOTS * BIG_SLOT);
           allowed = true;
         }
-        hipLaunchKernelGGL((gemm_bf16_big_kernel<EPI>), dim3(bm * bn), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w, out, M, N, K, ldx,
+        BW_LAUNCH((gemm_bf16_big_kernel<EPI>), dim3(bm * bn), dim3(512), BIG_SLOTS * BIG_SLOT, s, x, w, out, M, N, K, ldx,
                            ldo, bm, bn, rp, (size_t)0);
         return BW_LAUNCH_CHECK();
       }
@@ -2234,17 +2655,17 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                                     T128_STAGES * T128_STAGE);
           allowed = true;
         }
-        hipLaunchKernelGGL((gemm_bf16_tile128_kernel<EPI>), grid, dim3(512), T128_STAGES * T128_STAGE, s, x, w, out, M, N, K, ldx,
+        BW_LAUNCH((gemm_bf16_tile128_kernel<EPI>), grid, dim3(512), T128_STAGES * T128_STAGE, s, x, w, out, M, N, K, ldx,
                            ldo, m_tiles, n_tiles, rp, (size_t)0);
         return BW_LAUNCH_CHECK();
       }
     }
     if (S > 1)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
+      BW_LAUNCH((gemm_bf16_wide_kernel<EPI, true, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else if (K % (2 * WIDE_BK) == 0)
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
+      BW_LAUNCH((gemm_bf16_wide_kernel<EPI, false, true>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
     else
-      hipLaunchKernelGGL((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
+      BW_LAUNCH((gemm_bf16_wide_kernel<EPI, false, false>), grid, block, 0, s, x, w, out, M, N, K, ldx, ldo, m_tiles, n_tiles, rp);
   }
   return BW_LAUNCH_CHECK();
 }
@@ -2394,7 +2815,7 @@ extern "C" int bw_gemm_add_bf16_static(const void* x, const void* w, void* out, 
   // The counters must be zero when the kernel starts.  Every launch leaves them so, but the array outlives a
   // launch that was aborted half way; a small kernel clears them (a memset node in a captured graph is no
   // safe thing on this hardware's runtime).  The sums need no clearing: every cell is written before it is read.
-  hipLaunchKernelGGL(zero_words_kernel, dim3((need_counters + 255) / 256), dim3(256), 0, (hipStream_t)stream, count,
+  BW_LAUNCH(zero_words_kernel, dim3((need_counters + 255) / 256), dim3(256), 0, (hipStream_t)stream, count,
                      need_counters);
   return launch_gemm_bf16<EPI_ADD_F32>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldx, ldo, (hipStream_t)stream,
                                        QkvRopeArgs{}, MidSplitArgs{base, count}, (size_t)need_floats, need_counters);

@@ -69,14 +69,32 @@ _SIGS = {
     "bw_norm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                               c_int, c_int, c_int, c_void_p],
+    "bw_chain_sync_words": [],
+    "bw_chain_begin": [c_void_p, c_int, c_void_p, c_int],
+    "bw_chain_flush": [c_void_p],
+    "bw_chain_end": [c_void_p],
     "bw_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_fingerprint": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
 }
 
 _fns = {}
 
+# While a chain is open (``chain`` below) the library keeps the decode products that can run as phases of one
+# launch back; these entry points may be called meanwhile (they join the chain, launch through the library's own
+# path that sends the waiting phases first, or launch nothing).  Every other one is a launch that must come after
+# what waits.
+_CHAIN_KEEPS = frozenset({
+    "bw_gemm_bf16", "bw_gemm_add_bf16", "bw_norm_gemm_bf16", "bw_norm_qkv_rope_bf16",
+    "bw_gemm_add_scratch", "bw_norm_gemm_supported", "bw_norm_gemm_wide_supported", "bw_attention_decode_scratch",
+    "bw_attention_fold_group_tiles", "bw_gemm_add_bf16_static_max", "bw_chain_sync_words", "bw_chain_begin",
+    "bw_chain_flush", "bw_chain_end",
+})
+_chain_open = False
+
 
 def _fn(name: str):
+    if _chain_open and name not in _CHAIN_KEEPS:
+        _check(_fn("bw_chain_flush")(_stream()), "chain flush")
     f = _fns.get(name)
     if f is None:
         lib = _build.load()
@@ -130,6 +148,47 @@ def _is_bf16(t: torch.Tensor, what: str) -> int:
     if t.dtype == torch.float32:
         return 0
     raise ValueError(f"{what} must be bfloat16 or float32, got {t.dtype}")
+
+
+# ------------------------------------------------------------------------------ several products, one launch
+
+CHAIN_SPIN_LIMIT = 200000      # looks at a phase's flag before a wait gives up (some tenths of a second)
+
+
+def chain_sync_words() -> int:
+    return int(_fn("bw_chain_sync_words")())
+
+
+class chain:
+    """``with ops.chain(sync, err):`` the decode products of up to 16 rows asked for inside (RMSNorm + product with SwiGLU,
+    with a 32-bit store, or with rotation and cache write; residual adds) do not leave one by one: they wait and
+    run as phases of one launch, in the order they were asked for, when anything else is launched through this
+    module or the block ends.  A phase asks for its weights while the phase before it still runs, and waits inside
+    the kernel only for what that phase writes: the same bits, fewer kernel boundaries.  ``sync``: int32 zeros,
+    ``chain_sync_words()`` of them (left zero by every launch); ``err``: an int32 word that gets a bit if a wait
+    inside a launch gave up (then the step's results are void and ``sync`` has to be zeroed).  Everything put on the
+    stream inside the block must come through this module: a launch from elsewhere would overtake what waits."""
+
+    def __init__(self, sync: torch.Tensor, err: torch.Tensor, spin_limit: int = CHAIN_SPIN_LIMIT):
+        _need(sync, torch.int32, "sync")
+        _need(err, torch.int32, "err")
+        if sync.numel() < chain_sync_words() or err.numel() < 1:
+            raise ValueError(f"chain: sync needs {chain_sync_words()} words and err one")
+        self.sync, self.err, self.spin_limit = sync, err, int(spin_limit)
+
+    def __enter__(self):
+        global _chain_open
+        if _chain_open:
+            raise RuntimeError("a chain is already open")
+        _check(_fn("bw_chain_begin")(self.sync.data_ptr(), self.sync.numel(), self.err.data_ptr(), self.spin_limit), "chain")
+        _chain_open = True
+        return self
+
+    def __exit__(self, *exc):
+        global _chain_open
+        _chain_open = False
+        _check(_fn("bw_chain_end")(_stream()), "chain")
+        return False
 
 
 # ------------------------------------------------------------------------------ row ops

@@ -30,15 +30,18 @@ AHEAD_TOKEN = -2       # the token id of a row whose token the step before is st
 class _Pending:
     """A step that has been launched: what it will leave in pinned host memory once its event has passed."""
 
-    def __init__(self, n: int, event, tokens_host, prints_host, graph_rows: int):
+    def __init__(self, n: int, event, tokens_host, prints_host, graph_rows: int, check=None):
         self.n, self.event, self.tokens_host, self.prints_host, self.graph_rows = n, event, tokens_host, prints_host, graph_rows
         self.prints_dev = None
+        self.check = check              # called once the device is through: raises if the step's results are void
 
     def result(self):
         """(tokens, fingerprints or []) of the sampled rows; waits for the device."""
         if self.n == 0:
             return [], []
         self.event.synchronize()
+        if self.check is not None:
+            self.check()
         tokens = self.tokens_host[:self.n].tolist()
         prints = self.prints_host[:self.n].numpy().view(np.uint64).tolist() if self.prints_host is not None else []
         return tokens, prints
@@ -116,12 +119,14 @@ class GpuExecutor:
         self.max_model_len = min(max_len, asm.spec.max_positions)
         max_logit_rows = min(config.max_num_seqs, config.max_batched_tokens)
         self.runner = ModelRunner(asm, self.storage, self.max_model_len, max_rows=config.max_batched_tokens,
-                                  max_logit_rows=max_logit_rows, use_graphs=config.use_graphs)
+                                  max_logit_rows=max_logit_rows, use_graphs=config.use_graphs,
+                                  decode_phases=config.decode_phases)
         self.sampler = Sampler(rt.device, max_logit_rows)
         # two steps may be under way at a time (one being read back, one launched ahead): two sets of buffers
         self._flip = 0
         self._events = [torch.cuda.Event(), torch.cuda.Event()]
         self._tokens_host = [torch.zeros(max_logit_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._phase_err_host = [torch.zeros(1, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._prints_host = [torch.zeros(max_logit_rows, dtype=torch.int64, pin_memory=True) for _ in range(2)]
         self._prints_dev = [torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device) for _ in range(2)]
         self._prints_in = torch.zeros(max_logit_rows, dtype=torch.int64, device=rt.device)
@@ -150,6 +155,11 @@ class GpuExecutor:
         slot = self._flip
         self._flip ^= 1
         pend = _Pending(n, self._events[slot], self._tokens_host[slot], None, self.runner.last_graph_rows)
+        if n and self.runner.chain_rows and self.runner.last_graph_rows:
+            # the word that says whether a wait inside a launch of several phases gave up comes back with the tokens
+            word = self._phase_err_host[slot]
+            word.copy_(self.runner.chain_err, non_blocking=True)
+            pend.check = lambda: self.runner.check_phases(int(word[0]))
         if n:
             sampled = self.runner.last_sampled
             if sampled is None:

@@ -22,6 +22,7 @@ from .batch import Segment, StepContext
 from .storage import CacheStorage
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+CHAIN_MAX_ROWS = 16       # the graph buckets whose products can run as phases of one launch (ops.chain)
 
 
 class _StaticDecodeContext:
@@ -122,7 +123,7 @@ class ModelRunner:
     storage's caches.  It keeps nothing in the model, so several runners may share one."""
 
     def __init__(self, model: AssembledModel, storage: CacheStorage, max_model_len: int, max_rows: int = 256,
-                 max_logit_rows: Optional[int] = None, use_graphs: bool = True):
+                 max_logit_rows: Optional[int] = None, use_graphs: bool = True, decode_phases: bool = False):
         self.model, self.storage = model, storage
         self.rt = model.rt
         self.use_graphs = bool(use_graphs) and model.graph_safe
@@ -139,6 +140,14 @@ class ModelRunner:
         self.ws = Workspace(model.rt.device, ws_rows, storage.page_size, ws_logit_rows,
                             max_table_width=(self.max_model_len + storage.page_size - 1) // storage.page_size)
         self._graphs: Dict[int, tuple] = {}
+        # decode_phases: captured decode steps of few rows in bfloat16 mode run their products as phases of a few
+        # launches (ops.chain), if every part launches through ops: the words the phases meet in, and the word that
+        # says that a wait inside a launch gave up.
+        self.chain_rows = CHAIN_MAX_ROWS if (decode_phases and self.use_graphs and model.rt.bf16 and model.launches_through_ops) else 0
+        self.chain_sync = self.chain_err = None
+        if self.chain_rows:
+            self.chain_sync = torch.zeros(ops.chain_sync_words(), dtype=torch.int32, device=model.rt.device)
+            self.chain_err = torch.zeros(1, dtype=torch.int32, device=model.rt.device)
         self.last_sampled: Optional[torch.Tensor] = None   # tokens the last step's graph sampled, if it did
         self.last_graph_rows = 0      # requests of the last step if it was replayed from a graph, else 0
 
@@ -177,6 +186,20 @@ class ModelRunner:
     def _context(self, segments: Sequence[Segment]) -> StepContext:
         return StepContext(segments, len(self.model.group_specs), self.ws, self.storage.bindings, self.storage.num_pages)
 
+    def check_phases(self, bits: Optional[int] = None) -> None:
+        """Raise if a wait inside one of the launches of several phases gave up since the last check.  ``bits``: the
+        error word as the caller has read it back (None: it is read here, which waits for the device).  The words
+        the phases meet in are cleared, so that the next step starts clean."""
+        if self.chain_err is None:
+            return
+        if bits is None:
+            bits = int(self.chain_err.item())
+        if bits:
+            self.chain_sync.zero_()
+            self.chain_err.zero_()
+            raise RuntimeError(f"a decode step's launch of several phases gave up waiting for a phase (phases {bits:#x}): "
+                               "the step's results are void")
+
     # ------------------------------------------------------------------ graph replay
     def _step_graph(self, segments: Sequence[Segment], sampling=None) -> torch.Tensor:
         n = len(segments)
@@ -207,7 +230,11 @@ class ModelRunner:
         torch.cuda.synchronize(ws.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            logits = self.model.forward(ctx)
+            if bucket <= self.chain_rows:
+                with ops.chain(self.chain_sync, self.chain_err):
+                    logits = self.model.forward(ctx)
+            else:
+                logits = self.model.forward(ctx)
             ops.sample(logits, bucket, ctx.temps, ctx.unis, ctx.sampled)
         entry = (ctx, graph, logits)
         self._graphs[bucket] = entry

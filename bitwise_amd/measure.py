@@ -21,12 +21,13 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return cfg["num_hidden_layers"] * (per_token * tokens + attn) + 2 * h * v      # the head runs for one row
 
 
-def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT):
+def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT, decode_phases: bool = False):
     block = 16
     per_request = context + steps_total + 2 * block
     cfg = bw.EngineConfig(num_blocks=batch * ((per_request + block - 1) // block) + 8, max_batched_tokens=2048,
                           max_num_seqs=max(batch, 1), prefix_caching=False, fingerprint_logits=False,
-                          block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024))
+                          block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024),
+                          decode_phases=decode_phases)
     return bw.Engine(model, None, cfg)
 
 
@@ -107,7 +108,7 @@ def measure_chunked_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops:
 
 
 def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
-                   context: int = CONTEXT) -> dict:
+                   context: int = CONTEXT, decode_phases: bool = False) -> dict:
     """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
     said otherwise): tokens a second, and the bytes a step has to read (every weight once, the cache of the live
     requests) over its time."""
@@ -117,7 +118,7 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     # timed steps, so that each timed step has all ``batch`` rows.
     chunks = (context + 2047) // 2048                  # steps a prompt takes under the 2,048-token budget
     new_tokens = steps + warmup + batch * chunks + 8
-    eng = make_engine(bw, model, batch, new_tokens, dtype, context)
+    eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases)
     fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch, context=context)
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)

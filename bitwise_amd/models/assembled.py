@@ -52,6 +52,8 @@ class AssembledModel:
         self._plan_caches(spec.schedule)
         every = [self.embedding, self.final_norm, self.lm_head] + [p for b in self.layers for p in (b, *b.parts.values())]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
+        # (a captured decode step may hold its launches back to join them only if none of them goes round ops)
+        self.launches_through_ops = all(getattr(p, "launches_through_ops", False) for p in every)
         # each mixer's own word on what the engine may do around it (parts.base.Mixer)
         mixers = [self.layers[c.layer].mixer for c in spec.schedule]
         self.prefix_reusable = all(m.prefix_reusable for m in mixers)

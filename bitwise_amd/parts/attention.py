@@ -67,6 +67,8 @@ class Attention(Mixer):
     """params: width, heads, kv_heads, head_dim, window (None = all keys), position (PartSpec
     of the position encoding).  tensors: q_proj/k_proj/v_proj/o_proj .weight."""
 
+    launches_through_ops = True
+
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
         p = params

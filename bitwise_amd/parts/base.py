@@ -124,6 +124,8 @@ class Part:
     to one engine (scratch buffers, page size, caches) arrives with every step's context."""
 
     graph_safe = False             # True if forward() launches only capturable device work
+    launches_through_ops = False   # True if everything forward() puts on the stream goes through bitwise_amd.csrc.ops
+                                   # (then a decode step may hold launches back to join them: ops.chain)
 
     def __init__(self, params: Dict[str, Any], runtime: "Any"):
         self.params = dict(params)

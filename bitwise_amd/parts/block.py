@@ -11,6 +11,7 @@ class PreNormBlock(Block):
 
     roles = {"mixer_norm": "norm", "ffn_norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
     graph_safe = True
+    launches_through_ops = True
 
     def forward(self, ctx, call, x) -> None:
         if not self.mixer.forward_with_norm(ctx, call, x, self.mixer_norm, x):

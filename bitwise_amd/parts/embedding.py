@@ -16,6 +16,7 @@ class TokenEmbedding(Embedding):
     """params: vocab, width.  tensor: weight [vocab, width], gathered as 32-bit rows."""
 
     graph_safe = True
+    launches_through_ops = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
@@ -44,6 +45,7 @@ class LMHead(Head):
     (src/model.cpp:170-171).  Only the wanted rows are normed and projected."""
 
     graph_safe = True
+    launches_through_ops = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)

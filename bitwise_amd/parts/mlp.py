@@ -18,6 +18,7 @@ class SwiGLU(FeedForward):
     """params: width, inter.  tensors: gate_proj/up_proj/down_proj .weight."""
 
     graph_safe = True
+    launches_through_ops = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)

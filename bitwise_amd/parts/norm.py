@@ -16,6 +16,7 @@ class RMSNorm(Norm):
     products are 32-bit; the output has the mode's activation dtype."""
 
     graph_safe = True
+    launches_through_ops = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)

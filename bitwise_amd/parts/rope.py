@@ -19,6 +19,7 @@ class RotaryTable(PositionEncoding):
     """params: theta, head_dim, max_positions.  No checkpoint tensors."""
 
     graph_safe = True
+    launches_through_ops = True
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)

@@ -21,8 +21,8 @@ MAX_STEP_ROWS = 4096
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, use_graphs: bool = True,
                  max_live: int = 64, model: Optional[Model] = None, poison_freed_pages: bool = False,
-                 fingerprint_logits: bool = False):
-        """``poison_freed_pages``: every page that comes back is filled with NaN at once (a fault finder: what a
+                 fingerprint_logits: bool = False, decode_phases: bool = False):
+        """``decode_phases``: EngineConfig.decode_phases.  ``poison_freed_pages``: every page that comes back is filled with NaN at once (a fault finder: what a
         later owner of the page reads before writing it shows up in its logits)."""
         self.model = model if model is not None else Model.load(model_dir, dtype)
         asm = self.model.assembled
@@ -33,7 +33,7 @@ class Replayer:
         self.storage = CacheStorage(asm, pages, max_live, block_size)
         max_len = min(asm.spec.max_positions, max(int(max_tokens), 1))
         self.runner = ModelRunner(asm, self.storage, max_model_len=max_len, max_rows=rows, max_logit_rows=rows,
-                                  use_graphs=use_graphs)
+                                  use_graphs=use_graphs, decode_phases=decode_phases)
         if poison_freed_pages:
             self.manager.on_free = lambda group, page: self.storage.poison_pages(group, [page])
         self.live: Dict[str, RequestCache] = {}

@@ -952,3 +952,89 @@ def test_decode_attention_beyond_one_pass_of_partials(gpu):
             want = w @ vv
             got = split[r].cpu().double().view(heads, hd)[h]
             assert (got - want).abs().max() <= 1.5e-2 * want.abs().max().clamp(min=0.05), (p, h)
+
+
+def _decode_layer_tail(gpu, g, M, width, inter, heads, kvh, hd, page, vocab):
+    """What follows a decode step's attention in one layer and opens the next (output projection, RMSNorm + gate|up +
+    SwiGLU, down projection, RMSNorm + q|k|v + rotation + cache write) and a head: random operands, and a function
+    that runs the five products on fresh outputs, one launch each or as phases (ops.chain)."""
+    cos, sin = rope_tables(10000.0, hd, 200, gpu)
+    per_row = (90 + page - 1) // page                    # every row a request of its own, with pages of its own
+    attn = torch.randn(M, heads * hd, generator=g).bfloat16().to(gpu)
+    resid = (torch.randn(M, width, generator=g) * 2).to(gpu)
+    w_o = (torch.randn(width, heads * hd, generator=g) * 0.05).bfloat16().to(gpu)
+    w_gu = (torch.randn(2 * inter, width, generator=g) * 0.05).bfloat16().to(gpu)
+    w_d = (torch.randn(width, inter, generator=g) * 0.05).bfloat16().to(gpu)
+    w_qkv = (torch.randn((heads + 2 * kvh) * hd, width, generator=g) * 0.05).bfloat16().to(gpu)
+    w_head = (torch.randn(vocab, width, generator=g) * 0.05).bfloat16().to(gpu)
+    n1 = (1 + 0.1 * torch.randn(width, generator=g)).bfloat16().to(gpu)
+    n2 = (1 + 0.1 * torch.randn(width, generator=g)).bfloat16().to(gpu)
+    positions = torch.tensor([(7 * i + 3) % 90 if i != 2 else -1 for i in range(M)], dtype=torch.int32, device=gpu)
+    row_seq = torch.arange(M, dtype=torch.int32, device=gpu)
+    table = torch.arange(M * per_row, dtype=torch.int32, device=gpu).reshape(M, per_row).contiguous()
+
+    def run(chained, sync=None, err=None, spin=None):
+        x = resid.clone()
+        h = torch.zeros(M, inter, dtype=torch.bfloat16, device=gpu)
+        q = torch.zeros(M, heads * hd, dtype=torch.bfloat16, device=gpu)
+        kc = torch.full((M * per_row, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+        vc = torch.full((M * per_row, kvh * page * hd), 3.0, dtype=torch.bfloat16, device=gpu)
+        logits = torch.zeros(M, vocab, device=gpu)
+
+        def products():
+            ops.gemm_bf16(attn, w_o, x, M, ops.EPI_ADD_F32)
+            ops.norm_gemm_bf16(x, n1, 1e-5, w_gu, h, M, ops.EPI_SWIGLU_BF16)
+            ops.gemm_bf16(h, w_d, x, M, ops.EPI_ADD_F32)
+            ops.norm_qkv_rope_bf16(x, n2, 1e-5, w_qkv, q, positions, row_seq, table, cos, sin, kc, vc, M, heads, kvh, hd, page)
+            ops.norm_gemm_bf16(x, n1, 1e-5, w_head, logits, M, ops.EPI_F32)
+        if chained:
+            with (ops.chain(sync, err) if spin is None else ops.chain(sync, err, spin)):
+                products()
+        else:
+            products()
+        torch.cuda.synchronize()
+        return x, h, q, kc, vc, logits
+    return run
+
+
+@pytest.mark.parametrize("M,width,inter,heads,kvh,hd,vocab", [
+    (8, 2048, 8192, 32, 32, 64, 49152),        # the layer sizes the decode benchmark runs (burst, stream with 8 rows a stage)
+    (13, 2048, 8192, 32, 32, 64, 4096),        # more than 8 rows (16 rows a stage, two rows a wave to normalise)
+    (8, 4096, 14336, 32, 8, 128, 4096),        # rows of two segments; the stream kernel with 16 columns a wave, seven segments
+    (3, 1024, 2816, 16, 4, 64, 8192),          # a feed-forward width that is no multiple of 2048
+])
+def test_products_as_phases_of_one_launch_equal_the_separate_launches(gpu, M, width, inter, heads, kvh, hd, vocab):
+    """The decode products run as phases of one launch (ops.chain) give the bits of one launch each; the launch leaves
+    its meeting words zero and reports no wait that gave up; and a second launch on the same words works like the first."""
+    g = torch.Generator().manual_seed(M * 1000 + width)
+    run = _decode_layer_tail(gpu, g, M, width, inter, heads, kvh, hd, 16, vocab)
+    sync = torch.zeros(ops.chain_sync_words(), dtype=torch.int32, device=gpu)
+    err = torch.zeros(1, dtype=torch.int32, device=gpu)
+    plain = run(False)
+    for _ in range(2):
+        chained = run(True, sync, err)
+        assert int(err.item()) == 0
+        assert int(sync.abs().sum().item()) == 0
+        for name, a, b in zip(("residual", "swiglu", "q", "k cache", "v cache", "logits"), plain, chained):
+            assert torch.equal(a, b), name
+
+
+def test_a_phase_that_gives_up_waiting_says_so_and_nothing_hangs(gpu):
+    """With no looks at the flag allowed, a phase that finds the phase before it unfinished gives up at once: the launch
+    ends normally, the error word names the phase, and after the caller has cleared the words the next launch is right.
+    (Whether a wait gives up depends on how far the phase before has got; with no looks allowed and megabytes of weights
+    to stream it has not finished.)"""
+    g = torch.Generator().manual_seed(5)
+    run = _decode_layer_tail(gpu, g, 8, 2048, 8192, 32, 32, 64, 16, 4096)
+    sync = torch.zeros(ops.chain_sync_words(), dtype=torch.int32, device=gpu)
+    err = torch.zeros(1, dtype=torch.int32, device=gpu)
+    plain = run(False)
+    run(True, sync, err, spin=0)                     # returns: nothing hangs
+    gave_up = int(err.item())
+    assert gave_up != 0 and gave_up < (1 << 6)
+    sync.zero_()
+    err.zero_()
+    chained = run(True, sync, err)
+    assert int(err.item()) == 0 and int(sync.abs().sum().item()) == 0
+    for a, b in zip(plain, chained):
+        assert torch.equal(a, b)

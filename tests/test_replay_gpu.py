@@ -352,7 +352,8 @@ def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
     """Two layers of real sizes, so that every shape-dependent route of the kernels runs at the shapes it was
     written for (K = 2048, 4096, 8192 and 14336; up to 128,256 columns), in bfloat16 and in 32-bit: a prompt whole;
     in portions of 900, 700, 300, 100, 61, 29 and 10 tokens; with its last 40 tokens decoded one by one from graphs;
-    and decoded beside 8 and then 19 other requests.  The logits of the last 40 positions are the same bits every time."""
+    and decoded beside 8 and then 19 other requests; in bfloat16 also with the decode steps' products run as phases of a
+    few launches (EngineConfig.decode_phases).  The logits of the last 40 positions are the same bits every time."""
     import bitwise_amd as bw
     from bitwise_amd.replay import Replayer
 
@@ -367,8 +368,8 @@ def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
     tail = 40
     head = len(toks) - tail
 
-    def last(rp_steps, max_tokens=4096):
-        rp = Replayer("", dtype, max_tokens, block_size=16, model=model)
+    def last(rp_steps, max_tokens=4096, decode_phases=False):
+        rp = Replayer("", dtype, max_tokens, block_size=16, model=model, decode_phases=decode_phases)
         rows = []
         for st in rp_steps:
             lg = rp.step(st["entries"], st.get("end", []))
@@ -378,6 +379,8 @@ def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
                     if e["id"] == "r":
                         rows.append(lg[row].copy())
                     row += 1
+        if decode_phases:
+            rp.runner.check_phases()              # no wait inside a launch gave up
         return np.stack(rows)
 
     whole = last([{"entries": [{"id": "r", "tokens": toks, "want": list(range(head, len(toks)))}]}])
@@ -391,6 +394,9 @@ def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
     one = [{"entries": [{"id": "r", "tokens": toks[:head + 1], "want": [head]}]}]
     one += [{"entries": [{"id": "r", "tokens": [t], "want": [0]}]} for t in toks[head + 1:]]
     assert np.array_equal(last(one), whole), "last tokens one by one"
+    if dtype == "bfloat16":
+        # the decode steps' products as phases of a few launches that wait for each other inside the kernel
+        assert np.array_equal(last(one, decode_phases=True), whole), "last tokens one by one, products as phases"
     for crowd in (8, 19):
         names = list(others)[:crowd]
         mixed = [{"entries": [{"id": "r", "tokens": toks[:head + 1], "want": [head]}] +
@@ -400,3 +406,5 @@ def test_real_layer_sizes_are_cut_invariant(gpu, shape, dtype):
                                      [{"id": "r", "tokens": [t], "want": [0]}] +
                                      [{"id": n, "tokens": [others[n][j % 30]], "want": [0]} for n in names[crowd // 2:]]})
         assert np.array_equal(last(mixed, max_tokens=8192), whole), f"decoded beside {crowd} others"
+        if dtype == "bfloat16" and crowd == 8:
+            assert np.array_equal(last(mixed, max_tokens=8192, decode_phases=True), whole), "decoded beside 8 others, products as phases"
