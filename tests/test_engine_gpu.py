@@ -104,6 +104,13 @@ def test_long_decoding_with_and_without_graphs(folders):
     assert outs[0].tokens == outs[1].tokens and outs[0].logits_fingerprint == outs[1].logits_fingerprint
     want = pl.generate(cfg_long, tiny.read_weights(folder), prompt, 100, 0.9, 3, True, **tiny.plain_mode(dtype))
     assert outs[0].tokens == want
+    # the same with the decode steps' products as phases of a few launches (what of them can run so at these sizes)
+    eng = bw.Engine(model, None, engine_config(name, dtype, decode_phases=True))
+    assert eng.exec.runner.chain_rows == 16
+    i = eng.add_request(prompt, sp)
+    while not eng.idle():
+        eng.step()
+    assert eng.result(i).tokens == want and eng.result(i).logits_fingerprint == outs[0].logits_fingerprint
 
 
 def test_many_requests_decode_from_the_large_graph_buckets(gpu):

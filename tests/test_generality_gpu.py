@@ -202,6 +202,8 @@ def test_stateful_mixer_through_the_engine_with_preemption(toy_folder):
     of a solo run, with graphs on and off."""
     dtype = "float32"
     model = bw.Model.load(toy_folder, dtype)
+    # (a part that does not say that all its launches go through ops keeps the engine from holding launches back)
+    assert not model.assembled.launches_through_ops
     g = torch.Generator().manual_seed(8)
     prompts = [torch.randint(0, TOY["vocab"], (n,), generator=g).tolist() for n in (9, 17, 5, 12)]
     sp = bw.SamplingParams(max_new_tokens=20, ignore_eos=True)
