@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--sweep]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -46,6 +46,28 @@ LLAMA3_8B = {
 }
 
 
+def sweep(bw, torch, steps: int) -> int:
+    """Decode steps over batch and context, prefills over length, at both shapes in bfloat16: one JSON object a line."""
+    from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
+    for name, shape in (("SmolLM2-1.7B", SMOLLM2_1_7B), ("Llama-3-8B", LLAMA3_8B)):
+        cfg = dict(shape, max_position_embeddings=16384)
+        model = bw.Model.random(cfg, seed=0, dtype="bfloat16", sigma=0.02, on_device=True)
+        for tokens in (128, 256, 512, 1024, 2048):
+            m = measure_prefill(bw, torch, model, cfg, "bfloat16", PEAK_FLOPS["bf16"], tokens)
+            print(json.dumps({"shape": name, "prefill_tokens": tokens, "ms": m["ms"], "tok_s": m["value"], "frac_of_2.5_PFLOPs": m["frac"]}),
+                  flush=True)
+        for context in (512, 2048, 8192):
+            for batch in (1, 2, 4, 8, 16, 32, 64, 128):
+                if batch * context > 512 * 1024:          # (a pool of at most half a million tokens)
+                    continue
+                m = measure_decode(bw, torch, model, cfg, "bfloat16", batch, steps, 4, context=context)
+                print(json.dumps({"shape": name, "decode_batch": batch, "context": context, "ms_per_step": m["ms_per_step"],
+                                  "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}), flush=True)
+        del model
+        torch.cuda.empty_cache()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -62,6 +84,9 @@ def main() -> int:
                     help="run nothing but the 128-request shared-prefix trace at Llama-3-8B's sizes and print its figures (for profiles)")
     ap.add_argument("--decode-phases", action="store_true",
                     help="the headline decode with EngineConfig.decode_phases (its products as phases of a few launches; for profiles)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="print a table instead of the line: decode at batches 1 to 128 and contexts of 512 to 8,192 tokens, prefills "
+                         "of 128 to 2,048 tokens, at both shapes (bfloat16)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -75,6 +100,8 @@ def main() -> int:
                                      measure_trace)
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    if args.sweep:
+        return sweep(bw, torch, args.steps)
     if args.trace_only:
         big = dict(LLAMA3_8B, max_position_embeddings=16384)
         model8 = bw.Model.random(big, seed=1, dtype=dtype, sigma=0.02, on_device=True)

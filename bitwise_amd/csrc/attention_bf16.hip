@@ -1023,7 +1023,7 @@ static void decode_split_shape(int num_tiles, int items, int table_stride, int p
   max_parts = (table_stride * page_size + ATT_PART - 1) / ATT_PART + 1;
   const int rounds = (max_parts + DECODE_W - 1) / DECODE_W;
   const int wgs = num_tiles * items;
-  nsplit = wgs >= 128 ? 1 : 256 / wgs;
+  nsplit = wgs >= 256 ? 1 : 256 / wgs;
   if (nsplit > rounds) nsplit = rounds;
   if (nsplit < 1) nsplit = 1;
 }

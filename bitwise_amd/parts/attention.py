@@ -209,7 +209,7 @@ class Attention(Mixer):
         sizes = ws.notes.get(key)
         if sizes is None:
             floats = counters = 0
-            for t in range(1, min(ws.max_rows, 128) + 1):            # (from 128 workgroups on nothing splits)
+            for t in range(1, min(ws.max_rows, 256) + 1):            # (from 256 workgroups on nothing splits)
                 f, c = ops.attention_decode_scratch(t, self.heads, self.kv_heads, self.head_dim, width, ws.page_size)
                 floats, counters = max(floats, f), max(counters, c)
             sizes = ws.notes[key] = (floats, counters)
