@@ -166,7 +166,7 @@ def test_randomized_scenarios(gpu, dtype):
     assert tally.requests_compared > 60 and tally.preemptions > 0 and tally.prefix_hit_tokens > 0
     assert tally.ended_by_eos > 0 and tally.cancelled > 0
     assert len(tally.knobs_seen["block_size"]) >= 3 and tally.knobs_seen["use_graphs"] == {True, False}
-    assert tally.knobs_seen["run_ahead"] == {True, False}
+    assert tally.knobs_seen["run_ahead"] == {True, False} and tally.knobs_seen["decode_phases"] == {True, False}
 
 
 def test_the_simulator_program_catches_every_injected_fault(gpu):
