@@ -14,6 +14,7 @@ int bw_embed(const int32_t* tokens, const int32_t* feedback, const void* table, 
 int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16, int rows,
                int dim, int ldy, float eps, void* stream);
 int bw_add(float* x, const float* y, long long n, void* stream);
+int bw_add_bias(float* x, const float* bias, int rows, int cols, int ldx, void* stream);
 int bw_convert(const void* src, int src_is_bf16, void* dst, int dst_is_bf16, int rows, int cols, int lds, int ldd,
                void* stream);
 int bw_swiglu_f32(const float* gate_up, float* h, int rows, int inter, void* stream);

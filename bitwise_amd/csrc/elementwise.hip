@@ -208,6 +208,22 @@ extern "C" int bw_add(float* x, const float* y, long long n, void* stream) {
   return BW_LAUNCH_CHECK();
 }
 
+// x[r, c] += bias[c] in 32-bit: a projection's bias, one addition behind the product's sum.
+__global__ void add_bias_kernel(float* __restrict__ x, const float* __restrict__ bias, int rows, int cols, int ldx) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)rows * cols) return;
+  const int r = (int)(i / cols), c = (int)(i % cols);
+  x[(size_t)r * ldx + c] += bias[c];
+}
+
+extern "C" int bw_add_bias(float* x, const float* bias, int rows, int cols, int ldx, void* stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (ldx < cols) return -2;
+  const size_t n = (size_t)rows * cols;
+  hipLaunchKernelGGL(add_bias_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, bias, rows, cols, ldx);
+  return BW_LAUNCH_CHECK();
+}
+
 // dst[r, c] = src[r, c] between 32-bit and bfloat16 rows (widening is exact; narrowing rounds to nearest even
 // with the hardware conversion).  For the routes on which a weight's dtype is not the mode's.
 template <typename S, typename D>

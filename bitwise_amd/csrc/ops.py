@@ -39,6 +39,7 @@ _SIGS = {
     "bw_embed": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "bw_add": [c_void_p, c_void_p, c_longlong, c_void_p],
+    "bw_add_bias": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_convert": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_swiglu_f32": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "bw_gather_rows_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -234,6 +235,15 @@ def add_(x: torch.Tensor, y: torch.Tensor, rows: int) -> None:
     if x.shape[1:] != y.shape[1:] or x.shape[0] < rows or y.shape[0] < rows:
         raise ValueError("add_: shapes differ")
     _check(_fn("bw_add")(x.data_ptr(), y.data_ptr(), rows * x.stride(0), _stream()), "add")
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor, rows: int) -> None:
+    """x[:rows] += bias (32-bit, one addition an element): a projection's bias behind its product."""
+    _need(x, torch.float32, "x")
+    _need(bias, torch.float32, "bias")
+    if bias.dim() != 1 or bias.shape[0] != x.shape[1] or x.shape[0] < rows:
+        raise ValueError(f"add_bias: x {tuple(x.shape)} and bias {tuple(bias.shape)} do not match")
+    _check(_fn("bw_add_bias")(x.data_ptr(), bias.data_ptr(), rows, x.shape[1], x.stride(0), _stream()), "add_bias")
 
 
 def convert(src: torch.Tensor, dst: torch.Tensor, rows: int) -> None:

@@ -58,6 +58,41 @@ def test_norm_part(gpu, mode):
 
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+@pytest.mark.parametrize("stored", [torch.bfloat16, torch.float32])
+def test_a_projection_with_a_bias(gpu, mode, stored):
+    """The reference's architecture has no biases; a part of another one passes ``bias`` to Linear: one 32-bit addition
+    behind the product's sum, stored in 32-bit or rounded to bfloat16, or the biased product added whole into the
+    residual stream.  Against 64-bit arithmetic at the product's tolerance, and to the bit against the same Linear
+    without a bias followed by the addition."""
+    from bitwise_amd.parts.linear import Linear
+    rt, ws = Runtime(mode, gpu), Workspace(gpu, max_rows=32, page_size=8)
+    g = torch.Generator().manual_seed(12)
+    n, k, rows = 88, 72, 19
+    w = (torch.randn(n, k, generator=g) * 0.3).to(stored)
+    b = torch.randn(n, generator=g).bfloat16()
+    x = torch.zeros(32, k, device=gpu, dtype=rt.act_dtype)
+    x[:rows] = torch.randn(rows, k, generator=g).to(rt.act_dtype).to(gpu)
+    with_bias, plain = Linear(w, rt, bias=b), Linear(w, rt)
+    ref = pl.linear(x[:rows].cpu().double(), w) + b.double()
+    y = torch.zeros(32, n, device=gpu)
+    with_bias.store(ws, x, y, rows)
+    check_rows(y[:rows].cpu().double(), ref, mode, "biased projection")
+    y0 = torch.zeros(32, n, device=gpu)
+    plain.store(ws, x, y0, rows)
+    assert torch.equal(y[:rows], y0[:rows] + b.float().to(gpu))
+    yb = torch.zeros(32, n, device=gpu, dtype=torch.bfloat16)
+    with_bias.store(ws, x, yb, rows)
+    assert torch.equal(yb[:rows], y[:rows].bfloat16())
+    res = torch.randn(32, n, generator=g).to(gpu)
+    before = res.clone()
+    with_bias.add_into(ws, x, res, rows)
+    assert torch.equal(res[:rows], before[:rows] + y[:rows]) and torch.equal(res[rows:], before[rows:])
+    assert with_bias.nbytes() == plain.nbytes() + 4 * n
+    with pytest.raises(ValueError):
+        Linear(w, rt, bias=b[:5])
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 def test_feed_forward_part(gpu, mode):
     rt, ws = Runtime(mode, gpu), Workspace(gpu, max_rows=64, page_size=8)
     part = base.FEED_FORWARDS["swiglu"]({"width": 40, "inter": 88}, rt)
