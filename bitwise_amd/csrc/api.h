@@ -71,6 +71,18 @@ int bw_norm_qkv_rope_bf16(const float* x, int ldx, const void* norm_w, int norm_
                           const int32_t* block_table, int table_stride, const float* cos_table,
                           const float* sin_table, void* k_cache, void* v_cache, int M, int heads, int kv_heads,
                           int head_dim, int K, int page_size, int write_cache, void* stream);
+// Between bw_chain_begin and bw_chain_end (in the calling thread) the decode products of up to 16 rows that can run as
+// phases of one launch (bw_norm_gemm_bf16 with SwiGLU or a 32-bit store, bw_norm_qkv_rope_bf16, the residual adds of
+// bw_gemm_bf16 / bw_gemm_add_bf16 of few columns) are not launched when they are asked for: they wait, and leave as one
+// launch whose phases wait for each other inside the kernel when anything else of gemm_bf16.hip or fused_decode.hip is
+// launched, at bw_chain_flush, or at the end.  A caller that launches anything else on the stream meanwhile (this
+// library's other entry points included) calls bw_chain_flush first.  sync: bw_chain_sync_words() 32-bit words, zero
+// before the first chain (every launch leaves them zero); err: a word that gets a bit for every phase one of whose
+// bounded waits gave up after spin_limit looks (then the results are void and the caller clears sync).  The same bits.
+int bw_chain_sync_words();
+int bw_chain_begin(void* sync, int sync_words, void* err, int spin_limit);
+int bw_chain_flush(void* stream);
+int bw_chain_end(void* stream);
 int bw_sample(const float* logits, int vocab, int ld, int rows, const float* temperature, const double* uniform,
               int32_t* out, void* stream);
 int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void* h_in, void* h_out, void* stream);
