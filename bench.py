@@ -46,23 +46,27 @@ LLAMA3_8B = {
 }
 
 
-def sweep(bw, torch, steps: int) -> int:
-    """Decode steps over batch and context, prefills over length, at both shapes in bfloat16: one JSON object a line."""
+def sweep(bw, torch, steps: int, dtype: str) -> int:
+    """Decode steps over batch and context, prefills over length: in bfloat16 at both shapes, in the 32-bit mode a
+    coarser grid at the small one.  One JSON object a line."""
     from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
-    for name, shape in (("SmolLM2-1.7B", SMOLLM2_1_7B), ("Llama-3-8B", LLAMA3_8B)):
+    bf16 = dtype == "bfloat16"
+    shapes = (("SmolLM2-1.7B", SMOLLM2_1_7B), ("Llama-3-8B", LLAMA3_8B)) if bf16 else (("SmolLM2-1.7B", SMOLLM2_1_7B),)
+    for name, shape in shapes:
         cfg = dict(shape, max_position_embeddings=16384)
-        model = bw.Model.random(cfg, seed=0, dtype="bfloat16", sigma=0.02, on_device=True)
-        for tokens in (128, 256, 512, 1024, 2048):
-            m = measure_prefill(bw, torch, model, cfg, "bfloat16", PEAK_FLOPS["bf16"], tokens)
-            print(json.dumps({"shape": name, "prefill_tokens": tokens, "ms": m["ms"], "tok_s": m["value"], "frac_of_2.5_PFLOPs": m["frac"]}),
-                  flush=True)
-        for context in (512, 2048, 8192):
-            for batch in (1, 2, 4, 8, 16, 32, 64, 128):
+        model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+        for tokens in ((128, 256, 512, 1024, 2048) if bf16 else (128, 512, 2048)):
+            m = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[dtype], tokens)
+            print(json.dumps({"shape": name, "dtype": dtype, "prefill_tokens": tokens, "ms": m["ms"], "tok_s": m["value"],
+                              "frac_of_matrix_peak": m["frac"]}), flush=True)
+        for context in ((512, 2048, 8192) if bf16 else (512, 2048)):
+            for batch in ((1, 2, 4, 8, 16, 32, 64, 128) if bf16 else (1, 8, 64)):
                 if batch * context > 512 * 1024:          # (a pool of at most half a million tokens)
                     continue
-                m = measure_decode(bw, torch, model, cfg, "bfloat16", batch, steps, 4, context=context)
-                print(json.dumps({"shape": name, "decode_batch": batch, "context": context, "ms_per_step": m["ms_per_step"],
-                                  "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}), flush=True)
+                m = measure_decode(bw, torch, model, cfg, dtype, batch, steps, 4, context=context)
+                print(json.dumps({"shape": name, "dtype": dtype, "decode_batch": batch, "context": context,
+                                  "ms_per_step": m["ms_per_step"], "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}),
+                      flush=True)
         del model
         torch.cuda.empty_cache()
     return 0
@@ -86,7 +90,7 @@ def main() -> int:
                     help="the headline decode with EngineConfig.decode_phases (its products as phases of a few launches; for profiles)")
     ap.add_argument("--sweep", action="store_true",
                     help="print a table instead of the line: decode at batches 1 to 128 and contexts of 512 to 8,192 tokens, prefills "
-                         "of 128 to 2,048 tokens, at both shapes (bfloat16)")
+                         "of 128 to 2,048 tokens, at both shapes (with --dtype fp32: a coarser grid at the small shape)")
     ap.add_argument("--no-points", action="store_true",
                     help="only the headline: skip decode at batch 1 and 64, the 32-bit path and the Llama-3-8B sizes")
     args = ap.parse_args()
@@ -101,7 +105,7 @@ def main() -> int:
 
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
-        return sweep(bw, torch, args.steps)
+        return sweep(bw, torch, args.steps, dtype)
     if args.trace_only:
         big = dict(LLAMA3_8B, max_position_embeddings=16384)
         model8 = bw.Model.random(big, seed=1, dtype=dtype, sigma=0.02, on_device=True)
