@@ -225,16 +225,19 @@ class ModelRunner:
         # One eager run first, on rows that are all padding: it creates every scratch buffer the capture
         # will use and touches neither cache nor state (a real step run here and then replayed from the
         # fresh graph would advance a stateful mixer twice).
+        def forward():
+            # (the warm-up runs what the capture will run: the kernels' one-time set-up happens outside the capture)
+            if bucket <= self.chain_rows:
+                with ops.chain(self.chain_sync, self.chain_err):
+                    return self.model.forward(ctx)
+            return self.model.forward(ctx)
+
         ctx.fill([])
-        self.model.forward(ctx)
+        forward()
         torch.cuda.synchronize(ws.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            if bucket <= self.chain_rows:
-                with ops.chain(self.chain_sync, self.chain_err):
-                    logits = self.model.forward(ctx)
-            else:
-                logits = self.model.forward(ctx)
+            logits = forward()
             ops.sample(logits, bucket, ctx.temps, ctx.unis, ctx.sampled)
         entry = (ctx, graph, logits)
         self._graphs[bucket] = entry
