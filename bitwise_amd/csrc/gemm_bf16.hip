@@ -1850,24 +1850,28 @@ int bw_norm_qkv_rope_mid(const float* x32, int ldx32, const void* norm_w, int no
 // hand.  Nothing is shared between waves, so the loop has no barrier.  K a multiple of 64.
 // XR: rows of x a stage holds, 16, or 8 where there are no more than 8 (lanes that stand for rows 8 to 15 read rows
 // 0 to 7 again; their products go nowhere): a load less a stage, so more stages of W in flight.
-template <int CW, int XR = 16>
+// DEPTH: loads a wave keeps in flight, 24, or fewer for a workgroup of more than four waves (a product of five to eight
+// segments of K: a wave a segment, all at once, where four waves would take the segments in two turns; the rings of
+// eight waves fit the compute unit's LDS only if they are shallower).
+template <int CW, int XR = 16, int DEPTH = 24>
 struct StreamShape {
   static constexpr int A_LOADS = XR / 8, B_LOADS = CW / 8, LPW = A_LOADS + B_LOADS;
   static constexpr int A_BYTES = A_LOADS * 1024;
   static constexpr int STAGE = A_BYTES + B_LOADS * 1024;            // x: XR rows of 128 bytes, then W
-  static constexpr int STAGES = 24 / LPW + 2;
+  static constexpr int STAGES = DEPTH / LPW + 2;
   static constexpr int RING = STAGES * STAGE;
-  static_assert(LPW * (STAGES - 2) == 24, "the wait below is written for 24 loads in flight");
+  static_assert(LPW * (STAGES - 2) == DEPTH, "the wait for a stage counts DEPTH loads in flight");
 };
+#define STREAM_DEPTH_MANY(CW) ((CW) == 16 ? 15 : 14)               // (with 8 rows of x a stage: seven and nine stages)
 
 // A wave's loads of one stage of its ring (a device function rather than a lambda in the kernel: the
 // host pass drops, without a word, kernel templates whose lambdas capture arrays of dependent size).
 // DO_X, DO_W: which of the stage's loads (a phase of a launch of several asks for the weights of its first stages
 // before the rows); DEV: x at device scope.
-template <int CW, int XR, bool DO_X = true, bool DO_W = true, bool DEV = false>
+template <int CW, int XR, bool DO_X = true, bool DO_W = true, bool DEV = false, int DEPTH = 24>
 __device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffer_rsrc_t rs_x, __amdgpu_buffer_rsrc_t rs_w,
                                              const int* voff_x, const int* voff_w, int step, int steps, int k_begin) {
-  using SH = StreamShape<CW, XR>;
+  using SH = StreamShape<CW, XR, DEPTH>;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   unsigned char* dst = ring + (step % SH::STAGES) * SH::STAGE;
   const bool real = step < steps;                                  // scalar; past the segment: outside the descriptors
@@ -1888,10 +1892,10 @@ __device__ __forceinline__ void stream_issue(unsigned char* ring, __amdgpu_buffe
 // wave asks for the weights of its first segment's first stages, waits, and asks for their rows of x then (loads
 // complete in the order they are issued: until the ring has turned once the wait for a stage lets fewer loads stay in
 // flight); x, old values and outputs travel at device scope.
-template <int EPI, int CW, int XR, bool CH>
+template <int EPI, int CW, int XR, bool CH, int DEPTH = 24>
 __device__ __forceinline__ void stream_body(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
                                             int K, int ldx, int ldo, int S, const ChainCtx& cc) {
-  using SH = StreamShape<CW, XR>;
+  using SH = StreamShape<CW, XR, DEPTH>;
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];   // [waves][ring], then [S][4][64] floats when S > 1
   const int wave = wave_index(), lane = threadIdx.x & 63, nwaves = cc.waves;
   const int r = lane & 15, g = lane >> 4;
@@ -1945,22 +1949,22 @@ __device__ __forceinline__ void stream_body(const bf16_t* __restrict__ x, const 
     const bool first_turn = CH && s == wave;                       // (scalar) the segment whose x had to wait
     if (first_turn) {
 #pragma unroll
-      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, false, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, false, true, CH, DEPTH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       chain_wait<CH>(cc);
       ask_old();
 #pragma unroll
-      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, false, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, false, CH, DEPTH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
     } else {
 #pragma unroll
-      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
+      for (int st = 0; st < SH::STAGES - 1; ++st) stream_issue<CW, XR, true, true, CH, DEPTH>(ring, rs_x, rs_w, voff_x, voff_w, st, steps, k_begin);
     }
     for (int step = 0; step < steps; ++step) {
       // the stage at hand has landed when all but the loads of the stages after it have: 24, or, while x of the
       // first stages was asked for behind their weights, what is left of x (B_LOADS fewer a stage) and what came since
       if (first_turn && step < SH::STAGES - 2) __builtin_amdgcn_s_waitcnt(vmcnt_only(SH::A_LOADS * (SH::STAGES - 2)));
-      else __builtin_amdgcn_s_waitcnt(0x4f78);                     // vmcnt(24)
+      else __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH));
       asm volatile("" ::: "memory");
       const unsigned char* stage = ring + (step % SH::STAGES) * SH::STAGE;
       u32x4 fa[2], fb[2];
@@ -1974,7 +1978,7 @@ __device__ __forceinline__ void stream_body(const bf16_t* __restrict__ x, const 
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[kk]), as_bf16x8(fb[kk]), acc, 0, 0, 0);
       // the reads above are done (their values were used) before the stage is asked for again
       asm volatile("" ::: "memory");
-      stream_issue<CW, XR, true, true, CH>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
+      stream_issue<CW, XR, true, true, CH, DEPTH>(ring, rs_x, rs_w, voff_x, voff_w, step + SH::STAGES - 1, steps, k_begin);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);                            // the padding loads too, before the ring is reused
     if (S > 1) {
@@ -2010,16 +2014,36 @@ __device__ __forceinline__ void stream_body(const bf16_t* __restrict__ x, const 
   }
 }
 
-template <int EPI, int CW, int XR = 16>
-__global__ __launch_bounds__(256) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                               void* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                               int S) {
-  stream_body<EPI, CW, XR, false>(x, w, out, M, N, K, ldx, ldo, S, launch_ctx());
+template <int EPI, int CW, int XR = 16, int DEPTH = 24>
+__global__ __launch_bounds__(DEPTH == 24 ? 256 : 512) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                                   void* __restrict__ out, int M, int N, int K, int ldx,
+                                                                                   int ldo, int S) {
+  stream_body<EPI, CW, XR, false, DEPTH>(x, w, out, M, N, K, ldx, ldo, S, launch_ctx());
+}
+
+// Five to eight segments of K and no more than 8 rows: a wave a segment, all at once, with shallower rings.
+template <int EPI, int CW>
+static int launch_stream_many(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
+  constexpr int DEPTH = STREAM_DEPTH_MANY(CW);
+  using SH = StreamShape<CW, 8, DEPTH>;
+  const size_t lds_bytes = (size_t)S * SH::RING + (size_t)S * 4 * 64 * sizeof(float);
+  if (S < 5 || S > 8 || lds_bytes > BW_LDS_LIMIT - 256) return -7;
+  static bool allowed = false;                       // more than 64 KB of dynamic LDS has to be asked for once
+  if (!allowed) {
+    (void)hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<EPI, CW, 8, DEPTH>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    allowed = true;
+  }
+  BW_LAUNCH((gemm_bf16_stream_kernel<EPI, CW, 8, DEPTH>), dim3((N + CW - 1) / CW), dim3(64 * S), lds_bytes, s, x, w, out, M, N, K, ldx, ldo, S);
+  return BW_LAUNCH_CHECK();
 }
 
 template <int EPI, int CW, int XR>
 static int launch_stream_rows(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, int S, hipStream_t s) {
   using SH = StreamShape<CW, XR>;
+  if constexpr (XR == 8) {
+    const int rc = launch_stream_many<EPI, CW>(x, w, out, M, N, K, ldx, ldo, S, s);
+    if (rc != -7) return rc;
+  }
   const int waves = S < 4 ? S : 4;
   const size_t lds_bytes = (size_t)waves * SH::RING + (S > 1 ? (size_t)S * 4 * 64 * sizeof(float) : 0);
   if (lds_bytes > 160 * 1024) return -2;
@@ -2508,6 +2532,8 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
         // one segment and few columns: everything asked for at once
         if ((N + 15) / 16 < 256 && K <= 64 * BURST_STEPS) return launch_burst<EPI>(x, w, out, M, N, K, ldx, ldo, s);
+        // (two segments and 256 strips, the 8B shape's output projection: half strips, 512 workgroups of two waves of which
+        // two share a compute unit, were slower: 10.7 us against 9.6)
         if ((N + 15) / 16 < 256) return launch_stream<EPI, 8>(x, w, out, M, N, K, ldx, ldo, S, s);
         return launch_stream<EPI, 16>(x, w, out, M, N, K, ldx, ldo, S, s);
       }

@@ -132,6 +132,8 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
                     (130, 2048, 256), (500, 2100, 128), (65, 1030, 64), (320, 1024, 2048),   # a residual add of one segment: all blocks of 64 rows in one launch
                     (2100, 2100, 128),                                    # more than 256 tiles: four waves a tile
                     (3, 40, 4096), (8, 64, 8192), (70, 80, 4160), (40, 48, 6144), (150, 200, 4096),
+                    (8, 4096, 14336), (5, 2050, 10240), (3, 1000, 16384), (7, 4100, 9280),   # five to eight segments, up to 8 rows: a wave a segment
+                    (8, 4096, 4096), (6, 3000, 2112), (9, 4096, 14336),   # one or two segments: half strips; more than 8 rows with seven segments
                     (129, 96, 6144)]:                                     # several 2048-segments of K
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = torch.randn(N, K, generator=g).bfloat16().to(gpu)
