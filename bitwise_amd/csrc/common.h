@@ -73,6 +73,11 @@ __device__ __forceinline__ float bw_expf(float x) {
 // exp(x) through the hardware exp2; one fixed instruction sequence wherever it is used.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
+// SiLU(g) * u as every bfloat16 kernel computes it: the exponential through the hardware exp2 and the quotient through
+// the hardware reciprocal (the correctly rounded division is ten instructions an element, and the result is
+// rounded to bfloat16 anyway); one fixed instruction sequence wherever it is used, so every route gives the same bits.
+__device__ __forceinline__ float silu_times(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + fast_exp(-g)) * u; }
+
 // Lane exchanges from register to register (no trip through LDS).  The halves and quarters of the wave by gfx950's
 // lane swaps: of (v, v) swapped, the first result holds in every lane the value of its partner or its own in the
 // lower half (32: lanes 0-31; 16: the even rows of 16 lanes), the second the one in the upper half; an operation

@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void decode_gemm_kernel(DecodeGemmArgs a) {
       else if constexpr (EPI == DEPI_ADD_F32) ((float*)a.out)[o] += v;
       else {
         const float uv = acc[NB - 1][q];
-        ((bf16_t*)a.out)[o] = f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * uv);
+        ((bf16_t*)a.out)[o] = f32_to_bf16(silu_times(v, uv));
       }
     }
   } else {

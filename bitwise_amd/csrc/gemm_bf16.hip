@@ -131,7 +131,7 @@ __device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o,
   if constexpr (EPI == EPI_F32) st_f32<DEV>((float*)out + o, v);
   else if constexpr (EPI == EPI_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v));
   else if constexpr (EPI == EPI_ADD_F32) st_f32<DEV>((float*)out + o, ld_f32<DEV>((const float*)out + o) + v);
-  else if constexpr (EPI == EPI_SWIGLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v * (1.0f / (1.0f + fast_exp(-v))) * u));
+  else if constexpr (EPI == EPI_SWIGLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(silu_times(v, u)));
 }
 
 // (host) The phases asked for while a chain is open wait in a list and leave as one launch (further down).
@@ -880,6 +880,36 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
   } else {
+    if constexpr (GLU) {
+      // Whole rows of the tile leave as 16-byte stores: the waves put their outputs into the ring (free now) as the tile
+      // lies in memory, [256 rows][128 columns] with 16 bytes between rows, and the threads then store a row's 256 bytes
+      // sixteen lanes wide.  (Two bytes a lane straight from the accumulators were 64 stores a wave, each of them four
+      // pieces of 32 bytes.)  Outputs that are not 16-byte aligned take the element-wise way below.
+      constexpr int TROW = 128 * 2 + 16;
+      const bool wide = (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (ldo & 7) == 0 && (N & 7) == 0;
+      if (wide) {
+        __syncthreads();                                              // every wave is done with the ring
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            unsigned char* row = big_lds + (128 * wy + 16 * i + 4 * g + q) * TROW + (32 * wx + r) * 2;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              *reinterpret_cast<bf16_t*>(row + 32 * j) = f32_to_bf16(silu_times(acc[i][j][q], acc[i][j + 2][q]));
+          }
+        __syncthreads();
+        const int chunk = threadIdx.x & 15, row0 = threadIdx.x >> 4;
+        const int n = n0 + 8 * chunk;
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) {
+          const int row = row0 + 32 * pass, m = m0 + row;
+          if (m < M && n < N)
+            *reinterpret_cast<u32x4*>((bf16_t*)out + (size_t)m * ldo + n) = *reinterpret_cast<const u32x4*>(big_lds + row * TROW + 16 * chunk);
+        }
+        return;
+      }
+    }
     tile_epilogue<EPI, 8>(acc, out, M, N, ldo, m0 + 128 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g, false, rp);
   }
 }
