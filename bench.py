@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--sweep]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -88,6 +88,10 @@ def main() -> int:
                     help="run nothing but the 128-request shared-prefix trace at Llama-3-8B's sizes and print its figures (for profiles)")
     ap.add_argument("--decode-phases", action="store_true",
                     help="the headline decode with EngineConfig.decode_phases (its products as phases of a few launches; for profiles)")
+    ap.add_argument("--portion-align", type=int, default=64,
+                    help="EngineConfig.portion_align of the headline decode's engine (1: prompts cut exactly at the budget; for profiles)")
+    ap.add_argument("--mixed", action="store_true",
+                    help="only: an 8,192-token prompt beside 7 decoding requests, with portions cut at the budget and cut to whole blocks")
     ap.add_argument("--sweep", action="store_true",
                     help="print a table instead of the line: decode at batches 1 to 128 and contexts of 512 to 8,192 tokens, prefills "
                          "of 128 to 2,048 tokens, at both shapes (with --dtype fp32: a coarser grid at the small shape)")
@@ -106,6 +110,14 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
+    if args.mixed:
+        from bitwise_amd.measure import measure_prefill_beside_decodes
+        cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B, max_position_embeddings=16384)
+        model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+        print(json.dumps({"shape": args.shape, "dtype": args.dtype,
+                          "prompt_beside_decodes": [measure_prefill_beside_decodes(bw, torch, model, cfg, dtype, portion_align=a)
+                                                    for a in (1, 64, 1, 64)]}))
+        return 0
     if args.trace_only:
         big = dict(LLAMA3_8B, max_position_embeddings=16384)
         model8 = bw.Model.random(big, seed=1, dtype=dtype, sigma=0.02, on_device=True)
@@ -127,7 +139,8 @@ def main() -> int:
         print(f"bench.py: --prefill-tokens {args.prefill_tokens} is outside 1..{PREFILL_TOKENS}")
         return 2
     prefill = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[args.dtype], args.prefill_tokens)
-    head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup, decode_phases=args.decode_phases)
+    head = measure_decode(bw, torch, model, cfg, dtype, args.batch, args.steps, args.warmup, decode_phases=args.decode_phases,
+                         portion_align=args.portion_align)
     points, point_rooflines = {}, {}
     extra = {}
     if not args.no_points:

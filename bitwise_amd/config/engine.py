@@ -46,6 +46,9 @@ class EngineConfig:
     decode_phases: bool = False      # captured decode steps of up to 16 rows run their products as phases of a few
                                      # launches that wait for each other inside the kernel (ops.chain): the same
                                      # bits; on MI355X some 5 % slower than a launch each, so off
+    portion_align: int = 64          # a prompt portion that ends before its prompt does ends at a multiple of this many
+                                     # tokens where the budget allows (whole pages and whole 64-key partitions: the
+                                     # kernels' rows of 16 then never straddle a page); 1: cut exactly at the budget
     fault: int = 0                   # a test-only bug (``Fault``) for the simulator to catch; 0: none
 
     def validate(self) -> None:
@@ -55,5 +58,7 @@ class EngineConfig:
             raise ValueError(f"block_size must be a power of two, got {self.block_size}")   # (which ones a model takes: its mixers say)
         if self.num_blocks < 1 or self.max_batched_tokens < 1 or self.max_num_seqs < 1:
             raise ValueError("num_blocks, max_batched_tokens and max_num_seqs must be positive")
+        if self.portion_align < 1:
+            raise ValueError(f"portion_align must be at least 1, got {self.portion_align}")
         if self.fault and self.fault not in Fault.NAMES:
             raise ValueError(f"fault must be 0 or one of {sorted(Fault.NAMES)}, got {self.fault}")

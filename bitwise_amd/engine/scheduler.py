@@ -107,6 +107,30 @@ class Scheduler:
         seq.done = True
 
     # ------------------------------------------------------------------ one step's decisions
+    def _cut(self, s: Sequence, n: int) -> int:
+        """The length of a portion of ``s`` that the budget ends after ``n`` tokens, short of the prompt's end: shortened
+        to end at a multiple of ``portion_align`` tokens, so that the next portion starts with a page (0: the request
+        waits a step, if nothing is left then) -- unless what an exact cut leaves is shorter than that anyway.  Only
+        where every step has room for such a portion whatever else runs (the budget exceeds the running requests'
+        single tokens by ``portion_align`` at least); else the portion is cut at the budget."""
+        a = self.cfg.portion_align
+        if a <= 1 or self.cfg.max_batched_tokens - self.cfg.max_num_seqs < a:
+            return n
+        if len(s.tokens) - s.computed - n < a:
+            return n
+        end = (s.computed + n) // a * a
+        return max(end - s.computed, 0)
+
+    def _in_row_order(self, plan: List[Work]) -> List[Work]:
+        """The step's rows: portions of whole blocks of 16 rows first, then the other portions, longest first, then
+        single tokens, so that a long portion's first row is a multiple of 16 whenever that can be had (the kernels
+        work on blocks of 16 rows, and a block of one request's consecutive tokens that starts with a page is one page)."""
+        def rank(w: Work):
+            if w.n == 1:
+                return (2, 0)
+            return (0, 0) if w.n % 16 == 0 else (1, -w.n)
+        return sorted(plan, key=rank)
+
     def plan(self) -> List[Work]:
         budget = self.cfg.max_batched_tokens
         plan: List[Work] = []
@@ -125,7 +149,9 @@ class Scheduler:
             if n > budget:
                 if budget <= 0:
                     continue                  # a decode row without budget waits for the next step
-                n = budget                    # cut the rest of the prompt to the budget
+                n = self._cut(s, budget)      # cut the rest of the prompt to the budget
+                if n == 0:
+                    continue
             ok = self.manager.ensure(s.cache, s.computed + n)
             while not ok:
                 victim = next((v for v in reversed(self.running) if v is not s and v not in scheduled), None)
@@ -155,7 +181,10 @@ class Scheduler:
             if not any(s.cache.tables):
                 hit = self.manager.admit_prefix(s.cache, s.tokens)
             need = len(s.tokens) - s.computed
-            n = min(need, budget)
+            n = need if need <= budget else self._cut(s, budget)
+            if n == 0 and need > 0:
+                self._drop_cache(s)           # (as below: nothing of this request is held while it waits)
+                break
             if not self.manager.ensure(s.cache, s.computed + n):
                 self._drop_cache(s)           # the prefix hit is retried at the next attempt
                 break
@@ -169,7 +198,7 @@ class Scheduler:
             if n > 0:
                 plan.append(Work(s, n, s.computed))
                 budget -= n
-        return plan
+        return self._in_row_order(plan)
 
     def commit(self, work: Work) -> None:
         """The step ran: ``work.n`` more tokens of the request are in the cache."""

@@ -21,13 +21,14 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return cfg["num_hidden_layers"] * (per_token * tokens + attn) + 2 * h * v      # the head runs for one row
 
 
-def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT, decode_phases: bool = False):
+def make_engine(bw, model, batch: int, steps_total: int, dtype: str, context: int = CONTEXT, decode_phases: bool = False,
+                portion_align: int = 64):
     block = 16
     per_request = context + steps_total + 2 * block
     cfg = bw.EngineConfig(num_blocks=batch * ((per_request + block - 1) // block) + 8, max_batched_tokens=2048,
                           max_num_seqs=max(batch, 1), prefix_caching=False, fingerprint_logits=False,
                           block_size=block, dtype=dtype, max_model_len=max(4096, context + 1024),
-                          decode_phases=decode_phases)
+                          decode_phases=decode_phases, portion_align=portion_align)
     return bw.Engine(model, None, cfg)
 
 
@@ -107,8 +108,42 @@ def measure_chunked_prefill(bw, torch, model, cfg: dict, dtype: str, peak_flops:
             "ms_mean": round(sum(timed) / len(timed), 3), "runs": len(timed)}
 
 
+def measure_prefill_beside_decodes(bw, torch, model, cfg: dict, dtype: str, tokens: int = 8192, decoders: int = 7,
+                                   portion_align: int = 64) -> dict:
+    """One prompt of ``tokens`` tokens arriving while ``decoders`` requests decode (512-token contexts): every step
+    holds the decoders' single tokens and a portion of the prompt under a budget of 2,048 tokens.  The time from the
+    prompt's arrival to its first token: the median of three after an untimed one."""
+    block = 16
+    ecfg = bw.EngineConfig(num_blocks=(tokens + decoders * 1024) // block + 16, max_batched_tokens=2048,
+                           max_num_seqs=decoders + 1, prefix_caching=False, fingerprint_logits=False, block_size=block,
+                           dtype=dtype, max_model_len=tokens + 1024, portion_align=portion_align)
+    engine = bw.Engine(model, None, ecfg)
+    g = torch.Generator().manual_seed(97)
+    for _ in range(decoders):
+        prompt = torch.randint(0, cfg["vocab_size"], (512,), generator=g).tolist()
+        engine.add_request(prompt, bw.SamplingParams(max_new_tokens=400, ignore_eos=True))
+    while engine.num_waiting or any(s.computed < s.prompt_len for s in engine.sched.running):
+        engine.step()
+    times, steps = [], 0
+    for _ in range(4):
+        prompt = torch.randint(0, cfg["vocab_size"], (tokens,), generator=g).tolist()
+        rid = engine.add_request(prompt, bw.SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = 0
+        while not engine.result(rid).finished:
+            engine.step()
+            steps += 1
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    assert len(engine.sched.running) == decoders, "a decoding request finished inside the measurement"
+    timed = sorted(times[1:])
+    return {"tokens": tokens, "decoders": decoders, "portion_align": portion_align, "steps": steps, "ms": round(timed[1], 3),
+            "ms_best": round(timed[0], 3), "prompt_tok_s": round(tokens / timed[1] * 1e3, 1)}
+
+
 def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
-                   context: int = CONTEXT, decode_phases: bool = False) -> dict:
+                   context: int = CONTEXT, decode_phases: bool = False, portion_align: int = 64) -> dict:
     """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
     said otherwise): tokens a second, and the bytes a step has to read (every weight once, the cache of the live
     requests) over its time."""
@@ -116,9 +151,11 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     # Requests admitted early decode while the later ones are still being prefilled (2,048 prompt
     # tokens a step): every request gets enough new tokens to outlast the prefills, the warm-up and the
     # timed steps, so that each timed step has all ``batch`` rows.
-    chunks = (context + 2047) // 2048                  # steps a prompt takes under the 2,048-token budget
-    new_tokens = steps + warmup + batch * chunks + 8
-    eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases)
+    # (a step of the fill holds at least 2,048 tokens less the decoded ones and less what a cut gives up to end on
+    # a whole block)
+    fill_steps = -(-batch * context // (2048 - batch - 64)) + 1
+    new_tokens = steps + warmup + fill_steps + 8
+    eng = make_engine(bw, model, batch, new_tokens, dtype, context, decode_phases, portion_align)
     fill(eng, bw, torch, batch, cfg["vocab_size"], new_tokens, seed=batch, context=context)
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)
@@ -128,7 +165,7 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     ms = secs / steps * 1e3
     # keys a decoded token reads, on average: the prompt, what the request decoded while later
     # prompts were prefilled, the warm-up, and half the timed steps
-    avg_ctx = context + chunks * (batch - 1) / 2 + warmup + (steps + 1) / 2
+    avg_ctx = context + batch * context / 2048 * (batch - 1) / (2 * batch) + warmup + (steps + 1) / 2
     step_bytes = model.weight_bytes + batch * avg_ctx * kv_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
     return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),

@@ -46,7 +46,7 @@ class Scenario:
         e = self.engine
         return (f"scenario {self.seed} [{self.kind}] {len(self.arrivals)} requests; page {e.block_size}, pool {e.num_blocks}, "
                 f"budget {e.max_batched_tokens}, seqs {e.max_num_seqs}, len {e.max_model_len}, graphs {e.use_graphs}, "
-                f"ahead {e.run_ahead}, prefix cache {e.prefix_caching}, decode phases {e.decode_phases}")
+                f"ahead {e.run_ahead}, prefix cache {e.prefix_caching}, decode phases {e.decode_phases}, portions to {e.portion_align}")
 
 
 @dataclass
@@ -172,13 +172,14 @@ class Simulator:
         cfg = EngineConfig(num_blocks=pool, max_batched_tokens=budget, max_num_seqs=seqs, prefix_caching=rng.random() < 0.7,
                            block_size=page, dtype=self.dtype, max_model_len=model_len, use_graphs=rng.random() < 0.7,
                            run_ahead=rng.random() < 0.7, fault=self.fault)
-        cfg.decode_phases = rng.random() < 0.3          # (the last draw: the scenarios of a seed are what they were without it)
+        cfg.decode_phases = rng.random() < 0.3          # (the last draws: the scenarios of a seed are what they were without them)
+        cfg.portion_align = rng.choice((1, 4, 16, 64))
         return Scenario(seed, kind, cfg, arrivals)
 
     # ------------------------------------------------------------------ running one
     def run_scenario(self, sc: Scenario, tally: Tally) -> None:
         tally.scenarios += 1
-        for name in ("block_size", "use_graphs", "run_ahead", "prefix_caching", "decode_phases"):
+        for name in ("block_size", "use_graphs", "run_ahead", "prefix_caching", "decode_phases", "portion_align"):
             tally.knobs_seen.setdefault(name, set()).add(getattr(sc.engine, name))
         tally.knobs_seen.setdefault("kind", set()).add(sc.kind)
         try:
