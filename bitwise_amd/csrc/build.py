@@ -24,7 +24,8 @@ from typing import List, Optional
 HERE = Path(__file__).resolve().parent
 SOURCES = ["elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "attention_bf16.hip",
            "fused_decode.hip", "sampling.hip"]
-HEADERS = ["common.h", "api.h", "layout.h"]
+HEADERS = ["common.h", "api.h", "layout.h", "gemm_bf16_skinny.h", "gemm_bf16_tiles.h", "gemm_bf16_rows.h",
+           "gemm_bf16_phases.h"]
 LIB_NAME = "libbitwise_hip.so"
 # -ffp-contract=off: a multiply-add is fused only where the source says fmaf.  Packed 32-bit
 # float instructions are switched off for the device pass.
