@@ -111,12 +111,13 @@ def main() -> int:
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
     if args.mixed:
-        from bitwise_amd.measure import measure_prefill_beside_decodes
+        from bitwise_amd.measure import measure_prefill_beside_decodes, measure_qkv_row_orders
         cfg = dict(SMOLLM2_1_7B if args.shape == "smollm2" else LLAMA3_8B, max_position_embeddings=16384)
         model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
         print(json.dumps({"shape": args.shape, "dtype": args.dtype,
                           "prompt_beside_decodes": [measure_prefill_beside_decodes(bw, torch, model, cfg, dtype, portion_align=a)
-                                                    for a in (1, 64, 1, 64)]}))
+                                                    for a in (1, 64, 1, 64)],
+                          "qkv_us_by_row_order": measure_qkv_row_orders(torch, cfg) if args.dtype == "bf16" else {}}))
         return 0
     if args.trace_only:
         big = dict(LLAMA3_8B, max_position_embeddings=16384)

@@ -142,6 +142,52 @@ def measure_prefill_beside_decodes(bw, torch, model, cfg: dict, dtype: str, toke
             "ms_best": round(timed[0], 3), "prompt_tok_s": round(tokens / timed[1] * 1e3, 1)}
 
 
+def measure_qkv_row_orders(torch, cfg: dict, calls: int = 30) -> dict:
+    """The q|k|v product with rotation and cache write in its epilogue, called alone on about 2,048 rows composed in
+    different ways (one request; portions of two requests and decoded tokens of others, behind or in front): microseconds
+    a call.  Heads of 64 only (other sizes rotate in a kernel of their own)."""
+    from bitwise_amd.csrc import ops
+    dev = torch.device("cuda:0")
+    heads, kvh, hd, K, ps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["hidden_size"], 16
+    if hd != 64:
+        return {}
+    N, pool = (heads + 2 * kvh) * hd, 1100
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16().to(dev)
+    kc = torch.zeros(pool, kvh, ps, hd, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros(pool, kvh, hd, ps, dtype=torch.bfloat16, device=dev)
+    ang = torch.arange(4096, dtype=torch.float64)[:, None] * (cfg["rope_theta"] ** (-torch.arange(0, hd, 2, dtype=torch.float64) / hd))[None, :]
+    cos, sin = ang.cos().float().to(dev), ang.sin().float().to(dev)
+    out = {}
+
+    def case(name, segs):                       # segs: (request, first position, rows)
+        M = sum(n for _, _, n in segs)
+        nseq = max(s for s, _, _ in segs) + 1
+        pos = torch.cat([torch.arange(p0, p0 + n, dtype=torch.int32) for _, p0, n in segs]).to(dev)
+        rs = torch.cat([torch.full((n,), s, dtype=torch.int32) for s, _, n in segs]).to(dev)
+        table = torch.zeros(nseq, 264, dtype=torch.int32)
+        for s in range(nseq):
+            table[s, :130] = torch.arange(130 * s, 130 * s + 130, dtype=torch.int32)
+        table = table.to(dev)
+        x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+        q = torch.zeros(M, heads * hd, dtype=torch.bfloat16, device=dev)
+        for i in range(calls + 5):
+            if i == 5:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            ops.gemm_qkv_rope_bf16(x, w, q, pos, rs, table, cos, sin, kc, vc, M, heads, kvh, hd, ps)
+        torch.cuda.synchronize()
+        out[name] = round((time.perf_counter() - t0) / calls * 1e6, 1)
+
+    decoded = [(2 + i, 2048, 1) for i in range(5)]
+    case("one request, positions 0..2047", [(0, 0, 2048)])
+    case("64 rows of one request, 1920 of another, 5 decoded tokens", [(0, 1984, 64), (1, 0, 1920)] + decoded)
+    case("the 5 decoded tokens in front", decoded + [(0, 1984, 64), (1, 0, 1920)])
+    case("1 decoded token in front of 2047 rows of a request", [(1, 2048, 1), (0, 0, 2047)])
+    case("2047 rows of a request, then 1 decoded token", [(0, 0, 2047), (1, 2048, 1)])
+    return out
+
+
 def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: int, warmup: int,
                    context: int = CONTEXT, decode_phases: bool = False, portion_align: int = 64) -> dict:
     """``steps`` decode steps of ``batch`` requests that each hold a context of ``context`` tokens (2,048 unless
