@@ -24,7 +24,12 @@ class Segment:
 
 
 class StepContext:
-    """Device arrays of one step.  Rows of a request are contiguous and in position order.
+    """Device arrays of one step.  Rows of a request are contiguous and in position order.  The requests' rows lie
+    in an order of the step's own (``segments`` and every per-request array follow it): portions of whole blocks of 16
+    rows first, then the other portions, the longest first, then single tokens.  The kernels work on blocks of 16
+    rows, and a block that is 16 consecutive tokens of one request from a page's first slot on is one page: a single
+    token in front of a long portion would shift every block of it across two pages.  The wanted rows keep the
+    order in which the caller gave the requests and their ``want``.
 
     ``ws``: the workspace of the engine that runs the step (scratch buffers, page size, limits).
     ``calls``: the model's layer calls bound to that engine's caches and state.  ``num_pages``:
@@ -35,7 +40,13 @@ class StepContext:
 
     def __init__(self, segments: Sequence[Segment], num_groups: int, ws, calls: Sequence[Any] = (),
                  num_pages: Optional[int] = None):
-        self.segments = list(segments)
+        given = list(segments)
+
+        def rank(i: int):
+            n = len(given[i].tokens)
+            return (2, 0, i) if n == 1 else ((0, 0, i) if n % 16 == 0 else (1, -n, i))
+        order = sorted(range(len(given)), key=rank)
+        self.segments = [given[i] for i in order]
         self.ws = ws
         self.calls = list(calls)
         self.device = device = ws.device
@@ -46,7 +57,6 @@ class StepContext:
         tokens = np.empty(rows, np.int32)
         positions = np.empty(rows, np.int32)
         row_seq = np.empty(rows, np.int32)
-        want: List[int] = []
         self.seq_start: List[int] = []
         r = 0
         for i, s in enumerate(self.segments):
@@ -55,8 +65,9 @@ class StepContext:
             tokens[r:r + n] = s.tokens
             positions[r:r + n] = np.arange(s.pos0, s.pos0 + n, dtype=np.int32)
             row_seq[r:r + n] = i
-            want.extend(r + w for w in s.want)
             r += n
+        first_row = {g: self.seq_start[k] for k, g in enumerate(order)}
+        want: List[int] = [first_row[g] + w for g, s in enumerate(given) for w in s.want]
         self.num_wanted = len(want)
         widths = [max((len(s.tables[g]) for s in self.segments), default=1) or 1 for g in range(num_groups)]
         tables = []

@@ -121,16 +121,6 @@ class Scheduler:
         end = (s.computed + n) // a * a
         return max(end - s.computed, 0)
 
-    def _in_row_order(self, plan: List[Work]) -> List[Work]:
-        """The step's rows: portions of whole blocks of 16 rows first, then the other portions, longest first, then
-        single tokens, so that a long portion's first row is a multiple of 16 whenever that can be had (the kernels
-        work on blocks of 16 rows, and a block of one request's consecutive tokens that starts with a page is one page)."""
-        def rank(w: Work):
-            if w.n == 1:
-                return (2, 0)
-            return (0, 0) if w.n % 16 == 0 else (1, -w.n)
-        return sorted(plan, key=rank)
-
     def plan(self) -> List[Work]:
         budget = self.cfg.max_batched_tokens
         plan: List[Work] = []
@@ -198,7 +188,7 @@ class Scheduler:
             if n > 0:
                 plan.append(Work(s, n, s.computed))
                 budget -= n
-        return self._in_row_order(plan)
+        return plan
 
     def commit(self, work: Work) -> None:
         """The step ran: ``work.n`` more tokens of the request are in the cache."""

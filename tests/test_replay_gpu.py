@@ -267,6 +267,42 @@ def test_first_tokens_of_a_sequence(folders):
             check_against_plain(one["a"], ref, dtype, f"first tokens {name}", median=True)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_order_of_a_steps_entries_changes_nothing(folders, dtype):
+    """A step lays its requests' rows out in an order of its own (portions of whole blocks of 16 rows, other portions,
+    single tokens); the wanted logits come back in the caller's order, and in any order of the entries they are the
+    same bits."""
+    from bitwise_amd.engine.batch import Segment, StepContext
+    from bitwise_amd.replay import Replayer
+    name = "B"
+    cfg = tiny.read_config(folders[name])
+    reqs = requests_for(cfg, 21, [40, 35, 32, 9])
+    first = [{"id": "r0", "tokens": reqs["r0"][:39], "want": []}, {"id": "r3", "tokens": reqs["r3"][:8], "want": []}]
+    second = [{"id": "r0", "tokens": reqs["r0"][39:], "want": [0]}, {"id": "r1", "tokens": reqs["r1"], "want": [0, 34]},
+              {"id": "r3", "tokens": reqs["r3"][8:], "want": [0]}, {"id": "r2", "tokens": reqs["r2"], "want": [31, 5]}]
+    got = []
+    for entries in (second, second[::-1], [second[1], second[3], second[0], second[2]]):
+        rp = Replayer(str(folders[name]), dtype, 256, block_size=tiny.CONFIGS[name][3])
+        rp.step(first)
+        lg = rp.step(entries)
+        rows, row = {}, 0
+        for e in entries:
+            for w in e["want"]:
+                rows[(e["id"], w)] = lg[row]
+                row += 1
+        got.append(rows)
+    for other in got[1:]:
+        assert got[0].keys() == other.keys() and all(np.array_equal(got[0][k], other[k]) for k in got[0])
+    ref = plain_logits(folders[name], reqs["r1"], dtype)
+    check_against_plain(np.stack([got[0][("r1", 0)], got[0][("r1", 34)]]), ref[[0, 34]], dtype, "a portion between single tokens")
+    # the layout itself
+    ctx = StepContext([Segment([1], 39, [[0, 1, 2, 3, 4]], 0, [0]), Segment([2] * 35, 0, [[5, 6, 7, 8, 9]], 1, [0, 34]),
+                       Segment([3] * 32, 0, [[10, 11, 12, 13]], 2, [31, 5])], 1, rp.runner.ws)
+    assert [len(sg.tokens) for sg in ctx.segments] == [32, 35, 1] and ctx.seq_start == [0, 32, 67]
+    assert ctx.want_rows.tolist() == [67, 32, 66, 31, 5] and ctx.slots.tolist() == [2, 1, 0]
+    assert ctx.row_seq.tolist() == [0] * 32 + [1] * 35 + [2]
+
+
 def test_trace_run_program(folders, tmp_path):
     """bin/trace_run as a user calls it: JSON steps on standard input, <step>.f32 files, a
     'done <step>' line after every step, exit 0; a request may pause and pages are reused."""
