@@ -341,6 +341,10 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
       // for 128 rows and 2048 columns, whatever is idle): the kernel for up to 64 rows, a workgroup per block of 64 rows,
       // 64 or 32 columns and segment of K, all blocks in one launch.
       if ((size_t)M * ldx * 2 < ((size_t)1 << 31)) {
+        // (one segment, and blocks of 32 rows by 32 columns still fit the chip at once: as for 33 to 64 rows above)
+        if (S == 1 && K % 64 == 0 && ((N + 31) / 32) * ((M + 31) / 32) <= 256 && ((N + 31) / 32) * ((M + 31) / 32) >= 32)
+          return launch_mid<EPI, 2, false, true>(x, w, out, M, N, K, ldx, ldo, (N + 31) / 32, s, MidNormArgs{}, QkvRopeArgs{}, 1,
+                                                 MidSplitArgs{}, (M + 31) / 32);
         int tiles, zb;
         bool narrow;
         add_blocks_shape(M, N, K, tiles, narrow, zb);
