@@ -1013,9 +1013,14 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
 
 #define DECODE_W 8
 #define BW_LDS_BYTES (160 * 1024 - 256)   // a compute unit's LDS less the kernels' few static words
-#define DECODE_W_MANY 4          // waves a workgroup where there are several workgroups for every compute unit
-#define DECODE_MANY 1024          // that many workgroups: a workgroup's last, partly empty round of partitions costs more
-                                  // than what a compute unit gains from eight waves' loads in flight
+#define DECODE_W_MANY 4          // waves a workgroup where there are two workgroups or more for every compute unit: two of
+                                 // these share a compute unit, and a token's first keys do not wait for a whole
+                                 // generation of eight-wave workgroups before it (16 requests of 32 heads: 2.61 -> 2.52 ms
+                                 // a step at 2,048-token contexts, 1.76 -> 1.69 at 512)
+#define DECODE_MANY 257          // that many workgroups: more than there are compute units
+#define DECODE_MANY_LONG 1024    // heads of 128 or more in a cache laid out for long contexts (more than 80 partitions a
+                                 // request): eight waves' loads in flight are worth more there up to this many (64
+                                 // requests of 8 heads of 128 at 8,192 tokens: 16.3 ms a step against 16.5)
 
 // How a decode launch over ``num_tiles`` tiles is split: workgroups per tile (1 = no split) and
 // the partitions a tile's scratch must hold.  Depends on nothing that changes from step to step.
@@ -1046,7 +1051,7 @@ static int launch_attention(const AttnBf16Args& a, int decode, float* scratch, s
     int nsplit, max_parts;
     decode_split_shape(a.num_tiles, items, a.table_stride, a.page_size, nsplit, max_parts);
     if (scratch == nullptr || counters == nullptr) nsplit = 1;
-    bool few_waves = nsplit == 1 && a.num_tiles * items >= DECODE_MANY;
+    bool few_waves = nsplit == 1 && a.num_tiles * items >= ((HD >= 128 && max_parts > 80) ? DECODE_MANY_LONG : DECODE_MANY);
     if (lds_bytes > BW_LDS_BYTES) {                // sixteen heads of 256 a workgroup: only four waves' partials fit
       few_waves = true;
       nsplit = 1;
