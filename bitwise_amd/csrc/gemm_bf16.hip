@@ -433,14 +433,15 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         return BW_LAUNCH_CHECK();
       }
     }
-    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16) {
+    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16 || EPI == EPI_QKV_ROPE) {
       // 128 x 256 tiles where they go round the compute units (the 256 x 256 kernel above took what it takes: one
-      // segment of K and enough of its tiles)
+      // segment of K and enough of its tiles); the q|k|v product of 600 to 1,200 rows among them (four heads of 64 a
+      // tile, a head a wave as in the 128 x 128 tiles: 1,024 rows 45.8 us there)
       constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
       const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
       // (in rounds of 256 workgroups; a step of these takes 1.0 us where a 128 x 128 tile's takes 0.58)
       const int rounds256 = (mt * nt + 255) / 256, rounds128 = (mt * ((N + COLS256 / 2 - 1) / (COLS256 / 2)) + 255) / 256;
-      if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) return launch_tile256<EPI>(x, w, out, M, N, K, ldx, ldo, s);
+      if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) return launch_tile256<EPI>(x, w, out, M, N, K, ldx, ldo, s, rp);
     }
     constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;

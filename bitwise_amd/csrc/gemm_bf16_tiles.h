@@ -807,7 +807,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // a step pulls 48 KB for twice the 128 x 128 tile's products (which pulls 32), and a wave's 64 accumulators leave room
 // for the sums of the segments before, so that a K of several segments, which the 256 x 256 kernel does not take,
 // runs on these where there are enough of them.  Three stages of 48 KB (x 16 KB | W 32 KB); a wave issues six loads a
-// stage.  Plain, residual and SwiGLU epilogues; segments joined left to right in registers (a residual add's chain
+// stage.  Plain, residual, SwiGLU and (one segment, heads of 64) rotary epilogues; segments joined left to right in registers (a residual add's chain
 // starts at the residual, which is read when the first segment ends).  K a multiple of 64.
 #define T256_STAGE (48 * 1024)
 #define T256_STAGES 3
@@ -815,8 +815,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile256_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles) {
-  static_assert(EPI != EPI_QKV_ROPE, "plain, residual and SwiGLU epilogues");
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char t256_lds[];   // [3 stages][x 16 KB | W 32 KB]
@@ -941,11 +940,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   // (a residual add of several segments has the residual in its sums; of one segment the epilogue adds it)
   tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (GLU ? 32 : 64) * wx, (n0 >> 6) + wx, r, g,
-                        EPI == EPI_ADD_F32 && K > GEMM_SEG, QkvRopeArgs{});
+                        EPI == EPI_ADD_F32 && K > GEMM_SEG, rp);
 }
 
 template <int EPI>
-static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s) {
+static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s,
+                          const QkvRopeArgs& rp = QkvRopeArgs{}) {
   constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
   const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
   static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
@@ -955,6 +955,6 @@ static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, in
     allowed = true;
   }
   BW_LAUNCH((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
-                     ldo, mt, nt);
+                     ldo, mt, nt, rp);
   return BW_LAUNCH_CHECK();
 }

@@ -888,6 +888,7 @@ def test_prompt_qkv_product_with_rotary_epilogue_equals_the_separate_kernels(gpu
     for case in [(3, 1, 256, 130, 16), (4, 4, 128, 200, 8), (5, 2, 320, 97, 32),
                                    (5, 2, 96, 150, 16), (2, 2, 40, 190, 8),   # K no multiple of 64: tiles through registers
                                    (40, 10, 128, 2100, 32),        # enough 256 x 256 tiles for the big-tile kernel
+                                   (40, 28, 128, 1000, 16), (41, 28, 192, 777, 8),   # 128 x 256 tiles (a ragged last one)
                                    (40, 12, 128, 64, 16), (44, 10, 192, 23, 8), (64, 8, 64, 9, 16),   # up to 64 rows, half a head a workgroup
                                    (200, 28, 64, 40, 16), (208, 24, 64, 12, 8), (230, 13, 128, 64, 32),   # a head a workgroup
                                    (40, 12, 128, 130, 16), (72, 12, 192, 300, 16), (64, 16, 2048, 190, 32),   # blocks of 64 rows in one launch
