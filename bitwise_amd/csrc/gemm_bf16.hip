@@ -202,7 +202,7 @@ static void add_rows_shape(int M, int N, int K, int& tiles, bool& narrow) {
 // a 256 x 256 tile counts twice); the join moves 8 bytes an element and segment (about 500,000 elements in the
 // time of a step) and is a launch more (8 steps); a split has to win by a tenth.  tiles64: what the 64-row
 // kernel's scratch is sized by.
-enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT, ADD_TILE256 };
+enum AddRoute { ADD_WHOLE, ADD_ROW_BLOCKS, ADD_TILE_SPLIT, ADD_BIG_SPLIT, ADD_TILE256, ADD_TILE256_SPLIT };
 
 // "Blocks at once" for a residual add of more than 64 rows: how many blocks of 64 rows, tiles of 64 or (narrow) 32
 // columns; tiles 0: it does not run that way (more than 512 workgroups, or too few to matter).  Several segments of K
@@ -235,13 +235,17 @@ static AddRoute add_route(int M, int N, int K, int ldo, int& tiles64) {
   const long long whole = ((t128 + 255) / 256) * (K / 64);
   const long long tile_split = ((t128 * S + 255) / 256) * (GEMM_SEG / 64) + join;
   const long long big_split = M >= 2 * BIG_BM ? ((tbig * S + 255) / 256) * 2 * (GEMM_SEG / 64) + join : whole;
-  const long long split = tile_split <= big_split ? tile_split : big_split;
-  // 128 x 256 tiles with all of K, the segments joined in registers: no scratch, no join; a step of theirs takes
-  // 1.0 us (1.6 of the 128 x 128 tile's)
+  // 128 x 256 tiles: a step of theirs takes 1.0 us (1.6 to 1.75 of the 128 x 128 tile's).  With all of K, the
+  // segments joined in registers: no scratch, no join.  A workgroup per tile and segment: where that is one round of
+  // the chip and 128 x 128 tiles would be two (1,024 rows of K = 8192 into 2048 columns).
   const long long t256 = (long long)((M + 127) / 128) * ((N + 255) / 256);
   const long long whole256 = ((t256 + 255) / 256) * (K / 64) * 8 / 5;
+  const long long t256_split = ((t256 * S + 255) / 256) * (GEMM_SEG / 64) * 7 / 4 + join;
+  const long long split3 = tile_split <= big_split ? tile_split : big_split;
+  const long long split = t256_split < split3 ? t256_split : split3;
   if (whole256 < whole && whole256 <= split) return ADD_TILE256;
   if (10 * split >= 9 * whole) return ADD_WHOLE;
+  if (t256_split < split3) return ADD_TILE256_SPLIT;
   return tile_split <= big_split ? ADD_TILE_SPLIT : ADD_BIG_SPLIT;
 }
 
@@ -386,6 +390,15 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                            M, N, ldo);
         return BW_LAUNCH_CHECK();
       }
+      if (route == ADD_TILE256_SPLIT && sp.scratch != nullptr && ((uintptr_t)out & 15) == 0) {
+        if (scratch_floats < (size_t)S * M * N) return -6;
+        const int rc = launch_tile256<EPI_F32>(x, w, (void*)sp.scratch, M, N, K, ldx, N, s, QkvRopeArgs{}, S, (size_t)M * N);
+        if (rc) return rc;
+        const size_t quads = (size_t)M * (N >> 2);
+        BW_LAUNCH(add_segments_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, (float*)out, sp.scratch, S,
+                           M, N, ldo);
+        return BW_LAUNCH_CHECK();
+      }
       if (route == ADD_TILE_SPLIT && sp.scratch != nullptr && ((uintptr_t)out & 15) == 0) {
         if (scratch_floats < (size_t)S * M * N) return -6;
         const int mt = (M + 127) / 128, nt = (N + 127) / 128;
@@ -486,7 +499,7 @@ extern "C" int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_float
     }
   }
   const AddRoute route = M > 64 && N > 0 ? add_route(M, N, K, 4, tiles) : ADD_WHOLE;
-  if (route == ADD_TILE_SPLIT || route == ADD_BIG_SPLIT) {      // a prompt portion: the segments' sums, whole
+  if (route == ADD_TILE_SPLIT || route == ADD_BIG_SPLIT || route == ADD_TILE256_SPLIT) {      // a prompt portion: the segments' sums, whole
     *scratch_floats = (long long)S * M * N;
     *counters = 1;                                          // (none is used)
     return 0;

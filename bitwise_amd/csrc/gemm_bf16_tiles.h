@@ -815,10 +815,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile256_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
-    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
+    int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
   constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char t256_lds[];   // [3 stages][x 16 KB | W 32 KB]
+  // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
+  // elements (a residual add's segments, joined in order by add_segments_kernel afterwards)
+  const int k_base = (int)blockIdx.y * GEMM_SEG, k_all = K;
+  if (gridDim.y > 1) {
+    out = (void*)((float*)out + (size_t)blockIdx.y * seg_stride);
+    K = min(GEMM_SEG, K - k_base);
+  }
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
   const int wy = wave >> 2, wx = wave & 3;
@@ -831,10 +838,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // (SwiGLU: W rows 0-127 of the tile are gate rows n0.., 128-255 the up rows N + n0..)
   const int a_rows = min(128, M - m0), b_rows = min(COLS, N - n0);
   const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + K) * 2), 0x00020000);
+      (void*)(x + (size_t)m0 * ldx), 0, (int)((((size_t)a_rows - 1) * ldx + k_all) * 2), 0x00020000);
   const bool up = GLU && wave >= 4;
   const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(w + ((size_t)(up ? N : 0) + n0) * K), 0, (int)((size_t)b_rows * K * 2), 0x00020000);
+      (void*)(w + ((size_t)(up ? N : 0) + n0) * k_all), 0, (int)((size_t)b_rows * k_all * 2), 0x00020000);
   const int b_row0 = GLU ? 32 * (wave & 3) : 32 * wave;
   const int lrow = lane >> 3, lslot = lane & 7;
   int voff_a[2], voff_b[4];
@@ -843,7 +850,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int r16 = (8 * t + lrow) & 15;                    // the row within its block of 16
     const int chunk = lslot ^ (r16 >> 1);
     if (t < 2) voff_a[t] = ((16 * wave + 8 * t + lrow) * ldx + 8 * chunk) * 2;
-    voff_b[t] = ((b_row0 + 8 * t + lrow) * K + 8 * chunk) * 2;
+    voff_b[t] = ((b_row0 + 8 * t + lrow) * k_all + 8 * chunk) * 2;
   }
   typedef __attribute__((address_space(3))) void* lds_ptr;
   const int steps = K / 64;
@@ -853,11 +860,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int t = 0; t < 2; ++t)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(dst + (2 * wave + t) * 1024), 16, real ? voff_a[t] : 0x7ffffff0,
-                                               step * 128, 0, 0);
+                                               k_base * 2 + step * 128, 0, 0);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lds_ptr)(dst + 16 * 1024 + (4 * wave + t) * 1024), 16,
-                                               real ? voff_b[t] : 0x7ffffff0, step * 128, 0, 0);
+                                               real ? voff_b[t] : 0x7ffffff0, k_base * 2 + step * 128, 0, 0);
   };
   f32x4 acc[4][4], tot[4][4];
 #pragma unroll
@@ -945,7 +952,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <int EPI>
 static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s,
-                          const QkvRopeArgs& rp = QkvRopeArgs{}) {
+                          const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1, size_t seg_stride = 0) {
   constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
   const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
   static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
@@ -954,7 +961,7 @@ static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, in
                               T256_STAGES * T256_STAGE);
     allowed = true;
   }
-  BW_LAUNCH((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
-                     ldo, mt, nt, rp);
+  BW_LAUNCH((gemm_bf16_tile256_kernel<EPI>), dim3(mt * nt, segments), dim3(512), T256_STAGES * T256_STAGE, s, x, w, out, M, N, K, ldx,
+                     ldo, mt, nt, rp, seg_stride);
   return BW_LAUNCH_CHECK();
 }

@@ -197,7 +197,7 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
             assert torch.equal(got, want) and not scratch[1].any(), (M, N, K)
     # a residual add of more than 64 rows whose 128 x 128 tiles with all of K would leave compute units idle: up to
     # 128 rows and three segments in blocks of 64 rows through that kernel (its scratch if K has several segments);
-    # else a workgroup per tile (128 x 128, or 256 x 256 from 512 rows) and segment, the segments' sums whole in
+    # else a workgroup per tile (128 x 128, 128 x 256, or 256 x 256 from 512 rows) and segment, the segments' sums whole in
     # scratch and joined in order afterwards; or 128 x 256 tiles with all of K where those go round the compute units
     # once (no scratch).  The bits of the rows alone, 16 at a time, with and without scratch,
     # twice on the same scratch (full of NaN at first, larger than needed); ragged edges, a short last segment
@@ -210,6 +210,8 @@ def test_gemm_bf16_rows_shapes_and_epilogues(gpu):
                           (65, 2048, 8192, "at once"), (145, 2048, 8192, "at once"), (300, 1000, 2 * 2048 + 192, "at once"),
                           (256, 2048, 8192, "at once"), (320, 2048, 8192, "sums"),
                           (768, 2048, 8192, "sums"), (700, 3000, 4 * 2048 + 128, "sums"), (2048, 2048, 8192, "sums"),
+                          (1000, 2000, 8128, "sums"),     # 128 x 256 tiles, a workgroup per tile and segment
+
                           (513, 8192, 4096, "sums")]:
         x = torch.randn(M, K, generator=g).bfloat16().to(gpu)
         w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(gpu)
